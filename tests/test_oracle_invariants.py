@@ -1,0 +1,320 @@
+"""Pins what the reference's literal vectors leave open: closed forms, the
+reference tests' own invariants, and brute-force fp64 numpy on tiny shapes.
+Each check is chosen so that a dropped term, a wrong sign/index or a
+transposed operand fails it."""
+import numpy as np
+import pytest
+
+from oracle import cpu_ref as ref
+
+
+def rnd(rows, cols, seed):
+    return ref.random_tensor(rows, cols, seed)
+
+
+def close(a, b, atol=1e-5, rtol=1e-5):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    assert a.shape == b.shape
+    assert np.all(np.abs(a - b) <= atol + rtol * np.abs(b)), float(np.max(np.abs(a - b)))
+
+
+# ── primitives against fp64 numpy (non-square shapes catch transposes) ───────
+
+def test_primitives_match_numpy_fp64():
+    a, b = rnd(7, 13, 1), rnd(13, 5, 2)
+    close(ref.matmul(a, b), a.astype(np.float64) @ b.astype(np.float64))
+    x = rnd(6, 11, 3)
+    close(ref.softmax_rows(x), np.exp(x - x.max(1, keepdims=True)) / np.exp(x - x.max(1, keepdims=True)).sum(1, keepdims=True))
+    close(ref.mean_along_rows(x), x.astype(np.float64).mean(1, keepdims=True))
+    close(ref.variance_along_rows(x), x.astype(np.float64).var(1, keepdims=True))
+    close(ref.max_along_rows(x), x.max(1, keepdims=True))
+    close(ref.sum_rows(x), x.astype(np.float64).sum(0, keepdims=True))
+    close(ref.sigmoid(x), 1 / (1 + np.exp(-x.astype(np.float64))))
+    close(ref.tanh(x), np.tanh(x.astype(np.float64)))
+    close(ref.exp(x), np.exp(x.astype(np.float64)))
+    close(ref.log(np.abs(x) + 0.5), np.log(np.abs(x.astype(np.float64)) + 0.5))
+    x64 = x.astype(np.float64)
+    close(ref.gelu(x), 0.5 * x64 * (1 + np.tanh(np.sqrt(2 / np.pi) * (x64 + 0.044715 * x64 ** 3))))
+    # gelu backward against a central finite difference of gelu (ActivationsTest.java:126-141)
+    h = 1e-3
+    fd = (ref.gelu(x + np.float32(h)).astype(np.float64) - ref.gelu(x - np.float32(h))) / (2 * h)
+    close(ref.gelu_backward(x, np.ones_like(x)), fd, atol=2e-3)
+
+
+def test_softmax_rows_sum_to_one_and_backward():
+    # ActivationsTest.java:72-85
+    p = ref.softmax_rows([[1, 2, 3], [-1, 0, 1]])
+    close(p.sum(1), [1.0, 1.0], atol=1e-6)
+    g, s = rnd(4, 9, 10), ref.softmax_rows(rnd(4, 9, 11))
+    s64, g64 = s.astype(np.float64), g.astype(np.float64)
+    close(ref.softmax_backward(g, s), s64 * (g64 - (g64 * s64).sum(1, keepdims=True)))
+
+
+def test_cross_entropy_loss_closed_form():
+    logits = rnd(5, 9, 20)
+    t = ref.JavaRandom(21).ints(5, 9)
+    l64 = logits.astype(np.float64)
+    lse = np.log(np.exp(l64 - l64.max(1, keepdims=True)).sum(1)) + l64.max(1)
+    close(ref.cross_entropy_loss(logits, t), np.mean(lse - l64[np.arange(5), t]))
+    g = ref.cross_entropy_gradient(logits, t)
+    close(g.sum(1), np.zeros(5), atol=1e-6)        # LossTest.java:37-53
+
+
+def test_adamw_and_layernorm_backward_closed_form():
+    w, g = rnd(3, 5, 30), rnd(3, 5, 31)
+    mt, vt = np.zeros_like(w), np.zeros_like(w)
+    w0 = w.copy()
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 0.01
+    ref.adamw_update(w, g, mt, vt, lr, b1, b2, eps, wd, 1 - b1, 1 - b2)
+    g64 = g.astype(np.float64)
+    m = (1 - b1) * g64; v = (1 - b2) * g64 ** 2
+    exp_w = w0 - (lr * (m / (1 - b1)) / (np.sqrt(v / (1 - b2)) + eps) + lr * wd * w0)
+    close(w, exp_w, atol=1e-6); close(mt, m, atol=1e-7); close(vt, v, atol=1e-8)
+    d, xh = rnd(4, 6, 32), rnd(4, 6, 33)
+    std = (0.5 + np.abs(xh[:, :1])).astype(np.float32)
+    d64, x64 = d.astype(np.float64), xh.astype(np.float64)
+    exp = (d64 - d64.mean(1, keepdims=True) - x64 * (d64 * x64).mean(1, keepdims=True)) / std
+    close(ref.layer_norm_backward(d, xh, std, 6), exp)
+
+
+def test_scatter_add_rows_with_duplicates():
+    target = rnd(10, 8, 124); t0 = target.copy()
+    grad = rnd(6, 8, 125); idx = [3, 1, 7, 1, 4, 3]     # MetalBackendTest.java:151-167
+    ref.scatter_add_rows(target, idx, grad)
+    exp = t0.astype(np.float64)
+    for i, r in enumerate(idx):
+        exp[r] += grad[i]
+    close(target, exp, atol=1e-6)
+
+
+# ── layers ──────────────────────────────────────────────────────────────────
+
+def test_rmsnorm_invariants():
+    # RMSNorm1DTest.java:59-111
+    y = ref.rmsnorm([[3.0, 0.0, 4.0, 0.0]], np.ones((1, 4)))
+    assert abs(np.sqrt(np.mean(y.astype(np.float64) ** 2)) - 1.0) < 1e-5
+    x = np.array([[1.0, 2.0, 3.0, 4.0]], np.float32)
+    y1, y2 = ref.rmsnorm(x, np.ones((1, 4))), ref.rmsnorm(x, 2 * np.ones((1, 4)))
+    assert np.array_equal(y1 * 2.0, y2)
+    close(ref.rmsnorm(2 * x, np.ones((1, 4))), y1, atol=1e-6, rtol=0)
+    # closed form incl. eps and a non-trivial gain, multi-row
+    x, gm = rnd(5, 12, 40), 1 + rnd(1, 12, 41)
+    x64 = x.astype(np.float64)
+    close(ref.rmsnorm(x, gm), gm * x64 / np.sqrt((x64 ** 2).mean(1, keepdims=True) + 1e-6))
+
+
+def test_swiglu_and_linear_against_numpy():
+    x = rnd(3, 8, 50)
+    wg, wu, wd = rnd(8, 20, 51), rnd(8, 20, 52), rnd(20, 8, 53)
+    bg, bu, bd = rnd(1, 20, 54), rnd(1, 20, 55), rnd(1, 8, 56)
+    x64 = x.astype(np.float64)
+    gate, up = x64 @ wg + bg, x64 @ wu + bu
+    exp = (gate / (1 + np.exp(-gate)) * up) @ wd + bd
+    close(ref.swiglu(x, wg, bg, wu, bu, wd, bd), exp)
+
+
+def test_rope_properties():
+    cos, sin = ref.rope_tables(8, 32)
+    # table closed form (RotaryEmbedding.java:63-70)
+    pos, i = np.arange(32)[:, None], np.arange(4)[None, :]
+    theta = pos / np.power(10000.0, 2.0 * i / 8)
+    close(cos, np.cos(theta), atol=1e-6); close(sin, np.sin(theta), atol=1e-6)
+    x = rnd(2 * 5, 8, 3)                       # nHeads=2, seqLen=5
+    y = ref.rope_apply(x, 5, 2, cos, sin)
+    close(np.linalg.norm(y, axis=1), np.linalg.norm(x, axis=1), atol=1e-6)      # :85-98
+    # interleaved pairing (2i,2i+1), not half-split: explicit complex rotation
+    z = (x[:, 0::2] + 1j * x[:, 1::2]).astype(np.complex128)
+    rot = np.exp(1j * np.tile(theta[:5], (2, 1)))
+    zr = z * rot
+    exp = np.empty_like(x, dtype=np.float64); exp[:, 0::2] = zr.real; exp[:, 1::2] = zr.imag
+    close(y, exp, atol=1e-6)
+    # both heads see the same positions (:120-142)
+    xs = rnd(2, 8, 4)
+    yd = ref.rope_apply(np.vstack([xs, xs]), 2, 2, cos, sin)
+    assert np.array_equal(yd[:2], yd[2:])
+    # pos0 offset = rows of a longer sequence
+    y_long = ref.rope_apply(rnd(7, 8, 5), 7, 1, cos, sin)
+    y_off = ref.rope_apply(rnd(7, 8, 5)[3:5], 2, 1, cos, sin, pos0=3)
+    assert np.array_equal(y_long[3:5], y_off)
+
+
+def test_split_merge_heads_roundtrip_and_layout():
+    x = rnd(5, 12, 60)
+    s = ref.split_heads(x, 3)
+    assert s.shape == (15, 4)
+    assert np.array_equal(s[1 * 5 + 2], x[2, 4:8])          # HeadOps.java:33-46
+    assert np.array_equal(ref.merge_heads(s, 3), x)
+
+
+def brute_attention(x, wq, wk, wv, wo, heads, theta=None, causal=True):
+    x, wq, wk, wv, wo = (t.astype(np.float64) for t in (x, wq, wk, wv, wo))
+    seq, d = x.shape
+    hd = d // heads
+    q, k, v = x @ wq, x @ wk, x @ wv
+    out = np.zeros((seq, d))
+    for h in range(heads):
+        qh, kh, vh = (t[:, h * hd:(h + 1) * hd].copy() for t in (q, k, v))
+        if theta is not None:
+            for t in (qh, kh):
+                z = (t[:, 0::2] + 1j * t[:, 1::2]) * np.exp(1j * theta[:seq])
+                t[:, 0::2], t[:, 1::2] = z.real, z.imag
+        s = qh @ kh.T / np.sqrt(hd)
+        if causal:
+            s = s + np.triu(np.full((seq, seq), -1e9), 1)
+        p = np.exp(s - s.max(1, keepdims=True)); p /= p.sum(1, keepdims=True)
+        out[:, h * hd:(h + 1) * hd] = p @ vh
+    return out @ wo
+
+
+def test_mhsa_matches_brute_force_fp64():
+    # shapes of TransformerBuilderTest.java:22-56 (d=8, H=2, S=4)
+    d, H, S = 8, 2, 4
+    x = rnd(S, d, 70)
+    w = [rnd(d, d, 71 + i) for i in range(4)]
+    cos, sin = ref.rope_tables(d // H, 16)
+    theta = np.arange(16)[:, None] / np.power(10000.0, 2.0 * np.arange(d // H // 2)[None, :] / (d // H))
+    close(ref.mhsa_forward(x, *w, H, cos, sin), brute_attention(x, *w, H, theta), atol=1e-6)
+    close(ref.mhsa_forward(x, *w, H), brute_attention(x, *w, H), atol=1e-6)
+    close(ref.mhsa_forward(x, *w, H, causal=False), brute_attention(x, *w, H, causal=False), atol=1e-6)
+
+
+def test_causal_mask_blocks_future_tokens():
+    # MultiHeadSelfAttentionTest.java:24-68: identity projections, change a future row
+    d, H, S = 8, 2, 5
+    eye = np.eye(d, dtype=np.float32)
+    x = rnd(S, d, 80)
+    y1 = ref.mhsa_forward(x, eye, eye, eye, eye, H)
+    x2 = x.copy(); x2[4] += 10.0
+    y2 = ref.mhsa_forward(x2, eye, eye, eye, eye, H)
+    assert np.array_equal(y1[:4], y2[:4]) and not np.allclose(y1[4], y2[4])
+
+
+def test_mla_matches_brute_force_fp64():
+    d, H, S, qr, kvr = 8, 2, 4, 4, 2
+    x = rnd(S, d, 90)
+    wdq, wuq, wdkv, wuk, wuv, wo = (rnd(*s, 91 + i) for i, s in enumerate(
+        [(d, qr), (qr, d), (d, kvr), (kvr, d), (kvr, d), (d, d)]))
+    cos, sin = ref.rope_tables(d // H, 16)
+    theta = np.arange(16)[:, None] / np.power(10000.0, 2.0 * np.arange(d // H // 2)[None, :] / (d // H))
+    f = np.float64
+    exp = brute_attention(x, (wdq.astype(f) @ wuq).astype(f), (wdkv.astype(f) @ wuk), (wdkv.astype(f) @ wuv),
+                          wo, H, theta)
+    close(ref.mla_forward(x, wdq, wuq, wdkv, wuk, wuv, wo, H, cos, sin), exp, atol=1e-6)
+
+
+# ── Q8 (this build's format: pinned by bounds and exact cases) ───────────────
+
+def test_q8_roundtrip_bounds_and_exact_cases():
+    w = rnd(70, 9, 100)                            # K=70: ragged last group (70 = 2*32 + 6)
+    q, s = ref.q8_quantize(w)
+    assert q.shape == (9, 96) and s.shape == (9, 3)
+    assert np.all(q[:, 70:] == 0) and np.all(np.abs(q.astype(int)) <= 127)
+    dq = ref.q8_dequantize(q, s, 70)
+    bound = np.repeat(s.T, 32, axis=0)[:70] / 2        # |w - dq| <= scale/2 per group
+    assert np.all(np.abs(w - dq) <= bound * (1 + 1e-6) + 1e-12)
+    # scale = absmax/127 and the absmax element is reproduced to 1 ulp of scale*127
+    for col in range(9):
+        for g in range(3):
+            blk = w[g * 32:min(70, g * 32 + 32), col]
+            assert s[col, g] == np.float32(np.max(np.abs(blk))) / np.float32(127.0)
+    # representable inputs are exact: integers in [-127,127] with absmax 127
+    wi = np.zeros((32, 2), np.float32); wi[:, 0] = np.arange(-16, 16) * 7.0; wi[0, 0] = -127.0; wi[5, 1] = 127.0
+    assert np.array_equal(ref.q8_roundtrip(wi), wi)
+    # all-zero group: scale 0, q 0, no NaN
+    assert np.array_equal(ref.q8_roundtrip(np.zeros((32, 3), np.float32)), np.zeros((32, 3), np.float32))
+    # idempotent
+    assert np.array_equal(ref.q8_roundtrip(dq), dq)
+
+
+# ── models ──────────────────────────────────────────────────────────────────
+
+TINY = dict(vocab=256, max_seq=16, d=32, heads=4, layers=2, dff=88)   # LlamaModelTest.java:18-29 scale
+
+
+def test_llama_init_order_and_forward_matches_layers():
+    m = ref.Model(seed=42, **TINY)
+    # §RNG wiring (LlamaModel.java:27-42): embedding and layer-0 Wq start with the same Gaussians
+    assert np.array_equal(m.weight("emb").reshape(-1)[:32 * 32], m.weight("L0.wq").reshape(-1))
+    r = ref.JavaRandom(42)
+    for name, shape in [("L0.wq", (32, 32)), ("L0.wk", (32, 32)), ("L0.wv", (32, 32)), ("L0.wo", (32, 32)),
+                        ("L0.wg", (32, 88)), ("L0.wu", (32, 88)), ("L0.wd", (88, 32)), ("L1.wq", (32, 32))]:
+        assert np.array_equal(m.weight(name), r.tensor(*shape)), name
+    assert np.array_equal(m.weight("wlm"), ref.JavaRandom(43).tensor(32, 256))
+    assert np.all(m.weight("L0.bg") == 0) and np.all(m.weight("gf") == 1)
+    # forward == composition of the layer functions
+    ids = ref.JavaRandom(7).ints(6, 256)
+    x = ref.slice_rows(m.weight("emb"), ids)
+    cos, sin = ref.rope_tables(8, 16)
+    for l in range(2):
+        w = lambda n: m.weight(f"L{l}.{n}")
+        x2 = ref.add(x, ref.mhsa_forward(ref.rmsnorm(x, w("g1")), w("wq"), w("wk"), w("wv"), w("wo"), 4, cos, sin))
+        x = ref.add(x2, ref.swiglu(ref.rmsnorm(x2, w("g2")), w("wg"), w("bg"), w("wu"), w("bu"), w("wd"), w("bd")))
+    exp = ref.linear(ref.rmsnorm(x, m.weight("gf")), m.weight("wlm"), m.weight("blm"))
+    assert np.array_equal(m.forward(ids), exp)
+    with pytest.raises(ValueError, match="out of range"):
+        m.forward([0, 256])                              # Embedding.java:30-32
+
+
+def test_cached_forward_is_bit_identical_to_full_context():
+    for cfg in (dict(TINY), dict(TINY, q_rank=16, kv_rank=8)):
+        m = ref.Model(seed=42, **cfg)
+        ids = ref.JavaRandom(7).ints(12, 256)
+        full = m.forward(ids)
+        m.reset_cache()
+        got = [m.forward_cached(ids[:5])]                # prompt chunk, then ragged chunks
+        got.append(m.forward_cached(ids[5:6]))
+        got.append(m.forward_cached(ids[6:12]))
+        assert np.array_equal(np.vstack(got), full), cfg
+        m.reset_cache()
+        assert np.array_equal(m.forward_cached(ids, last_only=True), full[-1:])
+
+
+def test_generate_greedy_properties_and_cache_equivalence():
+    m = ref.Model(seed=42, **TINY)
+    prompt = ref.JavaRandom(7).ints(4, 256)
+    a = m.generate(prompt, 8, temperature=1.0, top_k=1, seed=1)
+    b = m.generate(prompt, 8, temperature=0.7, top_k=1, seed=99)   # TextGeneratorTest.java:92-98
+    assert np.array_equal(a, b) and np.array_equal(a[:4], prompt)  # LlamaModelTest.java:120-127
+    c, logits = m.generate(prompt, 8, top_k=1, use_cache=True, return_logits=True)
+    assert np.array_equal(a, c)
+    assert np.array_equal(np.argmax(logits, axis=1), c[4:])
+    # sliding window past maxSeqLen (TextGenerator.java:93,172-175): still runs, window = last 16 ids
+    long = m.generate(prompt, 16, top_k=1)
+    assert len(long) == 20
+    ctx = long[-17:-1]
+    assert long[-1] == int(np.argmax(m.forward(ctx)[-1]))
+
+
+def test_sampler_semantics():
+    # ties -> lowest index (stable sort); one nextFloat per token; top-k restricts support
+    logits = np.array([1.0, 5.0, 5.0, -2.0], np.float32)
+    r = ref.JavaRandom(0)
+    assert ref.sample_from_logits(logits, 1.0, 1, r) == 1
+    r2 = ref.JavaRandom(0); r2.next_float()
+    assert r.next_float() == r2.next_float()
+    counts = np.zeros(4, int)
+    r = ref.JavaRandom(5)
+    for _ in range(4000):
+        counts[ref.sample_from_logits(np.array([0.0, 1.0, 2.0, -50.0], np.float32), 1.0, 3, r)] += 1
+    p = np.exp([0.0, 1.0, 2.0]); p /= p.sum()
+    assert counts[3] == 0 and np.allclose(counts[:3] / 4000, p, atol=0.03)
+
+
+def test_deepseek_param_layout():
+    m = ref.Model(seed=42, **dict(TINY, q_rank=16, kv_rank=8))
+    r = ref.JavaRandom(42)          # MultiHeadLatentAttention.java:81-86 order
+    for name, shape in [("L0.wdq", (32, 16)), ("L0.wuq", (16, 32)), ("L0.wdkv", (32, 8)), ("L0.wuk", (8, 32)),
+                        ("L0.wuv", (8, 32)), ("L0.wo", (32, 32)), ("L0.wg", (32, 88))]:
+        assert np.array_equal(m.weight(name), r.tensor(*shape)), name
+    per_block = [n for n in m.weight_names() if n.startswith("L0.")]
+    assert len(per_block) == 14                      # DeepSeekModelTest.java:92-99
+    assert len([n for n in ref.Model(seed=1, **TINY).weight_names() if n.startswith("L0.")]) == 12
+
+
+def test_threading_never_changes_results():
+    a, b = rnd(37, 19, 1), rnd(19, 23, 2)
+    ref.set_threads(1); y1 = ref.matmul(a, b); s1 = ref.softmax_rows(a)
+    ref.set_threads(5); y5 = ref.matmul(a, b); s5 = ref.softmax_rows(a)
+    ref.set_column_parallel(True); y5c = ref.matmul(a[:2], b); ref.set_column_parallel(False)
+    ref.set_threads(1)
+    assert np.array_equal(y1, y5) and np.array_equal(s1, s5) and np.array_equal(y1[:2], y5c)
