@@ -1,0 +1,11 @@
+"""deepj_amd: MI355X (gfx950) backend for DeepJ behind its TensorBackend / ComputeGraph /
+GpuRuntime boundary.  The compute lives in libdeepj_hip.so (hand-written HIP kernels
+reached through the C ABI in include/deepj_hip.h); this package is the host-side twin of
+the reference's Java classes around that boundary."""
+from . import opcodes
+from ._native import HipNative, LIB_PATH
+from .compute_graph import ComputeGraph, GpuBuffer
+from .hip_backend import HipBackend, HipGpuRuntime
+from .tensor import Tensor
+
+__all__ = ["opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor"]

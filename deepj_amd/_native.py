@@ -1,0 +1,159 @@
+"""ctypes binding of libdeepj_hip.so - the Python twin of the reference's
+MetalNative (src/main/java/io/github/kirstenali/deepj/tensor/metal/MetalNative.java:10-57):
+five calls into the native library plus the runtime-control extras.
+
+The HIP library is the product: if it is missing or fails to load, every entry
+point raises; there is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdeepj_hip.so")
+
+_i32p = C.POINTER(C.c_int32)
+_f32p = C.POINTER(C.c_float)
+
+_lib = None
+_load_error: Exception | None = None
+
+
+def _bind(lib: C.CDLL) -> None:
+    lib.deepj_hip_init.argtypes = [C.c_int32]
+    lib.deepj_hip_alloc_buffers.argtypes = [_i32p, _i32p, C.c_int32]
+    lib.deepj_hip_upload.argtypes = [C.c_int32, C.c_void_p, C.c_int64]
+    lib.deepj_hip_download.argtypes = [C.c_int32, C.c_void_p, C.c_int64]
+    lib.deepj_hip_release.argtypes = [_i32p, C.c_int32]
+    lib.deepj_hip_flush_ops.argtypes = [_i32p, C.c_int32]
+    lib.deepj_hip_last_error.restype = C.c_char_p
+    lib.deepj_hip_pool_stats.argtypes = [C.POINTER(C.c_int64)]
+    lib.deepj_hip_stream.restype = C.c_void_p
+    lib.deepj_hip_q8_floats.argtypes = [C.c_int32, C.c_int32]
+    lib.deepj_hip_q8_floats.restype = C.c_int64
+    lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
+    lib.deepj_hip_graph_capture.argtypes = [_i32p, C.c_int32, _i32p]
+    lib.deepj_hip_graph_launch.argtypes = [C.c_int32, C.c_int32]
+    lib.deepj_hip_graph_destroy.argtypes = [C.c_int32]
+    for name in ("deepj_hip_init", "deepj_hip_alloc_buffers", "deepj_hip_upload", "deepj_hip_download",
+                 "deepj_hip_release", "deepj_hip_flush_ops", "deepj_hip_synchronize", "deepj_hip_shutdown",
+                 "deepj_hip_trim", "deepj_hip_pool_stats", "deepj_hip_time_ops", "deepj_hip_graph_capture",
+                 "deepj_hip_graph_launch", "deepj_hip_graph_destroy"):
+        getattr(lib, name).restype = C.c_int
+
+
+def library() -> C.CDLL:
+    """The loaded native library; raises RuntimeError when it is not there."""
+    global _lib, _load_error
+    if _lib is not None:
+        return _lib
+    if _load_error is None:
+        try:
+            if not os.path.exists(LIB_PATH):
+                raise FileNotFoundError(f"{LIB_PATH} is not built (run: python -m deepj_amd.build)")
+            lib = C.CDLL(LIB_PATH)
+            _bind(lib)
+            _lib = lib
+            return lib
+        except Exception as exc:  # noqa: BLE001 - remembered and re-raised on every use
+            _load_error = exc
+    raise RuntimeError(f"[DeepJ/HIP] native library unavailable: {_load_error}")
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(library().deepj_hip_last_error().decode("utf-8", "replace"))
+
+
+def _ids(a) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int32))
+
+
+class HipNative:
+    """Static facade, one method per native entry point (names as in MetalNative)."""
+
+    @staticmethod
+    def available() -> bool:
+        try:
+            library()
+            return True
+        except RuntimeError:
+            return False
+
+    @staticmethod
+    def nativeAllocBuffers(ids, sizes, count: int) -> None:
+        ids, sizes = _ids(ids), _ids(sizes)
+        _check(library().deepj_hip_alloc_buffers(ids.ctypes.data_as(_i32p), sizes.ctypes.data_as(_i32p), count))
+
+    @staticmethod
+    def nativeUploadBuffer(buf_id: int, data: np.ndarray) -> None:
+        data = np.ascontiguousarray(data)
+        assert data.dtype.itemsize == 4, "buffers hold 32-bit words"
+        _check(library().deepj_hip_upload(buf_id, data.ctypes.data, data.size))
+
+    @staticmethod
+    def nativeDownloadBuffer(buf_id: int, out: np.ndarray) -> None:
+        assert out.flags["C_CONTIGUOUS"] and out.dtype.itemsize == 4
+        _check(library().deepj_hip_download(buf_id, out.ctypes.data, out.size))
+
+    @staticmethod
+    def nativeReleaseBuffers(ids, count: int) -> None:
+        ids = _ids(ids)
+        _check(library().deepj_hip_release(ids.ctypes.data_as(_i32p), count))
+
+    @staticmethod
+    def nativeFlushOps(cmd_stream, length: int) -> None:
+        cmd = _ids(cmd_stream)
+        _check(library().deepj_hip_flush_ops(cmd.ctypes.data_as(_i32p), length))
+
+    # ── runtime control ─────────────────────────────────────────────────────
+    @staticmethod
+    def init(device: int = 0) -> None:
+        _check(library().deepj_hip_init(device))
+
+    @staticmethod
+    def synchronize() -> None:
+        _check(library().deepj_hip_synchronize())
+
+    @staticmethod
+    def shutdown() -> None:
+        _check(library().deepj_hip_shutdown())
+
+    @staticmethod
+    def trim() -> None:
+        _check(library().deepj_hip_trim())
+
+    @staticmethod
+    def poolStats() -> dict:
+        out = (C.c_int64 * 4)()
+        _check(library().deepj_hip_pool_stats(out))
+        return {"live_buffers": out[0], "live_bytes": out[1], "cached_bytes": out[2], "driver_allocs": out[3]}
+
+    @staticmethod
+    def q8Floats(k: int, rows: int) -> int:
+        return int(library().deepj_hip_q8_floats(k, rows))
+
+    @staticmethod
+    def timeOps(cmd_stream, iters: int) -> float:
+        cmd = _ids(cmd_stream)
+        ms = C.c_float()
+        _check(library().deepj_hip_time_ops(cmd.ctypes.data_as(_i32p), cmd.size, iters, C.byref(ms)))
+        return float(ms.value)
+
+    @staticmethod
+    def graphCapture(cmd_stream) -> int:
+        cmd = _ids(cmd_stream)
+        h = C.c_int32()
+        _check(library().deepj_hip_graph_capture(cmd.ctypes.data_as(_i32p), cmd.size, C.byref(h)))
+        return int(h.value)
+
+    @staticmethod
+    def graphLaunch(handle: int, times: int = 1) -> None:
+        _check(library().deepj_hip_graph_launch(handle, times))
+
+    @staticmethod
+    def graphDestroy(handle: int) -> None:
+        _check(library().deepj_hip_graph_destroy(handle))

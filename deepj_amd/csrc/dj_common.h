@@ -1,0 +1,104 @@
+// Shared declarations of the device runtime: buffer records, error plumbing and
+// the launcher prototypes each kernel file exports to the stream interpreter.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "../../include/deepj_hip.h"
+
+namespace dj {
+
+constexpr int kQ8Group = 32;          // weights per fp32 scale, along the input (K) axis
+constexpr float kRmsEps = 1e-6f;      // RMSNorm1D.java:30 in the reference
+
+struct Error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+[[noreturn]] inline void fail(const std::string &msg) { throw Error(msg); }
+
+inline void hip_check(hipError_t e, const char *what) {
+    if (e != hipSuccess) fail(std::string(what) + ": " + hipGetErrorString(e));
+}
+#define DJ_HIP(expr) ::dj::hip_check((expr), #expr)
+
+inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+inline int q8_padded_k(int k) { return (int)round_up(k, kQ8Group); }
+// Q8 weight buffer: [rows x Kp] int8, padded to 256 B, then [rows x Kp/32] fp32 scales.
+inline int64_t q8_scale_offset_bytes(int k, int rows) { return round_up((int64_t)rows * q8_padded_k(k), 256); }
+inline int64_t q8_bytes(int k, int rows) {
+    return q8_scale_offset_bytes(k, rows) + (int64_t)rows * (q8_padded_k(k) / kQ8Group) * 4;
+}
+
+// ── launchers (each validates nothing: the interpreter has already checked
+//    ids, sizes and shapes on the host before any of these is called) ──────
+
+// kernels_elementwise.hip
+void launch_binary(hipStream_t s, int op, const float *a, const float *b, float *out, int64_t n);
+void launch_unary(hipStream_t s, int op, const float *a, float *out, int64_t n);
+void launch_scalar(hipStream_t s, int op, const float *a, float *out, float s0, float s1, int64_t n);
+void launch_broadcast(hipStream_t s, int op, const float *a, const float *v, float *out, int rows, int cols);
+void launch_transpose(hipStream_t s, const float *a, float *out, int rows, int cols);
+void launch_adamw(hipStream_t s, float *w, const float *g, float *mt, float *vt, int64_t n, float lr,
+                  float beta1, float beta2, float eps, float wd, float bc1, float bc2);
+void launch_scatter_add(hipStream_t s, float *target, const float *idx, const float *grad, int target_rows,
+                        int cols, int n_idx);
+void launch_fill(hipStream_t s, uint32_t *dst, uint32_t bits, int64_t n);
+void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n);
+void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n);
+void launch_embed_gather(hipStream_t s, const float *table, const int32_t *ids, float *out, int n_ids, int d,
+                         int vocab);
+void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity);
+
+// kernels_reduce.hip
+void launch_row_reduce(hipStream_t s, int op, const float *a, float *out, int rows, int cols);
+void launch_sum_rows(hipStream_t s, const float *a, float *out, int rows, int cols);
+void launch_sum_scalar(hipStream_t s, const float *a, float *out, int64_t n);
+void launch_softmax_rows(hipStream_t s, const float *a, float *out, int rows, int cols);
+void launch_softmax_backward(hipStream_t s, const float *g, const float *sm, float *out, int rows, int cols);
+void launch_layernorm_backward(hipStream_t s, const float *dxhat, const float *xhat, const float *stdv,
+                               float *out, int rows, int cols);
+void launch_cross_entropy(hipStream_t s, bool gradient, const float *logits, const float *targets, float *out,
+                          int rows, int cols);
+void launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int rows, int cols);
+void launch_argmax_rows(hipStream_t s, const float *a, int32_t *out, int rows, int cols);
+
+// kernels_matmul.hip
+void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out, int m, int n, int k);
+
+// kernels_q8.hip
+struct Q8Linear {
+    const float *x; const int8_t *wq; const float *scales; float *out;
+    int m, k, n, flags;
+    const float *gamma, *bias, *bias2, *residual;
+};
+void launch_q8_quantize(hipStream_t s, const float *w, int8_t *q, float *scales, int k, int n, int row_off,
+                        int row_step);
+void launch_q8_dequantize(hipStream_t s, const int8_t *q, const float *scales, float *w, int k, int n,
+                          int row_off, int row_step);
+void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_t workspace_floats);
+int64_t q8_linear_workspace_floats(int m, int k, int n, int flags);
+
+// kernels_attn.hip
+struct AttnArgs {
+    const float *q;        // [S x H*hd], already rotated
+    const float *k, *v;    // key/value base for this layer
+    int64_t k_tok_stride, k_head_stride;   // in floats
+    float *out;            // [S x H*hd]
+    const int32_t *state;  // state[0] = number of positions before this chunk
+    float *scratch; int64_t scratch_floats;
+    int s, h, hd, max_seq;
+};
+void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *k_cache, float *v_cache,
+                          const int32_t *state, const float *cos_t, const float *sin_t, int S, int H, int hd,
+                          int max_seq);
+void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *state, const float *cos_t,
+                      const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row);
+void launch_attention(hipStream_t s, const AttnArgs &a);
+int64_t attention_scratch_floats(int S, int H, int hd, int max_seq);
+
+}  // namespace dj

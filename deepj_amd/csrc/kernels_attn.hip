@@ -1,0 +1,255 @@
+// RoPE + KV-cache store, and causal softmax attention over a device-resident
+// KV cache (fp32).  Semantics follow the reference's Java composition:
+//   RotaryEmbedding.java:63-70,112-122   interleaved pairs (2i, 2i+1), tables via f64
+//   HeadOps.java:90-140                  s = (q.k) * scale, causal mask, softmax, p.v
+//   MultiHeadSelfAttention.java:45       scale = (float)(1/sqrt(headDim))
+// but nothing is materialised: no [H*S x S] score tensor, no mask tensor, no head
+// split/merge copies.  Keys later than the query position are simply not read
+// (the reference adds -1e9 to them, which makes their probability exactly 0).
+//
+// Cache layout (per layer): K and V as [H][maxSeq][hd] fp32, so one head's keys
+// are a single contiguous stream.  A key row is read by hd/4 lanes as float4
+// (a wavefront load covers 64/(hd/4) whole keys = 1 KiB, fully coalesced).
+//
+// Decode (S = 1): the key range is split over gridDim.z workgroups per head so the
+// HBM-bound KV read is spread over all CUs; each split keeps a running
+// (max, sum, weighted V) and the last split to finish - found with a counter in
+// the scratch buffer that it resets for the next launch - merges them.
+#include "dj_common.h"
+
+namespace dj {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kSplitKeys = 64;          // keys per decode split
+
+// ── RoPE on the fused projection + cache append ─────────────────────────────
+// qkv [S x 3d]: Q | K | V.  Row i sits at position state[0] + i.
+__global__ void __launch_bounds__(kThreads) k_rope_kv_store(const float *__restrict__ qkv, float *__restrict__ q_out,
+                                                            float *__restrict__ k_cache, float *__restrict__ v_cache,
+                                                            const int32_t *__restrict__ state,
+                                                            const float *__restrict__ cos_t,
+                                                            const float *__restrict__ sin_t, int S, int H, int hd,
+                                                            int max_seq) {
+    const int half = hd >> 1, d = H * hd;
+    const int pos0 = state[0];
+    int64_t total = (int64_t)S * H * half;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        int j = (int)(t % half);
+        int h = (int)((t / half) % H);
+        int i = (int)(t / ((int64_t)half * H));
+        int pos = pos0 + i;
+        if (pos < 0 || pos >= max_seq) continue;          // never write outside the cache
+        float c = cos_t[(int64_t)pos * half + j], s = sin_t[(int64_t)pos * half + j];
+        const float *row = qkv + (int64_t)i * 3 * d;
+        int e = h * hd + 2 * j;
+        float2 q = *reinterpret_cast<const float2 *>(row + e);
+        float2 k = *reinterpret_cast<const float2 *>(row + d + e);
+        float2 v = *reinterpret_cast<const float2 *>(row + 2 * d + e);
+        float2 qr = make_float2(q.x * c - q.y * s, q.x * s + q.y * c);
+        float2 kr = make_float2(k.x * c - k.y * s, k.x * s + k.y * c);
+        *reinterpret_cast<float2 *>(q_out + (int64_t)i * d + e) = qr;
+        int64_t ce = ((int64_t)h * max_seq + pos) * hd + 2 * j;
+        *reinterpret_cast<float2 *>(k_cache + ce) = kr;
+        *reinterpret_cast<float2 *>(v_cache + ce) = v;
+    }
+}
+
+// RoPE on token-major rows [rows x H*hd]; position = row (pos_from_row) or state[0] + row.
+__global__ void __launch_bounds__(kThreads) k_rope_rows(const float *__restrict__ x, float *__restrict__ out,
+                                                        const int32_t *__restrict__ state,
+                                                        const float *__restrict__ cos_t,
+                                                        const float *__restrict__ sin_t, int rows, int H, int hd,
+                                                        int max_seq, int pos_from_row) {
+    const int half = hd >> 1, d = H * hd;
+    const int pos0 = pos_from_row ? 0 : state[0];
+    int64_t total = (int64_t)rows * H * half;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        int j = (int)(t % half);
+        int h = (int)((t / half) % H);
+        int i = (int)(t / ((int64_t)half * H));
+        int pos = pos0 + i;
+        if (pos < 0 || pos >= max_seq) continue;
+        float c = cos_t[(int64_t)pos * half + j], s = sin_t[(int64_t)pos * half + j];
+        int64_t e = (int64_t)i * d + h * hd + 2 * j;
+        float2 v = *reinterpret_cast<const float2 *>(x + e);
+        *reinterpret_cast<float2 *>(out + e) = make_float2(v.x * c - v.y * s, v.x * s + v.y * c);
+    }
+}
+
+// ── attention ───────────────────────────────────────────────────────────────
+// grid (H, S, nsplit).  LPK = hd/4 lanes cooperate on one key; a wavefront handles
+// 64/LPK keys per step.  Scratch (only when nsplit > 1), per (query, head):
+//   [counter(1 int) pad(3)] [nsplit x (hd + 4)] floats: max, sum, pad, pad, o[hd]
+struct AttnKernelArgs {
+    const float *q; const float *k; const float *v; float *out;
+    const int32_t *state; float *scratch;
+    int64_t tok_stride, head_stride;
+    int S, H, hd, max_seq, nsplit;
+    float scale;
+};
+
+template <int LPK>
+__global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
+    constexpr int HD = LPK * 4;
+    constexpr int KPW = 64 / LPK;                 // keys per wavefront step
+    constexpr int NSUB = kWaves * KPW;            // independent running softmaxes per workgroup
+    __shared__ float s_m[NSUB], s_l[NSUB];
+    __shared__ __align__(16) float s_o[NSUB][HD];
+    __shared__ int s_last;
+
+    const int h = blockIdx.x, qi = blockIdx.y, split = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane / LPK, dl = lane % LPK;
+    const int d = a.H * HD;
+
+    const int pos = a.state[0] + qi;              // this query's position; keys 0..pos
+    int n_keys = pos + 1;
+    if (n_keys > a.max_seq) n_keys = a.max_seq;
+    int k_begin = 0, k_end = n_keys;
+    if (a.nsplit > 1) {
+        k_begin = split * kSplitKeys;
+        k_end = k_begin + kSplitKeys;
+        if (split == a.nsplit - 1) k_end = n_keys;          // the last split takes any tail
+        if (k_end > n_keys) k_end = n_keys;
+    }
+
+    const float4 qv = *reinterpret_cast<const float4 *>(a.q + (int64_t)qi * d + h * HD + dl * 4);
+    const float *kb = a.k + (int64_t)h * a.head_stride + dl * 4;
+    const float *vb = a.v + (int64_t)h * a.head_stride + dl * 4;
+
+    float m = -INFINITY, l = 0.0f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int key = k_begin + wave * KPW + sub; key < k_end; key += kWaves * KPW) {
+        float4 kk = *reinterpret_cast<const float4 *>(kb + (int64_t)key * a.tok_stride);
+        float4 vv = *reinterpret_cast<const float4 *>(vb + (int64_t)key * a.tok_stride);
+        float s = qv.x * kk.x + qv.y * kk.y + qv.z * kk.z + qv.w * kk.w;
+#pragma unroll
+        for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s *= a.scale;
+        float mn = fmaxf(m, s);
+        float corr = expf(m - mn);                // 0 when m = -inf
+        float p = expf(s - mn);
+        l = l * corr + p;
+        o.x = o.x * corr + p * vv.x; o.y = o.y * corr + p * vv.y;
+        o.z = o.z * corr + p * vv.z; o.w = o.w * corr + p * vv.w;
+        m = mn;
+    }
+    const int slot = wave * KPW + sub;
+    if (dl == 0) { s_m[slot] = m; s_l[slot] = l; }
+    *reinterpret_cast<float4 *>(&s_o[slot][dl * 4]) = o;
+    __syncthreads();
+
+    // merge the NSUB running states: thread j < HD owns output dim j
+    float M = -INFINITY, L = 0.0f, O = 0.0f;
+    if (tid < HD) {
+#pragma unroll
+        for (int i = 0; i < NSUB; i++) M = fmaxf(M, s_m[i]);
+        if (M != -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < NSUB; i++) {
+                float w = expf(s_m[i] - M);       // empty slots: exp(-inf) = 0
+                L += s_l[i] * w;
+                O += s_o[i][tid] * w;
+            }
+        }
+    }
+
+    float *outp = a.out + (int64_t)qi * d + h * HD;
+    if (a.nsplit == 1) {
+        if (tid < HD) outp[tid] = O / L;
+        return;
+    }
+
+    // ── cross-split merge ──
+    const int64_t rec = HD + 4;
+    float *base = a.scratch + ((int64_t)qi * a.H + h) * (4 + (int64_t)a.nsplit * rec);
+    int *counter = reinterpret_cast<int *>(base);
+    float *mine = base + 4 + (int64_t)split * rec;
+    if (tid < HD) mine[4 + tid] = O;
+    if (tid == 0) { mine[0] = M; mine[1] = L; }
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        int done = atomicAdd(counter, 1);
+        s_last = (done == a.nsplit - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();                              // acquire: the other splits' records are visible now
+    if (tid < HD) {
+        float GM = -INFINITY;
+        for (int i = 0; i < a.nsplit; i++) GM = fmaxf(GM, base[4 + i * rec]);
+        float GL = 0.0f, GO = 0.0f;
+        for (int i = 0; i < a.nsplit; i++) {
+            const float *r = base + 4 + i * rec;
+            float mi = r[0];
+            if (mi == -INFINITY) continue;
+            float w = expf(mi - GM);
+            GL += r[1] * w;
+            GO += r[4 + tid] * w;
+        }
+        outp[tid] = GO / GL;
+    }
+    if (tid == 0) *counter = 0;                   // ready for the next launch / graph replay
+}
+
+inline int decode_splits(int max_seq) { return (max_seq + kSplitKeys - 1) / kSplitKeys; }
+
+}  // namespace
+
+void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *k_cache, float *v_cache,
+                          const int32_t *state, const float *cos_t, const float *sin_t, int S, int H, int hd,
+                          int max_seq) {
+    int64_t total = (int64_t)S * H * (hd / 2);
+    if (total <= 0) return;
+    int64_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_rope_kv_store, dim3((int)blocks), dim3(kThreads), 0, s, qkv, q_out, k_cache, v_cache, state,
+                       cos_t, sin_t, S, H, hd, max_seq);
+}
+
+void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *state, const float *cos_t,
+                      const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row) {
+    int64_t total = (int64_t)rows * H * (hd / 2);
+    if (total <= 0) return;
+    int64_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_rope_rows, dim3((int)blocks), dim3(kThreads), 0, s, x, out, state, cos_t, sin_t, rows, H, hd,
+                       max_seq, pos_from_row);
+}
+
+// Decode launches always use the same number of splits (sized for max_seq) so that a
+// captured graph stays valid as the cache grows; splits beyond the live keys exit
+// after writing an empty record.
+int64_t attention_scratch_floats(int S, int H, int hd, int max_seq) {
+    if (S != 1) return 0;
+    return (int64_t)H * (4 + (int64_t)decode_splits(max_seq) * (hd + 4));
+}
+
+void launch_attention(hipStream_t s, const AttnArgs &p) {
+    if (p.s <= 0) return;
+    AttnKernelArgs a;
+    a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.state = p.state; a.scratch = p.scratch;
+    a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
+    a.S = p.s; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
+    a.scale = (float)(1.0 / sqrt((double)p.hd));
+    a.nsplit = 1;
+    if (p.s == 1) {
+        a.nsplit = decode_splits(p.max_seq);
+        if (a.nsplit > 1 && p.scratch_floats < attention_scratch_floats(1, p.h, p.hd, p.max_seq))
+            fail("attention: scratch buffer too small");
+    }
+    dim3 grid(p.h, p.s, a.nsplit);
+    switch (p.hd) {
+        case 32: hipLaunchKernelGGL(k_attention<8>, grid, dim3(kThreads), 0, s, a); break;
+        case 64: hipLaunchKernelGGL(k_attention<16>, grid, dim3(kThreads), 0, s, a); break;
+        case 128: hipLaunchKernelGGL(k_attention<32>, grid, dim3(kThreads), 0, s, a); break;
+        default: fail("attention: head dim must be 32, 64 or 128");
+    }
+}
+
+}  // namespace dj

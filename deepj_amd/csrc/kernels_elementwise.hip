@@ -1,0 +1,362 @@
+// Element-wise, broadcast and data-movement kernels of the 42 primitive opcodes
+// (semantics: CpuBackend.java:56-132,190-214,300-354,466-489,542-549 in the
+// reference) plus the small fused inference helpers.  All of them are HBM
+// bound: one pass, 128-bit accesses where the length allows it, grid sized to
+// a multiple of the 256 CUs.
+//
+// Transcendentals follow the CPU backend's convention - evaluate in f64, cast
+// to fp32 (CpuBackend.java:24-28) - so a GPU result differs from the CPU one by
+// at most the last f64 bit of the math library, not by an fp32 approximation.
+#include "dj_common.h"
+
+namespace dj {
+namespace {
+
+constexpr int kThreads = 256;
+
+inline int grid_for(int64_t work_items, int per_thread = 1) {
+    int64_t blocks = (work_items + (int64_t)kThreads * per_thread - 1) / ((int64_t)kThreads * per_thread);
+    if (blocks < 1) blocks = 1;
+    if (blocks > 256 * 32) blocks = 256 * 32;      // grid-stride beyond 32 blocks per CU
+    return (int)blocks;
+}
+
+__device__ __forceinline__ float d_exp(float x) { return (float)exp((double)x); }
+__device__ __forceinline__ float d_log(float x) { return (float)log((double)x); }
+__device__ __forceinline__ float d_tanh(float x) { return (float)tanh((double)x); }
+__device__ __forceinline__ float d_pow(float x, float e) { return (float)pow((double)x, (double)e); }
+__device__ __forceinline__ float d_sigmoid(float x) { return 1.0f / (1.0f + d_exp(-x)); }
+
+__device__ __forceinline__ float d_gelu(float x) {
+    float c = sqrtf(2.0f / 3.14159265358979323846f);
+    float x3 = x * x * x;
+    float t = c * (x + 0.044715f * x3);
+    return 0.5f * x * (1.0f + d_tanh(t));
+}
+__device__ __forceinline__ float d_gelu_deriv(float x) {
+    float c = sqrtf(2.0f / 3.14159265358979323846f);
+    float x2 = x * x;
+    float x3 = x2 * x;
+    float t = c * (x + 0.044715f * x3);
+    float th = d_tanh(t);
+    float sech2 = 1.0f - th * th;
+    float dtdx = c * (1.0f + 3.0f * 0.044715f * x2);
+    return 0.5f * (1.0f + th) + 0.5f * x * sech2 * dtdx;
+}
+
+template <int OP> __device__ __forceinline__ float binary_op(float x, float y) {
+    if constexpr (OP == DJ_OP_ADD) return x + y;
+    if constexpr (OP == DJ_OP_SUBTRACT) return x - y;
+    if constexpr (OP == DJ_OP_MULTIPLY) return x * y;
+    if constexpr (OP == DJ_OP_DIVIDE) return x / y;
+    if constexpr (OP == DJ_OP_RELU_BACKWARD) return x > 0.0f ? y : 0.0f;
+    if constexpr (OP == DJ_OP_GELU_BACKWARD) return y * d_gelu_deriv(x);
+    return 0.0f;
+}
+
+template <int OP> __device__ __forceinline__ float unary_op(float x) {
+    if constexpr (OP == DJ_OP_SQRT) return sqrtf(x);          // correctly rounded, as (float)Math.sqrt
+    if constexpr (OP == DJ_OP_NEG) return -x;
+    if constexpr (OP == DJ_OP_EXP) return d_exp(x);
+    if constexpr (OP == DJ_OP_LOG) return d_log(x);
+    if constexpr (OP == DJ_OP_TANH) return d_tanh(x);
+    if constexpr (OP == DJ_OP_SIGMOID) return d_sigmoid(x);
+    if constexpr (OP == DJ_OP_RELU) return x > 0.0f ? x : (x != x ? x : 0.0f);
+    if constexpr (OP == DJ_OP_GELU) return d_gelu(x);
+    return 0.0f;
+}
+
+template <int OP> __device__ __forceinline__ float scalar_op(float x, float s0, float s1) {
+    if constexpr (OP == DJ_OP_MULTIPLY_SCALAR) return x * s0;
+    if constexpr (OP == DJ_OP_ADD_SCALAR) return x + s0;
+    if constexpr (OP == DJ_OP_DIVIDE_SCALAR) return x / s0;
+    if constexpr (OP == DJ_OP_POW) return d_pow(x, s0);
+    if constexpr (OP == DJ_OP_CLAMP) {                         // Math.min(max, Math.max(min, x))
+        float mx = x > s0 ? x : s0;
+        if (x != x) mx = x;
+        float mn = mx < s1 ? mx : s1;
+        if (mx != mx) mn = mx;
+        return mn;
+    }
+    return 0.0f;
+}
+
+template <int OP>
+__global__ void __launch_bounds__(kThreads) k_binary(const float *__restrict__ a, const float *__restrict__ b,
+                                                     float *__restrict__ out, int64_t n) {
+    int64_t n4 = n >> 2;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const float4 *a4 = reinterpret_cast<const float4 *>(a);
+    const float4 *b4 = reinterpret_cast<const float4 *>(b);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    for (int64_t i = tid; i < n4; i += stride) {
+        float4 x = a4[i], y = b4[i], r;
+        r.x = binary_op<OP>(x.x, y.x); r.y = binary_op<OP>(x.y, y.y);
+        r.z = binary_op<OP>(x.z, y.z); r.w = binary_op<OP>(x.w, y.w);
+        o4[i] = r;
+    }
+    for (int64_t i = (n4 << 2) + tid; i < n; i += stride) out[i] = binary_op<OP>(a[i], b[i]);
+}
+
+template <int OP>
+__global__ void __launch_bounds__(kThreads) k_unary(const float *__restrict__ a, float *__restrict__ out, int64_t n) {
+    int64_t n4 = n >> 2;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const float4 *a4 = reinterpret_cast<const float4 *>(a);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    for (int64_t i = tid; i < n4; i += stride) {
+        float4 x = a4[i], r;
+        r.x = unary_op<OP>(x.x); r.y = unary_op<OP>(x.y); r.z = unary_op<OP>(x.z); r.w = unary_op<OP>(x.w);
+        o4[i] = r;
+    }
+    for (int64_t i = (n4 << 2) + tid; i < n; i += stride) out[i] = unary_op<OP>(a[i]);
+}
+
+template <int OP>
+__global__ void __launch_bounds__(kThreads) k_scalar(const float *__restrict__ a, float *__restrict__ out,
+                                                     float s0, float s1, int64_t n) {
+    int64_t n4 = n >> 2;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const float4 *a4 = reinterpret_cast<const float4 *>(a);
+    float4 *o4 = reinterpret_cast<float4 *>(out);
+    for (int64_t i = tid; i < n4; i += stride) {
+        float4 x = a4[i], r;
+        r.x = scalar_op<OP>(x.x, s0, s1); r.y = scalar_op<OP>(x.y, s0, s1);
+        r.z = scalar_op<OP>(x.z, s0, s1); r.w = scalar_op<OP>(x.w, s0, s1);
+        o4[i] = r;
+    }
+    for (int64_t i = (n4 << 2) + tid; i < n; i += stride) out[i] = scalar_op<OP>(a[i], s0, s1);
+}
+
+// out[r,c] = a[r,c] (op) v[c]  (ROWVEC)  or  a[r,c] (op) v[r]  (column vector)
+template <int OP, bool ROWVEC>
+__global__ void __launch_bounds__(kThreads) k_broadcast(const float *__restrict__ a, const float *__restrict__ v,
+                                                        float *__restrict__ out, int rows, int cols) {
+    int64_t n = (int64_t)rows * cols;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        int r = (int)(i / cols);
+        int c = (int)(i - (int64_t)r * cols);
+        float y = ROWVEC ? v[c] : v[r];
+        out[i] = binary_op<OP>(a[i], y);
+    }
+}
+
+// 32x32 tile through LDS (+1 padding: no bank conflicts on the transposed read).
+__global__ void __launch_bounds__(256) k_transpose(const float *__restrict__ a, float *__restrict__ out, int rows,
+                                                   int cols) {
+    __shared__ float tile[32][33];
+    int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;     // 32 x 8
+    int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int j = ty; j < 32; j += 8) {
+        int r = r0 + j, c = c0 + tx;
+        if (r < rows && c < cols) tile[j][tx] = a[(int64_t)r * cols + c];
+    }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) {
+        int c = c0 + j, r = r0 + tx;                       // out is [cols x rows]
+        if (r < rows && c < cols) out[(int64_t)c * rows + r] = tile[tx][j];
+    }
+}
+
+__global__ void __launch_bounds__(kThreads) k_adamw(float *__restrict__ w, const float *__restrict__ g,
+                                                    float *__restrict__ mt, float *__restrict__ vt, int64_t n,
+                                                    float lr, float beta1, float beta2, float eps, float wd,
+                                                    float bc1, float bc2) {
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float grad = g[i];
+        float m_new = beta1 * mt[i] + (1.0f - beta1) * grad;
+        float v_new = beta2 * vt[i] + (1.0f - beta2) * (grad * grad);
+        mt[i] = m_new;
+        vt[i] = v_new;
+        float m_hat = m_new / bc1;
+        float v_hat = v_new / bc2;
+        float update = (lr * m_hat) / (sqrtf(v_hat) + eps);
+        if (wd != 0.0f) update += lr * wd * w[i];
+        w[i] -= update;
+    }
+}
+
+// target[idx[i], c] += grad[i, c]; indices arrive as floats (MetalBackend.java:43-54),
+// rows outside the target are skipped (deepj_metal_jni.mm:606-607).
+__global__ void __launch_bounds__(kThreads) k_scatter_add(float *__restrict__ target, const float *__restrict__ idx,
+                                                          const float *__restrict__ grad, int target_rows, int cols,
+                                                          int n_idx) {
+    int64_t n = (int64_t)n_idx * cols;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride) {
+        int i = (int)(t / cols);
+        int c = (int)(t - (int64_t)i * cols);
+        float fi = idx[i];
+        if (!(fi >= 0.0f) || fi >= (float)target_rows) continue;
+        int row = (int)fi;
+        atomicAdd(&target[(int64_t)row * cols + c], grad[t]);
+    }
+}
+
+__global__ void __launch_bounds__(kThreads) k_fill(uint32_t *__restrict__ dst, uint32_t bits, int64_t n) {
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = bits;
+}
+
+__global__ void __launch_bounds__(kThreads) k_copy(const float *__restrict__ src, float *__restrict__ dst, int64_t n) {
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
+// SiLU.java:20-24 then SwiGLULayer.java:69: (g * sigmoid(g)) * up
+__global__ void __launch_bounds__(kThreads) k_silu_mul(const float *__restrict__ gate, const float *__restrict__ up,
+                                                       float *__restrict__ out, int64_t n) {
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float g = gate[i];
+        float sg = g * d_sigmoid(g);
+        out[i] = sg * up[i];
+    }
+}
+
+// Embedding.java:28-34 (Tensor.sliceRows): out[i,:] = table[ids[i],:].  Ids were range
+// checked on the host when they came from the host; ids produced on the device
+// (argmax) are always < vocab.  An out-of-range id writes NaN instead of reading.
+__global__ void __launch_bounds__(kThreads) k_embed_gather(const float *__restrict__ table,
+                                                           const int32_t *__restrict__ ids, float *__restrict__ out,
+                                                           int n_ids, int d, int vocab) {
+    int i = blockIdx.x;
+    if (i >= n_ids) return;
+    int id = ids[i];
+    bool ok = id >= 0 && id < vocab;
+    const float *src = table + (int64_t)(ok ? id : 0) * d;
+    float *dst = out + (int64_t)i * d;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) dst[c] = ok ? src[c] : __builtin_nanf("");
+}
+
+// state[0] = positions held in the cache, state[1] = current token, state[2] = tokens generated.
+__global__ void k_decode_advance(int32_t *state, const int32_t *token, int32_t *tokens, int capacity) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        int32_t t = token[0];
+        int32_t g = state[2];
+        if (g < capacity) tokens[g] = t;
+        state[1] = t;
+        state[0] = state[0] + 1;
+        state[2] = g + 1;
+    }
+}
+
+}  // namespace
+
+#define DJ_LAUNCH(kernel, grid, block, stream, ...) \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, __VA_ARGS__)
+
+void launch_binary(hipStream_t s, int op, const float *a, const float *b, float *out, int64_t n) {
+    if (n <= 0) return;
+    int grid = grid_for(n, 4);
+    switch (op) {
+        case DJ_OP_ADD: DJ_LAUNCH(k_binary<DJ_OP_ADD>, grid, kThreads, s, a, b, out, n); break;
+        case DJ_OP_SUBTRACT: DJ_LAUNCH(k_binary<DJ_OP_SUBTRACT>, grid, kThreads, s, a, b, out, n); break;
+        case DJ_OP_MULTIPLY: DJ_LAUNCH(k_binary<DJ_OP_MULTIPLY>, grid, kThreads, s, a, b, out, n); break;
+        case DJ_OP_DIVIDE: DJ_LAUNCH(k_binary<DJ_OP_DIVIDE>, grid, kThreads, s, a, b, out, n); break;
+        case DJ_OP_RELU_BACKWARD: DJ_LAUNCH(k_binary<DJ_OP_RELU_BACKWARD>, grid, kThreads, s, a, b, out, n); break;
+        case DJ_OP_GELU_BACKWARD: DJ_LAUNCH(k_binary<DJ_OP_GELU_BACKWARD>, grid, kThreads, s, a, b, out, n); break;
+        default: fail("launch_binary: bad op");
+    }
+}
+
+void launch_unary(hipStream_t s, int op, const float *a, float *out, int64_t n) {
+    if (n <= 0) return;
+    int grid = grid_for(n, 4);
+    switch (op) {
+        case DJ_OP_SQRT: DJ_LAUNCH(k_unary<DJ_OP_SQRT>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_NEG: DJ_LAUNCH(k_unary<DJ_OP_NEG>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_EXP: DJ_LAUNCH(k_unary<DJ_OP_EXP>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_LOG: DJ_LAUNCH(k_unary<DJ_OP_LOG>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_TANH: DJ_LAUNCH(k_unary<DJ_OP_TANH>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_SIGMOID: DJ_LAUNCH(k_unary<DJ_OP_SIGMOID>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_RELU: DJ_LAUNCH(k_unary<DJ_OP_RELU>, grid, kThreads, s, a, out, n); break;
+        case DJ_OP_GELU: DJ_LAUNCH(k_unary<DJ_OP_GELU>, grid, kThreads, s, a, out, n); break;
+        default: fail("launch_unary: bad op");
+    }
+}
+
+void launch_scalar(hipStream_t s, int op, const float *a, float *out, float s0, float s1, int64_t n) {
+    if (n <= 0) return;
+    int grid = grid_for(n, 4);
+    switch (op) {
+        case DJ_OP_MULTIPLY_SCALAR: DJ_LAUNCH(k_scalar<DJ_OP_MULTIPLY_SCALAR>, grid, kThreads, s, a, out, s0, s1, n); break;
+        case DJ_OP_ADD_SCALAR: DJ_LAUNCH(k_scalar<DJ_OP_ADD_SCALAR>, grid, kThreads, s, a, out, s0, s1, n); break;
+        case DJ_OP_DIVIDE_SCALAR: DJ_LAUNCH(k_scalar<DJ_OP_DIVIDE_SCALAR>, grid, kThreads, s, a, out, s0, s1, n); break;
+        case DJ_OP_POW: DJ_LAUNCH(k_scalar<DJ_OP_POW>, grid, kThreads, s, a, out, s0, s1, n); break;
+        case DJ_OP_CLAMP: DJ_LAUNCH(k_scalar<DJ_OP_CLAMP>, grid, kThreads, s, a, out, s0, s1, n); break;
+        default: fail("launch_scalar: bad op");
+    }
+}
+
+void launch_broadcast(hipStream_t s, int op, const float *a, const float *v, float *out, int rows, int cols) {
+    int64_t n = (int64_t)rows * cols;
+    if (n <= 0) return;
+    int grid = grid_for(n);
+    switch (op) {
+        case DJ_OP_ADD_ROW_VECTOR:
+            DJ_LAUNCH((k_broadcast<DJ_OP_ADD, true>), grid, kThreads, s, a, v, out, rows, cols); break;
+        case DJ_OP_MULTIPLY_BROADCAST_ROWS:
+            DJ_LAUNCH((k_broadcast<DJ_OP_MULTIPLY, true>), grid, kThreads, s, a, v, out, rows, cols); break;
+        case DJ_OP_ADD_BROADCAST_COLS:
+            DJ_LAUNCH((k_broadcast<DJ_OP_ADD, false>), grid, kThreads, s, a, v, out, rows, cols); break;
+        case DJ_OP_SUBTRACT_BROADCAST_COLS:
+            DJ_LAUNCH((k_broadcast<DJ_OP_SUBTRACT, false>), grid, kThreads, s, a, v, out, rows, cols); break;
+        case DJ_OP_DIVIDE_BROADCAST_COLS:
+            DJ_LAUNCH((k_broadcast<DJ_OP_DIVIDE, false>), grid, kThreads, s, a, v, out, rows, cols); break;
+        case DJ_OP_MULTIPLY_BROADCAST_COLS:
+            DJ_LAUNCH((k_broadcast<DJ_OP_MULTIPLY, false>), grid, kThreads, s, a, v, out, rows, cols); break;
+        default: fail("launch_broadcast: bad op");
+    }
+}
+
+void launch_transpose(hipStream_t s, const float *a, float *out, int rows, int cols) {
+    if (rows <= 0 || cols <= 0) return;
+    dim3 grid((cols + 31) / 32, (rows + 31) / 32);
+    hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, s, a, out, rows, cols);
+}
+
+void launch_adamw(hipStream_t s, float *w, const float *g, float *mt, float *vt, int64_t n, float lr, float beta1,
+                  float beta2, float eps, float wd, float bc1, float bc2) {
+    if (n <= 0) return;
+    DJ_LAUNCH(k_adamw, grid_for(n), kThreads, s, w, g, mt, vt, n, lr, beta1, beta2, eps, wd, bc1, bc2);
+}
+
+void launch_scatter_add(hipStream_t s, float *target, const float *idx, const float *grad, int target_rows, int cols,
+                        int n_idx) {
+    int64_t n = (int64_t)n_idx * cols;
+    if (n <= 0) return;
+    DJ_LAUNCH(k_scatter_add, grid_for(n), kThreads, s, target, idx, grad, target_rows, cols, n_idx);
+}
+
+void launch_fill(hipStream_t s, uint32_t *dst, uint32_t bits, int64_t n) {
+    if (n <= 0) return;
+    DJ_LAUNCH(k_fill, grid_for(n), kThreads, s, dst, bits, n);
+}
+
+void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n) {
+    if (n <= 0) return;
+    DJ_LAUNCH(k_copy, grid_for(n), kThreads, s, src, dst, n);
+}
+
+void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n) {
+    if (n <= 0) return;
+    DJ_LAUNCH(k_silu_mul, grid_for(n), kThreads, s, gate, up, out, n);
+}
+
+void launch_embed_gather(hipStream_t s, const float *table, const int32_t *ids, float *out, int n_ids, int d,
+                         int vocab) {
+    if (n_ids <= 0) return;
+    DJ_LAUNCH(k_embed_gather, n_ids, kThreads, s, table, ids, out, n_ids, d, vocab);
+}
+
+void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity) {
+    DJ_LAUNCH(k_decode_advance, 1, 64, s, state, token, tokens, capacity);
+}
+
+}  // namespace dj

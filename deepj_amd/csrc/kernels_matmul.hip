@@ -1,0 +1,165 @@
+// Dense contractions on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+//   C[M x N] = A[M x K] . B      A fp32 row-major, fp32 accumulate
+//
+// B is either fp32 [K x N] row-major (OP_MATMUL; CpuBackend.java:168-188 in the
+// reference) or a Q8 weight [N x Kp] int8 + one fp32 scale per 32-group, which is
+// dequantised while it is staged into LDS (prefill-time Q8 GEMM: a dense
+// contraction, so it belongs on MFMA; the M = 1 decode case is a separate
+// HBM-bound kernel in kernels_q8.hip).
+//
+// Tiling: 256 threads = 4 wavefronts, workgroup tile 64 x 64, each wavefront owns
+// one 32 x 32 accumulator (16 VGPRs), K advances 32 per step = one Q8 group.
+// Both operand tiles sit k-major in LDS so the 64 lanes of an MFMA operand read
+// 32 consecutive floats per half-wave (no bank conflicts).
+#include "dj_common.h"
+
+namespace dj {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BM = 64, BN = 64, BK = 32;
+constexpr int PAD = 4;
+
+struct GemmEpilogue {
+    const float *bias;      // [N] or null; with interleave: even col n -> bias[n/2], odd col -> bias2[n/2]
+    const float *bias2;
+    const float *residual;  // [M x N] or null
+    int interleaved_bias;
+};
+
+template <bool Q8>
+__global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const float *__restrict__ Bf,
+                                              const int8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                              float *__restrict__ C, int M, int N, int K, int kp,
+                                              GemmEpilogue ep) {
+    __shared__ float As[BK][BM + PAD];
+    __shared__ float Bl[BK][BN + PAD];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    floatx16 acc;
+#pragma unroll
+    for (int j = 0; j < 16; j++) acc[j] = 0.0f;
+
+    const int a_row = t >> 2;            // 0..63
+    const int a_k = (t & 3) * 8;         // 0,8,16,24
+    const bool a_vec = (K & 3) == 0;
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        // ── stage A: 64 rows x 32 k ────────────────────────────────────────
+        {
+            int gr = m0 + a_row;
+            float v[8];
+            if (gr < M && a_vec && k0 + a_k + 8 <= K) {
+                const float4 *p = reinterpret_cast<const float4 *>(A + (int64_t)gr * K + k0 + a_k);
+                float4 x = p[0], y = p[1];
+                v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w; v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    int gk = k0 + a_k + j;
+                    v[j] = (gr < M && gk < K) ? A[(int64_t)gr * K + gk] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) As[a_k + j][a_row] = v[j];
+        }
+        // ── stage B: 32 k x 64 cols ────────────────────────────────────────
+        if constexpr (Q8) {
+            int col = t >> 2, part = t & 3;          // 8 int8 per thread
+            int gn = n0 + col;
+            float w[8];
+            if (gn < N) {
+                const int8_t *p = Bq + (int64_t)gn * kp + k0 + part * 8;   // kp is a multiple of 32: in bounds
+                int2 raw = *reinterpret_cast<const int2 *>(p);
+                float sc = Bs[(int64_t)gn * (kp / kQ8Group) + k0 / kQ8Group];
+                int r0 = raw.x, r1 = raw.y;
+                w[0] = (float)(int8_t)(r0 & 0xff) * sc;         w[1] = (float)(int8_t)((r0 >> 8) & 0xff) * sc;
+                w[2] = (float)(int8_t)((r0 >> 16) & 0xff) * sc; w[3] = (float)(int8_t)((r0 >> 24) & 0xff) * sc;
+                w[4] = (float)(int8_t)(r1 & 0xff) * sc;         w[5] = (float)(int8_t)((r1 >> 8) & 0xff) * sc;
+                w[6] = (float)(int8_t)((r1 >> 16) & 0xff) * sc; w[7] = (float)(int8_t)((r1 >> 24) & 0xff) * sc;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) w[j] = 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) Bl[part * 8 + j][col] = w[j];
+        } else {
+            int bk = t >> 3, bn = (t & 7) * 8;       // 8 consecutive columns per thread
+            int gk = k0 + bk;
+            float w[8];
+            if (gk < K && (N & 3) == 0 && n0 + bn + 8 <= N) {
+                const float4 *p = reinterpret_cast<const float4 *>(Bf + (int64_t)gk * N + n0 + bn);
+                float4 x = p[0], y = p[1];
+                w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w; w[4] = y.x; w[5] = y.y; w[6] = y.z; w[7] = y.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    int gn = n0 + bn + j;
+                    w[j] = (gk < K && gn < N) ? Bf[(int64_t)gk * N + gn] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) Bl[bk][bn + j] = w[j];
+        }
+        __syncthreads();
+
+        // ── 16 MFMA steps of K = 2 ─────────────────────────────────────────
+        const int half = lane >> 5, l32 = lane & 31;
+#pragma unroll
+        for (int kk = 0; kk < BK / 2; kk++) {
+            float a = As[2 * kk + half][wm * 32 + l32];
+            float b = Bl[2 * kk + half][wn * 32 + l32];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // ── epilogue: acc[j] is C[8*(j/4) + 4*(lane/32) + j%4][lane%32] of the wave tile ──
+    const int col = n0 + wn * 32 + (lane & 31);
+    if (col < N) {
+        float badd = 0.0f;
+        if (ep.bias) badd = ep.interleaved_bias ? ((col & 1) ? ep.bias2[col >> 1] : ep.bias[col >> 1]) : ep.bias[col];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            int row = m0 + wm * 32 + 8 * (j >> 2) + 4 * (lane >> 5) + (j & 3);
+            if (row < M) {
+                float v = acc[j];
+                if (ep.bias) v = v + badd;
+                if (ep.residual) v = ep.residual[(int64_t)row * N + col] + v;
+                C[(int64_t)row * N + col] = v;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out, int m, int n, int k) {
+    if (m <= 0 || n <= 0) return;
+    if (k <= 0) { launch_fill(s, reinterpret_cast<uint32_t *>(out), 0u, (int64_t)m * n); return; }
+    dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM);
+    GemmEpilogue ep{nullptr, nullptr, nullptr, 0};
+    hipLaunchKernelGGL(k_gemm<false>, grid, dim3(256), 0, s, a, b, (const int8_t *)nullptr, (const float *)nullptr,
+                       out, m, n, k, 0, ep);
+}
+
+// Q8 GEMM used by launch_q8_linear for M > 1.  n_rows is the number of Q8 rows
+// (= output columns of this launch; 2N for an interleaved gate/up weight).
+void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
+                    int k, int n_rows, const float *bias, const float *bias2, const float *residual,
+                    int interleaved_bias) {
+    if (m <= 0 || n_rows <= 0) return;
+    dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
+    GemmEpilogue ep{bias, bias2, residual, interleaved_bias};
+    hipLaunchKernelGGL(k_gemm<true>, grid, dim3(256), 0, s, x, (const float *)nullptr, wq, scales, out, m, n_rows, k,
+                       q8_padded_k(k), ep);
+}
+
+}  // namespace dj

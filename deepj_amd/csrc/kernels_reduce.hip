@@ -1,0 +1,325 @@
+// Row/column reductions, softmax family, cross entropy, fused RMSNorm and argmax.
+// One 256-thread workgroup (4 wavefronts of 64) owns a row: lanes stride over the
+// row with coalesced loads, reduce inside the wavefront with DPP/shuffle steps,
+// then across the four wavefronts through 4 floats of LDS.  Reference semantics:
+// CpuBackend.java:220-294 (reductions), :360-464 (softmax, cross entropy),
+// :491-516 (layer-norm backward), RMSNorm1D.java:46-57.
+#include "dj_common.h"
+
+namespace dj {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Every thread of the block receives the result.
+__device__ __forceinline__ float block_sum(float v, float *lds) {
+    v = wave_sum(v);
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __syncthreads();                 // lds may still be read from a previous call
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    float r = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) r += lds[w];
+    return r;
+}
+__device__ __forceinline__ float block_max(float v, float *lds) {
+    v = wave_max(v);
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __syncthreads();
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    float r = lds[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) r = fmaxf(r, lds[w]);
+    return r;
+}
+
+__device__ __forceinline__ float d_exp(float x) { return (float)exp((double)x); }
+
+template <int OP>
+__global__ void __launch_bounds__(kThreads) k_row_reduce(const float *__restrict__ a, float *__restrict__ out,
+                                                         int rows, int cols) {
+    __shared__ float lds[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float *row = a + (int64_t)r * cols;
+        if constexpr (OP == DJ_OP_MAX_ALONG_ROWS) {
+            float m = -INFINITY;
+            for (int c = threadIdx.x; c < cols; c += kThreads) m = fmaxf(m, row[c]);
+            m = block_max(m, lds);
+            if (threadIdx.x == 0) out[r] = m;
+        } else if constexpr (OP == DJ_OP_VARIANCE_ALONG_ROWS) {
+            float s = 0.0f;
+            for (int c = threadIdx.x; c < cols; c += kThreads) s += row[c];
+            float inv = 1.0f / (float)cols;
+            float mean = block_sum(s, lds) * inv;
+            float acc = 0.0f;
+            for (int c = threadIdx.x; c < cols; c += kThreads) { float d = row[c] - mean; acc += d * d; }
+            acc = block_sum(acc, lds);
+            if (threadIdx.x == 0) out[r] = acc * inv;
+        } else {
+            float s = 0.0f;
+            for (int c = threadIdx.x; c < cols; c += kThreads) {
+                float x = row[c];
+                s += (OP == DJ_OP_SUM_ABS) ? fabsf(x) : x;
+            }
+            s = block_sum(s, lds);
+            if (threadIdx.x == 0) out[r] = (OP == DJ_OP_MEAN_ALONG_ROWS) ? s * (1.0f / (float)cols) : s;
+        }
+    }
+}
+
+// Column sums [rows x cols] -> [1 x cols]: 64 columns per workgroup (coalesced
+// 256 B rows), the four wavefronts take interleaved rows, LDS combines them.
+__global__ void __launch_bounds__(kThreads) k_sum_rows(const float *__restrict__ a, float *__restrict__ out, int rows,
+                                                       int cols) {
+    __shared__ float part[kWaves][64];
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int c = blockIdx.x * 64 + lane;
+    float s = 0.0f;
+    if (c < cols)
+        for (int r = wave; r < rows; r += kWaves) s += a[(int64_t)r * cols + c];
+    part[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && c < cols) out[c] = part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane];
+}
+
+// Whole-tensor sum into out[0]; one workgroup of 1024 threads (used for loss scalars).
+__global__ void __launch_bounds__(1024) k_sum_scalar(const float *__restrict__ a, float *__restrict__ out, int64_t n) {
+    __shared__ float lds[16];
+    float s = 0.0f;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) s += a[i];
+    s = wave_sum(s);
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) lds[wave] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float r = 0.0f;
+        for (int w = 0; w < 16; w++) r += lds[w];
+        out[0] = r;
+    }
+}
+
+// rowWriteSoftmax (CpuBackend.java:392-397): max, exp(x-max), sum of the same exps, divide.
+__global__ void __launch_bounds__(kThreads) k_softmax_rows(const float *__restrict__ a, float *__restrict__ out,
+                                                           int rows, int cols) {
+    __shared__ float lds[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float *row = a + (int64_t)r * cols;
+        float *orow = out + (int64_t)r * cols;
+        float m = -INFINITY;
+        for (int c = threadIdx.x; c < cols; c += kThreads) m = fmaxf(m, row[c]);
+        m = block_max(m, lds);
+        float s = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) {
+            float e = d_exp(row[c] - m);
+            orow[c] = e;
+            s += e;
+        }
+        s = block_sum(s, lds);
+        for (int c = threadIdx.x; c < cols; c += kThreads) orow[c] = orow[c] / s;
+    }
+}
+
+__global__ void __launch_bounds__(kThreads) k_softmax_backward(const float *__restrict__ g,
+                                                               const float *__restrict__ sm, float *__restrict__ out,
+                                                               int rows, int cols) {
+    __shared__ float lds[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        int64_t base = (int64_t)r * cols;
+        float dot = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) dot += g[base + c] * sm[base + c];
+        dot = block_sum(dot, lds);
+        for (int c = threadIdx.x; c < cols; c += kThreads) out[base + c] = sm[base + c] * (g[base + c] - dot);
+    }
+}
+
+__global__ void __launch_bounds__(kThreads) k_layernorm_backward(const float *__restrict__ dxhat,
+                                                                 const float *__restrict__ xhat,
+                                                                 const float *__restrict__ stdv,
+                                                                 float *__restrict__ out, int rows, int cols) {
+    __shared__ float lds[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        int64_t base = (int64_t)r * cols;
+        float inv_std = 1.0f / stdv[r];
+        float sd = 0.0f, sdx = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) {
+            float d = dxhat[base + c];
+            sd += d;
+            sdx += d * xhat[base + c];
+        }
+        sd = block_sum(sd, lds);
+        sdx = block_sum(sdx, lds);
+        float dim = (float)cols;
+        for (int c = threadIdx.x; c < cols; c += kThreads) {
+            float d = dxhat[base + c], xh = xhat[base + c];
+            out[base + c] = inv_std * (d - sd / dim - xh * (sdx / dim));
+        }
+    }
+}
+
+// Per-row loss log(sum exp(x-max)) + max - x[target] (GRAD=false, out [rows x 1]) or
+// (softmax - onehot)/rows (GRAD=true).  Targets arrive as floats; a target outside
+// [0, cols) yields NaN for that row, as the reference's GPU kernels do
+// (deepj_metal_jni.mm:472-476,497-503).
+template <bool GRAD>
+__global__ void __launch_bounds__(kThreads) k_cross_entropy(const float *__restrict__ logits,
+                                                            const float *__restrict__ targets,
+                                                            float *__restrict__ out, int rows, int cols) {
+    __shared__ float lds[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        int64_t base = (int64_t)r * cols;
+        float ft = targets[r];
+        bool ok = ft >= 0.0f && ft < (float)cols;
+        int target = ok ? (int)ft : 0;
+        float m = -INFINITY;
+        for (int c = threadIdx.x; c < cols; c += kThreads) m = fmaxf(m, logits[base + c]);
+        m = block_max(m, lds);
+        float s = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) s += d_exp(logits[base + c] - m);
+        s = block_sum(s, lds);
+        if constexpr (GRAD) {
+            float frows = (float)rows;
+            for (int c = threadIdx.x; c < cols; c += kThreads) {
+                float p = d_exp(logits[base + c] - m) / s;
+                if (c == target) p -= 1.0f;
+                out[base + c] = ok ? p / frows : __builtin_nanf("");
+            }
+        } else if (threadIdx.x == 0) {
+            out[r] = ok ? (float)log((double)s) + m - logits[base + target] : __builtin_nanf("");
+        }
+    }
+}
+
+// out = gamma * (x / sqrt(mean(x*x) + 1e-6)) in one pass over the row
+// (RMSNorm1D.java:46-57 folds six primitive ops and five temporaries into this).
+__global__ void __launch_bounds__(kThreads) k_rmsnorm(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                      float *__restrict__ out, int rows, int cols) {
+    __shared__ float lds[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float *row = x + (int64_t)r * cols;
+        float *orow = out + (int64_t)r * cols;
+        float s = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) { float v = row[c]; s += v * v; }
+        s = block_sum(s, lds);
+        float rms = sqrtf(s * (1.0f / (float)cols) + kRmsEps);
+        for (int c = threadIdx.x; c < cols; c += kThreads) orow[c] = (row[c] / rms) * gamma[c];
+    }
+}
+
+// Index of the row maximum, lowest index on ties: what topK=1 sampling reduces to
+// (TextGenerator.java:110-114,163-170: stable descending sort, first element).
+// NaN ranks above everything, as Float.compare orders it.
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
+    bool vn = v != v, bn = bv != bv;
+    if (vn != bn) return vn;
+    if (!vn && v != bv) return v > bv;
+    return i < bi;
+}
+__global__ void __launch_bounds__(kThreads) k_argmax_rows(const float *__restrict__ a, int32_t *__restrict__ out,
+                                                          int rows, int cols) {
+    __shared__ float sv[kWaves];
+    __shared__ int si[kWaves];
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float *row = a + (int64_t)r * cols;
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int c = threadIdx.x; c < cols; c += kThreads) {
+            float v = row[c];
+            if (better(v, c, bv, bi)) { bv = v; bi = c; }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            float ov = __shfl_xor(bv, off, 64);
+            int oi = __shfl_xor(bi, off, 64);
+            if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+        }
+        int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        __syncthreads();
+        if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < kWaves; w++)
+                if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+            out[r] = bi;
+        }
+    }
+}
+
+inline int row_grid(int rows) { return rows < 256 * 16 ? (rows < 1 ? 1 : rows) : 256 * 16; }
+
+}  // namespace
+
+void launch_row_reduce(hipStream_t s, int op, const float *a, float *out, int rows, int cols) {
+    if (rows <= 0) return;
+    dim3 grid(row_grid(rows)), block(kThreads);
+    switch (op) {
+        case DJ_OP_SUM_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_SUM_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_MEAN_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_MEAN_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_VARIANCE_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_VARIANCE_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_MAX_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_MAX_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_SUM_ABS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_SUM_ABS>, grid, block, 0, s, a, out, rows, cols); break;
+        default: fail("launch_row_reduce: bad op");
+    }
+}
+
+void launch_sum_rows(hipStream_t s, const float *a, float *out, int rows, int cols) {
+    if (cols <= 0) return;
+    hipLaunchKernelGGL(k_sum_rows, dim3((cols + 63) / 64), dim3(kThreads), 0, s, a, out, rows, cols);
+}
+
+void launch_sum_scalar(hipStream_t s, const float *a, float *out, int64_t n) {
+    hipLaunchKernelGGL(k_sum_scalar, dim3(1), dim3(1024), 0, s, a, out, n);
+}
+
+void launch_softmax_rows(hipStream_t s, const float *a, float *out, int rows, int cols) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(k_softmax_rows, dim3(row_grid(rows)), dim3(kThreads), 0, s, a, out, rows, cols);
+}
+
+void launch_softmax_backward(hipStream_t s, const float *g, const float *sm, float *out, int rows, int cols) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(k_softmax_backward, dim3(row_grid(rows)), dim3(kThreads), 0, s, g, sm, out, rows, cols);
+}
+
+void launch_layernorm_backward(hipStream_t s, const float *dxhat, const float *xhat, const float *stdv, float *out,
+                               int rows, int cols) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(k_layernorm_backward, dim3(row_grid(rows)), dim3(kThreads), 0, s, dxhat, xhat, stdv, out, rows,
+                       cols);
+}
+
+void launch_cross_entropy(hipStream_t s, bool gradient, const float *logits, const float *targets, float *out,
+                          int rows, int cols) {
+    if (rows <= 0) return;
+    if (gradient)
+        hipLaunchKernelGGL(k_cross_entropy<true>, dim3(row_grid(rows)), dim3(kThreads), 0, s, logits, targets, out,
+                           rows, cols);
+    else
+        hipLaunchKernelGGL(k_cross_entropy<false>, dim3(row_grid(rows)), dim3(kThreads), 0, s, logits, targets, out,
+                           rows, cols);
+}
+
+void launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int rows, int cols) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(k_rmsnorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, out, rows, cols);
+}
+
+void launch_argmax_rows(hipStream_t s, const float *a, int32_t *out, int rows, int cols) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(k_argmax_rows, dim3(row_grid(rows)), dim3(kThreads), 0, s, a, out, rows, cols);
+}
+
+}  // namespace dj

@@ -1,0 +1,801 @@
+// Device runtime behind the C ABI: the buffer/residency manager, the command-stream
+// interpreter and HIP-graph capture.  It takes the place of the reference's native
+// library (native/deepj_metal_jni.mm:1350-2140: gBufferPool + the opcode switch) and
+// keeps its observable contract: ids are chosen by the caller, allocating an existing
+// id and releasing an unknown id are no-ops, uploads copy the caller's array length,
+// and a stream is executed in program order.
+//
+// What is different by design:
+//  * Tensors stay resident in HBM between flushes; released buffers go to a
+//    size-class cache, so the "new output id + release the old id" pattern that
+//    in-place ops arrive as (MetalBackend.java:400-411) costs no hipMalloc/hipFree.
+//  * flush only enqueues on one in-order HIP stream; download is the single
+//    synchronisation point (the reference waits for the GPU in every flush,
+//    deepj_metal_jni.mm:2126-2127).
+//  * The whole stream is validated on the host - opcode, stride, ids, buffer sizes,
+//    shapes - before the first kernel is launched, so a malformed stream can never
+//    make a kernel touch memory it does not own.
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <unordered_map>
+#include <vector>
+
+#include "dj_common.h"
+
+namespace dj {
+namespace {
+
+struct Buffer {
+    void *ptr = nullptr;
+    size_t capacity = 0;      // bytes actually owned (size class)
+    int64_t floats = 0;       // size the caller asked for
+};
+
+struct Graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct Runtime {
+    bool ready = false;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::unordered_map<int32_t, Buffer> live;
+    std::map<size_t, std::vector<void *>> cache;   // size class -> free blocks
+    int64_t live_bytes = 0, cached_bytes = 0, driver_allocs = 0;
+    size_t cache_limit = (size_t)16 << 30;
+    float *workspace = nullptr;
+    int64_t workspace_floats = 0;
+    void *staging = nullptr;                       // pinned, for small uploads/downloads
+    size_t staging_bytes = 0;
+    bool capturing = false;
+    std::unordered_map<int32_t, Graph> graphs;
+    int32_t next_graph = 1;
+};
+
+Runtime g;
+thread_local std::string g_error;
+
+void ensure_init(int device = 0) {
+    if (g.ready) return;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) fail("deepj_hip: no HIP device available");
+    if (device < 0 || device >= count) fail("deepj_hip: bad device index " + std::to_string(device));
+    DJ_HIP(hipSetDevice(device));
+    DJ_HIP(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
+    g.staging_bytes = (size_t)1 << 20;
+    DJ_HIP(hipHostMalloc(&g.staging, g.staging_bytes, hipHostMallocDefault));
+    g.device = device;
+    g.ready = true;
+}
+
+// 256 B granularity up to 64 KiB, then four classes per power of two (<= 25 % slack).
+size_t size_class(size_t bytes) {
+    if (bytes < 256) return 256;
+    if (bytes <= (64u << 10)) return (bytes + 255) & ~(size_t)255;
+    size_t p = (size_t)1 << (63 - __builtin_clzll(bytes));      // largest power of two <= bytes
+    if (p == bytes) return bytes;
+    size_t step = p >> 2;
+    return (bytes + step - 1) / step * step;
+}
+
+void *pool_alloc(size_t cls) {
+    auto it = g.cache.find(cls);
+    if (it != g.cache.end() && !it->second.empty()) {
+        void *p = it->second.back();
+        it->second.pop_back();
+        g.cached_bytes -= (int64_t)cls;
+        return p;
+    }
+    if (g.capturing) fail("deepj_hip: device allocation requested while a graph is being captured");
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, cls);
+    if (e != hipSuccess) {
+        // give cached blocks back to the driver and retry once
+        (void)hipGetLastError();
+        DJ_HIP(hipStreamSynchronize(g.stream));
+        for (auto &kv : g.cache) {
+            for (void *q : kv.second) (void)hipFree(q);
+            kv.second.clear();
+        }
+        g.cached_bytes = 0;
+        e = hipMalloc(&p, cls);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            fail("Failed to allocate HIP buffer of " + std::to_string(cls) + " bytes: " + hipGetErrorString(e));
+        }
+    }
+    g.driver_allocs++;
+    return p;
+}
+
+void pool_free(void *p, size_t cls) {
+    // Work already queued on the stream may still use the block; any later user is
+    // queued behind it on the same in-order stream, so recycling needs no wait.
+    if ((size_t)g.cached_bytes + cls > g.cache_limit) {
+        DJ_HIP(hipStreamSynchronize(g.stream));
+        DJ_HIP(hipFree(p));
+        return;
+    }
+    g.cache[cls].push_back(p);
+    g.cached_bytes += (int64_t)cls;
+}
+
+void ensure_workspace(int64_t floats) {
+    if (floats <= g.workspace_floats) return;
+    if (g.capturing) fail("deepj_hip: workspace would have to grow during graph capture; run the stream once first");
+    DJ_HIP(hipStreamSynchronize(g.stream));
+    if (g.workspace) DJ_HIP(hipFree(g.workspace));
+    g.workspace = nullptr;
+    g.workspace_floats = 0;
+    int64_t want = std::max<int64_t>(floats, (int64_t)1 << 20);
+    DJ_HIP(hipMalloc((void **)&g.workspace, (size_t)want * 4));
+    g.driver_allocs++;
+    g.workspace_floats = want;
+}
+
+// ── stream interpreter ──────────────────────────────────────────────────────
+
+struct Cursor {
+    const int32_t *cmd;
+    int32_t len;
+    int32_t pos;
+    bool dry;          // validate only
+    int64_t ws_need;   // workspace floats the stream needs (collected in the dry pass)
+};
+
+const char *op_name(int op);
+
+int stride_of(int op) {
+    switch (op) {
+        case DJ_OP_SQRT: case DJ_OP_NEG: case DJ_OP_EXP: case DJ_OP_LOG: case DJ_OP_TANH: case DJ_OP_SIGMOID:
+        case DJ_OP_RELU: case DJ_OP_GELU:
+            return 4;
+        case DJ_OP_ADD: case DJ_OP_SUBTRACT: case DJ_OP_MULTIPLY: case DJ_OP_DIVIDE: case DJ_OP_RELU_BACKWARD:
+        case DJ_OP_GELU_BACKWARD: case DJ_OP_MULTIPLY_SCALAR: case DJ_OP_ADD_SCALAR: case DJ_OP_DIVIDE_SCALAR:
+        case DJ_OP_TRANSPOSE: case DJ_OP_SUM_ROWS: case DJ_OP_MEAN_ALONG_ROWS: case DJ_OP_VARIANCE_ALONG_ROWS:
+        case DJ_OP_SUM_ALONG_ROWS: case DJ_OP_MAX_ALONG_ROWS: case DJ_OP_SOFTMAX_ROWS: case DJ_OP_POW:
+        case DJ_OP_SUM_ABS: case DJ_OP_SUM_SCALAR:
+            return 5;
+        case DJ_OP_CLAMP: case DJ_OP_CROSS_ENTROPY_LOSS: case DJ_OP_CROSS_ENTROPY_GRADIENT:
+        case DJ_OP_SOFTMAX_BACKWARD: case DJ_OP_ADD_ROW_VECTOR: case DJ_OP_ADD_BROADCAST_COLS:
+        case DJ_OP_SUBTRACT_BROADCAST_COLS: case DJ_OP_DIVIDE_BROADCAST_COLS: case DJ_OP_MULTIPLY_BROADCAST_ROWS:
+        case DJ_OP_MULTIPLY_BROADCAST_COLS:
+            return 6;
+        case DJ_OP_MATMUL: case DJ_OP_LAYERNORM_BACKWARD: case DJ_OP_SCATTER_ADD_ROWS:
+        case DJ_OP_SCATTER_ADD_ROWS_ATOMIC:
+            return 7;
+        case DJ_OP_ADAMW_UPDATE: return 13;
+        case DJ_OP_Q8_QUANTIZE: case DJ_OP_Q8_DEQUANTIZE: return 8;
+        case DJ_OP_Q8_LINEAR: return 12;
+        case DJ_OP_RMSNORM: return 6;
+        case DJ_OP_SILU_MUL: return 5;
+        case DJ_OP_EMBED_GATHER: return 8;
+        case DJ_OP_ROPE_KV_STORE: return 13;
+        case DJ_OP_ATTENTION: return 12;
+        case DJ_OP_ARGMAX_ROWS: return 5;
+        case DJ_OP_DECODE_ADVANCE: return 5;
+        case DJ_OP_COPY: return 6;
+        case DJ_OP_FILL: return 4;
+        case DJ_OP_ROPE_ROWS: return 11;
+        case DJ_OP_ATTENTION_KV: return 12;
+        default: return -1;
+    }
+}
+
+float bits_to_float(int32_t b) { float f; std::memcpy(&f, &b, 4); return f; }
+
+// Pointer to buffer `id`, after checking that it exists and holds >= floats floats.
+float *buf(int32_t id, int64_t floats, int op, const char *role) {
+    auto it = g.live.find(id);
+    if (it == g.live.end())
+        fail(std::string(op_name(op)) + ": missing GPU buffer id=" + std::to_string(id) + " (" + role + ")");
+    if (floats < 0 || floats > it->second.floats)
+        fail(std::string(op_name(op)) + ": buffer id=" + std::to_string(id) + " (" + role + ") holds " +
+             std::to_string(it->second.floats) + " floats, op needs " + std::to_string(floats));
+    return static_cast<float *>(it->second.ptr);
+}
+float *buf_opt(int32_t id, int64_t floats, int op, const char *role) {
+    return id < 0 ? nullptr : buf(id, floats, op, role);
+}
+
+void need_positive(int op, const char *what, int64_t v) {
+    if (v < 0) fail(std::string(op_name(op)) + ": negative " + what + " " + std::to_string(v));
+}
+
+void exec_one(Cursor &c) {
+    const int32_t *w = c.cmd + c.pos;
+    const int op = w[0];
+    hipStream_t s = g.stream;
+    const bool run = !c.dry;
+    switch (op) {
+        case DJ_OP_ADD: case DJ_OP_SUBTRACT: case DJ_OP_MULTIPLY: case DJ_OP_DIVIDE: case DJ_OP_RELU_BACKWARD:
+        case DJ_OP_GELU_BACKWARD: {
+            int64_t n = w[4]; need_positive(op, "n", n);
+            const float *a = buf(w[1], n, op, "a"), *b = buf(w[2], n, op, "b");
+            float *o = buf(w[3], n, op, "out");
+            if (run) launch_binary(s, op, a, b, o, n);
+            break;
+        }
+        case DJ_OP_SQRT: case DJ_OP_NEG: case DJ_OP_EXP: case DJ_OP_LOG: case DJ_OP_TANH: case DJ_OP_SIGMOID:
+        case DJ_OP_RELU: case DJ_OP_GELU: {
+            int64_t n = w[3]; need_positive(op, "n", n);
+            const float *a = buf(w[1], n, op, "in");
+            float *o = buf(w[2], n, op, "out");
+            if (run) launch_unary(s, op, a, o, n);
+            break;
+        }
+        case DJ_OP_MULTIPLY_SCALAR: case DJ_OP_ADD_SCALAR: case DJ_OP_DIVIDE_SCALAR: case DJ_OP_POW: {
+            int64_t n = w[4]; need_positive(op, "n", n);
+            const float *a = buf(w[1], n, op, "in");
+            float *o = buf(w[2], n, op, "out");
+            if (run) launch_scalar(s, op, a, o, bits_to_float(w[3]), 0.0f, n);
+            break;
+        }
+        case DJ_OP_CLAMP: {
+            int64_t n = w[5]; need_positive(op, "n", n);
+            const float *a = buf(w[1], n, op, "in");
+            float *o = buf(w[2], n, op, "out");
+            if (run) launch_scalar(s, op, a, o, bits_to_float(w[3]), bits_to_float(w[4]), n);
+            break;
+        }
+        case DJ_OP_MATMUL: {
+            int64_t m = w[4], n = w[5], k = w[6];
+            need_positive(op, "m", m); need_positive(op, "n", n); need_positive(op, "k", k);
+            const float *a = buf(w[1], m * k, op, "a"), *b = buf(w[2], k * n, op, "b");
+            float *o = buf(w[3], m * n, op, "out");
+            if (run) launch_matmul_f32(s, a, b, o, (int)m, (int)n, (int)k);
+            break;
+        }
+        case DJ_OP_TRANSPOSE: {
+            int64_t rows = w[3], cols = w[4]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *a = buf(w[1], rows * cols, op, "in");
+            float *o = buf(w[2], rows * cols, op, "out");
+            if (run) launch_transpose(s, a, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_ADD_ROW_VECTOR: case DJ_OP_MULTIPLY_BROADCAST_ROWS: case DJ_OP_ADD_BROADCAST_COLS:
+        case DJ_OP_SUBTRACT_BROADCAST_COLS: case DJ_OP_DIVIDE_BROADCAST_COLS: case DJ_OP_MULTIPLY_BROADCAST_COLS: {
+            int64_t rows = w[4], cols = w[5]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            bool rowvec = (op == DJ_OP_ADD_ROW_VECTOR || op == DJ_OP_MULTIPLY_BROADCAST_ROWS);
+            const float *a = buf(w[1], rows * cols, op, "a");
+            const float *v = buf(w[2], rowvec ? cols : rows, op, "vector");
+            float *o = buf(w[3], rows * cols, op, "out");
+            if (run) launch_broadcast(s, op, a, v, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_SUM_ROWS: {
+            int64_t rows = w[3], cols = w[4]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *a = buf(w[1], rows * cols, op, "in");
+            float *o = buf(w[2], cols, op, "out");
+            if (run) launch_sum_rows(s, a, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_SUM_ALONG_ROWS: case DJ_OP_MEAN_ALONG_ROWS: case DJ_OP_VARIANCE_ALONG_ROWS:
+        case DJ_OP_MAX_ALONG_ROWS: case DJ_OP_SUM_ABS: {
+            int64_t rows = w[3], cols = w[4]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *a = buf(w[1], rows * cols, op, "in");
+            float *o = buf(w[2], rows, op, "out");
+            if (run) launch_row_reduce(s, op, a, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_SUM_SCALAR: {
+            int64_t rows = w[3], cols = w[4]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *a = buf(w[1], rows * cols, op, "in");
+            float *o = buf(w[2], 1, op, "out");
+            if (run) launch_sum_scalar(s, a, o, rows * cols);
+            break;
+        }
+        case DJ_OP_SOFTMAX_ROWS: {
+            int64_t rows = w[3], cols = w[4]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *a = buf(w[1], rows * cols, op, "in");
+            float *o = buf(w[2], rows * cols, op, "out");
+            if (run) launch_softmax_rows(s, a, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_SOFTMAX_BACKWARD: {
+            int64_t rows = w[4], cols = w[5]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *gr = buf(w[1], rows * cols, op, "grad"), *sm = buf(w[2], rows * cols, op, "softmax");
+            float *o = buf(w[3], rows * cols, op, "out");
+            if (run) launch_softmax_backward(s, gr, sm, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_LAYERNORM_BACKWARD: {
+            int64_t rows = w[5], cols = w[6]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *dx = buf(w[1], rows * cols, op, "dXHat"), *xh = buf(w[2], rows * cols, op, "xHat");
+            const float *sd = buf(w[3], rows, op, "std");
+            float *o = buf(w[4], rows * cols, op, "out");
+            if (run) launch_layernorm_backward(s, dx, xh, sd, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_ADAMW_UPDATE: {
+            int64_t n = w[12]; need_positive(op, "n", n);
+            float *wt = buf(w[1], n, op, "w");
+            const float *gr = buf(w[2], n, op, "g");
+            float *mt = buf(w[3], n, op, "mt"), *vt = buf(w[4], n, op, "vt");
+            if (run)
+                launch_adamw(s, wt, gr, mt, vt, n, bits_to_float(w[5]), bits_to_float(w[6]), bits_to_float(w[7]),
+                             bits_to_float(w[8]), bits_to_float(w[9]), bits_to_float(w[10]), bits_to_float(w[11]));
+            break;
+        }
+        case DJ_OP_SCATTER_ADD_ROWS: case DJ_OP_SCATTER_ADD_ROWS_ATOMIC: {
+            // Both opcodes accumulate atomically: the non-atomic variant is racy for
+            // duplicate indices by construction (deepj_metal_jni.mm:559-577).
+            int64_t trows = w[4], tcols = w[5], nidx = w[6];
+            need_positive(op, "rows", trows); need_positive(op, "cols", tcols); need_positive(op, "indices", nidx);
+            float *t = buf(w[1], trows * tcols, op, "target");
+            const float *idx = buf(w[2], nidx, op, "indices");
+            const float *gr = buf(w[3], nidx * tcols, op, "grad");
+            if (run) launch_scatter_add(s, t, idx, gr, (int)trows, (int)tcols, (int)nidx);
+            break;
+        }
+        case DJ_OP_CROSS_ENTROPY_LOSS: case DJ_OP_CROSS_ENTROPY_GRADIENT: {
+            int64_t rows = w[4], cols = w[5]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            bool grad = op == DJ_OP_CROSS_ENTROPY_GRADIENT;
+            const float *lg = buf(w[1], rows * cols, op, "logits"), *tg = buf(w[2], rows, op, "targets");
+            float *o = buf(w[3], grad ? rows * cols : rows, op, "out");
+            if (run) launch_cross_entropy(s, grad, lg, tg, o, (int)rows, (int)cols);
+            break;
+        }
+
+        // ── fused inference opcodes ────────────────────────────────────────
+        case DJ_OP_Q8_QUANTIZE: case DJ_OP_Q8_DEQUANTIZE: {
+            int64_t k = w[3], n = w[4], off = w[5], step = w[6], total = w[7];
+            if (k <= 0 || n <= 0 || total <= 0 || step <= 0 || off < 0) fail(std::string(op_name(op)) + ": bad shape");
+            if (off + (n - 1) * step >= total) fail(std::string(op_name(op)) + ": rows fall outside the Q8 buffer");
+            int64_t qfloats = (q8_bytes((int)k, (int)total) + 3) / 4;
+            bool quant = op == DJ_OP_Q8_QUANTIZE;
+            float *src = buf(w[1], quant ? k * n : qfloats, op, "src");
+            float *dst = buf(w[2], quant ? qfloats : k * n, op, "dst");
+            if (run) {
+                if (quant) {
+                    int8_t *q = reinterpret_cast<int8_t *>(dst);
+                    float *sc = reinterpret_cast<float *>(q + q8_scale_offset_bytes((int)k, (int)total));
+                    launch_q8_quantize(s, src, q, sc, (int)k, (int)n, (int)off, (int)step);
+                } else {
+                    const int8_t *q = reinterpret_cast<const int8_t *>(src);
+                    const float *sc = reinterpret_cast<const float *>(q + q8_scale_offset_bytes((int)k, (int)total));
+                    launch_q8_dequantize(s, q, sc, dst, (int)k, (int)n, (int)off, (int)step);
+                }
+            }
+            break;
+        }
+        case DJ_OP_Q8_LINEAR: {
+            int64_t m = w[4], k = w[5], n = w[6];
+            int flags = w[7];
+            if (m <= 0 || k <= 0 || n <= 0) fail("OP_Q8_LINEAR: bad shape");
+            if (flags & ~15) fail("OP_Q8_LINEAR: unknown flag bits");
+            bool sw = flags & DJ_LIN_SWIGLU;
+            if (sw && (flags & DJ_LIN_RESIDUAL)) fail("OP_Q8_LINEAR: SWIGLU cannot be combined with RESIDUAL");
+            int64_t rows = sw ? 2 * n : n;
+            Q8Linear p;
+            p.x = buf(w[1], m * k, op, "x");
+            const float *wq = buf(w[2], (q8_bytes((int)k, (int)rows) + 3) / 4, op, "weight");
+            p.wq = reinterpret_cast<const int8_t *>(wq);
+            p.scales = reinterpret_cast<const float *>(p.wq + q8_scale_offset_bytes((int)k, (int)rows));
+            p.out = buf(w[3], m * n, op, "out");
+            p.m = (int)m; p.k = (int)k; p.n = (int)n; p.flags = flags;
+            p.gamma = (flags & DJ_LIN_RMSNORM) ? buf(w[8], k, op, "gamma") : nullptr;
+            p.bias = (flags & DJ_LIN_BIAS) ? buf(w[9], n, op, "bias") : nullptr;
+            p.bias2 = ((flags & DJ_LIN_BIAS) && sw) ? buf(w[10], n, op, "bias2") : nullptr;
+            p.residual = (flags & DJ_LIN_RESIDUAL) ? buf(w[11], m * n, op, "residual") : nullptr;
+            int64_t ws = q8_linear_workspace_floats((int)m, (int)k, (int)n, flags);
+            if (c.dry) c.ws_need = std::max(c.ws_need, ws);
+            if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
+            break;
+        }
+        case DJ_OP_RMSNORM: {
+            int64_t rows = w[4], cols = w[5]; need_positive(op, "rows", rows); need_positive(op, "cols", cols);
+            const float *x = buf(w[1], rows * cols, op, "x"), *gm = buf(w[2], cols, op, "gamma");
+            float *o = buf(w[3], rows * cols, op, "out");
+            if (run) launch_rmsnorm(s, x, gm, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_SILU_MUL: {
+            int64_t n = w[4]; need_positive(op, "n", n);
+            const float *a = buf(w[1], n, op, "gate"), *b = buf(w[2], n, op, "up");
+            float *o = buf(w[3], n, op, "out");
+            if (run) launch_silu_mul(s, a, b, o, n);
+            break;
+        }
+        case DJ_OP_EMBED_GATHER: {
+            int64_t nids = w[4], d = w[5], vocab = w[6], ids_off = w[7];
+            if (nids < 0 || d <= 0 || vocab <= 0 || ids_off < 0) fail("OP_EMBED_GATHER: bad shape");
+            const float *t = buf(w[1], vocab * d, op, "table");
+            const float *ids = buf(w[2], ids_off + nids, op, "ids");
+            float *o = buf(w[3], nids * d, op, "out");
+            if (run)
+                launch_embed_gather(s, t, reinterpret_cast<const int32_t *>(ids) + ids_off, o, (int)nids, (int)d,
+                                    (int)vocab);
+            break;
+        }
+        case DJ_OP_ROPE_KV_STORE: {
+            int64_t S = w[8], H = w[9], hd = w[10], max_seq = w[11], layer = w[12];
+            if (S <= 0 || H <= 0 || hd <= 0 || (hd & 3) || max_seq <= 0 || layer < 0) fail("OP_ROPE_KV_STORE: bad shape");
+            int64_t d = H * hd, per_layer = H * max_seq * hd;
+            const float *qkv = buf(w[1], S * 3 * d, op, "qkv");
+            float *q_out = buf(w[2], S * d, op, "qOut");
+            float *kc = buf(w[3], (layer + 1) * per_layer, op, "kCache");
+            float *vc = buf(w[4], (layer + 1) * per_layer, op, "vCache");
+            const float *st = buf(w[5], 4, op, "state");
+            const float *ct = buf(w[6], max_seq * (hd / 2), op, "cos"), *sn = buf(w[7], max_seq * (hd / 2), op, "sin");
+            if (run)
+                launch_rope_kv_store(s, qkv, q_out, kc + layer * per_layer, vc + layer * per_layer,
+                                     reinterpret_cast<const int32_t *>(st), ct, sn, (int)S, (int)H, (int)hd,
+                                     (int)max_seq);
+            break;
+        }
+        case DJ_OP_ROPE_ROWS: {
+            // [op, x, out, state, cos, sin, rows, H, hd, maxSeq, posFromRow]
+            int64_t rows = w[6], H = w[7], hd = w[8], max_seq = w[9];
+            if (rows <= 0 || H <= 0 || hd <= 0 || (hd & 1) || max_seq <= 0) fail("OP_ROPE_ROWS: bad shape");
+            if (w[10] && rows > max_seq) fail("OP_ROPE_ROWS: more rows than RoPE table positions");
+            const float *x = buf(w[1], rows * H * hd, op, "x");
+            float *o = buf(w[2], rows * H * hd, op, "out");
+            const float *st = buf(w[3], 4, op, "state");
+            const float *ct = buf(w[4], max_seq * (hd / 2), op, "cos"), *sn = buf(w[5], max_seq * (hd / 2), op, "sin");
+            if (run)
+                launch_rope_rows(s, x, o, reinterpret_cast<const int32_t *>(st), ct, sn, (int)rows, (int)H, (int)hd,
+                                 (int)max_seq, w[10]);
+            break;
+        }
+        case DJ_OP_ATTENTION: case DJ_OP_ATTENTION_KV: {
+            // ATTENTION    [op, q, kCache, vCache, out, state, scratch, S, H, hd, maxSeq, layer]  head-major cache
+            // ATTENTION_KV [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0]  k,v token-major [maxSeq x H*hd]
+            int64_t S = w[7], H = w[8], hd = w[9], max_seq = w[10], layer = w[11];
+            if (S <= 0 || H <= 0 || max_seq <= 0 || layer < 0) fail(std::string(op_name(op)) + ": bad shape");
+            if (hd != 32 && hd != 64 && hd != 128) fail(std::string(op_name(op)) + ": head dim must be 32, 64 or 128");
+            int64_t d = H * hd, per_layer = H * max_seq * hd;
+            AttnArgs a;
+            a.q = buf(w[1], S * d, op, "q");
+            bool cache = op == DJ_OP_ATTENTION;
+            if (!cache && layer != 0) fail("OP_ATTENTION_KV: layer must be 0");
+            const float *kc = buf(w[2], (layer + 1) * per_layer, op, "k");
+            const float *vc = buf(w[3], (layer + 1) * per_layer, op, "v");
+            a.k = kc + layer * per_layer; a.v = vc + layer * per_layer;
+            a.k_tok_stride = cache ? hd : d;
+            a.k_head_stride = cache ? max_seq * hd : hd;
+            a.out = buf(w[4], S * d, op, "out");
+            a.state = reinterpret_cast<const int32_t *>(buf(w[5], 4, op, "state"));
+            int64_t sf = attention_scratch_floats((int)S, (int)H, (int)hd, (int)max_seq);
+            a.scratch = sf > 0 ? buf(w[6], sf, op, "scratch") : nullptr;
+            a.scratch_floats = sf;
+            a.s = (int)S; a.h = (int)H; a.hd = (int)hd; a.max_seq = (int)max_seq;
+            if (run) launch_attention(s, a);
+            break;
+        }
+        case DJ_OP_ARGMAX_ROWS: {
+            int64_t rows = w[3], cols = w[4];
+            if (rows <= 0 || cols <= 0) fail("OP_ARGMAX_ROWS: bad shape");
+            const float *a = buf(w[1], rows * cols, op, "logits");
+            float *o = buf(w[2], rows, op, "out");
+            if (run) launch_argmax_rows(s, a, reinterpret_cast<int32_t *>(o), (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_DECODE_ADVANCE: {
+            // [op, state, token, tokens, capacity]
+            int64_t cap = w[4]; need_positive(op, "capacity", cap);
+            float *st = buf(w[1], 4, op, "state");
+            const float *tk = buf(w[2], 1, op, "token");
+            float *out = buf(w[3], std::max<int64_t>(cap, 1), op, "tokens");
+            if (run)
+                launch_decode_advance(s, reinterpret_cast<int32_t *>(st), reinterpret_cast<const int32_t *>(tk),
+                                      reinterpret_cast<int32_t *>(out), (int)cap);
+            break;
+        }
+        case DJ_OP_COPY: {
+            int64_t n = w[3], so = w[4], dof = w[5];
+            if (n < 0 || so < 0 || dof < 0) fail("OP_COPY: bad range");
+            const float *a = buf(w[1], so + n, op, "src");
+            float *o = buf(w[2], dof + n, op, "dst");
+            if (run) launch_copy(s, a + so, o + dof, n);
+            break;
+        }
+        case DJ_OP_FILL: {
+            int64_t n = w[3]; need_positive(op, "n", n);
+            float *o = buf(w[1], n, op, "dst");
+            if (run) launch_fill(s, reinterpret_cast<uint32_t *>(o), (uint32_t)w[2], n);
+            break;
+        }
+        default:
+            fail("Unknown op code in graph: " + std::to_string(op));
+    }
+}
+
+void walk(const int32_t *cmd, int32_t len, bool dry, int64_t *ws_need) {
+    Cursor c{cmd, len, 0, dry, 0};
+    while (c.pos < len) {
+        int op = cmd[c.pos];
+        int stride = stride_of(op);
+        if (stride < 0) fail("Unknown op code in graph: " + std::to_string(op));
+        if (c.pos + stride > len)
+            fail(std::string(op_name(op)) + ": command stream truncated at word " + std::to_string(c.pos));
+        exec_one(c);
+        c.pos += stride;
+    }
+    if (ws_need) *ws_need = c.ws_need;
+}
+
+void run_stream(const int32_t *cmd, int32_t len) {
+    if (len < 0) fail("flushOps: negative stream length");
+    if (len > 0 && !cmd) fail("flushOps: null command stream");
+    int64_t ws = 0;
+    walk(cmd, len, true, &ws);      // validate everything first
+    ensure_workspace(ws);
+    walk(cmd, len, false, nullptr);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) fail(std::string("kernel launch failed: ") + hipGetErrorString(e));
+}
+
+const char *op_name(int op) {
+    static const char *names[] = {
+        "?", "OP_ADD", "OP_SUBTRACT", "OP_MULTIPLY", "OP_DIVIDE", "OP_MATMUL", "OP_MULTIPLY_SCALAR", "OP_SQRT",
+        "OP_NEG", "OP_EXP", "OP_LOG", "OP_TANH", "OP_SIGMOID", "OP_RELU", "OP_RELU_BACKWARD", "OP_GELU",
+        "OP_GELU_BACKWARD", "OP_SOFTMAX_ROWS", "OP_SOFTMAX_BACKWARD", "OP_LAYERNORM_BACKWARD", "OP_ADAMW_UPDATE",
+        "OP_ADD_SCALAR", "OP_DIVIDE_SCALAR", "OP_TRANSPOSE", "OP_ADD_ROW_VECTOR", "OP_ADD_BROADCAST_COLS",
+        "OP_SUBTRACT_BROADCAST_COLS", "OP_DIVIDE_BROADCAST_COLS", "OP_MULTIPLY_BROADCAST_ROWS", "OP_SUM_ROWS",
+        "OP_MEAN_ALONG_ROWS", "OP_VARIANCE_ALONG_ROWS", "OP_MULTIPLY_BROADCAST_COLS", "OP_SUM_ALONG_ROWS",
+        "OP_MAX_ALONG_ROWS", "OP_CLAMP", "OP_POW", "OP_SCATTER_ADD_ROWS", "OP_SUM_ABS", "OP_CROSS_ENTROPY_LOSS",
+        "OP_CROSS_ENTROPY_GRADIENT", "OP_SUM_SCALAR", "OP_SCATTER_ADD_ROWS_ATOMIC"};
+    if (op >= 1 && op <= 42) return names[op];
+    switch (op) {
+        case DJ_OP_Q8_QUANTIZE: return "OP_Q8_QUANTIZE";
+        case DJ_OP_Q8_DEQUANTIZE: return "OP_Q8_DEQUANTIZE";
+        case DJ_OP_Q8_LINEAR: return "OP_Q8_LINEAR";
+        case DJ_OP_RMSNORM: return "OP_RMSNORM";
+        case DJ_OP_SILU_MUL: return "OP_SILU_MUL";
+        case DJ_OP_EMBED_GATHER: return "OP_EMBED_GATHER";
+        case DJ_OP_ROPE_KV_STORE: return "OP_ROPE_KV_STORE";
+        case DJ_OP_ATTENTION: return "OP_ATTENTION";
+        case DJ_OP_ARGMAX_ROWS: return "OP_ARGMAX_ROWS";
+        case DJ_OP_DECODE_ADVANCE: return "OP_DECODE_ADVANCE";
+        case DJ_OP_COPY: return "OP_COPY";
+        case DJ_OP_FILL: return "OP_FILL";
+        case DJ_OP_ROPE_ROWS: return "OP_ROPE_ROWS";
+        case DJ_OP_ATTENTION_KV: return "OP_ATTENTION_KV";
+        default: return "OP_?";
+    }
+}
+
+template <class F> int guarded(F &&f) {
+    try {
+        f();
+        g_error.clear();
+        return 0;
+    } catch (const std::exception &ex) {
+        g_error = ex.what();
+        return 1;
+    } catch (...) {
+        g_error = "deepj_hip: unknown native error";
+        return 1;
+    }
+}
+
+}  // namespace
+}  // namespace dj
+
+using namespace dj;
+
+extern "C" {
+
+int deepj_hip_init(int32_t device) {
+    return guarded([&] { ensure_init(device); });
+}
+
+int deepj_hip_alloc_buffers(const int32_t *ids, const int32_t *sizes, int32_t count) {
+    return guarded([&] {
+        ensure_init();
+        if (count < 0) fail("allocBuffers: negative count");
+        if (count > 0 && (!ids || !sizes)) fail("allocBuffers: null array");
+        for (int i = 0; i < count; i++) {
+            if (g.live.count(ids[i])) continue;          // existing id: silent no-op
+            if (sizes[i] < 0) fail("allocBuffers: negative size for id " + std::to_string(ids[i]));
+            size_t bytes = (size_t)sizes[i] * 4;
+            size_t cls = size_class(bytes);
+            Buffer b;
+            b.ptr = pool_alloc(cls);
+            b.capacity = cls;
+            b.floats = sizes[i];
+            g.live.emplace(ids[i], b);
+            g.live_bytes += (int64_t)cls;
+        }
+    });
+}
+
+int deepj_hip_upload(int32_t id, const float *src, int64_t n) {
+    return guarded([&] {
+        ensure_init();
+        auto it = g.live.find(id);
+        if (it == g.live.end()) fail("Buffer not found for upload");
+        if (n < 0 || n > it->second.floats)
+            fail("uploadBuffer: " + std::to_string(n) + " floats do not fit buffer id=" + std::to_string(id) + " of " +
+                 std::to_string(it->second.floats));
+        if (n == 0) return;
+        if (!src) fail("uploadBuffer: null source");
+        size_t bytes = (size_t)n * 4;
+        // The caller's array is only borrowed: the copy out of it has finished on return.
+        if (bytes <= g.staging_bytes) {
+            DJ_HIP(hipStreamSynchronize(g.stream));      // staging block may still be in flight
+            std::memcpy(g.staging, src, bytes);
+            DJ_HIP(hipMemcpyAsync(it->second.ptr, g.staging, bytes, hipMemcpyHostToDevice, g.stream));
+        } else {
+            DJ_HIP(hipMemcpyAsync(it->second.ptr, src, bytes, hipMemcpyHostToDevice, g.stream));
+            DJ_HIP(hipStreamSynchronize(g.stream));
+        }
+    });
+}
+
+int deepj_hip_download(int32_t id, float *dst, int64_t n) {
+    return guarded([&] {
+        ensure_init();
+        auto it = g.live.find(id);
+        if (it == g.live.end()) fail("Buffer not found for download");
+        if (n < 0 || n > it->second.floats)
+            fail("downloadBuffer: " + std::to_string(n) + " floats exceed buffer id=" + std::to_string(id) + " of " +
+                 std::to_string(it->second.floats));
+        if (n > 0 && !dst) fail("downloadBuffer: null destination");
+        if (n > 0) DJ_HIP(hipMemcpyAsync(dst, it->second.ptr, (size_t)n * 4, hipMemcpyDeviceToHost, g.stream));
+        DJ_HIP(hipStreamSynchronize(g.stream));
+    });
+}
+
+int deepj_hip_release(const int32_t *ids, int32_t count) {
+    return guarded([&] {
+        if (!g.ready) return;
+        if (count > 0 && !ids) fail("releaseBuffers: null array");
+        for (int i = 0; i < count; i++) {
+            auto it = g.live.find(ids[i]);
+            if (it == g.live.end()) continue;            // unknown id: silent no-op
+            g.live_bytes -= (int64_t)it->second.capacity;
+            pool_free(it->second.ptr, it->second.capacity);
+            g.live.erase(it);
+        }
+    });
+}
+
+int deepj_hip_flush_ops(const int32_t *cmd, int32_t len) {
+    return guarded([&] {
+        ensure_init();
+        run_stream(cmd, len);
+    });
+}
+
+const char *deepj_hip_last_error(void) { return g_error.c_str(); }
+
+int deepj_hip_synchronize(void) {
+    return guarded([&] {
+        if (g.ready) DJ_HIP(hipStreamSynchronize(g.stream));
+    });
+}
+
+int deepj_hip_trim(void) {
+    return guarded([&] {
+        if (!g.ready) return;
+        DJ_HIP(hipStreamSynchronize(g.stream));
+        for (auto &kv : g.cache) {
+            for (void *p : kv.second) DJ_HIP(hipFree(p));
+            kv.second.clear();
+        }
+        g.cached_bytes = 0;
+    });
+}
+
+int deepj_hip_shutdown(void) {
+    return guarded([&] {
+        if (!g.ready) return;
+        DJ_HIP(hipStreamSynchronize(g.stream));
+        for (auto &kv : g.graphs) {
+            if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+            if (kv.second.graph) (void)hipGraphDestroy(kv.second.graph);
+        }
+        g.graphs.clear();
+        for (auto &kv : g.live) (void)hipFree(kv.second.ptr);
+        g.live.clear();
+        for (auto &kv : g.cache)
+            for (void *p : kv.second) (void)hipFree(p);
+        g.cache.clear();
+        if (g.workspace) (void)hipFree(g.workspace);
+        g.workspace = nullptr; g.workspace_floats = 0;
+        if (g.staging) (void)hipHostFree(g.staging);
+        g.staging = nullptr;
+        (void)hipStreamDestroy(g.stream);
+        g.stream = nullptr;
+        g.live_bytes = g.cached_bytes = 0;
+        g.ready = false;
+    });
+}
+
+int deepj_hip_pool_stats(int64_t out[4]) {
+    return guarded([&] {
+        if (!out) fail("pool_stats: null output");
+        out[0] = (int64_t)g.live.size();
+        out[1] = g.live_bytes;
+        out[2] = g.cached_bytes;
+        out[3] = g.driver_allocs;
+    });
+}
+
+void *deepj_hip_stream(void) { return g.ready ? (void *)g.stream : nullptr; }
+
+int64_t deepj_hip_q8_floats(int32_t k, int32_t rows) {
+    if (k <= 0 || rows <= 0) return 0;
+    return (q8_bytes(k, rows) + 3) / 4;
+}
+
+int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total) {
+    return guarded([&] {
+        ensure_init();
+        if (iters <= 0 || !ms_total) fail("time_ops: bad arguments");
+        int64_t ws = 0;
+        walk(cmd, len, true, &ws);
+        ensure_workspace(ws);
+        hipEvent_t e0, e1;
+        DJ_HIP(hipEventCreate(&e0));
+        DJ_HIP(hipEventCreate(&e1));
+        DJ_HIP(hipEventRecord(e0, g.stream));
+        for (int i = 0; i < iters; i++) walk(cmd, len, false, nullptr);
+        DJ_HIP(hipEventRecord(e1, g.stream));
+        DJ_HIP(hipEventSynchronize(e1));
+        DJ_HIP(hipEventElapsedTime(ms_total, e0, e1));
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) fail(std::string("kernel launch failed: ") + hipGetErrorString(e));
+    });
+}
+
+int deepj_hip_graph_capture(const int32_t *cmd, int32_t len, int32_t *handle) {
+    return guarded([&] {
+        ensure_init();
+        if (!handle) fail("graph_capture: null handle");
+        int64_t ws = 0;
+        walk(cmd, len, true, &ws);
+        ensure_workspace(ws);
+        DJ_HIP(hipStreamSynchronize(g.stream));
+        Graph gr;
+        DJ_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal));
+        g.capturing = true;
+        try {
+            walk(cmd, len, false, nullptr);
+        } catch (...) {
+            g.capturing = false;
+            hipGraph_t tmp = nullptr;
+            (void)hipStreamEndCapture(g.stream, &tmp);
+            if (tmp) (void)hipGraphDestroy(tmp);
+            throw;
+        }
+        g.capturing = false;
+        DJ_HIP(hipStreamEndCapture(g.stream, &gr.graph));
+        hipError_t e = hipGraphInstantiate(&gr.exec, gr.graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) {
+            (void)hipGraphDestroy(gr.graph);
+            fail(std::string("hipGraphInstantiate: ") + hipGetErrorString(e));
+        }
+        int32_t h = g.next_graph++;
+        g.graphs.emplace(h, gr);
+        *handle = h;
+    });
+}
+
+int deepj_hip_graph_launch(int32_t handle, int32_t times) {
+    return guarded([&] {
+        auto it = g.graphs.find(handle);
+        if (it == g.graphs.end()) fail("graph_launch: unknown graph handle " + std::to_string(handle));
+        for (int i = 0; i < times; i++) DJ_HIP(hipGraphLaunch(it->second.exec, g.stream));
+    });
+}
+
+int deepj_hip_graph_destroy(int32_t handle) {
+    return guarded([&] {
+        auto it = g.graphs.find(handle);
+        if (it == g.graphs.end()) return;
+        DJ_HIP(hipStreamSynchronize(g.stream));
+        (void)hipGraphExecDestroy(it->second.exec);
+        (void)hipGraphDestroy(it->second.graph);
+        g.graphs.erase(it);
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,129 @@
+"""Direct access to the native runtime for the fused inference opcodes: buffer ids in a
+range of their own (so they never collide with the ids a ComputeGraph hands out, which
+restart at 0 after releaseAll - ComputeGraph.java:739 in the reference) and a small
+encoder for the opcodes the reference's ComputeGraph has no record* method for.
+
+The encodings are the ones include/deepj_hip.h documents; the native decode driver
+emits exactly the same words.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import opcodes as op
+from ._native import HipNative
+
+FUSED_ID_BASE = 1 << 28
+
+
+class DeviceBuffers:
+    """Id allocator + upload/download helpers on top of the five GpuRuntime calls."""
+
+    def __init__(self, base: int = FUSED_ID_BASE):
+        self._next = base
+        self._sizes: dict[int, int] = {}
+
+    def alloc(self, floats: int) -> int:
+        buf_id = self._next
+        self._next += 1
+        HipNative.nativeAllocBuffers([buf_id], [int(floats)], 1)
+        self._sizes[buf_id] = int(floats)
+        return buf_id
+
+    def upload(self, array) -> int:
+        a = np.ascontiguousarray(array)
+        if a.dtype not in (np.float32, np.int32):
+            a = a.astype(np.float32)
+        buf_id = self.alloc(a.size)
+        HipNative.nativeUploadBuffer(buf_id, a.reshape(-1))
+        return buf_id
+
+    def write(self, buf_id: int, array) -> None:
+        a = np.ascontiguousarray(array)
+        HipNative.nativeUploadBuffer(buf_id, a.reshape(-1))
+
+    def download(self, buf_id: int, shape, dtype=np.float32) -> np.ndarray:
+        out = np.empty(int(np.prod(shape)), dtype=dtype)
+        HipNative.nativeDownloadBuffer(buf_id, out)
+        return out.reshape(shape)
+
+    def size(self, buf_id: int) -> int:
+        return self._sizes[buf_id]
+
+    def release(self, *ids: int) -> None:
+        ids = [i for i in ids if i in self._sizes]
+        for i in ids:
+            del self._sizes[i]
+        if ids:
+            HipNative.nativeReleaseBuffers(ids, len(ids))
+
+    def release_all(self) -> None:
+        self.release(*list(self._sizes))
+
+
+class Stream:
+    """Accumulates command words; run() hands them to flushOps."""
+
+    def __init__(self):
+        self.words: list[int] = []
+
+    def emit(self, *w: int) -> "Stream":
+        self.words.extend(int(x) for x in w)
+        return self
+
+    # fused opcodes -----------------------------------------------------------
+    def q8_quantize(self, src, dst, k, n, row_off=0, row_step=1, total_rows=None):
+        return self.emit(op.OP_Q8_QUANTIZE, src, dst, k, n, row_off, row_step, n if total_rows is None else total_rows)
+
+    def q8_dequantize(self, src, dst, k, n, row_off=0, row_step=1, total_rows=None):
+        return self.emit(op.OP_Q8_DEQUANTIZE, src, dst, k, n, row_off, row_step, n if total_rows is None else total_rows)
+
+    def q8_linear(self, x, w, out, m, k, n, *, gamma=-1, bias=-1, bias2=-1, residual=-1, swiglu=False):
+        flags = ((op.LIN_RMSNORM if gamma >= 0 else 0) | (op.LIN_BIAS if bias >= 0 else 0) |
+                 (op.LIN_RESIDUAL if residual >= 0 else 0) | (op.LIN_SWIGLU if swiglu else 0))
+        return self.emit(op.OP_Q8_LINEAR, x, w, out, m, k, n, flags, gamma, bias, bias2, residual)
+
+    def rmsnorm(self, x, gamma, out, rows, cols): return self.emit(op.OP_RMSNORM, x, gamma, out, rows, cols)
+    def silu_mul(self, gate, up, out, n): return self.emit(op.OP_SILU_MUL, gate, up, out, n)
+
+    def embed_gather(self, table, ids, out, n_ids, d, vocab, ids_off=0):
+        return self.emit(op.OP_EMBED_GATHER, table, ids, out, n_ids, d, vocab, ids_off)
+
+    def rope_kv_store(self, qkv, q_out, k_cache, v_cache, state, cos, sin, S, H, hd, max_seq, layer):
+        return self.emit(op.OP_ROPE_KV_STORE, qkv, q_out, k_cache, v_cache, state, cos, sin, S, H, hd, max_seq, layer)
+
+    def rope_rows(self, x, out, state, cos, sin, rows, H, hd, max_seq, pos_from_row):
+        return self.emit(op.OP_ROPE_ROWS, x, out, state, cos, sin, rows, H, hd, max_seq, 1 if pos_from_row else 0)
+
+    def attention(self, q, k_cache, v_cache, out, state, scratch, S, H, hd, max_seq, layer):
+        return self.emit(op.OP_ATTENTION, q, k_cache, v_cache, out, state, scratch, S, H, hd, max_seq, layer)
+
+    def attention_kv(self, q, k, v, out, state, scratch, S, H, hd, max_seq):
+        return self.emit(op.OP_ATTENTION_KV, q, k, v, out, state, scratch, S, H, hd, max_seq, 0)
+
+    def argmax_rows(self, logits, out, rows, cols): return self.emit(op.OP_ARGMAX_ROWS, logits, out, rows, cols)
+
+    def decode_advance(self, state, token, tokens, capacity):
+        return self.emit(op.OP_DECODE_ADVANCE, state, token, tokens, capacity)
+
+    def copy(self, src, dst, n, src_off=0, dst_off=0): return self.emit(op.OP_COPY, src, dst, n, src_off, dst_off)
+    def fill(self, dst, bits, n): return self.emit(op.OP_FILL, dst, bits, n)
+    def matmul(self, a, b, out, m, n, k): return self.emit(op.OP_MATMUL, a, b, out, m, n, k)
+
+    # execution -----------------------------------------------------------------
+    def array(self) -> np.ndarray:
+        return np.asarray(self.words, dtype=np.int32)
+
+    def run(self) -> None:
+        a = self.array()
+        HipNative.nativeFlushOps(a, a.size)
+
+    def time(self, iters: int) -> float:
+        """Milliseconds for `iters` back-to-back executions (HIP events on the library's stream)."""
+        return HipNative.timeOps(self.array(), iters)
+
+
+def attention_scratch_floats(H: int, hd: int, max_seq: int) -> int:
+    """Floats the decode (S = 1) attention scratch buffer must hold; it must start zeroed."""
+    splits = (max_seq + 63) // 64
+    return H * (4 + splits * (hd + 4))

@@ -1,0 +1,139 @@
+/*
+ * deepj_hip.h - C ABI of libdeepj_hip.so, the MI355X (gfx950) device runtime
+ * behind DeepJ's GpuRuntime boundary.
+ *
+ * Every function returns 0 on success and a non-zero code on failure; the
+ * message is then available from deepj_hip_last_error().  Nothing throws
+ * across this boundary.  A single caller thread is assumed, as in the
+ * reference (its ComputeGraph and native pool are unsynchronised globals:
+ * src/main/java/io/github/kirstenali/deepj/tensor/ComputeGraph.java:67-78,
+ * native/deepj_metal_jni.mm:63,1358).
+ *
+ * Paths cited below are relative to the reference tree:
+ *   J/ = src/main/java/io/github/kirstenali/deepj/
+ */
+#ifndef DEEPJ_HIP_H
+#define DEEPJ_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ── the five GpuRuntime calls (J/tensor/GpuRuntime.java:9-28) ─────────────
+ * These are what HipNative's five `static native` methods bind, one to one,
+ * the way J/tensor/metal/MetalNative.java:41-57 binds the Metal library. */
+
+/* GpuRuntime.allocBuffers (native/deepj_metal_jni.mm:1480-1505).
+ * sizes are in floats.  Allocating an id that already exists is a no-op. */
+int deepj_hip_alloc_buffers(const int32_t *ids, const int32_t *sizes_in_floats, int32_t count);
+
+/* GpuRuntime.uploadBuffer (deepj_metal_jni.mm:1509-1521).  Copies n floats
+ * (the Java array length) into the buffer; src is only borrowed for the
+ * call.  Unknown id: error "Buffer not found for upload". */
+int deepj_hip_upload(int32_t id, const float *src, int64_t n);
+
+/* GpuRuntime.downloadBuffer (deepj_metal_jni.mm:1525-1537).  Waits for all
+ * work queued so far, then copies n floats out.  This is the only call that
+ * synchronises with the device.  Unknown id: "Buffer not found for download". */
+int deepj_hip_download(int32_t id, float *dst, int64_t n);
+
+/* GpuRuntime.releaseBuffers (deepj_metal_jni.mm:1541-1549).  Unknown ids are
+ * ignored.  Memory returns to the size-class cache, not to the driver. */
+int deepj_hip_release(const int32_t *ids, int32_t count);
+
+/* GpuRuntime.flushOps (deepj_metal_jni.mm:1554-2140).  Executes the int32
+ * command stream recorded by ComputeGraph (opcodes 1..42 exactly as encoded
+ * by J/tensor/ComputeGraph.java:260-518) plus the fused inference opcodes
+ * listed below.  The whole stream is validated first (opcode, stride, buffer
+ * ids, sizes); on error nothing is launched.  An unknown opcode N fails with
+ * "Unknown op code in graph: N" (deepj_metal_jni.mm:2120-2121).  The call
+ * only enqueues work: results are observable through deepj_hip_download. */
+int deepj_hip_flush_ops(const int32_t *cmd, int32_t len);
+
+/* Message of the last failure on this thread ("" if none). */
+const char *deepj_hip_last_error(void);
+
+/* ── runtime control (no counterpart in the reference: Metal's context is
+ * created lazily, deepj_metal_jni.mm:909-984) ──────────────────────────── */
+int deepj_hip_init(int32_t device);        /* optional; first use initialises device 0 */
+int deepj_hip_synchronize(void);
+int deepj_hip_shutdown(void);              /* frees every buffer and the cache */
+int deepj_hip_trim(void);                  /* returns cached (released) memory to the driver */
+/* out[0]=live buffers, out[1]=live bytes, out[2]=cached bytes, out[3]=driver allocations so far */
+int deepj_hip_pool_stats(int64_t out[4]);
+/* The HIP stream all work is queued on, as a hipStream_t, for callers that time with HIP events. */
+void *deepj_hip_stream(void);
+
+/* Times `iters` back-to-back executions of a validated stream with HIP events
+ * recorded on the library's stream; *ms_total receives the elapsed time. */
+int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total);
+
+/* Captures a command stream into a HIP graph (no allocation may be pending:
+ * every buffer it names must exist) and replays it.  Used for the per-token
+ * decode stream, whose position and token live in device memory. */
+int deepj_hip_graph_capture(const int32_t *cmd, int32_t len, int32_t *handle);
+int deepj_hip_graph_launch(int32_t handle, int32_t times);
+int deepj_hip_graph_destroy(int32_t handle);
+
+/* ── opcodes ──────────────────────────────────────────────────────────── */
+/* 1..42: J/tensor/ComputeGraph.java:19-60 (same numbers, same encodings). */
+enum {
+    DJ_OP_ADD = 1, DJ_OP_SUBTRACT = 2, DJ_OP_MULTIPLY = 3, DJ_OP_DIVIDE = 4, DJ_OP_MATMUL = 5,
+    DJ_OP_MULTIPLY_SCALAR = 6, DJ_OP_SQRT = 7, DJ_OP_NEG = 8, DJ_OP_EXP = 9, DJ_OP_LOG = 10,
+    DJ_OP_TANH = 11, DJ_OP_SIGMOID = 12, DJ_OP_RELU = 13, DJ_OP_RELU_BACKWARD = 14, DJ_OP_GELU = 15,
+    DJ_OP_GELU_BACKWARD = 16, DJ_OP_SOFTMAX_ROWS = 17, DJ_OP_SOFTMAX_BACKWARD = 18,
+    DJ_OP_LAYERNORM_BACKWARD = 19, DJ_OP_ADAMW_UPDATE = 20, DJ_OP_ADD_SCALAR = 21,
+    DJ_OP_DIVIDE_SCALAR = 22, DJ_OP_TRANSPOSE = 23, DJ_OP_ADD_ROW_VECTOR = 24,
+    DJ_OP_ADD_BROADCAST_COLS = 25, DJ_OP_SUBTRACT_BROADCAST_COLS = 26, DJ_OP_DIVIDE_BROADCAST_COLS = 27,
+    DJ_OP_MULTIPLY_BROADCAST_ROWS = 28, DJ_OP_SUM_ROWS = 29, DJ_OP_MEAN_ALONG_ROWS = 30,
+    DJ_OP_VARIANCE_ALONG_ROWS = 31, DJ_OP_MULTIPLY_BROADCAST_COLS = 32, DJ_OP_SUM_ALONG_ROWS = 33,
+    DJ_OP_MAX_ALONG_ROWS = 34, DJ_OP_CLAMP = 35, DJ_OP_POW = 36, DJ_OP_SCATTER_ADD_ROWS = 37,
+    DJ_OP_SUM_ABS = 38, DJ_OP_CROSS_ENTROPY_LOSS = 39, DJ_OP_CROSS_ENTROPY_GRADIENT = 40,
+    DJ_OP_SUM_SCALAR = 41, DJ_OP_SCATTER_ADD_ROWS_ATOMIC = 42,
+
+    /* Fused inference opcodes.  The reference has none of these: it composes
+     * them from primitives in Java (J/layers/transformer/norm/RMSNorm1D.java:46-57,
+     * J/layers/transformer/SwiGLULayer.java:63-70, J/transformer/embeddings/
+     * RotaryEmbedding.java:81-122, J/layers/transformer/attention/HeadOps.java:33-140).
+     * Encodings (all words int32; "buf" = buffer id, -1 = absent):
+     *
+     * Q8_QUANTIZE   [op, src, dst, K, N, rowOff, rowStep, totalRows]
+     *     src fp32 [K x N] (Linear weight orientation, J/layers/Linear.java:13);
+     *     column n becomes Q8 row rowOff + n*rowStep of dst, which holds
+     *     totalRows rows of Kp = roundup(K,32) int8 plus one fp32 scale per
+     *     32-group.  dst must hold deepj_hip_q8_floats(K, totalRows) floats.
+     * Q8_DEQUANTIZE [op, src, dst, K, N, rowOff, rowStep, totalRows]   inverse view, dst fp32 [K x N]
+     * Q8_LINEAR     [op, x, w, out, M, K, N, flags, gamma, bias, bias2, residual]
+     *     out[M x N] = f(x[M x K]) . W  (+ bias) (+ residual)
+     *     flags bit0: RMSNorm prologue, f(x) = gamma * x / sqrt(mean(x^2)+1e-6)
+     *           bit1: add bias[N]          bit2: add residual[M x N]
+     *           bit3: SwiGLU: w has 2N rows (gate n at row 2n, up n at 2n+1),
+     *                 out = SiLU(gate + bias) * (up + bias2)
+     * RMSNORM       [op, x, gamma, out, rows, cols]
+     * SILU_MUL      [op, gate, up, out, n]            out = gate*sigmoid(gate)*up
+     * EMBED_GATHER  [op, table, ids, out, nIds, d, vocab, idsOff]  ids are int32 words
+     * ROPE_KV_STORE [op, qkv, qOut, kCache, vCache, state, cosT, sinT, S, H, hd, maxSeq, layer]
+     *     qkv [S x 3d]; rows sit at positions state[0]..state[0]+S-1
+     * ATTENTION     [op, q, kCache, vCache, out, state, scratch, S, H, hd, maxSeq, layer]
+     * ARGMAX_ROWS   [op, logits, out, rows, cols]      out int32 words, ties -> lowest index
+     * DECODE_ADVANCE[op, state, tokens, capacity]      see DESIGN.md
+     * COPY          [op, src, dst, n, srcOff, dstOff]
+     * FILL          [op, dst, bits, n]
+     */
+    DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
+    DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
+    DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
+    DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77
+};
+
+enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8 };
+
+/* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
+int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEPJ_HIP_H */

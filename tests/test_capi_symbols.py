@@ -1,0 +1,42 @@
+"""The C-ABI library loads without a GPU and exports every function include/deepj_hip.h declares;
+compute entry points fail loudly (no CPU fallback) when no device is present."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from deepj_amd import HipNative, LIB_PATH
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "deepj_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(deepj_(?:hip|runner|host)_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(LIB_PATH)
+    names = declared_functions()
+    assert "deepj_hip_flush_ops" in names and len(names) >= 12
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_opcode_numbers_match_header():
+    from deepj_amd import opcodes
+    text = open(os.path.join(ROOT, "include", "deepj_hip.h")).read()
+    for name, value in re.findall(r"DJ_(OP_[A-Z0-9_]+)\s*=\s*(\d+)", text):
+        assert getattr(opcodes, name) == int(value), name
+
+
+@pytest.mark.skipif(os.path.exists("/dev/kfd"), reason="checks the no-GPU failure path")
+def test_no_silent_cpu_fallback_without_a_device():
+    with pytest.raises(RuntimeError, match="no HIP device"):
+        HipNative.nativeAllocBuffers([0], [4], 1)
+    with pytest.raises(RuntimeError):
+        HipNative.nativeFlushOps(np.array([1, 0, 0, 0, 4], dtype=np.int32), 5)
+    assert HipNative.q8Floats(64, 2) == (256 + 2 * 2 * 4) // 4      # pure size arithmetic needs no device

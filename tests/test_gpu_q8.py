@@ -1,0 +1,167 @@
+"""Q8 weight path through the C ABI: quantiser bit-exact against the host quantiser, decode
+matvec and prefill GEMM (with their fused prologue/epilogues) against the CPU oracle run on
+the dequantised weights.  Shapes of BASELINE.json's isolated linear-op sweep at reduced N
+where the oracle would be slow, plus ragged K (688 = 21*32 + 16)."""
+import numpy as np
+import pytest
+
+from deepj_amd import HipNative
+from deepj_amd.fused import DeviceBuffers, Stream
+from oracle import cpu_ref as ref
+from gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def gaussian(rows, cols, seed, scale):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
+
+
+@pytest.fixture
+def dev():
+    d = DeviceBuffers()
+    yield d
+    d.release_all()
+
+
+def quantize_on_device(dev, w, row_off=0, row_step=1, total_rows=None, dst=None):
+    k, n = w.shape
+    total = n if total_rows is None else total_rows
+    src = dev.upload(w)
+    if dst is None:
+        dst = dev.alloc(HipNative.q8Floats(k, total))
+    Stream().q8_quantize(src, dst, k, n, row_off, row_step, total).run()
+    dev.release(src)
+    return dst
+
+
+@pytest.mark.parametrize("k,n", [(64, 3), (688, 70), (2048, 256), (70, 9)])
+def test_quantize_and_dequantize_bit_exact_vs_host(dev, k, n):
+    w = gaussian(k, n, 1, 0.02)
+    w[:, 0] = 0.0                                   # an all-zero column: scale 0, no NaN
+    wq = quantize_on_device(dev, w)
+    kp = (k + 31) // 32 * 32
+    raw = dev.download(wq, (HipNative.q8Floats(k, n),), np.float32).view(np.int8)
+    q_dev = raw[: n * kp].reshape(n, kp)
+    sc_off = (n * kp + 255) // 256 * 256
+    s_dev = raw[sc_off: sc_off + n * (kp // 32) * 4].view(np.float32).reshape(n, kp // 32)
+    q_ref, s_ref = ref.q8_quantize(w)
+    assert np.array_equal(q_dev, q_ref), "int8 payload differs from the host quantiser"
+    assert np.array_equal(s_dev.view(np.int32), s_ref.view(np.int32)), "scales differ bitwise"
+    out = dev.alloc(k * n)
+    Stream().q8_dequantize(wq, out, k, n).run()
+    dq = dev.download(out, (k, n))
+    assert np.array_equal(dq.view(np.int32), ref.q8_dequantize(q_ref, s_ref, k).view(np.int32))
+
+
+def test_quantize_into_interleaved_rows(dev):
+    k, n = 96, 10
+    wg, wu = gaussian(k, n, 2, 0.02), gaussian(k, n, 3, 0.02)
+    dst = dev.alloc(HipNative.q8Floats(k, 2 * n))
+    quantize_on_device(dev, wg, 0, 2, 2 * n, dst)
+    quantize_on_device(dev, wu, 1, 2, 2 * n, dst)
+    og, ou = dev.alloc(k * n), dev.alloc(k * n)
+    Stream().q8_dequantize(dst, og, k, n, 0, 2, 2 * n).q8_dequantize(dst, ou, k, n, 1, 2, 2 * n).run()
+    assert np.array_equal(dev.download(og, (k, n)), ref.q8_roundtrip(wg))
+    assert np.array_equal(dev.download(ou, (k, n)), ref.q8_roundtrip(wu))
+
+
+def linear_case(dev, m, k, n, *, norm=False, bias=False, residual=False, seed=0):
+    w = gaussian(k, n, seed + 1, 0.02)
+    x = gaussian(m, k, seed + 2, 1.0)
+    wdq = ref.q8_roundtrip(w)
+    wq = quantize_on_device(dev, w)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    kw, h = {}, x
+    if norm:
+        gamma = (1.0 + gaussian(1, k, seed + 3, 0.02))
+        kw["gamma"] = dev.upload(gamma)
+        h = ref.rmsnorm(x, gamma)
+    exp = ref.matmul(h, wdq)
+    if bias:
+        b = gaussian(1, n, seed + 4, 0.1)
+        kw["bias"] = dev.upload(b)
+        exp = ref.add_row_vector(exp, b)
+    if residual:
+        r = gaussian(m, n, seed + 5, 1.0)
+        kw["residual"] = dev.upload(r)
+        exp = ref.add(r, exp)
+    Stream().q8_linear(xb, wq, ob, m, k, n, **kw).run()
+    return exp, dev.download(ob, (m, n))
+
+
+@pytest.mark.parametrize("k,n", [(2048, 2048), (2048, 5632), (5632, 2048), (4096, 1100), (11008, 512),
+                                 (688, 256), (256, 688), (32, 1), (1024, 5)])
+def test_q8_matvec_matches_oracle(dev, k, n):
+    exp, got = linear_case(dev, 1, k, n)
+    # fp32 sums of K terms in a different order: |err| <~ 1e-6 * sqrt(K) * |x||w|; outputs can sit near 0
+    scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+    assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"matvec {k}x{n}")
+
+
+@pytest.mark.parametrize("flags", [dict(norm=True), dict(bias=True), dict(residual=True),
+                                   dict(norm=True, bias=True, residual=True)])
+def test_q8_matvec_fused_prologue_epilogue(dev, flags):
+    for k, n in [(2048, 768), (688, 256)]:
+        exp, got = linear_case(dev, 1, k, n, seed=10, **flags)
+        scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+        assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"{flags} {k}x{n}")
+
+
+@pytest.mark.parametrize("m", [1, 64])
+def test_q8_swiglu_gate_up(dev, m):
+    k, n = 256, 688
+    wg, wu = gaussian(k, n, 21, 0.05), gaussian(k, n, 22, 0.05)
+    bg, bu = gaussian(1, n, 23, 0.1), gaussian(1, n, 24, 0.1)
+    x, gamma = gaussian(m, k, 25, 1.0), 1.0 + gaussian(1, k, 26, 0.02)
+    wq = dev.alloc(HipNative.q8Floats(k, 2 * n))
+    quantize_on_device(dev, wg, 0, 2, 2 * n, wq)
+    quantize_on_device(dev, wu, 1, 2, 2 * n, wq)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    Stream().q8_linear(xb, wq, ob, m, k, n, gamma=dev.upload(gamma), bias=dev.upload(bg), bias2=dev.upload(bu),
+                       swiglu=True).run()
+    h = ref.rmsnorm(x, gamma)
+    gate = ref.linear(h, ref.q8_roundtrip(wg), bg)
+    up = ref.linear(h, ref.q8_roundtrip(wu), bu)
+    exp = ref.multiply(ref.silu(gate), up)
+    assert_close(exp, dev.download(ob, (m, n)), atol=2e-6, rtol=1e-4, what=f"swiglu m={m}")
+
+
+@pytest.mark.parametrize("m,k,n", [(64, 2048, 512), (512, 2048, 256), (64, 688, 256), (7, 96, 33), (130, 5632, 128)])
+def test_q8_gemm_matches_oracle(dev, m, k, n):
+    exp, got = linear_case(dev, m, k, n, norm=True, bias=True, residual=True, seed=30)
+    scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+    assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"gemm {m}x{k}x{n}")
+
+
+def test_q8_linear_rejects_bad_streams(dev):
+    x, w, out = dev.alloc(64), dev.alloc(HipNative.q8Floats(64, 4)), dev.alloc(4)
+    with pytest.raises(RuntimeError, match="op needs"):
+        Stream().q8_linear(x, w, out, 1, 64, 8).run()                 # weight buffer too small for N=8
+    with pytest.raises(RuntimeError, match="SWIGLU cannot be combined"):
+        Stream().q8_linear(x, w, out, 1, 64, 2, residual=out, swiglu=True).run()
+    with pytest.raises(RuntimeError, match="rows fall outside"):
+        Stream().q8_quantize(x, w, 64, 1, 4, 1, 4).run()
+
+
+def test_fused_rmsnorm_silu_mul_embed_argmax(dev):
+    x, gamma = gaussian(9, 2048, 40, 1.0), 1.0 + gaussian(1, 2048, 41, 0.02)
+    xb, gb, ob = dev.upload(x), dev.upload(gamma), dev.alloc(x.size)
+    Stream().rmsnorm(xb, gb, ob, 9, 2048).run()
+    assert_close(ref.rmsnorm(x, gamma), dev.download(ob, x.shape), 1e-6, 1e-5)
+    g, u = gaussian(5, 5632, 42, 2.0), gaussian(5, 5632, 43, 1.0)
+    o2 = dev.alloc(g.size)
+    Stream().silu_mul(dev.upload(g), dev.upload(u), o2, g.size).run()
+    assert_close(ref.multiply(ref.silu(g), u), dev.download(o2, g.shape), 1e-7, 1e-6)
+    table = gaussian(100, 64, 44, 1.0)
+    ids = np.array([5, 99, 0, 5], np.int32)
+    o3 = dev.alloc(4 * 64)
+    Stream().embed_gather(dev.upload(table), dev.upload(ids), o3, 4, 64, 100).run()
+    assert np.array_equal(dev.download(o3, (4, 64)), table[ids])
+    logits = gaussian(3, 32000, 45, 4.0)
+    logits[1, 777] = logits[1, 31999] = 100.0          # tie -> lowest index
+    o4 = dev.alloc(3)
+    Stream().argmax_rows(dev.upload(logits), o4, 3, 32000).run()
+    got = dev.download(o4, (3,), np.int32)
+    assert list(got) == [int(np.argmax(logits[0])), 777, int(np.argmax(logits[2]))]
