@@ -7,5 +7,7 @@ from ._native import HipNative, LIB_PATH
 from .compute_graph import ComputeGraph, GpuBuffer
 from .hip_backend import HipBackend, HipGpuRuntime
 from .tensor import Tensor
+from .models import DeepSeekConfig, DeepSeekModel, JavaRandom, LlamaConfig, LlamaModel, TextGenerator
 
-__all__ = ["opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor"]
+__all__ = ["opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor",
+           "LlamaConfig", "LlamaModel", "DeepSeekConfig", "DeepSeekModel", "TextGenerator", "JavaRandom"]

@@ -52,7 +52,8 @@ void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n);
 void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n);
 void launch_embed_gather(hipStream_t s, const float *table, const int32_t *ids, float *out, int n_ids, int d,
                          int vocab);
-void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity);
+void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity,
+                           int n_positions);
 
 // kernels_reduce.hip
 void launch_row_reduce(hipStream_t s, int op, const float *a, float *out, int rows, int cols);

@@ -235,13 +235,14 @@ __global__ void __launch_bounds__(kThreads) k_embed_gather(const float *__restri
 }
 
 // state[0] = positions held in the cache, state[1] = current token, state[2] = tokens generated.
-__global__ void k_decode_advance(int32_t *state, const int32_t *token, int32_t *tokens, int capacity) {
+__global__ void k_decode_advance(int32_t *state, const int32_t *token, int32_t *tokens, int capacity,
+                                 int n_positions) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         int32_t t = token[0];
         int32_t g = state[2];
         if (g < capacity) tokens[g] = t;
         state[1] = t;
-        state[0] = state[0] + 1;
+        state[0] = state[0] + n_positions;
         state[2] = g + 1;
     }
 }
@@ -355,8 +356,9 @@ void launch_embed_gather(hipStream_t s, const float *table, const int32_t *ids, 
     DJ_LAUNCH(k_embed_gather, n_ids, kThreads, s, table, ids, out, n_ids, d, vocab);
 }
 
-void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity) {
-    DJ_LAUNCH(k_decode_advance, 1, 64, s, state, token, tokens, capacity);
+void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity,
+                           int n_positions) {
+    DJ_LAUNCH(k_decode_advance, 1, 64, s, state, token, tokens, capacity, n_positions);
 }
 
 }  // namespace dj

@@ -1,0 +1,592 @@
+// Native decode driver: the caller on the host side of the C ABI.  It plays the part of
+// the reference's LlamaModel / DeepSeekModel + TextGenerator
+//   (src/main/java/io/github/kirstenali/deepj/models/{DecoderOnlyModel,TextGenerator}.java,
+//    models/llama/LlamaModel.java, models/deepseek/DeepSeekModel.java)
+// for inference, but instead of re-running the whole context for every token
+// (TextGenerator.java:91-100) it keeps a KV cache in HBM, records ONE fused command
+// stream per token and replays it as a HIP graph.  Position, current token and the
+// generated ids live in device memory, so a run of N tokens needs no host round trip.
+//
+// Everything here goes through the public deepj_hip_* functions only: buffers are named
+// by int ids, work is submitted as int32 command streams - the same boundary a Java
+// HipBackend uses - so a Java facade can emit the identical streams.
+//
+// Weight names: "emb", "gf", "wlm", "blm" and per layer "L<i>.<w>" with w in
+//   g1 g2 wq wk wv wo           (Llama;  MultiHeadSelfAttention.java:47-50)
+//   g1 g2 wdq wuq wdkv wuk wuv wo (DeepSeek; MultiHeadLatentAttention.java:81-86)
+//   wg bg wu bu wd bd           (SwiGLULayer.java:56-58)
+// Matrices are given in the reference's orientation, fp32 [dIn x dOut] row-major.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/deepj_hip.h"
+
+extern "C" {
+void *deepj_host_random_create(int64_t seed);
+void deepj_host_random_destroy(void *h);
+void deepj_host_random_fill(void *h, float *out, int64_t n, double scale, int32_t threads);
+float deepj_host_random_next_float(void *h);
+}
+
+namespace {
+
+struct Config {
+    int32_t kind;       // 0 Llama, 1 DeepSeek (MLA)
+    int32_t vocab, max_seq, d, heads, layers, dff, q_rank, kv_rank;
+};
+
+struct Error : std::runtime_error { using std::runtime_error::runtime_error; };
+
+void hip(int rc) {
+    if (rc != 0) throw Error(deepj_hip_last_error());
+}
+
+struct Layer {
+    int32_t g1 = -1, g2 = -1;
+    int32_t wqkv = -1, wo = -1;                       // Llama: fused [3d x d]
+    int32_t wdq = -1, wuq = -1, wdkv = -1, wukv = -1;  // MLA: wukv = Wuk|Wuv fused [2d x kvRank]
+    int32_t wgu = -1, bg = -1, bu = -1, wd = -1, bd = -1;
+};
+
+struct Acts {          // activation buffers for S rows
+    int32_t rows = 0;
+    int32_t x = -1, x2 = -1, qkv = -1, q = -1, att = -1, ff = -1, ids = -1;
+    int32_t cq = -1, ckv = -1, kfull = -1, vfull = -1, kvexp = -1;   // MLA
+};
+
+struct Runner {
+    Config cfg{};
+    int32_t next_id = 0;
+    std::map<std::string, bool> have;
+    std::vector<Layer> layers;
+    int32_t emb = -1, gf = -1, wlm = -1, blm = -1;
+    int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
+    int32_t state = -1, tok = -1, tokens = -1, scratch = -1, logits = -1, last_x = -1;
+    Acts dec, pre;
+    int32_t graph = 0;
+    bool finalized = false;
+    int32_t pos = 0;          // host mirror of state[0]
+    int32_t generated = 0;    // host mirror of state[2]
+    std::string error;
+
+    int hd() const { return cfg.d / cfg.heads; }
+
+    int32_t alloc(int64_t floats) {
+        if (floats > 0x7fffffffLL) throw Error("buffer too large for an int32 float count");
+        int32_t id = next_id++;
+        int32_t sz = (int32_t)floats;
+        hip(deepj_hip_alloc_buffers(&id, &sz, 1));
+        return id;
+    }
+    void release(int32_t &id) {
+        if (id >= 0) { hip(deepj_hip_release(&id, 1)); id = -1; }
+    }
+    int32_t upload_new(const float *data, int64_t n) {
+        int32_t id = alloc(n);
+        hip(deepj_hip_upload(id, data, n));
+        return id;
+    }
+    void run(const std::vector<int32_t> &s) { hip(deepj_hip_flush_ops(s.data(), (int32_t)s.size())); }
+};
+
+using Stream = std::vector<int32_t>;
+template <class... A> void emit(Stream &s, A... words) { (s.push_back((int32_t)words), ...); }
+
+void q8_linear(Stream &s, int32_t x, int32_t w, int32_t out, int m, int k, int n, int flags, int32_t gamma = -1,
+               int32_t bias = -1, int32_t bias2 = -1, int32_t residual = -1) {
+    emit(s, DJ_OP_Q8_LINEAR, x, w, out, m, k, n, flags, gamma, bias, bias2, residual);
+}
+
+// ── weights ────────────────────────────────────────────────────────────────
+
+void quantize_into(Runner &r, int32_t &dst, const float *data, int k, int n, int row_off, int row_step, int total) {
+    if (dst < 0) dst = r.alloc(deepj_hip_q8_floats(k, total));
+    int32_t tmp = r.upload_new(data, (int64_t)k * n);
+    Stream s;
+    emit(s, DJ_OP_Q8_QUANTIZE, tmp, dst, k, n, row_off, row_step, total);
+    r.run(s);
+    r.release(tmp);
+}
+
+void expect_shape(const std::string &name, int rows, int cols, int er, int ec) {
+    if (rows != er || cols != ec)
+        throw Error("weight " + name + ": expected " + std::to_string(er) + "x" + std::to_string(ec) + " but got " +
+                    std::to_string(rows) + "x" + std::to_string(cols));
+}
+
+void set_weight(Runner &r, const std::string &name, const float *data, int rows, int cols) {
+    const Config &c = r.cfg;
+    const int d = c.d;
+    if (r.finalized) throw Error("set_weight after finalize");
+    if (name == "emb") { expect_shape(name, rows, cols, c.vocab, d); r.emb = r.upload_new(data, (int64_t)rows * cols); }
+    else if (name == "gf") { expect_shape(name, rows, cols, 1, d); r.gf = r.upload_new(data, d); }
+    else if (name == "blm") { expect_shape(name, rows, cols, 1, c.vocab); r.blm = r.upload_new(data, c.vocab); }
+    else if (name == "wlm") { expect_shape(name, rows, cols, d, c.vocab); quantize_into(r, r.wlm, data, d, c.vocab, 0, 1, c.vocab); }
+    else if (name.size() > 2 && name[0] == 'L') {
+        size_t dot = name.find('.');
+        if (dot == std::string::npos) throw Error("unknown weight " + name);
+        int l = std::atoi(name.substr(1, dot - 1).c_str());
+        if (l < 0 || l >= c.layers) throw Error("weight " + name + ": no such layer");
+        Layer &L = r.layers[l];
+        std::string w = name.substr(dot + 1);
+        if (w == "g1") { expect_shape(name, rows, cols, 1, d); L.g1 = r.upload_new(data, d); }
+        else if (w == "g2") { expect_shape(name, rows, cols, 1, d); L.g2 = r.upload_new(data, d); }
+        else if (w == "bg") { expect_shape(name, rows, cols, 1, c.dff); L.bg = r.upload_new(data, c.dff); }
+        else if (w == "bu") { expect_shape(name, rows, cols, 1, c.dff); L.bu = r.upload_new(data, c.dff); }
+        else if (w == "bd") { expect_shape(name, rows, cols, 1, d); L.bd = r.upload_new(data, d); }
+        else if (w == "wg") { expect_shape(name, rows, cols, d, c.dff); quantize_into(r, L.wgu, data, d, c.dff, 0, 2, 2 * c.dff); }
+        else if (w == "wu") { expect_shape(name, rows, cols, d, c.dff); quantize_into(r, L.wgu, data, d, c.dff, 1, 2, 2 * c.dff); }
+        else if (w == "wd") { expect_shape(name, rows, cols, c.dff, d); quantize_into(r, L.wd, data, c.dff, d, 0, 1, d); }
+        else if (w == "wo") { expect_shape(name, rows, cols, d, d); quantize_into(r, L.wo, data, d, d, 0, 1, d); }
+        else if (c.kind == 0 && (w == "wq" || w == "wk" || w == "wv")) {
+            expect_shape(name, rows, cols, d, d);
+            int part = w == "wq" ? 0 : (w == "wk" ? 1 : 2);
+            quantize_into(r, L.wqkv, data, d, d, part * d, 1, 3 * d);
+        }
+        else if (c.kind == 1 && w == "wdq") { expect_shape(name, rows, cols, d, c.q_rank); quantize_into(r, L.wdq, data, d, c.q_rank, 0, 1, c.q_rank); }
+        else if (c.kind == 1 && w == "wuq") { expect_shape(name, rows, cols, c.q_rank, d); quantize_into(r, L.wuq, data, c.q_rank, d, 0, 1, d); }
+        else if (c.kind == 1 && w == "wdkv") { expect_shape(name, rows, cols, d, c.kv_rank); quantize_into(r, L.wdkv, data, d, c.kv_rank, 0, 1, c.kv_rank); }
+        else if (c.kind == 1 && (w == "wuk" || w == "wuv")) {
+            expect_shape(name, rows, cols, c.kv_rank, d);
+            quantize_into(r, L.wukv, data, c.kv_rank, d, w == "wuk" ? 0 : d, 1, 2 * d);
+        }
+        else throw Error("unknown weight " + name);
+    } else throw Error("unknown weight " + name);
+    r.have[name] = true;
+}
+
+std::vector<std::string> weight_names(const Config &c) {
+    std::vector<std::string> names{"emb"};
+    for (int l = 0; l < c.layers; l++) {
+        std::string p = "L" + std::to_string(l) + ".";
+        for (const char *w : {"g1", "g2"}) names.push_back(p + w);
+        if (c.kind == 0) for (const char *w : {"wq", "wk", "wv", "wo"}) names.push_back(p + w);
+        else for (const char *w : {"wdq", "wuq", "wdkv", "wuk", "wuv", "wo"}) names.push_back(p + w);
+        for (const char *w : {"wg", "bg", "wu", "bu", "wd", "bd"}) names.push_back(p + w);
+    }
+    names.insert(names.end(), {"gf", "wlm", "blm"});
+    return names;
+}
+
+// new LlamaModel(cfg, seed) / new DeepSeekModel(cfg, seed): same RNG wiring and draw order
+// (LlamaModel.java:27-42, LlamaTransformerBuilder.java:45-55, DeepSeekTransformerBuilder.java:56-68).
+void init_seeded(Runner &r, int64_t seed, int threads) {
+    const Config &c = r.cfg;
+    const int d = c.d;
+    std::vector<float> buf;
+    auto draw = [&](void *rng, const std::string &name, int rows, int cols) {
+        buf.resize((size_t)rows * cols);
+        deepj_host_random_fill(rng, buf.data(), (int64_t)rows * cols, 0.1, threads);
+        set_weight(r, name, buf.data(), rows, cols);
+    };
+    auto constant = [&](const std::string &name, int cols, float v) {
+        buf.assign((size_t)cols, v);
+        set_weight(r, name, buf.data(), 1, cols);
+    };
+    void *emb_rng = deepj_host_random_create(seed);
+    void *stack_rng = deepj_host_random_create(seed);
+    void *head_rng = deepj_host_random_create(seed + 1);
+    try {
+        draw(emb_rng, "emb", c.vocab, d);
+        for (int l = 0; l < c.layers; l++) {
+            std::string p = "L" + std::to_string(l) + ".";
+            constant(p + "g1", d, 1.0f);
+            constant(p + "g2", d, 1.0f);
+            if (c.kind == 0) {
+                for (const char *w : {"wq", "wk", "wv", "wo"}) draw(stack_rng, p + w, d, d);
+            } else {
+                draw(stack_rng, p + "wdq", d, c.q_rank);
+                draw(stack_rng, p + "wuq", c.q_rank, d);
+                draw(stack_rng, p + "wdkv", d, c.kv_rank);
+                draw(stack_rng, p + "wuk", c.kv_rank, d);
+                draw(stack_rng, p + "wuv", c.kv_rank, d);
+                draw(stack_rng, p + "wo", d, d);
+            }
+            draw(stack_rng, p + "wg", d, c.dff);  constant(p + "bg", c.dff, 0.0f);
+            draw(stack_rng, p + "wu", d, c.dff);  constant(p + "bu", c.dff, 0.0f);
+            draw(stack_rng, p + "wd", c.dff, d);  constant(p + "bd", d, 0.0f);
+        }
+        constant("gf", d, 1.0f);
+        draw(head_rng, "wlm", d, c.vocab);
+        constant("blm", c.vocab, 0.0f);
+    } catch (...) {
+        deepj_host_random_destroy(emb_rng); deepj_host_random_destroy(stack_rng); deepj_host_random_destroy(head_rng);
+        throw;
+    }
+    deepj_host_random_destroy(emb_rng); deepj_host_random_destroy(stack_rng); deepj_host_random_destroy(head_rng);
+}
+
+// ── buffers ────────────────────────────────────────────────────────────────
+
+void alloc_acts(Runner &r, Acts &a, int rows) {
+    const Config &c = r.cfg;
+    if (a.rows == rows) return;
+    for (int32_t *id : {&a.x, &a.x2, &a.qkv, &a.q, &a.att, &a.ff, &a.ids, &a.cq, &a.ckv}) r.release(*id);
+    int64_t S = rows, d = c.d;
+    a.x = r.alloc(S * d); a.x2 = r.alloc(S * d); a.q = r.alloc(S * d); a.att = r.alloc(S * d);
+    a.ff = r.alloc(S * c.dff); a.ids = r.alloc(std::max<int64_t>(S, 4));
+    if (c.kind == 0) a.qkv = r.alloc(S * 3 * d);
+    else { a.cq = r.alloc(S * c.q_rank); a.ckv = r.alloc(S * c.kv_rank); a.qkv = r.alloc(S * d); }
+    a.rows = rows;
+}
+
+void finalize(Runner &r) {
+    const Config &c = r.cfg;
+    if (r.finalized) return;
+    for (const auto &n : weight_names(c))
+        if (!r.have.count(n)) throw Error("weight " + n + " was never set");
+    const int hd = r.hd(), half = hd / 2;
+    // RotaryEmbedding.java:63-70
+    std::vector<float> ct((size_t)c.max_seq * half), st((size_t)c.max_seq * half);
+    for (int pos = 0; pos < c.max_seq; pos++)
+        for (int i = 0; i < half; i++) {
+            float expo = (2.0f * (float)i) / (float)hd;
+            float theta = (float)((double)pos / std::pow((double)10000.0f, (double)expo));
+            ct[(size_t)pos * half + i] = (float)std::cos((double)theta);
+            st[(size_t)pos * half + i] = (float)std::sin((double)theta);
+        }
+    r.cos_t = r.upload_new(ct.data(), (int64_t)ct.size());
+    r.sin_t = r.upload_new(st.data(), (int64_t)st.size());
+    int64_t per_layer = (int64_t)c.max_seq * c.d;
+    if (c.kind == 0) {
+        r.kc = r.alloc(per_layer * c.layers);
+        r.vc = r.alloc(per_layer * c.layers);
+    } else {
+        r.latent = r.alloc((int64_t)c.layers * c.max_seq * c.kv_rank);   // cKV rows, the only per-token state
+        r.kc = r.alloc(per_layer);                                        // K re-expanded + rotated, one layer at a time
+        r.vc = r.alloc(per_layer);
+        r.dec.kvexp = r.alloc((int64_t)c.max_seq * 2 * c.d);              // [maxSeq x (K|V)] expansion output
+    }
+    r.state = r.alloc(4);
+    r.tok = r.alloc(4);
+    r.tokens = r.alloc(c.max_seq);
+    r.logits = r.alloc(c.vocab);
+    r.last_x = r.alloc(c.d);
+    int splits = (c.max_seq + 63) / 64;
+    int64_t sf = (int64_t)c.heads * (4 + (int64_t)splits * (hd + 4));
+    r.scratch = r.alloc(sf);
+    Stream s;
+    emit(s, DJ_OP_FILL, r.scratch, 0, (int32_t)sf);
+    emit(s, DJ_OP_FILL, r.state, 0, 4);
+    emit(s, DJ_OP_FILL, r.tok, 0, 4);
+    r.run(s);
+    alloc_acts(r, r.dec, 1);
+    r.finalized = true;
+}
+
+// ── command streams ────────────────────────────────────────────────────────
+
+// One transformer block on S rows held in a.x; result back in a.x.
+void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
+    const Config &c = r.cfg;
+    const Layer &L = r.layers[l];
+    const int d = c.d, H = c.heads, hd = r.hd();
+    if (c.kind == 0) {
+        // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
+        q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
+        emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
+        emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
+    } else {
+        throw Error("MLA streams are built by mla_block_stream");
+    }
+    q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
+    // x = x2 + down(SiLU(gate(norm2(x2))) * up(norm2(x2)))                  LlamaTransformerBlock.java:52
+    q8_linear(s, a.x2, L.wgu, a.ff, S, d, c.dff, DJ_LIN_RMSNORM | DJ_LIN_BIAS | DJ_LIN_SWIGLU, L.g2, L.bg, L.bu);
+    q8_linear(s, a.ff, L.wd, a.x, S, c.dff, d, DJ_LIN_BIAS | DJ_LIN_RESIDUAL, -1, L.bd, -1, a.x2);
+}
+
+void head_stream(Runner &r, Stream &s, int32_t x_row) {
+    const Config &c = r.cfg;
+    q8_linear(s, x_row, r.wlm, r.logits, 1, c.d, c.vocab, DJ_LIN_RMSNORM | DJ_LIN_BIAS, r.gf, r.blm);
+}
+
+Stream decode_stream(Runner &r, bool sample_on_device) {
+    const Config &c = r.cfg;
+    Stream s;
+    emit(s, DJ_OP_EMBED_GATHER, r.emb, r.state, r.dec.x, 1, c.d, c.vocab, 1);    // token = state[1]
+    for (int l = 0; l < c.layers; l++) block_stream(r, s, r.dec, l, 1);
+    head_stream(r, s, r.dec.x);
+    if (sample_on_device) {
+        emit(s, DJ_OP_ARGMAX_ROWS, r.logits, r.tok, 1, c.vocab);
+        emit(s, DJ_OP_DECODE_ADVANCE, r.state, r.tok, r.tokens, c.max_seq, 1);
+    }
+    return s;
+}
+
+void check_ids(const Config &c, const int32_t *ids, int n) {
+    for (int i = 0; i < n; i++)
+        if (ids[i] < 0 || ids[i] >= c.vocab) throw Error("Token id out of range: " + std::to_string(ids[i]));   // Embedding.java:30-32
+}
+
+// Runs the prompt rows through the model, filling the cache.  Leaves the last row's
+// logits in r.logits; with choose != 0 also picks the next token greedily on the device.
+void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choose) {
+    const Config &c = r.cfg;
+    if (!r.finalized) finalize(r);
+    if (n <= 0) throw Error("prefill: empty prompt");
+    check_ids(c, ids, n);
+    if (r.pos + n > c.max_seq)
+        throw Error("context of " + std::to_string(r.pos + n) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
+    alloc_acts(r, r.pre, n);
+    hip(deepj_hip_upload(r.pre.ids, reinterpret_cast<const float *>(ids), n));
+    Stream s;
+    emit(s, DJ_OP_EMBED_GATHER, r.emb, r.pre.ids, r.pre.x, n, c.d, c.vocab, 0);
+    for (int l = 0; l < c.layers; l++) block_stream(r, s, r.pre, l, n);
+    emit(s, DJ_OP_COPY, r.pre.x, r.last_x, c.d, (int64_t)(n - 1) * c.d, 0);
+    head_stream(r, s, r.last_x);
+    if (choose) {
+        emit(s, DJ_OP_ARGMAX_ROWS, r.logits, r.tok, 1, c.vocab);
+        emit(s, DJ_OP_DECODE_ADVANCE, r.state, r.tok, r.tokens, c.max_seq, n);
+    }
+    r.run(s);
+    if (all_logits) {
+        // DecoderOnlyModel.forward returns logits for every row; only parity tests ask for them.
+        int32_t full = r.alloc((int64_t)n * c.vocab);
+        Stream t;
+        q8_linear(t, r.pre.x, r.wlm, full, n, c.d, c.vocab, DJ_LIN_RMSNORM | DJ_LIN_BIAS, r.gf, r.blm);
+        r.run(t);
+        hip(deepj_hip_download(full, all_logits, (int64_t)n * c.vocab));
+        r.release(full);
+    }
+    if (choose) { r.pos += n; r.generated += 1; }
+    else {
+        // advance the position without choosing a token
+        int32_t st[4] = {r.pos + n, 0, r.generated, 0};
+        hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
+        r.pos += n;
+    }
+}
+
+void reset(Runner &r) {
+    if (!r.finalized) finalize(r);
+    int32_t st[4] = {0, 0, 0, 0};
+    hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
+    r.pos = 0;
+    r.generated = 0;
+}
+
+// Greedy steps on the device: each consumes state[1] at position state[0] and appends the argmax.
+void decode_greedy(Runner &r, int steps, bool use_graph) {
+    const Config &c = r.cfg;
+    if (steps <= 0) return;
+    if (r.pos + steps > c.max_seq)
+        throw Error("context of " + std::to_string(r.pos + steps) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
+    if (use_graph) {
+        if (!r.graph) {
+            Stream s = decode_stream(r, true);
+            hip(deepj_hip_graph_capture(s.data(), (int32_t)s.size(), &r.graph));
+        }
+        hip(deepj_hip_graph_launch(r.graph, steps));
+    } else {
+        Stream s = decode_stream(r, true);
+        for (int i = 0; i < steps; i++) r.run(s);
+    }
+    r.pos += steps;
+    r.generated += steps;
+}
+
+// ── TextGenerator.sampleFromLogits on the host (temperature / top-k > 1) ────
+
+int java_float_compare(float x, float y) {
+    if (x < y) return -1;
+    if (x > y) return 1;
+    int32_t bx, by;
+    std::memcpy(&bx, &x, 4); std::memcpy(&by, &y, 4);
+    if (x != x) bx = 0x7fc00000;
+    if (y != y) by = 0x7fc00000;
+    return bx == by ? 0 : (bx < by ? -1 : 1);
+}
+
+int32_t sample_from_logits(const std::vector<float> &logits, float temperature, int top_k, void *rng) {
+    int n = (int)logits.size();
+    std::vector<int32_t> order(n);
+    for (int i = 0; i < n; i++) order[i] = i;
+    // stable sort, descending (TextGenerator.java:163-170)
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int32_t i, int32_t j) { return java_float_compare(logits[j], logits[i]) < 0; });
+    int k = top_k == 0 ? n : std::min(top_k, n);
+    float mx = -INFINITY;
+    for (int i = 0; i < k; i++) mx = std::max(mx, logits[order[i]] / temperature);
+    std::vector<float> probs(k);
+    float sum = 0.0f;
+    for (int i = 0; i < k; i++) {
+        float p = (float)std::exp((double)(logits[order[i]] / temperature - mx));
+        probs[i] = p;
+        sum += p;
+    }
+    for (float &p : probs) p /= sum;
+    float u = deepj_host_random_next_float(rng), cum = 0.0f;
+    for (int i = 0; i < k; i++) {
+        cum += probs[i];
+        if (u <= cum) return order[i];
+    }
+    return order[k - 1];
+}
+
+// TextGenerator.generate on token ids (TextGenerator.java:66-87).  out holds n_prompt + max_new ids.
+void generate(Runner &r, const int32_t *prompt, int n_prompt, int max_new, float temperature, int top_k,
+              int64_t seed, int32_t *out, bool use_graph) {
+    const Config &c = r.cfg;
+    if (max_new < 0) throw Error("maxNewTokens must be >= 0");
+    if (!(temperature > 0.0f)) throw Error("temperature must be > 0");
+    if (top_k < 0) throw Error("topK must be >= 0");
+    if (max_new > 0 && n_prompt + max_new - 1 > c.max_seq)
+        throw Error("context of " + std::to_string(n_prompt + max_new - 1) + " tokens exceeds maxSeqLen " +
+                    std::to_string(c.max_seq) + " (the sliding window of TextGenerator is not cached)");
+    std::memcpy(out, prompt, (size_t)n_prompt * sizeof(int32_t));
+    if (max_new == 0) return;
+    reset(r);
+    if (top_k == 1) {
+        // argmax needs no random draw to pick, and greedy output is seed independent
+        prefill(r, prompt, n_prompt, nullptr, true);
+        decode_greedy(r, max_new - 1, use_graph);
+        hip(deepj_hip_download(r.tokens, reinterpret_cast<float *>(out + n_prompt), max_new));
+        return;
+    }
+    void *rng = deepj_host_random_create(seed);
+    try {
+        std::vector<float> logits((size_t)c.vocab);
+        Stream fwd = decode_stream(r, false);
+        prefill(r, prompt, n_prompt, nullptr, false);
+        for (int t = 0; t < max_new; t++) {
+            if (t > 0) {
+                r.run(fwd);          // consumes the token in state[1] at position state[0]
+                r.pos += 1;
+            }
+            hip(deepj_hip_download(r.logits, logits.data(), c.vocab));
+            int32_t next = sample_from_logits(logits, temperature, top_k, rng);
+            out[n_prompt + t] = next;
+            int32_t st[4] = {r.pos, next, t + 1, 0};
+            hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
+            r.generated = t + 1;
+        }
+    } catch (...) {
+        deepj_host_random_destroy(rng);
+        throw;
+    }
+    deepj_host_random_destroy(rng);
+}
+
+template <class F> int guarded(Runner *r, F &&f) {
+    try {
+        f();
+        if (r) r->error.clear();
+        return 0;
+    } catch (const std::exception &ex) {
+        if (r) r->error = ex.what();
+        return 1;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+// cfg: {kind, vocab, maxSeq, dModel, nHeads, nLayers, dFF, qRank, kvRank}; id_base: first buffer id this
+// runner may use (pick a range the ComputeGraph never reaches, e.g. 1 << 29).
+void *deepj_runner_create(const int32_t cfg[9], int32_t id_base) {
+    Config c{cfg[0], cfg[1], cfg[2], cfg[3], cfg[4], cfg[5], cfg[6], cfg[7], cfg[8]};
+    // TransformerConfig.validateCommon (models/TransformerConfig.java:19-31) + DeepSeekConfig.java:31-35
+    if (c.vocab <= 0 || c.max_seq <= 0 || c.d <= 0 || c.heads <= 0 || c.layers <= 0 || c.dff <= 0) return nullptr;
+    if (c.d % c.heads != 0) return nullptr;
+    if (c.kind == 1 && (c.q_rank <= 0 || c.kv_rank <= 0)) return nullptr;
+    if (c.kind != 0 && c.kind != 1) return nullptr;
+    int hd = c.d / c.heads;
+    if (hd != 32 && hd != 64 && hd != 128) return nullptr;
+    auto *r = new Runner;
+    r->cfg = c;
+    r->next_id = id_base;
+    r->layers.resize((size_t)c.layers);
+    return r;
+}
+
+void deepj_runner_destroy(void *h) {
+    auto *r = static_cast<Runner *>(h);
+    if (!r) return;
+    if (r->graph) deepj_hip_graph_destroy(r->graph);
+    deepj_hip_synchronize();
+    // every id in [id_base, next_id) that is still live belongs to this runner
+    std::vector<int32_t> ids;
+    auto add = [&](int32_t id) { if (id >= 0) ids.push_back(id); };
+    for (auto &L : r->layers)
+        for (int32_t id : {L.g1, L.g2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wukv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
+    for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state, r->tok,
+                       r->tokens, r->scratch, r->logits, r->last_x})
+        add(id);
+    for (Acts *a : {&r->dec, &r->pre})
+        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv, a->kfull, a->vfull, a->kvexp}) add(id);
+    if (!ids.empty()) deepj_hip_release(ids.data(), (int32_t)ids.size());
+    delete r;
+}
+
+const char *deepj_runner_last_error(void *h) { return h ? static_cast<Runner *>(h)->error.c_str() : "null runner"; }
+
+int deepj_runner_set_weight(void *h, const char *name, const float *data, int32_t rows, int32_t cols) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { set_weight(*r, name, data, rows, cols); });
+}
+
+int deepj_runner_init_seeded(void *h, int64_t seed, int32_t threads) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { init_seeded(*r, seed, threads); });
+}
+
+int deepj_runner_finalize(void *h) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { finalize(*r); });
+}
+
+int deepj_runner_reset(void *h) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { reset(*r); });
+}
+
+// all_logits: null, or room for n*vocab floats (logits of every prompt row, as DecoderOnlyModel.forward returns)
+int deepj_runner_prefill(void *h, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { prefill(*r, ids, n, all_logits, choose_next != 0); });
+}
+
+int deepj_runner_decode(void *h, int32_t steps, int32_t use_graph) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { decode_greedy(*r, steps, use_graph != 0); });
+}
+
+int deepj_runner_last_logits(void *h, float *out) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { hip(deepj_hip_download(r->logits, out, r->cfg.vocab)); });
+}
+
+// tokens generated so far in this sequence (device order); returns the count through *n
+int deepj_runner_tokens(void *h, int32_t *out, int32_t capacity, int32_t *n) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] {
+        int32_t count = std::min(r->generated, capacity);
+        if (count > 0) hip(deepj_hip_download(r->tokens, reinterpret_cast<float *>(out), count));
+        else hip(deepj_hip_synchronize());
+        if (n) *n = count;
+    });
+}
+
+int deepj_runner_generate(void *h, const int32_t *prompt, int32_t n_prompt, int32_t max_new, float temperature,
+                          int32_t top_k, int64_t seed, int32_t use_graph, int32_t *out) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { generate(*r, prompt, n_prompt, max_new, temperature, top_k, seed, out, use_graph != 0); });
+}
+
+// The per-token command stream (for inspection, timing and graph capture by the caller).
+int deepj_runner_decode_stream(void *h, int32_t *out, int32_t capacity, int32_t *len) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] {
+        if (!r->finalized) finalize(*r);
+        Stream s = decode_stream(*r, true);
+        if (len) *len = (int32_t)s.size();
+        if (out && capacity >= (int32_t)s.size()) std::memcpy(out, s.data(), s.size() * sizeof(int32_t));
+    });
+}
+
+}  // extern "C"

@@ -176,7 +176,7 @@ int stride_of(int op) {
         case DJ_OP_ROPE_KV_STORE: return 13;
         case DJ_OP_ATTENTION: return 12;
         case DJ_OP_ARGMAX_ROWS: return 5;
-        case DJ_OP_DECODE_ADVANCE: return 5;
+        case DJ_OP_DECODE_ADVANCE: return 6;
         case DJ_OP_COPY: return 6;
         case DJ_OP_FILL: return 4;
         case DJ_OP_ROPE_ROWS: return 11;
@@ -475,14 +475,15 @@ void exec_one(Cursor &c) {
             break;
         }
         case DJ_OP_DECODE_ADVANCE: {
-            // [op, state, token, tokens, capacity]
+            // [op, state, token, tokens, capacity, nPositions]
             int64_t cap = w[4]; need_positive(op, "capacity", cap);
+            need_positive(op, "positions", w[5]);
             float *st = buf(w[1], 4, op, "state");
             const float *tk = buf(w[2], 1, op, "token");
             float *out = buf(w[3], std::max<int64_t>(cap, 1), op, "tokens");
             if (run)
                 launch_decode_advance(s, reinterpret_cast<int32_t *>(st), reinterpret_cast<const int32_t *>(tk),
-                                      reinterpret_cast<int32_t *>(out), (int)cap);
+                                      reinterpret_cast<int32_t *>(out), (int)cap, w[5]);
             break;
         }
         case DJ_OP_COPY: {

@@ -103,8 +103,8 @@ class Stream:
 
     def argmax_rows(self, logits, out, rows, cols): return self.emit(op.OP_ARGMAX_ROWS, logits, out, rows, cols)
 
-    def decode_advance(self, state, token, tokens, capacity):
-        return self.emit(op.OP_DECODE_ADVANCE, state, token, tokens, capacity)
+    def decode_advance(self, state, token, tokens, capacity, n_pos=1):
+        return self.emit(op.OP_DECODE_ADVANCE, state, token, tokens, capacity, n_pos)
 
     def copy(self, src, dst, n, src_off=0, dst_off=0): return self.emit(op.OP_COPY, src, dst, n, src_off, dst_off)
     def fill(self, dst, bits, n): return self.emit(op.OP_FILL, dst, bits, n)

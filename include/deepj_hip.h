@@ -118,9 +118,13 @@ enum {
      *     qkv [S x 3d]; rows sit at positions state[0]..state[0]+S-1
      * ATTENTION     [op, q, kCache, vCache, out, state, scratch, S, H, hd, maxSeq, layer]
      * ARGMAX_ROWS   [op, logits, out, rows, cols]      out int32 words, ties -> lowest index
-     * DECODE_ADVANCE[op, state, tokens, capacity]      see DESIGN.md
+     * DECODE_ADVANCE[op, state, token, tokens, capacity, nPos]
+     *     state (int32 words): [0] positions held in the cache, [1] current token, [2] tokens generated;
+     *     tokens[state[2]++] = token[0]; state[1] = token[0]; state[0] += nPos
      * COPY          [op, src, dst, n, srcOff, dstOff]
      * FILL          [op, dst, bits, n]
+     * ROPE_ROWS     [op, x, out, state, cosT, sinT, rows, H, hd, maxSeq, posFromRow]  token-major rows
+     * ATTENTION_KV  [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0]  k, v token-major [maxSeq x H*hd]
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
@@ -132,6 +136,41 @@ enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU =
 
 /* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
+
+/* ── host side: java.util.Random twin ─────────────────────────────────────
+ * Tensor.random(rows, cols, Random) of the reference (J/tensor/cpu/CpuBackend.java:148-152)
+ * reproduced bit for bit (JDK-specified LCG + polar nextGaussian with StrictMath.log),
+ * multi-threaded for large tensors. */
+void   *deepj_host_random_create(int64_t seed);
+void    deepj_host_random_destroy(void *rng);
+void    deepj_host_random_fill(void *rng, float *out, int64_t n, double scale, int32_t threads);
+double  deepj_host_random_next_gaussian(void *rng);
+int32_t deepj_host_random_next_int(void *rng, int32_t bound);   /* bound <= 0: nextInt() */
+float   deepj_host_random_next_float(void *rng);
+
+/* ── host side: decode driver ─────────────────────────────────────────────
+ * The inference caller above the five GpuRuntime calls: LlamaModel / DeepSeekModel +
+ * TextGenerator of the reference (J/models/DecoderOnlyModel.java:58-64,
+ * J/models/TextGenerator.java:66-181) with a device-resident KV cache, Q8 weights and one
+ * fused command stream per token replayed as a HIP graph.  It uses only the functions
+ * above.  cfg = {kind (0 Llama, 1 DeepSeek), vocab, maxSeq, dModel, nHeads, nLayers, dFF,
+ * qRank, kvRank}; id_base = first buffer id the runner may use.  Weight names: "emb",
+ * "gf", "wlm", "blm", "L<i>.g1|g2|wq|wk|wv|wo|wdq|wuq|wdkv|wuk|wuv|wg|bg|wu|bu|wd|bd";
+ * matrices in the reference's [dIn x dOut] fp32 orientation. */
+void       *deepj_runner_create(const int32_t cfg[9], int32_t id_base);   /* NULL: invalid config */
+void        deepj_runner_destroy(void *runner);
+const char *deepj_runner_last_error(void *runner);
+int deepj_runner_set_weight(void *runner, const char *name, const float *data, int32_t rows, int32_t cols);
+int deepj_runner_init_seeded(void *runner, int64_t seed, int32_t threads);  /* new LlamaModel(cfg, seed) */
+int deepj_runner_finalize(void *runner);
+int deepj_runner_reset(void *runner);
+int deepj_runner_prefill(void *runner, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next);
+int deepj_runner_decode(void *runner, int32_t steps, int32_t use_graph);
+int deepj_runner_last_logits(void *runner, float *out);
+int deepj_runner_tokens(void *runner, int32_t *out, int32_t capacity, int32_t *n);
+int deepj_runner_generate(void *runner, const int32_t *prompt, int32_t n_prompt, int32_t max_new,
+                          float temperature, int32_t top_k, int64_t seed, int32_t use_graph, int32_t *out);
+int deepj_runner_decode_stream(void *runner, int32_t *out, int32_t capacity, int32_t *len);
 
 #ifdef __cplusplus
 }

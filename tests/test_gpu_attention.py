@@ -1,0 +1,102 @@
+"""RoPE + KV-cache store and causal attention kernels against the oracle's literal
+MultiHeadSelfAttention pieces (split heads, RoPE, per-head q.k^T*scale + mask, softmax, p.v,
+merge) on the same inputs: prefill chunks, then single-row decode steps over the growing
+cache (split-K path), for head dims 32/64/128."""
+import numpy as np
+import pytest
+
+from deepj_amd.fused import DeviceBuffers, Stream, attention_scratch_floats
+from oracle import cpu_ref as ref
+from gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def gaussian(rows, cols, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal((rows, cols)) * scale).astype(np.float32)
+
+
+def oracle_attention(q, k, v, H, cos, sin):
+    """merged attention output for all rows, literal reference path."""
+    qh = ref.rope_apply(ref.split_heads(q, H), q.shape[0], H, cos, sin)
+    kh = ref.rope_apply(ref.split_heads(k, H), q.shape[0], H, cos, sin)
+    vh = ref.split_heads(v, H)
+    return ref.merge_heads(ref.attention_heads(qh, kh, vh, H, causal=True), H)
+
+
+@pytest.mark.parametrize("H,hd,max_seq,chunks", [(8, 32, 256, [32, 1, 1, 1]), (4, 64, 200, [70, 1, 1, 60, 1]),
+                                                 (2, 128, 130, [5, 1, 124]), (32, 64, 2048, [3, 1])])
+def test_rope_store_attention_prefill_and_decode(H, hd, max_seq, chunks):
+    d = H * hd
+    total = sum(chunks)
+    layers, layer = 2, 1                                 # exercise the per-layer offset
+    q, k, v = (gaussian(total, d, 10 + i) for i in range(3))
+    cos, sin = ref.rope_tables(hd, max_seq)
+    exp = oracle_attention(q, k, v, H, cos, sin)
+
+    dev = DeviceBuffers()
+    try:
+        kc, vc = dev.alloc(layers * max_seq * d), dev.alloc(layers * max_seq * d)
+        state = dev.upload(np.zeros(4, np.int32))
+        cos_b, sin_b = dev.upload(cos), dev.upload(sin)
+        sf = attention_scratch_floats(H, hd, max_seq)
+        scratch = dev.alloc(sf)
+        tok, tokens = dev.upload(np.zeros(4, np.int32)), dev.alloc(max_seq)
+        Stream().fill(scratch, 0, sf).run()
+        pos = 0
+        for S in chunks:
+            qkv = np.concatenate([q[pos:pos + S], k[pos:pos + S], v[pos:pos + S]], axis=1)
+            qkv_b, q_b, out_b = dev.upload(qkv), dev.alloc(S * d), dev.alloc(S * d)
+            (Stream().rope_kv_store(qkv_b, q_b, kc, vc, state, cos_b, sin_b, S, H, hd, max_seq, layer)
+             .attention(q_b, kc, vc, out_b, state, scratch, S, H, hd, max_seq, layer)
+             .decode_advance(state, tok, tokens, max_seq, S).run())
+            got = dev.download(out_b, (S, d))
+            assert_close(exp[pos:pos + S], got, atol=2e-5, rtol=1e-4, what=f"rows {pos}..{pos + S} of {chunks}")
+            dev.release(qkv_b, q_b, out_b)
+            pos += S
+        st = dev.download(state, (4,), np.int32)
+        assert st[0] == total and st[2] == len(chunks)
+        # the scratch counters are back to zero (ready for a graph replay)
+        sc = dev.download(scratch, (sf,), np.int32).reshape(H, -1)
+        assert np.all(sc[:, 0] == 0)
+    finally:
+        dev.release_all()
+
+
+def test_rope_rows_and_attention_over_token_major_kv():
+    H, hd, max_seq, n = 4, 32, 64, 37
+    d = H * hd
+    q, k, v = (gaussian(n, d, 20 + i) for i in range(3))
+    cos, sin = ref.rope_tables(hd, max_seq)
+    exp = oracle_attention(q, k, v, H, cos, sin)
+    dev = DeviceBuffers()
+    try:
+        state = dev.upload(np.array([n - 1, 0, 0, 0], np.int32))      # the query is the last row
+        cos_b, sin_b = dev.upload(cos), dev.upload(sin)
+        kpad = np.zeros((max_seq, d), np.float32); kpad[:n] = k
+        vpad = np.zeros((max_seq, d), np.float32); vpad[:n] = v
+        k_b, kr_b, v_b = dev.upload(kpad), dev.alloc(max_seq * d), dev.upload(vpad)
+        q_b, qr_b, out_b = dev.upload(q[n - 1:]), dev.alloc(d), dev.alloc(d)
+        sf = attention_scratch_floats(H, hd, max_seq)
+        scratch = dev.alloc(sf)
+        (Stream().fill(scratch, 0, sf)
+         .rope_rows(k_b, kr_b, state, cos_b, sin_b, max_seq, H, hd, max_seq, True)      # position = row
+         .rope_rows(q_b, qr_b, state, cos_b, sin_b, 1, H, hd, max_seq, False)           # position = state[0]
+         .attention_kv(qr_b, kr_b, v_b, out_b, state, scratch, 1, H, hd, max_seq).run())
+        assert_close(exp[n - 1:], dev.download(out_b, (1, d)), atol=2e-5, rtol=1e-4)
+        kr = dev.download(kr_b, (max_seq, d))
+        assert_close(ref.merge_heads(ref.rope_apply(ref.split_heads(k, H), n, H, cos, sin), H), kr[:n], 1e-6, 1e-6)
+    finally:
+        dev.release_all()
+
+
+def test_attention_rejects_bad_shapes():
+    dev = DeviceBuffers()
+    try:
+        b = dev.alloc(64)
+        with pytest.raises(RuntimeError, match="head dim must be 32, 64 or 128"):
+            Stream().attention(b, b, b, b, b, b, 1, 1, 48, 1, 0).run()
+        with pytest.raises(RuntimeError, match="op needs"):
+            Stream().attention(b, b, b, b, b, b, 1, 2, 32, 64, 0).run()       # cache too small
+    finally:
+        dev.release_all()

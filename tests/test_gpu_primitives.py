@@ -74,8 +74,9 @@ def test_reductions_and_transpose_match_cpu(rows, cols):              # :115-135
         assert_close(ref.mean_along_rows(a), be.meanAlongRows(ta))
         assert_close(ref.variance_along_rows(a), be.varianceAlongRows(ta))
         assert_close(ref.max_along_rows(a), be.maxAlongRows(ta), 0, 0)
-        assert abs(ref.sum_(a) - be.sum(ta)) <= 1e-4 + 1e-5 * cols
-        assert abs(ref.sum_abs(a) - be.sumAbs(ta)) <= 1e-3
+        # whole-tensor fp32 sums: the CPU's sequential sum itself carries ~n*eps relative error
+        assert abs(ref.sum_(a) - be.sum(ta)) <= 1e-4 + 1e-5 * ref.sum_abs(a)
+        assert abs(ref.sum_abs(a) - be.sumAbs(ta)) <= 1e-4 + 1e-5 * ref.sum_abs(a)
 
 
 def test_unary_math_and_activations():
@@ -141,7 +142,7 @@ def test_scalar_sum_abs_and_cross_entropy_loss_match_cpu():           # :199-238
             targets = list(ref.JavaRandom(ts).ints(rows, cols))
             assert abs(ref.cross_entropy_loss(logits, targets) - be.crossEntropyLoss(tensor(logits), targets)) <= tol
         wide = rnd(29, 513, 132)
-        assert abs(ref.sum_abs(wide) - be.sumAbs(tensor(wide))) <= 1e-3
+        assert abs(ref.sum_abs(wide) - be.sumAbs(tensor(wide))) <= 1e-3 + 1e-5 * ref.sum_abs(wide)
 
 
 def test_softmax_backward_matches_cpu():                              # :240-266
