@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Decode benchmark of the MI355X HipBackend path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[2], the configuration the headline metric is quoted on):
+Llama decode, dModel 2048, 16 layers, 32 heads (head dim 64), SwiGLU hidden 5632, vocab
+32000, maxSeq 2048; weights = new LlamaModel(cfg, 42) (java.util.Random Gaussians x 0.1),
+all matmul weights Q8; prompt = 512 ids from Random(3).nextInt(32000); batch-1 greedy decode
+with a device-resident fp32 KV cache.  A step = one decoded token (one replay of the
+per-token HIP graph).  Prints ONE JSON line.
+
+Besides tok/s the line carries
+  roofline     - the Q8 matvec kernel (the dominant kernel): algorithmic bytes per launch /
+                 average launch duration, measured with HIP events on the library's stream
+                 over back-to-back launches on the model's own weights (1 GB of distinct
+                 weights per token, so nothing is served from the 256 MB Infinity Cache)
+  cpu_baseline - the CPU oracle (a C restatement of the reference's CpuBackend + layers,
+                 not the JVM) on this box's host cores, on a bounded sample of the workload
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+
+
+def q8_linear_bytes(k: int, n_rows: int) -> int:
+    """Algorithmic bytes of one M = 1 Q8 matvec: int8 weights + one fp32 scale per 32 + x + y."""
+    return k * n_rows + 4 * k * n_rows // 32 + 4 * k + 4 * n_rows
+
+
+def matvec_roofline(model, iters: int = 20):
+    """Times only the Q8_LINEAR ops of the per-token stream, in order, on the real weights."""
+    from deepj_amd import HipNative, opcodes as op
+    stream = model.decodeStream()
+    strides = op.FUSED_STRIDES
+    pos, lin, total_bytes, launches = 0, [], 0, 0
+    while pos < len(stream):
+        code = int(stream[pos])
+        n = strides[code]
+        if code == op.OP_Q8_LINEAR:
+            w = stream[pos:pos + n]
+            m, k, nn, flags = int(w[4]), int(w[5]), int(w[6]), int(w[7])
+            if m == 1:
+                rows = 2 * nn if flags & op.LIN_SWIGLU else nn
+                total_bytes += q8_linear_bytes(k, rows)
+                launches += 1
+                lin.extend(int(x) for x in w)
+        pos += n
+    lin = np.asarray(lin, dtype=np.int32)
+    HipNative.timeOps(lin, 2)                                   # warm-up
+    ms = HipNative.timeOps(lin, iters)
+    avg_launch_s = ms * 1e-3 / (iters * launches)
+    achieved = (total_bytes / launches) / avg_launch_s / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "k_q8_matvec", "launches_per_token": launches,
+            "bytes_per_launch": total_bytes // launches, "avg_launch_us": round(avg_launch_s * 1e6, 3)}
+
+
+def cpu_baseline(cfg, ctx: int, tokens: int = 6):
+    """Oracle timing, like for like: S = 1 with a KV cache at context `ctx`.
+
+    Sample: a model with the workload's dims but ONE of its 16 layers; the per-token time is
+    split into layer and head parts and scaled to all layers.  CpuBackend.matmul parallelises
+    over the rows of A only (CpuBackend.java:175), so M = 1 runs on one thread by construction."""
+    from oracle import cpu_ref as ref
+    threads = ref.default_threads()
+    ref.set_threads(threads)
+    m = ref.Model(vocab=cfg.vocabSize, max_seq=cfg.maxSeqLen, d=cfg.dModel, heads=cfg.nHeads, layers=1,
+                  dff=cfg.dFF, seed=42)
+    ids = ref.JavaRandom(3).ints(ctx + tokens, cfg.vocabSize)
+    m.reset_cache()
+    t0 = time.perf_counter()
+    m.forward_cached(ids[:ctx], last_only=True)                  # fills the cache (rows run in parallel)
+    t_prefill = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for i in range(tokens):
+        m.forward_cached(ids[ctx + i:ctx + i + 1], last_only=True)
+    t_tok = (time.perf_counter() - t0) / tokens
+    x = np.ones((1, cfg.dModel), np.float32)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        ref.linear(ref.rmsnorm(x, m.weight("gf")), m.weight("wlm"), m.weight("blm"))
+    t_head = (time.perf_counter() - t0) / 3
+    t_layer = max(t_tok - t_head, 1e-9)
+    per_token = cfg.nLayers * t_layer + t_head
+    # reference-faithful figure: no KV cache, the whole context re-run per token (TextGenerator.java:91-100)
+    full_ctx_s = cfg.nLayers * max(t_prefill - 0.0, 0.0) * (ctx + 1) / ctx
+    m.close()
+    ref.set_threads(1)
+    return {"value": round(1.0 / per_token, 4), "unit": "tok/s", "cores": 1, "kind": "port",
+            "sample": f"C restatement of CpuBackend (not the JVM); 1 of {cfg.nLayers} layers + LM head at context "
+                      f"{ctx}, {tokens} tokens, scaled to {cfg.nLayers} layers; S=1 matmul is single-threaded by "
+                      f"construction",
+            "no_kv_cache_s_per_token": round(full_ctx_s, 2), "no_kv_cache_threads": threads}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--prompt", type=int, default=512)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (one MI355X per box); --gpus > 1 is not supported", file=sys.stderr)
+        return 2
+
+    from deepj_amd import HipNative, JavaRandom, LlamaConfig, LlamaModel
+
+    cfg = LlamaConfig(vocabSize=32000, maxSeqLen=2048, dModel=2048, nHeads=32, nLayers=16, dFF=5632)
+    if args.prompt + args.warmup + args.steps > cfg.maxSeqLen:
+        print("bench.py: prompt + warmup + steps exceeds maxSeq 2048", file=sys.stderr)
+        return 2
+    t0 = time.perf_counter()
+    model = LlamaModel(cfg, 42)
+    t_build = time.perf_counter() - t0
+    prompt = JavaRandom(3).ints(args.prompt, cfg.vocabSize)
+
+    model.reset()
+    t0 = time.perf_counter()
+    model.prefill(prompt)
+    HipNative.synchronize()
+    t_prefill = time.perf_counter() - t0
+
+    model.decode(args.warmup)                       # captures the graph on first use
+    HipNative.synchronize()
+    t0 = time.perf_counter()
+    model.decode(args.steps)
+    HipNative.synchronize()
+    elapsed = time.perf_counter() - t0
+    toks = model.tokens()
+    assert len(toks) == 1 + args.warmup + args.steps
+
+    roof = matvec_roofline(model)
+    cpu = None if args.no_cpu_baseline else cpu_baseline(cfg, args.prompt)
+
+    # per-token algorithmic bytes at the mean decoded position (weights + fp32 KV read)
+    weights = sum(q8_linear_bytes(k, n) for k, n in
+                  [(2048, 6144), (2048, 2048), (2048, 11264), (5632, 2048)]) * cfg.nLayers + q8_linear_bytes(2048, 32000)
+    mean_pos = args.prompt + args.warmup + args.steps / 2
+    kv = cfg.nLayers * 2 * mean_pos * cfg.dModel * 4
+    tok_s = args.steps / elapsed
+    line = {
+        "metric": "decode tok/s, Q8 Llama d=2048 L=16, 1 GPU; Q8 matvec HBM GB/s vs peak",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "q8 weights (int8 + fp32 scale per 32), fp32 activations/accumulate",
+        "data": "synthetic: seeded random-init weights (java.util.Random seed 42), random prompt ids (seed 3)",
+        "config": {"workload": "llama-decode d2048 L16 H32 dFF5632 V32000, prompt 512, batch 1, greedy, fp32 KV cache",
+                   "prompt_tokens": args.prompt, "decode_tokens": args.steps},
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "end_to_end": {"bytes_per_token": int(weights + kv), "achieved_GBs": round((weights + kv) * tok_s / 1e9, 1),
+                       "frac_of_hbm_peak": round((weights + kv) * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+                       "prefill_tok_s": round(args.prompt / t_prefill, 1), "model_build_s": round(t_build, 1)},
+    }
+    print(json.dumps(line))
+    model.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

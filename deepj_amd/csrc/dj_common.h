@@ -100,6 +100,12 @@ void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *
 void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *state, const float *cos_t,
                       const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row);
 void launch_attention(hipStream_t s, const AttnArgs &a);
+void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *out,
+                        const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,
+                        int max_seq);
+int64_t attn_decode_scratch_floats(int H, int hd);
+void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
+                        const float *table, float *x, int vocab, int d, int n_positions);
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq);
 
 }  // namespace dj

@@ -11,10 +11,12 @@
 // are a single contiguous stream.  A key row is read by hd/4 lanes as float4
 // (a wavefront load covers 64/(hd/4) whole keys = 1 KiB, fully coalesced).
 //
-// Decode (S = 1): the key range is split over gridDim.z workgroups per head so the
-// HBM-bound KV read is spread over all CUs; each split keeps a running
-// (max, sum, weighted V) and the last split to finish - found with a counter in
-// the scratch buffer that it resets for the next launch - merges them.
+// Decode (S = 1) is one fused op: the query and the new key are rotated in registers,
+// the new key/value row is appended to the cache by the workgroup that owns it, the key
+// range is split evenly (computed on the device from the live position, so a captured
+// graph stays valid as the cache grows) over gridDim.y workgroups per head so the
+// HBM-bound KV read is spread over all CUs, and a second tiny kernel merges the
+// per-split (max, sum, weighted V) records.
 #include "dj_common.h"
 
 namespace dj {
@@ -199,6 +201,132 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 
 inline int decode_splits(int max_seq) { return (max_seq + kSplitKeys - 1) / kSplitKeys; }
 
+// ── fused decode attention ──────────────────────────────────────────────────
+// Record layout in scratch, per (head, split): [max, sum, pad, pad, o[hd]].
+struct DecodeArgs {
+    const float *qkv;          // [3d]: q | k | v of the new token (not rotated)
+    float *k_cache, *v_cache;  // this layer, [H][maxSeq][hd]
+    float *out;                // [d]
+    const int32_t *state;
+    float *scratch;
+    const float *cos_t, *sin_t;
+    int H, hd, max_seq, nsplit;
+    float scale;
+};
+
+template <int LPK>
+__global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) {
+    constexpr int HD = LPK * 4;
+    constexpr int KPW = 64 / LPK;
+    constexpr int NSUB = kWaves * KPW;
+    __shared__ float s_m[NSUB], s_l[NSUB];
+    __shared__ __align__(16) float s_o[NSUB][HD];
+
+    const int h = blockIdx.x, split = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane / LPK, dl = lane % LPK;
+    const int d = a.H * HD, half = HD / 2;
+
+    int pos = a.state[0];
+    if (pos < 0) pos = 0;
+    if (pos >= a.max_seq) pos = a.max_seq - 1;             // the host never lets this happen; stay in bounds
+    const int n_keys = pos + 1;
+    const int per = (n_keys + a.nsplit - 1) / a.nsplit;
+    const int k_begin = split * per;
+    const int k_end = k_begin + per < n_keys ? k_begin + per : n_keys;
+
+    // rotate this lane's two (even, odd) pairs of q and of the new k
+    const float2 c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
+    const float2 s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
+    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
+    const float4 qv = make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
+                                  q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y);
+    float *kb = a.k_cache + (int64_t)h * a.max_seq * HD + dl * 4;
+    float *vb = a.v_cache + (int64_t)h * a.max_seq * HD + dl * 4;
+
+    float m = -INFINITY, l = 0.0f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int key = k_begin + wave * KPW + sub; key < k_end; key += kWaves * KPW) {
+        float4 kk, vv;
+        if (key == pos) {                                   // the new token: rotate, use, append
+            const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
+            kk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
+                             k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
+            vv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
+            *reinterpret_cast<float4 *>(kb + (int64_t)key * HD) = kk;
+            *reinterpret_cast<float4 *>(vb + (int64_t)key * HD) = vv;
+        } else {
+            kk = *reinterpret_cast<const float4 *>(kb + (int64_t)key * HD);
+            vv = *reinterpret_cast<const float4 *>(vb + (int64_t)key * HD);
+        }
+        float s = qv.x * kk.x + qv.y * kk.y + qv.z * kk.z + qv.w * kk.w;
+#pragma unroll
+        for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s *= a.scale;
+        float mn = fmaxf(m, s);
+        float corr = expf(m - mn);
+        float p = expf(s - mn);
+        l = l * corr + p;
+        o.x = o.x * corr + p * vv.x; o.y = o.y * corr + p * vv.y;
+        o.z = o.z * corr + p * vv.z; o.w = o.w * corr + p * vv.w;
+        m = mn;
+    }
+    const int slot = wave * KPW + sub;
+    if (dl == 0) { s_m[slot] = m; s_l[slot] = l; }
+    *reinterpret_cast<float4 *>(&s_o[slot][dl * 4]) = o;
+    __syncthreads();
+    if (tid < HD) {
+        float M = -INFINITY, L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NSUB; i++) M = fmaxf(M, s_m[i]);
+        if (M != -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < NSUB; i++) {
+                float w = expf(s_m[i] - M);
+                L += s_l[i] * w;
+                O += s_o[i][tid] * w;
+            }
+        }
+        float *rec = a.scratch + ((int64_t)h * a.nsplit + split) * (HD + 4);
+        rec[4 + tid] = O;
+        if (tid == 0) { rec[0] = M; rec[1] = L; }
+    }
+}
+
+// grid H, block hd threads: out[h*hd + j] = sum_i w_i o_i[j] / sum_i w_i l_i.  All record
+// loads are issued before the first use (nsplit <= 16), so the merge is one L2 round trip.
+__global__ void k_attn_decode_merge(const float *__restrict__ scratch, float *__restrict__ out, int hd, int nsplit) {
+    const int h = blockIdx.x, j = threadIdx.x;
+    const float *base = scratch + (int64_t)h * nsplit * (hd + 4);
+    float m[16], l[16], o[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float *r = base + (int64_t)(i < nsplit ? i : 0) * (hd + 4);
+        m[i] = r[0]; l[i] = r[1]; o[i] = r[4 + j];
+    }
+    float M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; i++) if (i < nsplit) M = fmaxf(M, m[i]);
+    float L = 0.0f, O = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        if (i < nsplit && m[i] != -INFINITY) {
+            float w = expf(m[i] - M);
+            L += l[i] * w;
+            O += o[i] * w;
+        }
+    }
+    out[h * hd + j] = O / L;
+}
+
+// Splits per head for the fused decode op: about two workgroups per CU in total.
+inline int fused_decode_splits(int H) {
+    int ns = 512 / H;
+    if (ns < 1) ns = 1;
+    if (ns > 16) ns = 16;
+    return ns;
+}
+
 }  // namespace
 
 void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *k_cache, float *v_cache,
@@ -228,6 +356,26 @@ void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq) {
     if (S != 1) return 0;
     return (int64_t)H * (4 + (int64_t)decode_splits(max_seq) * (hd + 4));
+}
+
+int64_t attn_decode_scratch_floats(int H, int hd) { return (int64_t)H * fused_decode_splits(H) * (hd + 4); }
+
+void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *out,
+                        const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,
+                        int max_seq) {
+    DecodeArgs a;
+    a.qkv = qkv; a.k_cache = k_cache; a.v_cache = v_cache; a.out = out; a.state = state; a.scratch = scratch;
+    a.cos_t = cos_t; a.sin_t = sin_t; a.H = H; a.hd = hd; a.max_seq = max_seq;
+    a.nsplit = fused_decode_splits(H);
+    a.scale = (float)(1.0 / sqrt((double)hd));
+    dim3 grid(H, a.nsplit);
+    switch (hd) {
+        case 32: hipLaunchKernelGGL(k_attn_decode_partial<8>, grid, dim3(kThreads), 0, s, a); break;
+        case 64: hipLaunchKernelGGL(k_attn_decode_partial<16>, grid, dim3(kThreads), 0, s, a); break;
+        case 128: hipLaunchKernelGGL(k_attn_decode_partial<32>, grid, dim3(kThreads), 0, s, a); break;
+        default: fail("attention: head dim must be 32, 64 or 128");
+    }
+    hipLaunchKernelGGL(k_attn_decode_merge, dim3(H), dim3(hd), 0, s, scratch, out, hd, a.nsplit);
 }
 
 void launch_attention(hipStream_t s, const AttnArgs &p) {

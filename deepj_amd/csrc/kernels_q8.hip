@@ -16,6 +16,8 @@
 // once per workgroup through LDS, where the optional RMSNorm prologue is applied,
 // so norm + projection (+ bias, + residual, or the SwiGLU gate) is one launch.
 // M > 1 goes to the MFMA GEMM in kernels_matmul.hip.
+#include <cstdlib>
+
 #include "dj_common.h"
 
 namespace dj {
@@ -109,81 +111,65 @@ __device__ __forceinline__ float dot16(const int4 &w, const float *xr) {
     return d;
 }
 
-// NC: 1 KiB chunks of one row a lane visits (ceil(Kp/1024)); RU: outputs per iteration.
-template <int NC, int RU, bool SWIGLU>
-__global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
-    extern __shared__ __align__(16) float xs[];   // Kp floats
-    __shared__ float red[kWaves];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// Sum over the 64 lanes with DPP row operations (no LDS traffic); every lane gets the total.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    auto dpp = [](float x, int ctrl_unused) { return x; };
+    (void)dpp;
+#define DJ_DPP_ADD(ctrl, row_mask)                                                                        \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, false))
+    DJ_DPP_ADD(0xB1, 0xf);    // quad_perm [1,0,3,2]
+    DJ_DPP_ADD(0x4E, 0xf);    // quad_perm [2,3,0,1]
+    DJ_DPP_ADD(0x141, 0xf);   // row_half_mirror
+    DJ_DPP_ADD(0x140, 0xf);   // row_mirror: every lane of a 16-lane row holds the row sum
+    DJ_DPP_ADD(0x142, 0xa);   // row_bcast:15 into rows 1 and 3
+    DJ_DPP_ADD(0x143, 0xc);   // row_bcast:31 into rows 2 and 3: lane 63 holds the total
+#undef DJ_DPP_ADD
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
 
-    // stage the activation row (zero beyond K so padded weights meet zeros)
-    float ss = 0.0f;
-    for (int i = tid; i < p.kp; i += kThreads) {
-        float v = i < p.k ? p.x[i] : 0.0f;
-        xs[i] = v;
-        ss += v * v;
-    }
-    if (p.gamma) {                                // RMSNorm prologue, fp32 like the reference
-        ss = wave_sum(ss);
-        if (lane == 0) red[wave] = ss;
-        __syncthreads();
-        float tot = red[0] + red[1] + red[2] + red[3];
-        float rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
-        for (int i = tid; i < p.k; i += kThreads) xs[i] = (xs[i] / rms) * p.gamma[i];
-    }
-    __syncthreads();
+// One batch of Q8 rows held in registers by a wavefront: R rows x NC chunks.
+template <int NC, int R> struct RowBatch {
+    int4 w[R][NC];
+    float sc[R][NC];
+};
 
-    // this lane's activation slice: 16 consecutive k of each 1 KiB chunk
-    float xr[NC][16];
-    bool active[NC];
+// Loads are unconditional: rows past the wave's range are clamped to its last row and
+// chunks past Kp to chunk 0 (their activations are zero), so no load sits under a branch.
+template <int NC, int R>
+__device__ __forceinline__ void load_batch(RowBatch<NC, R> &b, const MatvecArgs &p, int row0, int row_last, int lane,
+                                           int groups) {
 #pragma unroll
-    for (int c = 0; c < NC; c++) {
-        int kb = (c * 64 + lane) * 16;
-        active[c] = kb < p.kp;
+    for (int u = 0; u < R; u++) {
+        int row = row0 + u < row_last ? row0 + u : row_last;
+        const int8_t *wrow = p.wq + (int64_t)row * p.kp;
+        const float *srow = p.scales + (int64_t)row * groups;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float4 v = active[c] ? *reinterpret_cast<const float4 *>(xs + kb + 4 * j) : make_float4(0, 0, 0, 0);
-            xr[c][4 * j] = v.x; xr[c][4 * j + 1] = v.y; xr[c][4 * j + 2] = v.z; xr[c][4 * j + 3] = v.w;
+        for (int c = 0; c < NC; c++) {
+            int chunk = c * 64 + lane;
+            if (chunk * 16 >= p.kp) chunk = 0;
+            b.w[u][c] = *reinterpret_cast<const int4 *>(wrow + chunk * 16);
+            b.sc[u][c] = srow[chunk >> 1];
         }
     }
+}
 
-    constexpr int RPO = SWIGLU ? 2 : 1;           // Q8 rows per output
-    const int groups = p.kp / kQ8Group;
-    const int wave_global = blockIdx.x * kWaves + wave;
-    const int wave_count = gridDim.x * kWaves;
-
-    for (int o0 = wave_global * RU; o0 < p.n_out; o0 += wave_count * RU) {
-        int4 w[RU * RPO][NC];
-        float sc[RU * RPO][NC];
+template <int NC, int B, bool SWIGLU>
+__device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 : 1)> &b, const float (&xr)[NC][16],
+                                             const MatvecArgs &p, int o0, int o_end, int lane) {
+    constexpr int R = B * (SWIGLU ? 2 : 1);
+    float acc[R];
 #pragma unroll
-        for (int u = 0; u < RU * RPO; u++) {
-            int row = o0 * RPO + u;
-            bool row_ok = row < p.n_out * RPO;
+    for (int u = 0; u < R; u++) {
+        float a = 0.0f;
 #pragma unroll
-            for (int c = 0; c < NC; c++) {
-                int chunk = c * 64 + lane;
-                if (row_ok && active[c]) {
-                    w[u][c] = *reinterpret_cast<const int4 *>(p.wq + (int64_t)row * p.kp + chunk * 16);
-                    sc[u][c] = p.scales[(int64_t)row * groups + (chunk >> 1)];
-                } else {
-                    w[u][c] = make_int4(0, 0, 0, 0);
-                    sc[u][c] = 0.0f;
-                }
-            }
-        }
-        float acc[RU * RPO];
+        for (int c = 0; c < NC; c++) a = fmaf(dot16(b.w[u][c], xr[c]), b.sc[u][c], a);
+        acc[u] = wave_sum_dpp(a);
+    }
+    if (lane == 0) {
 #pragma unroll
-        for (int u = 0; u < RU * RPO; u++) {
-            float a = 0.0f;
-#pragma unroll
-            for (int c = 0; c < NC; c++) a = fmaf(dot16(w[u][c], xr[c]), sc[u][c], a);
-            acc[u] = wave_sum(a);
-        }
-        if (lane == 0) {
-#pragma unroll
-            for (int u = 0; u < RU; u++) {
-                int o = o0 + u;
-                if (o >= p.n_out) break;
+        for (int u = 0; u < B; u++) {
+            int o = o0 + u;
+            if (o < o_end) {
                 float v;
                 if constexpr (SWIGLU) {
                     float gate = acc[2 * u], up = acc[2 * u + 1];
@@ -202,24 +188,155 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     }
 }
 
-template <int NC, int RU, bool SW>
-void launch_mv(hipStream_t s, const MatvecArgs &a, int grid) {
+// NC: 1 KiB chunks of one row a lane visits (ceil(Kp/1024)); B: outputs per batch.
+//
+// Batches of outputs are dealt round-robin to the wavefronts.  The weight loads of a
+// wavefront's first batch are issued before anything else - they do not depend on the activations - so
+// the HBM stream is already running while the workgroup stages x through LDS and
+// applies the RMSNorm prologue; after that the next batch is always in flight while
+// the current one is multiplied (two register buffers used in turn).
+template <int NC, int B, bool SWIGLU>
+__global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
+    extern __shared__ __align__(16) float xs[];   // Kp floats
+    __shared__ float red[kWaves];
+    constexpr int RPO = SWIGLU ? 2 : 1;           // Q8 rows per output
+    constexpr int R = B * RPO;                    // rows per batch
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int groups = p.kp / kQ8Group;
+    const int wave_global = blockIdx.x * kWaves + wave;
+    const int wave_count = gridDim.x * kWaves;
+    // Batches are dealt round-robin: batch j of wave w is batch w + j*wave_count of the
+    // matrix, so at any moment the rows in flight across the chip are neighbours in memory.
+    const int n_batches = (p.n_out + B - 1) / B;
+    const bool has_work = wave_global < n_batches;    // wave-uniform
+    const int row_last = p.n_out * RPO - 1;
+    const int o_end = p.n_out;
+    const int o_begin = wave_global * B;
+    const int o_step = wave_count * B;
+
+    RowBatch<NC, R> ba, bb;
+    const bool vec = (p.k & 3) == 0;              // kernel-uniform
+    float4 xv[NC], gv[NC];
+    if (vec) {
+        // The activation (and gain) loads go out first: they hit in L2 and come back while
+        // the weight loads issued right behind them are still on their way from HBM.
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            int e = (tid + kThreads * j) * 4;
+            bool ok = e < p.k;
+            xv[j] = ok ? *reinterpret_cast<const float4 *>(p.x + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+            gv[j] = (ok && p.gamma) ? *reinterpret_cast<const float4 *>(p.gamma + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    if (has_work) load_batch<NC, R>(ba, p, o_begin * RPO, row_last, lane, groups);
+
+    // Stage the activation row through LDS (zero beyond K so padded weights meet zeros).
+    // All global loads of the prologue - x and, for the RMSNorm prologue, gamma - were
+    // issued together, so it costs one memory round trip, not one per element.
+    if (vec) {
+        if (p.gamma) {                            // RMSNorm prologue, fp32 like the reference
+            float ss = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NC; j++) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+            ss = wave_sum_dpp(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = red[0] + red[1] + red[2] + red[3];
+            float rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
+#pragma unroll
+            for (int j = 0; j < NC; j++) {
+                xv[j].x = (xv[j].x / rms) * gv[j].x; xv[j].y = (xv[j].y / rms) * gv[j].y;
+                xv[j].z = (xv[j].z / rms) * gv[j].z; xv[j].w = (xv[j].w / rms) * gv[j].w;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            int e = (tid + kThreads * j) * 4;
+            if (e < p.kp) *reinterpret_cast<float4 *>(xs + e) = xv[j];
+        }
+    } else {
+        float ss = 0.0f;
+        for (int i = tid; i < p.kp; i += kThreads) {
+            float v = i < p.k ? p.x[i] : 0.0f;
+            xs[i] = v;
+            ss += v * v;
+        }
+        if (p.gamma) {
+            ss = wave_sum_dpp(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = red[0] + red[1] + red[2] + red[3];
+            float rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
+            for (int i = tid; i < p.k; i += kThreads) xs[i] = (xs[i] / rms) * p.gamma[i];
+        }
+    }
+    __syncthreads();
+    if (!has_work) return;
+
+    // this lane's activation slice: 16 consecutive k of each 1 KiB chunk
+    float xr[NC][16];
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        int kb = (c * 64 + lane) * 16;
+        bool active = kb < p.kp;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float4 v = active ? *reinterpret_cast<const float4 *>(xs + kb + 4 * j) : make_float4(0, 0, 0, 0);
+            xr[c][4 * j] = v.x; xr[c][4 * j + 1] = v.y; xr[c][4 * j + 2] = v.z; xr[c][4 * j + 3] = v.w;
+        }
+    }
+
+    for (int o0 = o_begin; o0 < o_end; o0 += 2 * o_step) {
+        if (o0 + o_step < o_end) load_batch<NC, R>(bb, p, (o0 + o_step) * RPO, row_last, lane, groups);
+        finish_batch<NC, B, SWIGLU>(ba, xr, p, o0, o_end, lane);
+        if (o0 + o_step >= o_end) break;
+        if (o0 + 2 * o_step < o_end) load_batch<NC, R>(ba, p, (o0 + 2 * o_step) * RPO, row_last, lane, groups);
+        finish_batch<NC, B, SWIGLU>(bb, xr, p, o0 + o_step, o_end, lane);
+    }
+}
+
+inline int mv_grid_cap() {
+    static int cap = [] { const char *e = getenv("DJ_MV_GRID"); return e ? atoi(e) : 768; }();
+    return cap;
+}
+
+template <int NC, int B, bool SW>
+void launch_mv(hipStream_t s, const MatvecArgs &a) {
+    // Three workgroups (12 wavefronts) per CU when there are outputs for them; never
+    // more wavefronts than outputs.
+    int batches = (a.n_out + B - 1) / B;
+    int grid = (batches + kWaves - 1) / kWaves;
+    if (grid > mv_grid_cap()) grid = mv_grid_cap();
+    if (grid < 1) grid = 1;
     size_t lds = (size_t)a.kp * sizeof(float);
-    hipLaunchKernelGGL((k_q8_matvec<NC, RU, SW>), dim3(grid), dim3(kThreads), lds, s, a);
+    hipLaunchKernelGGL((k_q8_matvec<NC, B, SW>), dim3(grid), dim3(kThreads), lds, s, a);
+}
+
+// Batch depth B (outputs a wavefront multiplies per step).  Small matrices want B = 1: every
+// row gets its own wavefront, so the whole matrix is requested at once and the serial work
+// after the data arrives is one row.  Large matrices want deeper batches (about eight 128-bit
+// loads per lane in flight per buffer) so ~3000 resident wavefronts keep the HBM queues full.
+inline int mv_target_waves() {
+    static int t = [] { const char *e = getenv("DJ_MV_WAVES"); return e ? atoi(e) : 3072; }();
+    return t;
 }
 
 template <int NC>
 void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu) {
-    // Enough workgroups to put >= 8 wavefronts on each of the 256 CUs when the
-    // matrix has the rows for it; two outputs per iteration once rows are plentiful.
-    int ru = (!swiglu && a.n_out >= 8192 && NC <= 4) ? 2 : 1;
-    int per_block = kWaves * ru;
-    int grid = (a.n_out + per_block - 1) / per_block;
-    if (grid > 2048) grid = 2048;
-    if (grid < 1) grid = 1;
-    if (swiglu) launch_mv<NC, 1, true>(s, a, grid);
-    else if (ru == 2) launch_mv<(NC <= 4 ? NC : 1), 2, false>(s, a, grid);
-    else launch_mv<NC, 1, false>(s, a, grid);
+    constexpr int BMAX = NC == 1 ? 8 : (NC == 2 ? 4 : (NC <= 4 ? 2 : 1));
+    int rows = swiglu ? 2 * a.n_out : a.n_out;
+    int want = (rows + mv_target_waves() - 1) / mv_target_waves();      // rows per wavefront per step
+    if (swiglu) {
+        constexpr int BS = BMAX >= 2 ? BMAX / 2 : 1;
+        if (BS >= 4 && want >= 8) launch_mv<NC, (BS >= 4 ? 4 : 1), true>(s, a);
+        else if (BS >= 2 && want >= 4) launch_mv<NC, (BS >= 2 ? 2 : 1), true>(s, a);
+        else launch_mv<NC, 1, true>(s, a);
+    } else {
+        if (BMAX >= 8 && want >= 8) launch_mv<NC, (BMAX >= 8 ? 8 : 1), false>(s, a);
+        else if (BMAX >= 4 && want >= 4) launch_mv<NC, (BMAX >= 4 ? 4 : 1), false>(s, a);
+        else if (BMAX >= 2 && want >= 2) launch_mv<NC, (BMAX >= 2 ? 2 : 1), false>(s, a);
+        else launch_mv<NC, 1, false>(s, a);
+    }
 }
 
 // out[m, j] = SiLU(t[m, 2j]) * t[m, 2j+1] for the GEMM path's interleaved gate/up result

@@ -258,6 +258,69 @@ __global__ void __launch_bounds__(kThreads) k_argmax_rows(const float *__restric
     }
 }
 
+// End of a greedy decode step in one launch: argmax over the logits (ties -> lowest
+// index), record the token, advance the position, and gather the token's embedding row
+// as the next step's input (Embedding.java:28-34).
+__global__ void __launch_bounds__(1024) k_decode_next(const float *__restrict__ logits, int32_t *__restrict__ state,
+                                                      int32_t *__restrict__ tokens, int capacity,
+                                                      const float *__restrict__ table, float *__restrict__ x,
+                                                      int vocab, int d, int n_positions) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    __shared__ int s_tok;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    // eight independent 128-bit loads per thread per round: one memory round trip per 32768 logits
+    const int v4 = vocab >> 2;
+    const float4 *l4 = reinterpret_cast<const float4 *>(logits);
+    for (int base = 0; base < v4; base += 1024 * 8) {
+        float4 t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            int i = base + u * 1024 + threadIdx.x;
+            t[u] = i < v4 ? l4[i] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            int c = (base + u * 1024 + threadIdx.x) * 4;
+            if (c < (v4 << 2)) {
+                if (better(t[u].x, c, bv, bi)) { bv = t[u].x; bi = c; }
+                if (better(t[u].y, c + 1, bv, bi)) { bv = t[u].y; bi = c + 1; }
+                if (better(t[u].z, c + 2, bv, bi)) { bv = t[u].z; bi = c + 2; }
+                if (better(t[u].w, c + 3, bv, bi)) { bv = t[u].w; bi = c + 3; }
+            }
+        }
+    }
+    for (int c = (v4 << 2) + threadIdx.x; c < vocab; c += 1024) {
+        float v = logits[c];
+        if (better(v, c, bv, bi)) { bv = v; bi = c; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(bv, off, 64);
+        int oi = __shfl_xor(bi, off, 64);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; w++)
+            if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+        int g = state[2];
+        if (g < capacity) tokens[g] = bi;
+        state[1] = bi;
+        state[0] = state[0] + n_positions;
+        state[2] = g + 1;
+        s_tok = bi;
+    }
+    __syncthreads();
+    int tok = s_tok;
+    bool ok = tok >= 0 && tok < vocab;
+    const float *src = table + (int64_t)(ok ? tok : 0) * d;
+    for (int c = threadIdx.x; c < d; c += 1024) x[c] = ok ? src[c] : __builtin_nanf("");
+}
+
 inline int row_grid(int rows) { return rows < 256 * 16 ? (rows < 1 ? 1 : rows) : 256 * 16; }
 
 }  // namespace
@@ -315,6 +378,12 @@ void launch_cross_entropy(hipStream_t s, bool gradient, const float *logits, con
 void launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int rows, int cols) {
     if (rows <= 0) return;
     hipLaunchKernelGGL(k_rmsnorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, out, rows, cols);
+}
+
+void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
+                        const float *table, float *x, int vocab, int d, int n_positions) {
+    hipLaunchKernelGGL(k_decode_next, dim3(1), dim3(1024), 0, s, logits, state, tokens, capacity, table, x, vocab, d,
+                       n_positions);
 }
 
 void launch_argmax_rows(hipStream_t s, const float *a, int32_t *out, int rows, int cols) {

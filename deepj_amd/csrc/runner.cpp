@@ -65,7 +65,7 @@ struct Runner {
     std::vector<Layer> layers;
     int32_t emb = -1, gf = -1, wlm = -1, blm = -1;
     int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
-    int32_t state = -1, tok = -1, tokens = -1, scratch = -1, logits = -1, last_x = -1;
+    int32_t state = -1, tok = -1, tokens = -1, scratch = -1, scratch_dec = -1, logits = -1, last_x = -1;
     Acts dec, pre;
     int32_t graph = 0;
     bool finalized = false;
@@ -269,6 +269,8 @@ void finalize(Runner &r) {
     int splits = (c.max_seq + 63) / 64;
     int64_t sf = (int64_t)c.heads * (4 + (int64_t)splits * (hd + 4));
     r.scratch = r.alloc(sf);
+    int ns = std::max(1, std::min(16, 512 / c.heads));
+    r.scratch_dec = r.alloc((int64_t)c.heads * ns * (hd + 4));
     Stream s;
     emit(s, DJ_OP_FILL, r.scratch, 0, (int32_t)sf);
     emit(s, DJ_OP_FILL, r.state, 0, 4);
@@ -288,8 +290,13 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     if (c.kind == 0) {
         // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
         q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
-        emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
-        emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
+        if (S == 1 && &a == &r.dec) {
+            emit(s, DJ_OP_ATTN_DECODE, a.qkv, r.kc, r.vc, a.att, r.state, r.scratch_dec, r.cos_t, r.sin_t, H, hd,
+                 c.max_seq, l);
+        } else {
+            emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
+            emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
+        }
     } else {
         throw Error("MLA streams are built by mla_block_stream");
     }
@@ -307,13 +314,13 @@ void head_stream(Runner &r, Stream &s, int32_t x_row) {
 Stream decode_stream(Runner &r, bool sample_on_device) {
     const Config &c = r.cfg;
     Stream s;
-    emit(s, DJ_OP_EMBED_GATHER, r.emb, r.state, r.dec.x, 1, c.d, c.vocab, 1);    // token = state[1]
+    // Greedy on the device: the previous step (or the prefill) already left the embedding of
+    // the token to process in dec.x.  Host sampling: gather it from state[1] first.
+    if (!sample_on_device) emit(s, DJ_OP_EMBED_GATHER, r.emb, r.state, r.dec.x, 1, c.d, c.vocab, 1);
     for (int l = 0; l < c.layers; l++) block_stream(r, s, r.dec, l, 1);
     head_stream(r, s, r.dec.x);
-    if (sample_on_device) {
-        emit(s, DJ_OP_ARGMAX_ROWS, r.logits, r.tok, 1, c.vocab);
-        emit(s, DJ_OP_DECODE_ADVANCE, r.state, r.tok, r.tokens, c.max_seq, 1);
-    }
+    if (sample_on_device)
+        emit(s, DJ_OP_DECODE_NEXT, r.logits, r.state, r.tokens, c.max_seq, r.emb, r.dec.x, c.vocab, c.d, 1);
     return s;
 }
 
@@ -338,10 +345,7 @@ void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choos
     for (int l = 0; l < c.layers; l++) block_stream(r, s, r.pre, l, n);
     emit(s, DJ_OP_COPY, r.pre.x, r.last_x, c.d, (int64_t)(n - 1) * c.d, 0);
     head_stream(r, s, r.last_x);
-    if (choose) {
-        emit(s, DJ_OP_ARGMAX_ROWS, r.logits, r.tok, 1, c.vocab);
-        emit(s, DJ_OP_DECODE_ADVANCE, r.state, r.tok, r.tokens, c.max_seq, n);
-    }
+    if (choose) emit(s, DJ_OP_DECODE_NEXT, r.logits, r.state, r.tokens, c.max_seq, r.emb, r.dec.x, c.vocab, c.d, n);
     r.run(s);
     if (all_logits) {
         // DecoderOnlyModel.forward returns logits for every row; only parity tests ask for them.
@@ -387,6 +391,23 @@ void decode_greedy(Runner &r, int steps, bool use_graph) {
     }
     r.pos += steps;
     r.generated += steps;
+}
+
+// One token through the single-row path with the token chosen by the caller: logits of the
+// new position end up in r.logits.  (Incremental decode with sampling done elsewhere.)
+void step_token(Runner &r, int32_t token) {
+    const Config &c = r.cfg;
+    if (!r.finalized) finalize(r);
+    check_ids(c, &token, 1);
+    if (r.pos + 1 > c.max_seq)
+        throw Error("context of " + std::to_string(r.pos + 1) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
+    int32_t st[4] = {r.pos, token, r.generated, 0};
+    hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
+    Stream fwd = decode_stream(r, false);
+    r.run(fwd);
+    r.pos += 1;
+    st[0] = r.pos;
+    hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
 }
 
 // ── TextGenerator.sampleFromLogits on the host (temperature / top-k > 1) ────
@@ -515,7 +536,7 @@ void deepj_runner_destroy(void *h) {
     for (auto &L : r->layers)
         for (int32_t id : {L.g1, L.g2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wukv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
     for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state, r->tok,
-                       r->tokens, r->scratch, r->logits, r->last_x})
+                       r->tokens, r->scratch, r->scratch_dec, r->logits, r->last_x})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
         for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv, a->kfull, a->vfull, a->kvexp}) add(id);
@@ -554,6 +575,11 @@ int deepj_runner_prefill(void *h, const int32_t *ids, int32_t n, float *all_logi
 int deepj_runner_decode(void *h, int32_t steps, int32_t use_graph) {
     auto *r = static_cast<Runner *>(h);
     return guarded(r, [&] { decode_greedy(*r, steps, use_graph != 0); });
+}
+
+int deepj_runner_step(void *h, int32_t token) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] { step_token(*r, token); });
 }
 
 int deepj_runner_last_logits(void *h, float *out) {

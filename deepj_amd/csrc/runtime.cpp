@@ -181,6 +181,8 @@ int stride_of(int op) {
         case DJ_OP_FILL: return 4;
         case DJ_OP_ROPE_ROWS: return 11;
         case DJ_OP_ATTENTION_KV: return 12;
+        case DJ_OP_DECODE_NEXT: return 10;
+        case DJ_OP_ATTN_DECODE: return 13;
         default: return -1;
     }
 }
@@ -486,6 +488,38 @@ void exec_one(Cursor &c) {
                                       reinterpret_cast<int32_t *>(out), (int)cap, w[5]);
             break;
         }
+        case DJ_OP_DECODE_NEXT: {
+            // [op, logits, state, tokens, capacity, table, x, vocab, d, nPos]
+            int64_t cap = w[4], vocab = w[7], d = w[8];
+            if (cap < 0 || vocab <= 0 || d <= 0 || w[9] < 0) fail("OP_DECODE_NEXT: bad shape");
+            const float *lg = buf(w[1], vocab, op, "logits");
+            float *st = buf(w[2], 4, op, "state");
+            float *tk = buf(w[3], std::max<int64_t>(cap, 1), op, "tokens");
+            const float *tb = buf(w[5], vocab * d, op, "table");
+            float *x = buf(w[6], d, op, "x");
+            if (run)
+                launch_decode_next(s, lg, reinterpret_cast<int32_t *>(st), reinterpret_cast<int32_t *>(tk), (int)cap,
+                                   tb, x, (int)vocab, (int)d, w[9]);
+            break;
+        }
+        case DJ_OP_ATTN_DECODE: {
+            // [op, qkv, kCache, vCache, out, state, scratch, cos, sin, H, hd, maxSeq, layer]
+            int64_t H = w[9], hd = w[10], max_seq = w[11], layer = w[12];
+            if (H <= 0 || max_seq <= 0 || layer < 0) fail("OP_ATTN_DECODE: bad shape");
+            if (hd != 32 && hd != 64 && hd != 128) fail("OP_ATTN_DECODE: head dim must be 32, 64 or 128");
+            int64_t d = H * hd, per_layer = H * max_seq * hd;
+            const float *qkv = buf(w[1], 3 * d, op, "qkv");
+            float *kc = buf(w[2], (layer + 1) * per_layer, op, "kCache");
+            float *vc = buf(w[3], (layer + 1) * per_layer, op, "vCache");
+            float *o = buf(w[4], d, op, "out");
+            const float *st = buf(w[5], 4, op, "state");
+            float *sc = buf(w[6], attn_decode_scratch_floats((int)H, (int)hd), op, "scratch");
+            const float *ct = buf(w[7], max_seq * (hd / 2), op, "cos"), *sn = buf(w[8], max_seq * (hd / 2), op, "sin");
+            if (run)
+                launch_attn_decode(s, qkv, kc + layer * per_layer, vc + layer * per_layer, o,
+                                   reinterpret_cast<const int32_t *>(st), sc, ct, sn, (int)H, (int)hd, (int)max_seq);
+            break;
+        }
         case DJ_OP_COPY: {
             int64_t n = w[3], so = w[4], dof = w[5];
             if (n < 0 || so < 0 || dof < 0) fail("OP_COPY: bad range");
@@ -556,6 +590,8 @@ const char *op_name(int op) {
         case DJ_OP_FILL: return "OP_FILL";
         case DJ_OP_ROPE_ROWS: return "OP_ROPE_ROWS";
         case DJ_OP_ATTENTION_KV: return "OP_ATTENTION_KV";
+        case DJ_OP_DECODE_NEXT: return "OP_DECODE_NEXT";
+        case DJ_OP_ATTN_DECODE: return "OP_ATTN_DECODE";
         default: return "OP_?";
     }
 }

@@ -106,6 +106,12 @@ class Stream:
     def decode_advance(self, state, token, tokens, capacity, n_pos=1):
         return self.emit(op.OP_DECODE_ADVANCE, state, token, tokens, capacity, n_pos)
 
+    def decode_next(self, logits, state, tokens, capacity, table, x, vocab, d, n_pos=1):
+        return self.emit(op.OP_DECODE_NEXT, logits, state, tokens, capacity, table, x, vocab, d, n_pos)
+
+    def attn_decode(self, qkv, k_cache, v_cache, out, state, scratch, cos, sin, H, hd, max_seq, layer):
+        return self.emit(op.OP_ATTN_DECODE, qkv, k_cache, v_cache, out, state, scratch, cos, sin, H, hd, max_seq, layer)
+
     def copy(self, src, dst, n, src_off=0, dst_off=0): return self.emit(op.OP_COPY, src, dst, n, src_off, dst_off)
     def fill(self, dst, bits, n): return self.emit(op.OP_FILL, dst, bits, n)
     def matmul(self, a, b, out, m, n, k): return self.emit(op.OP_MATMUL, a, b, out, m, n, k)
@@ -121,6 +127,11 @@ class Stream:
     def time(self, iters: int) -> float:
         """Milliseconds for `iters` back-to-back executions (HIP events on the library's stream)."""
         return HipNative.timeOps(self.array(), iters)
+
+
+def attn_decode_scratch_floats(H: int, hd: int) -> int:
+    """Floats of the scratch buffer the fused ATTN_DECODE op needs (no initialisation required)."""
+    return H * max(1, min(16, 512 // H)) * (hd + 4)
 
 
 def attention_scratch_floats(H: int, hd: int, max_seq: int) -> int:

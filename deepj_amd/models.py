@@ -37,6 +37,7 @@ def _lib():
         lib.deepj_runner_reset.argtypes = [C.c_void_p]
         lib.deepj_runner_prefill.argtypes = [C.c_void_p, _i32p, C.c_int32, C.c_void_p, C.c_int32]
         lib.deepj_runner_decode.argtypes = [C.c_void_p, C.c_int32, C.c_int32]
+        lib.deepj_runner_step.argtypes = [C.c_void_p, C.c_int32]
         lib.deepj_runner_last_logits.argtypes = [C.c_void_p, C.c_void_p]
         lib.deepj_runner_tokens.argtypes = [C.c_void_p, _i32p, C.c_int32, _i32p]
         lib.deepj_runner_generate.argtypes = [C.c_void_p, _i32p, C.c_int32, C.c_int32, C.c_float, C.c_int32,
@@ -195,6 +196,10 @@ class _DecoderOnlyModel:
 
     def decode(self, steps: int, use_graph: bool = True) -> None:
         self._check(_lib().deepj_runner_decode(self._h, steps, 1 if use_graph else 0))
+
+    def step(self, token: int) -> None:
+        """Feed one caller-chosen token through the single-row (cached) path; see lastLogits()."""
+        self._check(_lib().deepj_runner_step(self._h, int(token)))
 
     def lastLogits(self) -> np.ndarray:
         out = np.empty(self.cfg.vocabSize, dtype=np.float32)

@@ -125,11 +125,15 @@ enum {
      * FILL          [op, dst, bits, n]
      * ROPE_ROWS     [op, x, out, state, cosT, sinT, rows, H, hd, maxSeq, posFromRow]  token-major rows
      * ATTENTION_KV  [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0]  k, v token-major [maxSeq x H*hd]
+     * DECODE_NEXT   [op, logits, state, tokens, capacity, table, x, vocab, d, nPos]
+     *     argmax + DECODE_ADVANCE + EMBED_GATHER of the chosen token into x, one launch
+     * ATTN_DECODE   [op, qkv, kCache, vCache, out, state, scratch, cosT, sinT, H, hd, maxSeq, layer]
+     *     ROPE_KV_STORE + ATTENTION for one new row (S = 1) in two launches
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
-    DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77
+    DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8 };
@@ -166,6 +170,7 @@ int deepj_runner_finalize(void *runner);
 int deepj_runner_reset(void *runner);
 int deepj_runner_prefill(void *runner, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next);
 int deepj_runner_decode(void *runner, int32_t steps, int32_t use_graph);
+int deepj_runner_step(void *runner, int32_t token);     /* one caller-chosen token through the S=1 path */
 int deepj_runner_last_logits(void *runner, float *out);
 int deepj_runner_tokens(void *runner, int32_t *out, int32_t capacity, int32_t *n);
 int deepj_runner_generate(void *runner, const int32_t *prompt, int32_t n_prompt, int32_t max_new,

@@ -5,7 +5,7 @@ cache (split-K path), for head dims 32/64/128."""
 import numpy as np
 import pytest
 
-from deepj_amd.fused import DeviceBuffers, Stream, attention_scratch_floats
+from deepj_amd.fused import DeviceBuffers, Stream, attention_scratch_floats, attn_decode_scratch_floats
 from oracle import cpu_ref as ref
 from gpu_util import assert_close
 
@@ -59,6 +59,54 @@ def test_rope_store_attention_prefill_and_decode(H, hd, max_seq, chunks):
         # the scratch counters are back to zero (ready for a graph replay)
         sc = dev.download(scratch, (sf,), np.int32).reshape(H, -1)
         assert np.all(sc[:, 0] == 0)
+    finally:
+        dev.release_all()
+
+
+@pytest.mark.parametrize("H,hd,max_seq,prefill,steps", [(8, 32, 256, 32, 5), (32, 64, 2048, 515, 3), (4, 128, 96, 1, 40)])
+def test_fused_decode_attention_and_decode_next(H, hd, max_seq, prefill, steps):
+    """ATTN_DECODE (rotate + append + split attention + merge) over a growing cache, then
+    DECODE_NEXT (argmax, advance, embedding gather) - the two fused ops of a decode step."""
+    d = H * hd
+    total = prefill + steps
+    q, k, v = (gaussian(total, d, 30 + i) for i in range(3))
+    cos, sin = ref.rope_tables(hd, max_seq)
+    exp = oracle_attention(q, k, v, H, cos, sin)
+    dev = DeviceBuffers()
+    try:
+        kc, vc = dev.alloc(max_seq * d), dev.alloc(max_seq * d)
+        state = dev.upload(np.zeros(4, np.int32))
+        cos_b, sin_b = dev.upload(cos), dev.upload(sin)
+        sf = attention_scratch_floats(H, hd, max_seq)
+        scratch, scratch_dec = dev.alloc(sf), dev.alloc(attn_decode_scratch_floats(H, hd))
+        Stream().fill(scratch, 0, sf).run()
+        tok, tokens = dev.upload(np.zeros(4, np.int32)), dev.alloc(max_seq)
+        qkv0 = np.concatenate([q[:prefill], k[:prefill], v[:prefill]], axis=1)
+        qkv_b, q_b, out_b = dev.upload(qkv0), dev.alloc(prefill * d), dev.alloc(prefill * d)
+        (Stream().rope_kv_store(qkv_b, q_b, kc, vc, state, cos_b, sin_b, prefill, H, hd, max_seq, 0)
+         .attention(q_b, kc, vc, out_b, state, scratch, prefill, H, hd, max_seq, 0)
+         .decode_advance(state, tok, tokens, max_seq, prefill).run())
+        assert_close(exp[:prefill], dev.download(out_b, (prefill, d)), atol=2e-5, rtol=1e-4)
+        vocab = 50
+        table = gaussian(vocab, d, 40)
+        logits_b, x_b, row_b, o_b = dev.alloc(vocab), dev.alloc(d), dev.alloc(3 * d), dev.alloc(d)
+        for i in range(steps):
+            p = prefill + i
+            dev.write(row_b, np.concatenate([q[p], k[p], v[p]]))
+            logits = gaussian(1, vocab, 50 + i)
+            dev.write(logits_b, logits)
+            (Stream().attn_decode(row_b, kc, vc, o_b, state, scratch_dec, cos_b, sin_b, H, hd, max_seq, 0)
+             .decode_next(logits_b, state, tokens, max_seq, dev.upload(table), x_b, vocab, d).run())
+            assert_close(exp[p:p + 1], dev.download(o_b, (1, d)), atol=2e-5, rtol=1e-4, what=f"decode step {i}")
+            st = dev.download(state, (4,), np.int32)
+            best = int(np.argmax(logits))
+            assert (st[0], st[1], st[2]) == (p + 1, best, 2 + i)
+            assert np.array_equal(dev.download(x_b, (d,)), table[best])
+        # the appended rows really are in the cache: a plain ATTENTION over the cache agrees
+        st = np.array([total - 1, 0, 0, 0], np.int32); dev.write(state, st)
+        qr = ref.merge_heads(ref.rope_apply(ref.split_heads(q, H), total, H, cos, sin), H)[total - 1:]
+        (Stream().attention(dev.upload(qr), kc, vc, o_b, state, scratch, 1, H, hd, max_seq, 0).run())
+        assert_close(exp[total - 1:], dev.download(o_b, (1, d)), atol=2e-5, rtol=1e-4)
     finally:
         dev.release_all()
 

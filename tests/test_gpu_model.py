@@ -75,14 +75,7 @@ def test_c1_decode_row_equals_prefill_row(c1):
     full = gpu.forward(ids)
     gpu.reset()
     gpu.prefill(ids[:19], choose_next=False)
-    # feed token 19 through the single-row path
-    from deepj_amd.models import _lib
-    import ctypes as C
-    st = np.array([19, int(ids[19]), 0, 0], np.int32)
-    stream = gpu.decodeStream()
-    state_id = int(stream[2])                       # EMBED_GATHER [op, table, ids=state, ...]
-    HipNative.nativeUploadBuffer(state_id, st)
-    HipNative.nativeFlushOps(stream, stream.size)
+    gpu.step(int(ids[19]))                          # token 19 through the single-row path
     row = gpu.lastLogits()
     assert float(np.max(np.abs(row - full[19]))) <= 2e-4
 
