@@ -50,6 +50,8 @@ void launch_scatter_add(hipStream_t s, float *target, const float *idx, const fl
 void launch_fill(hipStream_t s, uint32_t *dst, uint32_t bits, int64_t n);
 void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n);
 void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n);
+void launch_append_rows(hipStream_t s, const float *src, float *dst, const int32_t *state, int rows, int row_floats,
+                        int max_rows);
 void launch_embed_gather(hipStream_t s, const float *table, const int32_t *ids, float *out, int n_ids, int d,
                          int vocab);
 void launch_decode_advance(hipStream_t s, int32_t *state, const int32_t *token, int32_t *tokens, int capacity,
@@ -76,6 +78,8 @@ struct Q8Linear {
     const float *x; const int8_t *wq; const float *scales; float *out;
     int m, k, n, flags;
     const float *gamma, *bias, *bias2, *residual;
+    const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
+    int m_extra = 0;
 };
 void launch_q8_quantize(hipStream_t s, const float *w, int8_t *q, float *scales, int k, int n, int row_off,
                         int row_step);

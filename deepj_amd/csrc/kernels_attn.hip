@@ -24,7 +24,6 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kSplitKeys = 64;          // keys per decode split
 
 // ── RoPE on the fused projection + cache append ─────────────────────────────
 // qkv [S x 3d]: Q | K | V.  Row i sits at position state[0] + i.
@@ -60,7 +59,7 @@ __global__ void __launch_bounds__(kThreads) k_rope_kv_store(const float *__restr
 }
 
 // RoPE on token-major rows [rows x H*hd]; position = row (pos_from_row) or state[0] + row.
-__global__ void __launch_bounds__(kThreads) k_rope_rows(const float *__restrict__ x, float *__restrict__ out,
+__global__ void __launch_bounds__(kThreads) k_rope_rows(const float *x, float *out,   // may alias (in place)
                                                         const int32_t *__restrict__ state,
                                                         const float *__restrict__ cos_t,
                                                         const float *__restrict__ sin_t, int rows, int H, int hd,
@@ -82,15 +81,14 @@ __global__ void __launch_bounds__(kThreads) k_rope_rows(const float *__restrict_
     }
 }
 
-// ── attention ───────────────────────────────────────────────────────────────
-// grid (H, S, nsplit).  LPK = hd/4 lanes cooperate on one key; a wavefront handles
-// 64/LPK keys per step.  Scratch (only when nsplit > 1), per (query, head):
-//   [counter(1 int) pad(3)] [nsplit x (hd + 4)] floats: max, sum, pad, pad, o[hd]
+// ── attention, several query rows (prefill) ─────────────────────────────────
+// grid (H, S).  LPK = hd/4 lanes cooperate on one key; a wavefront handles 64/LPK keys per
+// step; the 4*(64/LPK) running softmax states of a workgroup are merged through LDS.
 struct AttnKernelArgs {
     const float *q; const float *k; const float *v; float *out;
-    const int32_t *state; float *scratch;
+    const int32_t *state;
     int64_t tok_stride, head_stride;
-    int S, H, hd, max_seq, nsplit;
+    int S, H, hd, max_seq;
     float scale;
 };
 
@@ -101,9 +99,8 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
     constexpr int NSUB = kWaves * KPW;            // independent running softmaxes per workgroup
     __shared__ float s_m[NSUB], s_l[NSUB];
     __shared__ __align__(16) float s_o[NSUB][HD];
-    __shared__ int s_last;
 
-    const int h = blockIdx.x, qi = blockIdx.y, split = blockIdx.z;
+    const int h = blockIdx.x, qi = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane / LPK, dl = lane % LPK;
     const int d = a.H * HD;
@@ -111,13 +108,6 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
     const int pos = a.state[0] + qi;              // this query's position; keys 0..pos
     int n_keys = pos + 1;
     if (n_keys > a.max_seq) n_keys = a.max_seq;
-    int k_begin = 0, k_end = n_keys;
-    if (a.nsplit > 1) {
-        k_begin = split * kSplitKeys;
-        k_end = k_begin + kSplitKeys;
-        if (split == a.nsplit - 1) k_end = n_keys;          // the last split takes any tail
-        if (k_end > n_keys) k_end = n_keys;
-    }
 
     const float4 qv = *reinterpret_cast<const float4 *>(a.q + (int64_t)qi * d + h * HD + dl * 4);
     const float *kb = a.k + (int64_t)h * a.head_stride + dl * 4;
@@ -125,7 +115,7 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int key = k_begin + wave * KPW + sub; key < k_end; key += kWaves * KPW) {
+    for (int key = wave * KPW + sub; key < n_keys; key += kWaves * KPW) {
         float4 kk = *reinterpret_cast<const float4 *>(kb + (int64_t)key * a.tok_stride);
         float4 vv = *reinterpret_cast<const float4 *>(vb + (int64_t)key * a.tok_stride);
         float s = qv.x * kk.x + qv.y * kk.y + qv.z * kk.z + qv.w * kk.w;
@@ -144,68 +134,26 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
     if (dl == 0) { s_m[slot] = m; s_l[slot] = l; }
     *reinterpret_cast<float4 *>(&s_o[slot][dl * 4]) = o;
     __syncthreads();
-
-    // merge the NSUB running states: thread j < HD owns output dim j
-    float M = -INFINITY, L = 0.0f, O = 0.0f;
     if (tid < HD) {
+        float M = -INFINITY, L = 0.0f, O = 0.0f;
 #pragma unroll
         for (int i = 0; i < NSUB; i++) M = fmaxf(M, s_m[i]);
-        if (M != -INFINITY) {
 #pragma unroll
-            for (int i = 0; i < NSUB; i++) {
-                float w = expf(s_m[i] - M);       // empty slots: exp(-inf) = 0
-                L += s_l[i] * w;
-                O += s_o[i][tid] * w;
-            }
+        for (int i = 0; i < NSUB; i++) {
+            float w = expf(s_m[i] - M);           // empty slots: exp(-inf) = 0
+            L += s_l[i] * w;
+            O += s_o[i][tid] * w;
         }
+        a.out[(int64_t)qi * d + h * HD + tid] = O / L;
     }
-
-    float *outp = a.out + (int64_t)qi * d + h * HD;
-    if (a.nsplit == 1) {
-        if (tid < HD) outp[tid] = O / L;
-        return;
-    }
-
-    // ── cross-split merge ──
-    const int64_t rec = HD + 4;
-    float *base = a.scratch + ((int64_t)qi * a.H + h) * (4 + (int64_t)a.nsplit * rec);
-    int *counter = reinterpret_cast<int *>(base);
-    float *mine = base + 4 + (int64_t)split * rec;
-    if (tid < HD) mine[4 + tid] = O;
-    if (tid == 0) { mine[0] = M; mine[1] = L; }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        int done = atomicAdd(counter, 1);
-        s_last = (done == a.nsplit - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();                              // acquire: the other splits' records are visible now
-    if (tid < HD) {
-        float GM = -INFINITY;
-        for (int i = 0; i < a.nsplit; i++) GM = fmaxf(GM, base[4 + i * rec]);
-        float GL = 0.0f, GO = 0.0f;
-        for (int i = 0; i < a.nsplit; i++) {
-            const float *r = base + 4 + i * rec;
-            float mi = r[0];
-            if (mi == -INFINITY) continue;
-            float w = expf(mi - GM);
-            GL += r[1] * w;
-            GO += r[4 + tid] * w;
-        }
-        outp[tid] = GO / GL;
-    }
-    if (tid == 0) *counter = 0;                   // ready for the next launch / graph replay
 }
-
-inline int decode_splits(int max_seq) { return (max_seq + kSplitKeys - 1) / kSplitKeys; }
 
 // ── fused decode attention ──────────────────────────────────────────────────
 // Record layout in scratch, per (head, split): [max, sum, pad, pad, o[hd]].
 struct DecodeArgs {
-    const float *qkv;          // [3d]: q | k | v of the new token (not rotated)
-    float *k_cache, *v_cache;  // this layer, [H][maxSeq][hd]
+    const float *qkv;          // FUSED: [3d] q | k | v of the new token (not rotated); else q [d], rotated
+    float *k_cache, *v_cache;  // keys / values: element (key, h, j) at [h*head_stride + key*tok_stride + j]
+    int64_t tok_stride, head_stride;
     float *out;                // [d]
     const int32_t *state;
     float *scratch;
@@ -214,7 +162,8 @@ struct DecodeArgs {
     float scale;
 };
 
-template <int LPK>
+// FUSED: rotate q and the new key in registers and append the new key/value row to the cache.
+template <int LPK, bool FUSED>
 __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) {
     constexpr int HD = LPK * 4;
     constexpr int KPW = 64 / LPK;
@@ -236,28 +185,32 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     const int k_end = k_begin + per < n_keys ? k_begin + per : n_keys;
 
     // rotate this lane's two (even, odd) pairs of q and of the new k
-    const float2 c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
-    const float2 s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
+    float2 c2 = make_float2(1.f, 1.f), s2 = make_float2(0.f, 0.f);
+    if constexpr (FUSED) {
+        c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
+        s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
+    }
     const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
-    const float4 qv = make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
-                                  q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y);
-    float *kb = a.k_cache + (int64_t)h * a.max_seq * HD + dl * 4;
-    float *vb = a.v_cache + (int64_t)h * a.max_seq * HD + dl * 4;
+    const float4 qv = FUSED ? make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
+                                          q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y)
+                            : q0;
+    float *kb = a.k_cache + (int64_t)h * a.head_stride + dl * 4;
+    float *vb = a.v_cache + (int64_t)h * a.head_stride + dl * 4;
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int key = k_begin + wave * KPW + sub; key < k_end; key += kWaves * KPW) {
         float4 kk, vv;
-        if (key == pos) {                                   // the new token: rotate, use, append
+        if (FUSED && key == pos) {                          // the new token: rotate, use, append
             const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
             kk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
                              k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
             vv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
-            *reinterpret_cast<float4 *>(kb + (int64_t)key * HD) = kk;
-            *reinterpret_cast<float4 *>(vb + (int64_t)key * HD) = vv;
+            *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = kk;
+            *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = vv;
         } else {
-            kk = *reinterpret_cast<const float4 *>(kb + (int64_t)key * HD);
-            vv = *reinterpret_cast<const float4 *>(vb + (int64_t)key * HD);
+            kk = *reinterpret_cast<const float4 *>(kb + (int64_t)key * a.tok_stride);
+            vv = *reinterpret_cast<const float4 *>(vb + (int64_t)key * a.tok_stride);
         }
         float s = qv.x * kk.x + qv.y * kk.y + qv.z * kk.z + qv.w * kk.w;
 #pragma unroll
@@ -350,48 +303,55 @@ void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *
                        max_seq, pos_from_row);
 }
 
-// Decode launches always use the same number of splits (sized for max_seq) so that a
-// captured graph stays valid as the cache grows; splits beyond the live keys exit
-// after writing an empty record.
+// S = 1 uses the split kernels (scratch: attn_decode_scratch_floats); S > 1 needs no scratch.
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq) {
-    if (S != 1) return 0;
-    return (int64_t)H * (4 + (int64_t)decode_splits(max_seq) * (hd + 4));
+    (void)max_seq;
+    return S == 1 ? attn_decode_scratch_floats(H, hd) : 0;
 }
 
 int64_t attn_decode_scratch_floats(int H, int hd) { return (int64_t)H * fused_decode_splits(H) * (hd + 4); }
+
+template <bool FUSED>
+static void launch_decode_kernels(hipStream_t s, DecodeArgs &a) {
+    a.nsplit = fused_decode_splits(a.H);
+    a.scale = (float)(1.0 / sqrt((double)a.hd));
+    dim3 grid(a.H, a.nsplit);
+    switch (a.hd) {
+        case 32: hipLaunchKernelGGL((k_attn_decode_partial<8, FUSED>), grid, dim3(kThreads), 0, s, a); break;
+        case 64: hipLaunchKernelGGL((k_attn_decode_partial<16, FUSED>), grid, dim3(kThreads), 0, s, a); break;
+        case 128: hipLaunchKernelGGL((k_attn_decode_partial<32, FUSED>), grid, dim3(kThreads), 0, s, a); break;
+        default: fail("attention: head dim must be 32, 64 or 128");
+    }
+    hipLaunchKernelGGL(k_attn_decode_merge, dim3(a.H), dim3(a.hd), 0, s, a.scratch, a.out, a.hd, a.nsplit);
+}
 
 void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *out,
                         const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,
                         int max_seq) {
     DecodeArgs a;
     a.qkv = qkv; a.k_cache = k_cache; a.v_cache = v_cache; a.out = out; a.state = state; a.scratch = scratch;
+    a.tok_stride = hd; a.head_stride = (int64_t)max_seq * hd;
     a.cos_t = cos_t; a.sin_t = sin_t; a.H = H; a.hd = hd; a.max_seq = max_seq;
-    a.nsplit = fused_decode_splits(H);
-    a.scale = (float)(1.0 / sqrt((double)hd));
-    dim3 grid(H, a.nsplit);
-    switch (hd) {
-        case 32: hipLaunchKernelGGL(k_attn_decode_partial<8>, grid, dim3(kThreads), 0, s, a); break;
-        case 64: hipLaunchKernelGGL(k_attn_decode_partial<16>, grid, dim3(kThreads), 0, s, a); break;
-        case 128: hipLaunchKernelGGL(k_attn_decode_partial<32>, grid, dim3(kThreads), 0, s, a); break;
-        default: fail("attention: head dim must be 32, 64 or 128");
-    }
-    hipLaunchKernelGGL(k_attn_decode_merge, dim3(H), dim3(hd), 0, s, scratch, out, hd, a.nsplit);
+    launch_decode_kernels<true>(s, a);
 }
 
 void launch_attention(hipStream_t s, const AttnArgs &p) {
     if (p.s <= 0) return;
+    if (p.s == 1) {
+        if (p.scratch_floats < attn_decode_scratch_floats(p.h, p.hd)) fail("attention: scratch buffer too small");
+        DecodeArgs a;
+        a.qkv = p.q; a.k_cache = const_cast<float *>(p.k); a.v_cache = const_cast<float *>(p.v); a.out = p.out;
+        a.state = p.state; a.scratch = p.scratch; a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
+        a.cos_t = a.sin_t = nullptr; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
+        launch_decode_kernels<false>(s, a);
+        return;
+    }
     AttnKernelArgs a;
-    a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.state = p.state; a.scratch = p.scratch;
+    a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.state = p.state;
     a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
     a.S = p.s; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
     a.scale = (float)(1.0 / sqrt((double)p.hd));
-    a.nsplit = 1;
-    if (p.s == 1) {
-        a.nsplit = decode_splits(p.max_seq);
-        if (a.nsplit > 1 && p.scratch_floats < attention_scratch_floats(1, p.h, p.hd, p.max_seq))
-            fail("attention: scratch buffer too small");
-    }
-    dim3 grid(p.h, p.s, a.nsplit);
+    dim3 grid(p.h, p.s);
     switch (p.hd) {
         case 32: hipLaunchKernelGGL(k_attention<8>, grid, dim3(kThreads), 0, s, a); break;
         case 64: hipLaunchKernelGGL(k_attention<16>, grid, dim3(kThreads), 0, s, a); break;

@@ -234,6 +234,21 @@ __global__ void __launch_bounds__(kThreads) k_embed_gather(const float *__restri
     for (int c = threadIdx.x; c < d; c += blockDim.x) dst[c] = ok ? src[c] : __builtin_nanf("");
 }
 
+// dst[(state[0] + i), :] = src[i, :] for i < rows: append to a cache whose fill level lives on the device.
+__global__ void __launch_bounds__(kThreads) k_append_rows(const float *__restrict__ src, float *__restrict__ dst,
+                                                          const int32_t *__restrict__ state, int rows, int row_floats,
+                                                          int max_rows) {
+    const int pos0 = state[0];
+    int64_t n = (int64_t)rows * row_floats;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride) {
+        int i = (int)(t / row_floats);
+        int j = (int)(t - (int64_t)i * row_floats);
+        int r = pos0 + i;
+        if (r >= 0 && r < max_rows) dst[(int64_t)r * row_floats + j] = src[t];
+    }
+}
+
 // state[0] = positions held in the cache, state[1] = current token, state[2] = tokens generated.
 __global__ void k_decode_advance(int32_t *state, const int32_t *token, int32_t *tokens, int capacity,
                                  int n_positions) {
@@ -348,6 +363,13 @@ void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n) {
 void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n) {
     if (n <= 0) return;
     DJ_LAUNCH(k_silu_mul, grid_for(n), kThreads, s, gate, up, out, n);
+}
+
+void launch_append_rows(hipStream_t s, const float *src, float *dst, const int32_t *state, int rows, int row_floats,
+                        int max_rows) {
+    int64_t n = (int64_t)rows * row_floats;
+    if (n <= 0) return;
+    DJ_LAUNCH(k_append_rows, grid_for(n), kThreads, s, src, dst, state, rows, row_floats, max_rows);
 }
 
 void launch_embed_gather(hipStream_t s, const float *table, const int32_t *ids, float *out, int n_ids, int d,

@@ -28,12 +28,14 @@ struct GemmEpilogue {
     const float *bias2;
     const float *residual;  // [M x N] or null
     int interleaved_bias;
+    const int32_t *m_dev;   // when set, only rows < min(M, m_dev[0] + m_extra) exist (row count kept on the device)
+    int m_extra;
 };
 
 template <bool Q8>
 __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const float *__restrict__ Bf,
                                               const int8_t *__restrict__ Bq, const float *__restrict__ Bs,
-                                              float *__restrict__ C, int M, int N, int K, int kp,
+                                              float *__restrict__ C, int M, const int N, const int K, const int kp,
                                               GemmEpilogue ep) {
     __shared__ float As[BK][BM + PAD];
     __shared__ float Bl[BK][BN + PAD];
@@ -42,6 +44,11 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
     const int lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    if (ep.m_dev) {
+        int live = ep.m_dev[0] + ep.m_extra;
+        if (live < M) M = live;
+        if (m0 >= M) return;                 // workgroup-uniform
+    }
 
     floatx16 acc;
 #pragma unroll
@@ -145,7 +152,7 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
     if (m <= 0 || n <= 0) return;
     if (k <= 0) { launch_fill(s, reinterpret_cast<uint32_t *>(out), 0u, (int64_t)m * n); return; }
     dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM);
-    GemmEpilogue ep{nullptr, nullptr, nullptr, 0};
+    GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0};
     hipLaunchKernelGGL(k_gemm<false>, grid, dim3(256), 0, s, a, b, (const int8_t *)nullptr, (const float *)nullptr,
                        out, m, n, k, 0, ep);
 }
@@ -154,10 +161,10 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
 // (= output columns of this launch; 2N for an interleaved gate/up weight).
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias) {
+                    int interleaved_bias, const int32_t *m_dev, int m_extra) {
     if (m <= 0 || n_rows <= 0) return;
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
-    GemmEpilogue ep{bias, bias2, residual, interleaved_bias};
+    GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra};
     hipLaunchKernelGGL(k_gemm<true>, grid, dim3(256), 0, s, x, (const float *)nullptr, wq, scales, out, m, n_rows, k,
                        q8_padded_k(k), ep);
 }

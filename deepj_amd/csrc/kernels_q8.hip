@@ -24,7 +24,7 @@ namespace dj {
 
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias);
+                    int interleaved_bias, const int32_t *m_dev, int m_extra);
 
 namespace {
 
@@ -391,7 +391,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     const float *residual = (p.flags & DJ_LIN_RESIDUAL) ? p.residual : nullptr;
     const int kp = q8_padded_k(p.k);
 
-    if (p.m == 1 && matvec_supported(p.k)) {
+    if (p.m == 1 && !p.m_dev && matvec_supported(p.k)) {
         MatvecArgs a{p.x, p.wq, p.scales, p.out, p.k, kp, p.n, gamma, bias, bias2, residual};
         int nc = (kp + 1023) / 1024;
         switch (nc) {
@@ -420,7 +420,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
         ws += (int64_t)p.m * p.k;
     }
     if (swiglu) {
-        launch_q8_gemm(s, x, p.wq, p.scales, ws, p.m, p.k, 2 * p.n, bias, bias2, nullptr, 1);
+        launch_q8_gemm(s, x, p.wq, p.scales, ws, p.m, p.k, 2 * p.n, bias, bias2, nullptr, 1, nullptr, 0);
         int64_t n_out = (int64_t)p.m * p.n;
         int64_t blocks = (n_out + kThreads - 1) / kThreads;
         if (blocks > 8192) blocks = 8192;
@@ -428,7 +428,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
         if (residual) fail("q8_linear: SWIGLU with RESIDUAL is not supported");
         hipLaunchKernelGGL(k_swiglu_combine, dim3((int)blocks), dim3(kThreads), 0, s, ws, p.out, n_out);
     } else {
-        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0);
+        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0, p.m_dev, p.m_extra);
     }
 }
 

@@ -48,7 +48,7 @@ void hip(int rc) {
 struct Layer {
     int32_t g1 = -1, g2 = -1;
     int32_t wqkv = -1, wo = -1;                       // Llama: fused [3d x d]
-    int32_t wdq = -1, wuq = -1, wdkv = -1, wukv = -1;  // MLA: wukv = Wuk|Wuv fused [2d x kvRank]
+    int32_t wdq = -1, wuq = -1, wdkv = -1, wuk = -1, wuv = -1;   // MLA
     int32_t wgu = -1, bg = -1, bu = -1, wd = -1, bd = -1;
 };
 
@@ -150,10 +150,8 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
         else if (c.kind == 1 && w == "wdq") { expect_shape(name, rows, cols, d, c.q_rank); quantize_into(r, L.wdq, data, d, c.q_rank, 0, 1, c.q_rank); }
         else if (c.kind == 1 && w == "wuq") { expect_shape(name, rows, cols, c.q_rank, d); quantize_into(r, L.wuq, data, c.q_rank, d, 0, 1, d); }
         else if (c.kind == 1 && w == "wdkv") { expect_shape(name, rows, cols, d, c.kv_rank); quantize_into(r, L.wdkv, data, d, c.kv_rank, 0, 1, c.kv_rank); }
-        else if (c.kind == 1 && (w == "wuk" || w == "wuv")) {
-            expect_shape(name, rows, cols, c.kv_rank, d);
-            quantize_into(r, L.wukv, data, c.kv_rank, d, w == "wuk" ? 0 : d, 1, 2 * d);
-        }
+        else if (c.kind == 1 && w == "wuk") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuk, data, c.kv_rank, d, 0, 1, d); }
+        else if (c.kind == 1 && w == "wuv") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuv, data, c.kv_rank, d, 0, 1, d); }
         else throw Error("unknown weight " + name);
     } else throw Error("unknown weight " + name);
     r.have[name] = true;
@@ -256,23 +254,24 @@ void finalize(Runner &r) {
         r.kc = r.alloc(per_layer * c.layers);
         r.vc = r.alloc(per_layer * c.layers);
     } else {
-        r.latent = r.alloc((int64_t)c.layers * c.max_seq * c.kv_rank);   // cKV rows, the only per-token state
-        r.kc = r.alloc(per_layer);                                        // K re-expanded + rotated, one layer at a time
+        // The latent rows cKV = norm1(x).Wdkv are the only per-token state that is kept
+        // (kvRank floats per token per layer instead of 2*dModel); K and V of every cached
+        // position are re-expanded from them - and K re-rotated - for each layer of each step,
+        // into these two scratch tensors (token-major [maxSeq x d]).
+        r.latent = r.alloc((int64_t)c.layers * c.max_seq * c.kv_rank);
+        r.kc = r.alloc(per_layer);
         r.vc = r.alloc(per_layer);
-        r.dec.kvexp = r.alloc((int64_t)c.max_seq * 2 * c.d);              // [maxSeq x (K|V)] expansion output
     }
     r.state = r.alloc(4);
     r.tok = r.alloc(4);
     r.tokens = r.alloc(c.max_seq);
     r.logits = r.alloc(c.vocab);
     r.last_x = r.alloc(c.d);
-    int splits = (c.max_seq + 63) / 64;
-    int64_t sf = (int64_t)c.heads * (4 + (int64_t)splits * (hd + 4));
-    r.scratch = r.alloc(sf);
     int ns = std::max(1, std::min(16, 512 / c.heads));
-    r.scratch_dec = r.alloc((int64_t)c.heads * ns * (hd + 4));
+    int64_t sf = (int64_t)c.heads * ns * (hd + 4);           // split-attention records (S = 1 paths)
+    r.scratch = r.alloc(sf);
+    r.scratch_dec = r.alloc(sf);
     Stream s;
-    emit(s, DJ_OP_FILL, r.scratch, 0, (int32_t)sf);
     emit(s, DJ_OP_FILL, r.state, 0, 4);
     emit(s, DJ_OP_FILL, r.tok, 0, 4);
     r.run(s);
@@ -298,7 +297,18 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
             emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
         }
     } else {
-        throw Error("MLA streams are built by mla_block_stream");
+        // MultiHeadLatentAttention.java:92-123 with a latent cache
+        const int qr = c.q_rank, kvr = c.kv_rank;
+        const int64_t lat_off = (int64_t)l * c.max_seq * kvr;
+        q8_linear(s, a.x, L.wdq, a.cq, S, d, qr, DJ_LIN_RMSNORM, L.g1);            // cQ = norm1(x).Wdq
+        q8_linear(s, a.cq, L.wuq, a.qkv, S, qr, d, 0);                               // Q  = cQ.Wuq
+        q8_linear(s, a.x, L.wdkv, a.ckv, S, d, kvr, DJ_LIN_RMSNORM, L.g1);          // cKV = norm1(x).Wdkv
+        emit(s, DJ_OP_APPEND_ROWS, a.ckv, r.latent, r.state, S, kvr, c.max_seq, lat_off);
+        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wuk, r.kc, c.max_seq, kvr, d, r.state, S, lat_off);   // K = cKV.Wuk, all rows
+        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wuv, r.vc, c.max_seq, kvr, d, r.state, S, lat_off);   // V = cKV.Wuv
+        emit(s, DJ_OP_ROPE_ROWS, r.kc, r.kc, r.state, r.cos_t, r.sin_t, c.max_seq, H, hd, c.max_seq, 1);  // row = position
+        emit(s, DJ_OP_ROPE_ROWS, a.qkv, a.q, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, 0);
+        emit(s, DJ_OP_ATTENTION_KV, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0);
     }
     q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
     // x = x2 + down(SiLU(gate(norm2(x2))) * up(norm2(x2)))                  LlamaTransformerBlock.java:52
@@ -534,7 +544,7 @@ void deepj_runner_destroy(void *h) {
     std::vector<int32_t> ids;
     auto add = [&](int32_t id) { if (id >= 0) ids.push_back(id); };
     for (auto &L : r->layers)
-        for (int32_t id : {L.g1, L.g2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wukv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
+        for (int32_t id : {L.g1, L.g2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wuk, L.wuv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
     for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state, r->tok,
                        r->tokens, r->scratch, r->scratch_dec, r->logits, r->last_x})
         add(id);

@@ -183,6 +183,8 @@ int stride_of(int op) {
         case DJ_OP_ATTENTION_KV: return 12;
         case DJ_OP_DECODE_NEXT: return 10;
         case DJ_OP_ATTN_DECODE: return 13;
+        case DJ_OP_APPEND_ROWS: return 8;
+        case DJ_OP_Q8_LINEAR_DYN: return 10;
         default: return -1;
     }
 }
@@ -520,6 +522,33 @@ void exec_one(Cursor &c) {
                                    reinterpret_cast<const int32_t *>(st), sc, ct, sn, (int)H, (int)hd, (int)max_seq);
             break;
         }
+        case DJ_OP_APPEND_ROWS: {
+            // [op, src, dst, state, rows, rowFloats, maxRows, dstOff]: dst[dstOff + (state[0]+i)*rowFloats ..] = src row i
+            int64_t rows = w[4], rf = w[5], max_rows = w[6], off = w[7];
+            if (rows <= 0 || rf <= 0 || max_rows <= 0 || off < 0) fail("OP_APPEND_ROWS: bad shape");
+            const float *src = buf(w[1], rows * rf, op, "src");
+            float *dst = buf(w[2], off + max_rows * rf, op, "dst");
+            const float *st = buf(w[3], 4, op, "state");
+            if (run) launch_append_rows(s, src, dst + off, reinterpret_cast<const int32_t *>(st), (int)rows, (int)rf, (int)max_rows);
+            break;
+        }
+        case DJ_OP_Q8_LINEAR_DYN: {
+            // [op, x, w, out, Mmax, K, N, state, extraRows, xOff]: rows [0, min(Mmax, state[0]+extraRows)) of x + xOff
+            int64_t m = w[4], k = w[5], n = w[6], extra = w[8], xoff = w[9];
+            if (m <= 0 || k <= 0 || n <= 0 || extra < 0 || xoff < 0) fail("OP_Q8_LINEAR_DYN: bad shape");
+            Q8Linear p;
+            p.x = buf(w[1], xoff + m * k, op, "x") + xoff;
+            const float *wq = buf(w[2], (q8_bytes((int)k, (int)n) + 3) / 4, op, "weight");
+            p.wq = reinterpret_cast<const int8_t *>(wq);
+            p.scales = reinterpret_cast<const float *>(p.wq + q8_scale_offset_bytes((int)k, (int)n));
+            p.out = buf(w[3], m * n, op, "out");
+            p.m = (int)m; p.k = (int)k; p.n = (int)n; p.flags = 0;
+            p.gamma = p.bias = p.bias2 = p.residual = nullptr;
+            p.m_dev = reinterpret_cast<const int32_t *>(buf(w[7], 4, op, "state"));
+            p.m_extra = (int)extra;
+            if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
+            break;
+        }
         case DJ_OP_COPY: {
             int64_t n = w[3], so = w[4], dof = w[5];
             if (n < 0 || so < 0 || dof < 0) fail("OP_COPY: bad range");
@@ -592,6 +621,8 @@ const char *op_name(int op) {
         case DJ_OP_ATTENTION_KV: return "OP_ATTENTION_KV";
         case DJ_OP_DECODE_NEXT: return "OP_DECODE_NEXT";
         case DJ_OP_ATTN_DECODE: return "OP_ATTN_DECODE";
+        case DJ_OP_APPEND_ROWS: return "OP_APPEND_ROWS";
+        case DJ_OP_Q8_LINEAR_DYN: return "OP_Q8_LINEAR_DYN";
         default: return "OP_?";
     }
 }

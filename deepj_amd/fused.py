@@ -112,6 +112,12 @@ class Stream:
     def attn_decode(self, qkv, k_cache, v_cache, out, state, scratch, cos, sin, H, hd, max_seq, layer):
         return self.emit(op.OP_ATTN_DECODE, qkv, k_cache, v_cache, out, state, scratch, cos, sin, H, hd, max_seq, layer)
 
+    def append_rows(self, src, dst, state, rows, row_floats, max_rows, dst_off=0):
+        return self.emit(op.OP_APPEND_ROWS, src, dst, state, rows, row_floats, max_rows, dst_off)
+
+    def q8_linear_dyn(self, x, w, out, m_max, k, n, state, extra_rows, x_off=0):
+        return self.emit(op.OP_Q8_LINEAR_DYN, x, w, out, m_max, k, n, state, extra_rows, x_off)
+
     def copy(self, src, dst, n, src_off=0, dst_off=0): return self.emit(op.OP_COPY, src, dst, n, src_off, dst_off)
     def fill(self, dst, bits, n): return self.emit(op.OP_FILL, dst, bits, n)
     def matmul(self, a, b, out, m, n, k): return self.emit(op.OP_MATMUL, a, b, out, m, n, k)
@@ -134,7 +140,6 @@ def attn_decode_scratch_floats(H: int, hd: int) -> int:
     return H * max(1, min(16, 512 // H)) * (hd + 4)
 
 
-def attention_scratch_floats(H: int, hd: int, max_seq: int) -> int:
-    """Floats the decode (S = 1) attention scratch buffer must hold; it must start zeroed."""
-    splits = (max_seq + 63) // 64
-    return H * (4 + splits * (hd + 4))
+def attention_scratch_floats(H: int, hd: int, max_seq: int = 0) -> int:
+    """Floats the scratch buffer of ATTENTION / ATTENTION_KV must hold when S = 1."""
+    return attn_decode_scratch_floats(H, hd)

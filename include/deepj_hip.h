@@ -117,6 +117,7 @@ enum {
      * ROPE_KV_STORE [op, qkv, qOut, kCache, vCache, state, cosT, sinT, S, H, hd, maxSeq, layer]
      *     qkv [S x 3d]; rows sit at positions state[0]..state[0]+S-1
      * ATTENTION     [op, q, kCache, vCache, out, state, scratch, S, H, hd, maxSeq, layer]
+     *     scratch is only used when S = 1 (H * min(16, max(1, 512/H)) * (hd+4) floats, no initialisation)
      * ARGMAX_ROWS   [op, logits, out, rows, cols]      out int32 words, ties -> lowest index
      * DECODE_ADVANCE[op, state, token, tokens, capacity, nPos]
      *     state (int32 words): [0] positions held in the cache, [1] current token, [2] tokens generated;
@@ -129,11 +130,17 @@ enum {
      *     argmax + DECODE_ADVANCE + EMBED_GATHER of the chosen token into x, one launch
      * ATTN_DECODE   [op, qkv, kCache, vCache, out, state, scratch, cosT, sinT, H, hd, maxSeq, layer]
      *     ROPE_KV_STORE + ATTENTION for one new row (S = 1) in two launches
+     * APPEND_ROWS   [op, src, dst, state, rows, rowFloats, maxRows, dstOff]
+     *     dst[dstOff + (state[0]+i)*rowFloats ...] = src row i: append to a cache whose fill level is state[0]
+     * Q8_LINEAR_DYN [op, x, w, out, Mmax, K, N, state, extraRows, xOff]
+     *     Q8_LINEAR (no prologue/epilogue) on rows [0, min(Mmax, state[0]+extraRows)) of x + xOff: the row count
+     *     lives on the device, so the op can sit in a replayed graph while a cache grows
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
-    DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79
+    DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
+    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8 };

@@ -1,0 +1,81 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/model_greedy.json: greedy token ids (and a few logits) of the CPU oracle for
+the baseline's full-size model configurations, which are too slow to run inside the test suite.
+
+The numbers come from this repository's oracle (oracle/, a C restatement of the reference's
+CpuBackend, layers, LlamaModel/DeepSeekModel and TextGenerator) run on the Q8-dequantised seeded
+weights; nothing from the reference tree is imported or executed.  The reference's own tests hold
+no logits or token values for any model, so these fixtures pin the GPU path to the oracle, not to
+a JVM run.
+
+    python tests/golden/make_model_goldens.py c3 [c5]      # minutes per config on 8 cores
+"""
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import cpu_ref as ref  # noqa: E402
+
+CONFIGS = {
+    # BASELINE.json configs[2]: Llama decode workload
+    "c3": dict(model=dict(vocab=32000, max_seq=2048, d=2048, heads=32, layers=16, dff=5632), seed=42,
+               prompt_seed=3, prompt_len=512, new_tokens=64),
+    # BASELINE.json configs[4]: DeepSeek-style MLA (qRank = d/2, kvRank = d/4 as the reference's README suggests).
+    # With the reference's initialiser (N(0,1)*0.1, Tensor.java random) at this width the attention scores
+    # q.k/sqrt(hd) have a standard deviation near 150: every softmax row is a hard arg-max, and any change of
+    # fp32 summation order flips near-ties, so two correct fp32 implementations differ by O(1) in the logits
+    # after a few layers (measured: 1e-3 after 1 layer, 2.5e-2 after 2, 0.7 after 4).  The fixture therefore
+    # scales the five MLA projection matrices by 0.25 (exact in fp32) before quantisation, which brings the
+    # scores to a standard deviation near 0.6 and makes the comparison meaningful; everything else is the
+    # seeded reference initialisation.
+    "c5": dict(model=dict(vocab=32000, max_seq=512, d=2048, heads=16, layers=16, dff=5632, q_rank=1024, kv_rank=512),
+               seed=42, prompt_seed=5, prompt_len=256, new_tokens=64, mla_weight_scale=0.25),
+}
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "model_greedy.json")
+
+
+def run(name):
+    c = CONFIGS[name]
+    ref.set_threads(os.cpu_count() or 1)
+    ref.set_column_parallel(True)           # bit-identical, only faster for single-row matmuls
+    t0 = time.time()
+    m = ref.Model(seed=c["seed"], **c["model"])
+    if "mla_weight_scale" in c:
+        for n in m.weight_names():
+            if n.split(".")[-1] in ("wdq", "wuq", "wdkv", "wuk", "wuv"):
+                m.weight(n)[...] *= np.float32(c["mla_weight_scale"])
+    m.q8_roundtrip()
+    print(f"[{name}] model built in {time.time() - t0:.0f}s", flush=True)
+    prompt = ref.JavaRandom(c["prompt_seed"]).ints(c["prompt_len"], c["model"]["vocab"])
+    t0 = time.time()
+    ids, logits = m.generate(prompt, c["new_tokens"], temperature=1.0, top_k=1, seed=0, use_cache=True,
+                             return_logits=True)
+    print(f"[{name}] generated {c['new_tokens']} tokens in {time.time() - t0:.0f}s", flush=True)
+    srt = np.sort(logits, axis=1)
+    gaps = srt[:, -1] - srt[:, -2]
+    probe = [0, 1, 2, 3, 100, 1000, 31999]
+    return {
+        "config": c,
+        "prompt_head": [int(x) for x in prompt[:8]],
+        "tokens": [int(x) for x in ids[c["prompt_len"]:]],
+        "min_top2_gap": float(gaps.min()),
+        "top_logit": [float(x) for x in srt[:, -1]],
+        "logit_probe_cols": probe,
+        "logit_probe_step0": [float(logits[0, j]) for j in probe],
+        "logit_probe_last": [float(logits[-1, j]) for j in probe],
+        "logits_step0_sum_abs": float(np.abs(logits[0].astype(np.float64)).sum()),
+    }
+
+
+if __name__ == "__main__":
+    names = sys.argv[1:] or ["c3"]
+    data = json.load(open(OUT)) if os.path.exists(OUT) else {}
+    for n in names:
+        data[n] = run(n)
+        json.dump(data, open(OUT, "w"), indent=1)
+        print(f"[{n}] written to {OUT}", flush=True)

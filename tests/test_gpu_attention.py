@@ -56,9 +56,6 @@ def test_rope_store_attention_prefill_and_decode(H, hd, max_seq, chunks):
             pos += S
         st = dev.download(state, (4,), np.int32)
         assert st[0] == total and st[2] == len(chunks)
-        # the scratch counters are back to zero (ready for a graph replay)
-        sc = dev.download(scratch, (sf,), np.int32).reshape(H, -1)
-        assert np.all(sc[:, 0] == 0)
     finally:
         dev.release_all()
 

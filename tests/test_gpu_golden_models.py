@@ -1,0 +1,114 @@
+"""Full-size model configurations of the baseline against fixtures written by the CPU oracle
+(tests/golden/model_greedy.json, made by tests/golden/make_model_goldens.py; the oracle needs
+minutes per configuration, so it does not run inside the suite).
+
+Gates: greedy token ids identical over the first 64 generated tokens.  Logits: at this size the
+CPU path's own fp32 arithmetic is 3.4e-3 (max-abs) away from a float64 evaluation of the same
+model (fixture "fp64_step0", tests/golden/make_fp64_probe.py), so two different fp32 summation
+orders cannot agree to 1e-3; asserted instead: GPU-vs-float64 error no larger than the CPU
+path's (x1.25), and GPU-vs-oracle <= FULL_SIZE_LOGIT_ATOL.  (The 1e-3 gate is asserted on the
+small models in test_gpu_model.py.)  The DeepSeek fixture scales the MLA projections by 0.25: with the
+reference's initialiser at this width the attention softmax is a hard arg-max (scores with a standard
+deviation near 150) and two correct fp32 implementations diverge by O(1) within a few layers (see
+tests/golden/make_model_goldens.py).  Also size-independent properties at full size: graph
+replay == eager, decode row == prefill row (KV-cache causality)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from deepj_amd import DeepSeekConfig, DeepSeekModel, JavaRandom, LlamaConfig, LlamaModel, TextGenerator
+
+pytestmark = pytest.mark.gpu
+
+PATH = os.path.join(os.path.dirname(__file__), "golden", "model_greedy.json")
+GOLD = json.load(open(PATH)) if os.path.exists(PATH) else {}
+FULL_SIZE_LOGIT_ATOL = 5e-3
+
+
+MLA_PROJECTIONS = ("wdq", "wuq", "wdkv", "wuk", "wuv")
+
+
+def seeded_deepseek_with_scaled_mla(cfg, seed, scale):
+    """new DeepSeekModel(cfg, seed) (DeepSeekModel.java:31-47: embedding from Random(seed), the block
+    stack from its own Random(seed), the LM head from Random(seed+1); Tensor.random = N(0,1)*0.1) with the
+    five MLA projection matrices multiplied by `scale`, loaded through setWeight."""
+    model = DeepSeekModel(cfg, None)
+    emb_r, stack_r, head_r = JavaRandom(seed), JavaRandom(seed), JavaRandom(seed + 1)
+    d = cfg.dModel
+    model.setWeight("emb", emb_r.tensor(cfg.vocabSize, d))
+    shapes = dict(wdq=(d, cfg.qRank), wuq=(cfg.qRank, d), wdkv=(d, cfg.kvRank), wuk=(cfg.kvRank, d),
+                  wuv=(cfg.kvRank, d), wo=(d, d), wg=(d, cfg.dFF), wu=(d, cfg.dFF), wd=(cfg.dFF, d))
+    for l in range(cfg.nLayers):
+        model.setWeight(f"L{l}.g1", np.ones((1, d), np.float32))
+        model.setWeight(f"L{l}.g2", np.ones((1, d), np.float32))
+        for w, (r, c) in shapes.items():
+            t = stack_r.tensor(r, c)
+            model.setWeight(f"L{l}.{w}", t * np.float32(scale) if w in MLA_PROJECTIONS else t)
+        for b, n in (("bg", cfg.dFF), ("bu", cfg.dFF), ("bd", d)):
+            model.setWeight(f"L{l}.{b}", np.zeros((1, n), np.float32))
+    model.setWeight("gf", np.ones((1, d), np.float32))
+    model.setWeight("wlm", head_r.tensor(d, cfg.vocabSize))
+    model.setWeight("blm", np.zeros((1, cfg.vocabSize), np.float32))
+    model.finalize()
+    return model
+
+
+def build(name):
+    c = GOLD[name]["config"]
+    m = c["model"]
+    if "q_rank" in m:
+        cfg = DeepSeekConfig(m["vocab"], m["max_seq"], m["d"], m["heads"], m["layers"], m["dff"], m["q_rank"], m["kv_rank"])
+        if "mla_weight_scale" in c:
+            return seeded_deepseek_with_scaled_mla(cfg, c["seed"], c["mla_weight_scale"]), c
+        return DeepSeekModel(cfg, c["seed"]), c
+    cfg = LlamaConfig(m["vocab"], m["max_seq"], m["d"], m["heads"], m["layers"], m["dff"])
+    return LlamaModel(cfg, c["seed"]), c
+
+
+@pytest.mark.parametrize("name", ["c3", "c5"])
+def test_full_size_greedy_tokens_and_logits_match_oracle_fixture(name):
+    if name not in GOLD:
+        pytest.skip(f"no fixture for {name} (run tests/golden/make_model_goldens.py {name})")
+    g = GOLD[name]
+    model, c = build(name)
+    try:
+        prompt = JavaRandom(c["prompt_seed"]).ints(c["prompt_len"], c["model"]["vocab"])
+        assert [int(x) for x in prompt[:8]] == g["prompt_head"]
+        n_new = c["new_tokens"]
+        # step 0: logits of the last prompt row
+        model.reset()
+        model.prefill(prompt, choose_next=False)
+        l0 = model.lastLogits()
+        probe = g["logit_probe_cols"]
+        assert np.max(np.abs(l0[probe] - np.array(g["logit_probe_step0"]))) <= FULL_SIZE_LOGIT_ATOL
+        assert abs(float(l0.max()) - g["top_logit"][0]) <= FULL_SIZE_LOGIT_ATOL
+        if "fp64_step0" in g:
+            f = g["fp64_step0"]
+            exact, cpu = np.array(f["fp64"]), np.array(f["oracle_fp32"])
+            gpu_err = float(np.max(np.abs(l0[f["cols"]] - exact)))
+            cpu_err = float(np.max(np.abs(cpu - exact)))
+            print(f"\n[{name}] max-abs error vs float64 on {len(exact)} logits: GPU {gpu_err:.2e}, CPU oracle {cpu_err:.2e}")
+            assert gpu_err <= 1.25 * cpu_err + 1e-4
+            assert float(np.max(np.abs(l0[f["cols"]] - cpu))) <= FULL_SIZE_LOGIT_ATOL
+        # greedy generation through the captured graph
+        got = TextGenerator.generate(model, prompt, n_new, top_k=1, use_graph=True)
+        exp = np.array(g["tokens"], dtype=np.int32)
+        assert np.array_equal(got[c["prompt_len"]:], exp), f"first mismatch at token {int(np.argmax(got[c['prompt_len']:] != exp))}"
+        last = model.lastLogits()
+        assert np.max(np.abs(last[probe] - np.array(g["logit_probe_last"]))) <= FULL_SIZE_LOGIT_ATOL
+        print(f"\n[{name}] 64 greedy tokens identical; oracle min top-1/top-2 gap {g['min_top2_gap']:.4f}")
+        # eager execution of the same stream gives the same ids
+        eager = TextGenerator.generate(model, prompt, 16, top_k=1, use_graph=False)
+        assert np.array_equal(eager[c["prompt_len"]:], exp[:16])
+        # decode row == prefill row at full size
+        ids = np.concatenate([prompt[:40], exp[:3]])
+        full = model.forward(ids)
+        model.reset()
+        model.prefill(ids[:40], choose_next=False)
+        for t in range(40, 43):
+            model.step(int(ids[t]))
+            assert float(np.max(np.abs(model.lastLogits() - full[t]))) <= FULL_SIZE_LOGIT_ATOL
+    finally:
+        model.close()
