@@ -474,6 +474,8 @@ class _Cfg(C.Structure):
                 ("dff", _I), ("q_rank", _I), ("kv_rank", _I)]
 
 
+lib.ref_set_fast_fill.argtypes = [_I]
+lib.ref_set_fast_fill.restype = None
 lib.ref_model_create.argtypes = [C.POINTER(_Cfg), C.c_int64]
 lib.ref_model_create.restype = C.c_void_p
 lib.ref_model_free.argtypes = [C.c_void_p]
@@ -494,7 +496,9 @@ lib.ref_generate.restype = _I
 class Model:
     """LlamaModel / DeepSeekModel of the reference, seeded init included."""
 
-    def __init__(self, *, vocab, max_seq, d, heads, layers, dff, seed, q_rank=0, kv_rank=0):
+    def __init__(self, *, vocab, max_seq, d, heads, layers, dff, seed, q_rank=0, kv_rank=0, timing_only_fill=False):
+        """timing_only_fill: weights from a cheap hash instead of the seeded Gaussian stream - same
+        sizes and arithmetic, different values; only for measuring the CPU path's speed."""
         self.kind = 1 if q_rank else 0
         if vocab <= 0 or max_seq <= 0 or d <= 0 or heads <= 0 or layers <= 0 or dff <= 0:
             raise ValueError("config values must be > 0")
@@ -503,7 +507,11 @@ class Model:
         self.cfg = _Cfg(self.kind, vocab, max_seq, d, heads, layers, dff, q_rank, kv_rank)
         self.vocab, self.max_seq, self.d, self.heads, self.layers, self.dff = vocab, max_seq, d, heads, layers, dff
         self.q_rank, self.kv_rank = q_rank, kv_rank
-        self._h = lib.ref_model_create(C.byref(self.cfg), seed)
+        lib.ref_set_fast_fill(1 if timing_only_fill else 0)
+        try:
+            self._h = lib.ref_model_create(C.byref(self.cfg), seed)
+        finally:
+            lib.ref_set_fast_fill(0)
 
     def close(self):
         if self._h:

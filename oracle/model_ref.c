@@ -243,9 +243,29 @@ static void q8_roundtrip(float *w, int k, int n) {
 
 /* ── models ─────────────────────────────────────────────────────────── */
 
+/* Timing-only switch: fill weights with a cheap counter hash (uniform, variance of N(0,1)*0.1)
+ * instead of the java.util.Random Gaussian stream, which is sequential and takes minutes for a
+ * full-size model.  Such a model has the memory footprint and arithmetic of the real one but NOT
+ * its values: it is for measuring the CPU path's speed only, never for parity. */
+static int g_fast_fill = 0;
+void ref_set_fast_fill(int on) { g_fast_fill = on; }
+
 static float *rand_tensor(int rows, int cols, jrandom *r) {
-    float *t = falloc((int64_t)rows * cols);
-    ref_random(t, (int64_t)rows * cols, r);
+    int64_t n = (int64_t)rows * cols;
+    float *t = falloc(n);
+    if (g_fast_fill) {
+        uint64_t salt = (uint64_t)jr_next_int(r);
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < n; i++) {
+            uint64_t z = (uint64_t)i * 0x9E3779B97F4A7C15ull + salt;
+            z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+            z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+            z ^= z >> 31;
+            t[i] = ((float)(z >> 40) * (1.0f / 16777216.0f) - 0.5f) * 0.34641016f;   /* sqrt(12) * 0.1 */
+        }
+        return t;
+    }
+    ref_random(t, n, r);
     return t;
 }
 static float *ones(int n) {

@@ -93,6 +93,8 @@ typedef struct {
 } ref_model;
 
 ref_model *ref_model_create(const ref_config *cfg, int64_t seed);
+/* timing-only: later ref_model_create calls fill weights with a cheap hash instead of java.util.Random */
+void       ref_set_fast_fill(int on);
 void       ref_model_free(ref_model *m);
 /* Replace every matmul weight (attention/MLA projections, SwiGLU, LM head) by
  * dequant(quant(W)); embedding, gains and biases stay fp32. */
