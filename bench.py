@@ -32,6 +32,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+# HBM bytes read + written per matvec launch (mean over the 65 launches of one token), from rocprofv3
+# FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
+# (profiles/q8_matvec_llama_d2048_decode_hbm_traffic.txt); algorithmic bytes are 15.40 MB.
+MATVEC_TRAFFIC_BYTES_PER_LAUNCH = 15_700_000
 
 
 def q8_linear_bytes(k: int, n_rows: int) -> int:
@@ -63,9 +67,23 @@ def matvec_roofline(model, iters: int = 20):
     avg_launch_s = ms * 1e-3 / (iters * launches)
     achieved = (total_bytes / launches) / avg_launch_s / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MATVEC_TRAFFIC_BYTES_PER_LAUNCH,
             "kernel": "k_q8_matvec", "launches_per_token": launches,
             "bytes_per_launch": total_bytes // launches, "avg_launch_us": round(avg_launch_s * 1e6, 3)}
+
+
+def calibration_copy(mib: int = 256, repeats: int = 3) -> None:
+    """A plain device copy of known size (reads `mib` MiB, writes `mib` MiB per launch), so that a
+    hardware-counter run of this script has a kernel (k_copy) whose FETCH_SIZE / WRITE_SIZE readings
+    can be compared with its known traffic."""
+    from deepj_amd.fused import DeviceBuffers, Stream
+    dev = DeviceBuffers()
+    n = mib * (1 << 20) // 4
+    src, dst = dev.alloc(n), dev.alloc(n)
+    Stream().fill(src, 0x3F800000, n).run()
+    for _ in range(repeats):
+        Stream().copy(src, dst, n).run()
+    dev.release_all()
 
 
 def cpu_baseline(cfg, ctx: int, tokens: int = 12):
@@ -142,6 +160,7 @@ def main() -> int:
     assert len(toks) == 1 + args.warmup + args.steps
 
     roof = matvec_roofline(model)
+    calibration_copy()
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg, args.prompt)
 
     # per-token algorithmic bytes at the mean decoded position (weights + fp32 KV read)

@@ -851,7 +851,20 @@ int deepj_hip_graph_launch(int32_t handle, int32_t times) {
     return guarded([&] {
         auto it = g.graphs.find(handle);
         if (it == g.graphs.end()) fail("graph_launch: unknown graph handle " + std::to_string(handle));
-        for (int i = 0; i < times; i++) DJ_HIP(hipGraphLaunch(it->second.exec, g.stream));
+        // Bounded run-ahead: at most kRing windows of kWindow replays are queued behind the one the
+        // device is executing, so a long run never piles tens of thousands of dispatches (and their
+        // kernel-argument blocks) into the queue; the device is never left idle by this.
+        constexpr int kWindow = 16, kRing = 4;
+        static hipEvent_t ring[kRing] = {};
+        for (int i = 0; i < times; i++) {
+            if (i % kWindow == 0) {
+                int w = i / kWindow, slot = w % kRing;
+                if (!ring[slot]) DJ_HIP(hipEventCreateWithFlags(&ring[slot], hipEventDisableTiming));
+                if (w >= kRing) DJ_HIP(hipEventSynchronize(ring[slot]));
+                if (w > 0) DJ_HIP(hipEventRecord(ring[(w - 1) % kRing], g.stream));
+            }
+            DJ_HIP(hipGraphLaunch(it->second.exec, g.stream));
+        }
     });
 }
 
