@@ -30,6 +30,7 @@ SOURCES = {
     "kernels_matmul.hip": [],
     "kernels_q8.hip": [],
     "kernels_attn.hip": [],
+    "kernels_decode.hip": [],
     "runner.cpp": [],
     "host_random.cpp": [],
 }

@@ -112,4 +112,30 @@ void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int3
                         const float *table, float *x, int vocab, int d, int n_positions);
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq);
 
+// kernels_decode.hip: persistent greedy decode of the Llama block stack
+struct Q8Mat {
+    const int8_t *w; const float *sc;
+    int k, kp, rows;                       // rows = Q8 rows (gate/up: 2 * dFF, interleaved)
+};
+struct DecodeLayer {
+    Q8Mat qkv, wo, gu, down;
+    const float *g1, *g2, *bg, *bu, *bd;
+};
+struct DecodeParams {
+    int d, H, hd, dff, vocab, max_seq, L, steps, nsplit, capacity;
+    unsigned slot_count, xs_bytes;
+    const DecodeLayer *layers;             // device copy of the layer table
+    const DecodeLayer *layers_host;        // the same table on the host (launch-time checks only)
+    Q8Mat lm;
+    const float *gf, *blm, *emb, *cos_t, *sin_t;
+    float *kc, *vc;                        // [L][H][max_seq][hd]
+    float *x, *x2, *qkv, *att, *ff, *logits, *scratch, *argbuf;
+    int32_t *state, *tokens;
+    unsigned *sync;
+    float scale;
+};
+int64_t llama_decode_sync_words();
+void llama_decode_plan(int H, int hd, int *grid, int *nsplit, int64_t *scratch_floats, int64_t *argbuf_floats);
+void launch_llama_decode(hipStream_t s, DecodeParams &p);
+
 }  // namespace dj

@@ -66,6 +66,9 @@ struct Runner {
     int32_t emb = -1, gf = -1, wlm = -1, blm = -1;
     int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
     int32_t state = -1, tok = -1, tokens = -1, scratch = -1, scratch_dec = -1, logits = -1, last_x = -1;
+    int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
+    int64_t p_sync_floats = 0;
+    bool p_pending = false;                                // a persistent launch has not been checked yet
     Acts dec, pre;
     int32_t graph = 0;
     bool finalized = false;
@@ -274,6 +277,15 @@ void finalize(Runner &r) {
     Stream s;
     emit(s, DJ_OP_FILL, r.state, 0, 4);
     emit(s, DJ_OP_FILL, r.tok, 0, 4);
+    if (c.kind == 0) {
+        int64_t psf = 0, paf = 0;
+        hip(deepj_hip_llama_decode_plan(c.heads, hd, nullptr, nullptr, &psf, &paf));
+        r.p_scratch = r.alloc(psf);
+        r.p_argbuf = r.alloc(paf);
+        r.p_sync_floats = deepj_hip_llama_decode_sync_floats();
+        r.p_sync = r.alloc(r.p_sync_floats);
+        emit(s, DJ_OP_FILL, r.p_sync, 0, r.p_sync_floats);
+    }
     r.run(s);
     alloc_acts(r, r.dec, 1);
     r.finalized = true;
@@ -383,13 +395,48 @@ void reset(Runner &r) {
     r.generated = 0;
 }
 
+// All `steps` tokens in one launch of the persistent decode kernel.
+Stream persistent_stream(Runner &r, int steps) {
+    const Config &c = r.cfg;
+    Stream s;
+    emit(s, DJ_OP_LLAMA_DECODE, 29 + 9 * c.layers, steps, c.d, c.heads, c.dff, c.vocab, c.max_seq, c.layers, c.max_seq,
+         r.emb, r.cos_t, r.sin_t, r.kc, r.vc, r.state, r.tokens, r.dec.x, r.dec.x2, r.dec.qkv, r.dec.att, r.dec.ff,
+         r.logits, r.p_scratch, r.p_argbuf, r.p_sync, r.gf, r.wlm, r.blm);
+    for (const Layer &L : r.layers) emit(s, L.wqkv, L.wo, L.wgu, L.wd, L.g1, L.g2, L.bg, L.bu, L.bd);
+    return s;
+}
+
+// After a persistent launch: state[3] != 0 means a grid barrier timed out and the result is void.
+void check_persistent(Runner &r) {
+    if (!r.p_pending) return;
+    r.p_pending = false;
+    int32_t st[4] = {0, 0, 0, 0};
+    hip(deepj_hip_download(r.state, reinterpret_cast<float *>(st), 4));
+    if (st[3] != 0) {
+        Stream s;
+        emit(s, DJ_OP_FILL, r.p_sync, 0, r.p_sync_floats);
+        r.run(s);
+        st[3] = 0;
+        hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
+        throw Error("persistent decode: a grid barrier timed out (were all compute units available?); the sequence "
+                    "state is invalid, reset and run again");
+    }
+}
+
 // Greedy steps on the device: each consumes state[1] at position state[0] and appends the argmax.
-void decode_greedy(Runner &r, int steps, bool use_graph) {
+// mode 0: the per-token stream, eagerly; 1: the same stream as a replayed HIP graph; 2: persistent kernel.
+void decode_greedy(Runner &r, int steps, int mode) {
     const Config &c = r.cfg;
     if (steps <= 0) return;
     if (r.pos + steps > c.max_seq)
         throw Error("context of " + std::to_string(r.pos + steps) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
-    if (use_graph) {
+    if (mode == 2 && c.kind != 0) throw Error("the persistent decode kernel covers the Llama block only");
+    const bool use_graph = mode == 1;
+    if (mode == 2) {
+        check_persistent(r);
+        r.run(persistent_stream(r, steps));
+        r.p_pending = true;
+    } else if (use_graph) {
         if (!r.graph) {
             Stream s = decode_stream(r, true);
             hip(deepj_hip_graph_capture(s.data(), (int32_t)s.size(), &r.graph));
@@ -460,7 +507,7 @@ int32_t sample_from_logits(const std::vector<float> &logits, float temperature, 
 
 // TextGenerator.generate on token ids (TextGenerator.java:66-87).  out holds n_prompt + max_new ids.
 void generate(Runner &r, const int32_t *prompt, int n_prompt, int max_new, float temperature, int top_k,
-              int64_t seed, int32_t *out, bool use_graph) {
+              int64_t seed, int32_t *out, int mode) {
     const Config &c = r.cfg;
     if (max_new < 0) throw Error("maxNewTokens must be >= 0");
     if (!(temperature > 0.0f)) throw Error("temperature must be > 0");
@@ -474,7 +521,8 @@ void generate(Runner &r, const int32_t *prompt, int n_prompt, int max_new, float
     if (top_k == 1) {
         // argmax needs no random draw to pick, and greedy output is seed independent
         prefill(r, prompt, n_prompt, nullptr, true);
-        decode_greedy(r, max_new - 1, use_graph);
+        decode_greedy(r, max_new - 1, mode);
+        check_persistent(r);
         hip(deepj_hip_download(r.tokens, reinterpret_cast<float *>(out + n_prompt), max_new));
         return;
     }
@@ -582,9 +630,12 @@ int deepj_runner_prefill(void *h, const int32_t *ids, int32_t n, float *all_logi
     return guarded(r, [&] { prefill(*r, ids, n, all_logits, choose_next != 0); });
 }
 
-int deepj_runner_decode(void *h, int32_t steps, int32_t use_graph) {
+int deepj_runner_decode(void *h, int32_t steps, int32_t mode) {
     auto *r = static_cast<Runner *>(h);
-    return guarded(r, [&] { decode_greedy(*r, steps, use_graph != 0); });
+    return guarded(r, [&] {
+        if (mode < 0 || mode > 2) throw Error("decode: mode must be 0 (eager), 1 (graph) or 2 (persistent kernel)");
+        decode_greedy(*r, steps, mode);
+    });
 }
 
 int deepj_runner_step(void *h, int32_t token) {
@@ -594,13 +645,17 @@ int deepj_runner_step(void *h, int32_t token) {
 
 int deepj_runner_last_logits(void *h, float *out) {
     auto *r = static_cast<Runner *>(h);
-    return guarded(r, [&] { hip(deepj_hip_download(r->logits, out, r->cfg.vocab)); });
+    return guarded(r, [&] {
+        check_persistent(*r);
+        hip(deepj_hip_download(r->logits, out, r->cfg.vocab));
+    });
 }
 
 // tokens generated so far in this sequence (device order); returns the count through *n
 int deepj_runner_tokens(void *h, int32_t *out, int32_t capacity, int32_t *n) {
     auto *r = static_cast<Runner *>(h);
     return guarded(r, [&] {
+        check_persistent(*r);
         int32_t count = std::min(r->generated, capacity);
         if (count > 0) hip(deepj_hip_download(r->tokens, reinterpret_cast<float *>(out), count));
         else hip(deepj_hip_synchronize());
@@ -609,9 +664,12 @@ int deepj_runner_tokens(void *h, int32_t *out, int32_t capacity, int32_t *n) {
 }
 
 int deepj_runner_generate(void *h, const int32_t *prompt, int32_t n_prompt, int32_t max_new, float temperature,
-                          int32_t top_k, int64_t seed, int32_t use_graph, int32_t *out) {
+                          int32_t top_k, int64_t seed, int32_t mode, int32_t *out) {
     auto *r = static_cast<Runner *>(h);
-    return guarded(r, [&] { generate(*r, prompt, n_prompt, max_new, temperature, top_k, seed, out, use_graph != 0); });
+    return guarded(r, [&] {
+        if (mode < 0 || mode > 2) throw Error("generate: mode must be 0 (eager), 1 (graph) or 2 (persistent kernel)");
+        generate(*r, prompt, n_prompt, max_new, temperature, top_k, seed, out, mode);
+    });
 }
 
 // The per-token command stream (for inspection, timing and graph capture by the caller).

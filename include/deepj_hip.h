@@ -135,15 +135,33 @@ enum {
      * Q8_LINEAR_DYN [op, x, w, out, Mmax, K, N, state, extraRows, xOff]
      *     Q8_LINEAR (no prologue/epilogue) on rows [0, min(Mmax, state[0]+extraRows)) of x + xOff: the row count
      *     lives on the device, so the op can sit in a replayed graph while a cache grows
+     * LLAMA_DECODE  [op, len, steps, d, H, dFF, vocab, maxSeq, L, capacity,
+     *                emb, cosT, sinT, kCache, vCache, state, tokens, x, x2, qkv, att, ff, logits, scratch, argbuf, sync,
+     *                gf, wlm, blm,  then per layer: wqkv, wo, wgu, wd, g1, g2, bg, bu, bd]      (len = 29 + 9 L words)
+     *     `steps` greedy tokens of the whole Llama block stack (LlamaTransformerBlock.java:50-53,
+     *     DecoderOnlyModel.java:58-64, TextGenerator.java:91-114 with topK = 1) in ONE persistent launch: the
+     *     phases of a token are separated by grid-wide barriers instead of kernel boundaries and the Q8 rows of
+     *     the next phase stream into LDS while the current one finishes.  Starts from state[0] (positions in the
+     *     cache) and state[1] (token to process); appends to kCache/vCache and tokens, leaves the last logits in
+     *     `logits`, advances state[0..2]; state[3] != 0 afterwards means a grid barrier timed out (result invalid).
+     *     wqkv [3d x d], wgu interleaved [2 dFF x d], all weights Q8.  scratch >= H*nsplit*(hd+4) floats, argbuf >=
+     *     2*grid floats (deepj_hip_llama_decode_plan), sync = deepj_hip_llama_decode_sync_floats() floats, zero-filled
+     *     once.  Not capturable into a graph; calls that overlap on one device are not supported.
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
-    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81
+    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8 };
+
+/* Buffer sizes LLAMA_DECODE needs on this device: workgroups launched, key splits per head, floats of
+ * `scratch` and `argbuf`; and the floats of its `sync` buffer. */
+int deepj_hip_llama_decode_plan(int32_t heads, int32_t head_dim, int32_t *grid, int32_t *nsplit,
+                                int64_t *scratch_floats, int64_t *argbuf_floats);
+int64_t deepj_hip_llama_decode_sync_floats(void);
 
 /* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
@@ -176,12 +194,14 @@ int deepj_runner_init_seeded(void *runner, int64_t seed, int32_t threads);  /* n
 int deepj_runner_finalize(void *runner);
 int deepj_runner_reset(void *runner);
 int deepj_runner_prefill(void *runner, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next);
-int deepj_runner_decode(void *runner, int32_t steps, int32_t use_graph);
+/* Greedy decode of `steps` tokens on the device.  mode 0: the per-token stream, launched eagerly; 1: the same
+ * stream replayed as a HIP graph; 2: one launch of the persistent kernel (LLAMA_DECODE; Llama only). */
+int deepj_runner_decode(void *runner, int32_t steps, int32_t mode);
 int deepj_runner_step(void *runner, int32_t token);     /* one caller-chosen token through the S=1 path */
 int deepj_runner_last_logits(void *runner, float *out);
 int deepj_runner_tokens(void *runner, int32_t *out, int32_t capacity, int32_t *n);
 int deepj_runner_generate(void *runner, const int32_t *prompt, int32_t n_prompt, int32_t max_new,
-                          float temperature, int32_t top_k, int64_t seed, int32_t use_graph, int32_t *out);
+                          float temperature, int32_t top_k, int64_t seed, int32_t mode, int32_t *out);
 int deepj_runner_decode_stream(void *runner, int32_t *out, int32_t capacity, int32_t *len);
 
 #ifdef __cplusplus

@@ -59,6 +59,32 @@ def test_c1_greedy_64_tokens_identical_to_oracle(c1):
     assert gap > 1e-3
 
 
+@pytest.mark.skip(reason="the persistent decode kernel (OP_LLAMA_DECODE) ended its one GPU run in a memory fault whose "
+                         "cause is not yet found; the op refuses to launch until it is, and this test stays off the GPU")
+def test_c1_persistent_kernel_equals_graph_and_eager(c1):
+    """The persistent decode kernel (all tokens in one launch), the replayed graph of the per-token stream
+    and its eager execution produce the same ids; the persistent path is repeatable and can be entered
+    mid-sequence from the other paths and left again."""
+    gpu, cpu = c1
+    prompt = ref.JavaRandom(11).ints(20, 256)
+    exp = cpu.generate(prompt, 48, top_k=1, use_cache=True)
+    a = TextGenerator.generate(gpu, prompt, 48, top_k=1, persistent=True)
+    assert np.array_equal(a, exp), f"first mismatch at {int(np.argmax(a != exp))}"
+    logits_persistent = gpu.lastLogits()
+    b = TextGenerator.generate(gpu, prompt, 48, top_k=1, use_graph=True)
+    assert np.array_equal(b, exp)
+    assert float(np.max(np.abs(gpu.lastLogits() - logits_persistent))) <= 1e-4
+    assert np.array_equal(TextGenerator.generate(gpu, prompt, 48, top_k=1, persistent=True), exp)
+    # mixed: prefill, 5 tokens by the graph, 20 by the persistent kernel in two launches, 10 eagerly
+    gpu.reset()
+    gpu.prefill(prompt)
+    gpu.decode(5, use_graph=True)
+    gpu.decode(7, persistent=True)
+    gpu.decode(13, persistent=True)
+    gpu.decode(10, use_graph=False)
+    assert np.array_equal(gpu.tokens(), exp[20:20 + 36])
+
+
 def test_c1_graph_replay_equals_eager_and_is_repeatable(c1):
     gpu, _ = c1
     prompt = ref.JavaRandom(7).ints(32, 256)
