@@ -96,8 +96,10 @@ struct AttnArgs {
     float *out;            // [S x H*hd]
     const int32_t *state;  // state[0] = number of positions before this chunk
     float *scratch; int64_t scratch_floats;
+    unsigned *counters;    // S = 1: kAttnCounterHeads zeroed words owned by the runtime (split arrival counters)
     int s, h, hd, max_seq;
 };
+constexpr int kAttnCounterHeads = 1024;
 void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *k_cache, float *v_cache,
                           const int32_t *state, const float *cos_t, const float *sin_t, int S, int H, int hd,
                           int max_seq);
@@ -106,7 +108,7 @@ void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *
 void launch_attention(hipStream_t s, const AttnArgs &a);
 void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *out,
                         const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,
-                        int max_seq);
+                        int max_seq, unsigned *counters);
 int64_t attn_decode_scratch_floats(int H, int hd);
 void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
                         const float *table, float *x, int vocab, int d, int n_positions);

@@ -160,6 +160,7 @@ struct DecodeArgs {
     const float *cos_t, *sin_t;
     int H, hd, max_seq, nsplit;
     float scale;
+    unsigned *counters;        // one arrival counter per head, zero between launches
 };
 
 // FUSED: rotate q and the new key in registers and append the new key/value row to the cache.
@@ -240,36 +241,50 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
                 O += s_o[i][tid] * w;
             }
         }
+        // The record is written through to memory (agent-scope stores) so that the split that
+        // finishes last can read every record of its head without a cache flush.
         float *rec = a.scratch + ((int64_t)h * a.nsplit + split) * (HD + 4);
-        rec[4 + tid] = O;
-        if (tid == 0) { rec[0] = M; rec[1] = L; }
-    }
-}
-
-// grid H, block hd threads: out[h*hd + j] = sum_i w_i o_i[j] / sum_i w_i l_i.  All record
-// loads are issued before the first use (nsplit <= 16), so the merge is one L2 round trip.
-__global__ void k_attn_decode_merge(const float *__restrict__ scratch, float *__restrict__ out, int hd, int nsplit) {
-    const int h = blockIdx.x, j = threadIdx.x;
-    const float *base = scratch + (int64_t)h * nsplit * (hd + 4);
-    float m[16], l[16], o[16];
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const float *r = base + (int64_t)(i < nsplit ? i : 0) * (hd + 4);
-        m[i] = r[0]; l[i] = r[1]; o[i] = r[4 + j];
-    }
-    float M = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 16; i++) if (i < nsplit) M = fmaxf(M, m[i]);
-    float L = 0.0f, O = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        if (i < nsplit && m[i] != -INFINITY) {
-            float w = expf(m[i] - M);
-            L += l[i] * w;
-            O += o[i] * w;
+        __hip_atomic_store(rec + 4 + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) {
+            __hip_atomic_store(rec, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(rec + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    out[h * hd + j] = O / L;
+    // Last split of the head to arrive merges the head's records: out[h*hd + j] = sum_i w_i o_i[j] / sum_i w_i l_i.
+    __shared__ int s_last;
+    __builtin_amdgcn_s_waitcnt(0x0f70);            // vmcnt(0): this workgroup's record and appended row are in memory
+    __syncthreads();
+    if (tid == 0) {
+        unsigned old = __hip_atomic_fetch_add(a.counters + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bool last = old + 1 == (unsigned)a.nsplit;
+        if (last) __hip_atomic_store(a.counters + h, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = last ? 1 : 0;
+    }
+    __syncthreads();
+    if (s_last && tid < HD) {
+        const float *base = a.scratch + (int64_t)h * a.nsplit * (HD + 4);
+        float m[16], l[16], o[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float *r = base + (int64_t)(i < a.nsplit ? i : 0) * (HD + 4);
+            m[i] = __hip_atomic_load(r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            l[i] = __hip_atomic_load(r + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            o[i] = __hip_atomic_load(r + 4 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; i++) if (i < a.nsplit) M = fmaxf(M, m[i]);
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (i < a.nsplit && m[i] != -INFINITY) {
+                float w = expf(m[i] - M);
+                L += l[i] * w;
+                O += o[i] * w;
+            }
+        }
+        a.out[h * HD + tid] = O / L;
+    }
 }
 
 // Splits per head for the fused decode op: about two workgroups per CU in total.
@@ -322,13 +337,14 @@ static void launch_decode_kernels(hipStream_t s, DecodeArgs &a) {
         case 128: hipLaunchKernelGGL((k_attn_decode_partial<32, FUSED>), grid, dim3(kThreads), 0, s, a); break;
         default: fail("attention: head dim must be 32, 64 or 128");
     }
-    hipLaunchKernelGGL(k_attn_decode_merge, dim3(a.H), dim3(a.hd), 0, s, a.scratch, a.out, a.hd, a.nsplit);
 }
 
 void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *out,
                         const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,
-                        int max_seq) {
+                        int max_seq, unsigned *counters) {
+    if (H > kAttnCounterHeads) fail("attention: more than 1024 heads");
     DecodeArgs a;
+    a.counters = counters;
     a.qkv = qkv; a.k_cache = k_cache; a.v_cache = v_cache; a.out = out; a.state = state; a.scratch = scratch;
     a.tok_stride = hd; a.head_stride = (int64_t)max_seq * hd;
     a.cos_t = cos_t; a.sin_t = sin_t; a.H = H; a.hd = hd; a.max_seq = max_seq;
@@ -343,6 +359,8 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
         a.qkv = p.q; a.k_cache = const_cast<float *>(p.k); a.v_cache = const_cast<float *>(p.v); a.out = p.out;
         a.state = p.state; a.scratch = p.scratch; a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
         a.cos_t = a.sin_t = nullptr; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
+        if (p.h > kAttnCounterHeads) fail("attention: more than 1024 heads");
+        a.counters = p.counters;
         launch_decode_kernels<false>(s, a);
         return;
     }

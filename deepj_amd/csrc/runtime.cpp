@@ -52,6 +52,7 @@ struct Runtime {
     bool capturing = false;
     std::unordered_map<int32_t, Graph> graphs;
     int32_t next_graph = 1;
+    unsigned *attn_counters = nullptr;             // kAttnCounterHeads zeroed words: decode attention's split arrivals
     bool allow_persistent_decode = false;          // no caller sets this: OP_LLAMA_DECODE refuses to launch
     void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
     std::vector<int64_t> decode_table_key;
@@ -70,6 +71,8 @@ void ensure_init(int device = 0) {
     DJ_HIP(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
     g.staging_bytes = (size_t)1 << 20;
     DJ_HIP(hipHostMalloc(&g.staging, g.staging_bytes, hipHostMallocDefault));
+    DJ_HIP(hipMalloc((void **)&g.attn_counters, kAttnCounterHeads * sizeof(unsigned)));
+    DJ_HIP(hipMemset(g.attn_counters, 0, kAttnCounterHeads * sizeof(unsigned)));
     g.device = device;
     g.ready = true;
 }
@@ -470,6 +473,7 @@ void exec_one(Cursor &c) {
             int64_t sf = attention_scratch_floats((int)S, (int)H, (int)hd, (int)max_seq);
             a.scratch = sf > 0 ? buf(w[6], sf, op, "scratch") : nullptr;
             a.scratch_floats = sf;
+            a.counters = g.attn_counters;
             a.s = (int)S; a.h = (int)H; a.hd = (int)hd; a.max_seq = (int)max_seq;
             if (run) launch_attention(s, a);
             break;
@@ -523,7 +527,8 @@ void exec_one(Cursor &c) {
             const float *ct = buf(w[7], max_seq * (hd / 2), op, "cos"), *sn = buf(w[8], max_seq * (hd / 2), op, "sin");
             if (run)
                 launch_attn_decode(s, qkv, kc + layer * per_layer, vc + layer * per_layer, o,
-                                   reinterpret_cast<const int32_t *>(st), sc, ct, sn, (int)H, (int)hd, (int)max_seq);
+                                   reinterpret_cast<const int32_t *>(st), sc, ct, sn, (int)H, (int)hd, (int)max_seq,
+                                   g.attn_counters);
             break;
         }
         case DJ_OP_APPEND_ROWS: {
@@ -850,6 +855,8 @@ int deepj_hip_shutdown(void) {
         g.cache.clear();
         if (g.workspace) (void)hipFree(g.workspace);
         g.workspace = nullptr; g.workspace_floats = 0;
+        if (g.attn_counters) (void)hipFree(g.attn_counters);
+        g.attn_counters = nullptr;
         if (g.decode_table) (void)hipFree(g.decode_table);
         g.decode_table = nullptr; g.decode_table_key.clear();
         if (g.staging) (void)hipHostFree(g.staging);
