@@ -138,6 +138,7 @@ struct DecodeParams {
 };
 int64_t llama_decode_sync_words();
 void llama_decode_plan(int H, int hd, int *grid, int *nsplit, int64_t *scratch_floats, int64_t *argbuf_floats);
+bool llama_decode_supported(int d, int dff);
 void launch_llama_decode(hipStream_t s, DecodeParams &p);
 
 }  // namespace dj

@@ -1,28 +1,22 @@
 // Persistent greedy-decode kernel for the Llama block stack (batch 1, KV cache, Q8 weights).
 //
-// One launch runs `steps` whole tokens: every transformer block, the LM head, the arg-max
-// and the embedding lookup of the chosen token (LlamaTransformerBlock.java:50-53,
+// One launch runs `steps` whole tokens: every transformer block, the LM head, the arg-max and
+// the embedding lookup of the chosen token (LlamaTransformerBlock.java:50-53,
 // DecoderOnlyModel.java:58-64, TextGenerator.java:91-114 with topK = 1).  The grid is one
-// workgroup per CU, all resident at once; the phases of a token
+// workgroup of 512 threads per CU, all resident at once; the phases of a token
 //     qkv = Wqkv.norm1(x) | attention | x2 = x + Wo.att | ff = SwiGLU(norm2(x2)) | x = x2 + Wd.ff
-// are separated by grid-wide barriers (two-level arrival counters, bounded spinning) instead
-// of kernel boundaries.
+// are separated by grid-wide barriers (two-level arrival counters, bounded spinning) instead of
+// kernel boundaries.
 //
 // Why: at batch 1 every matrix-vector product is a few microseconds of HBM streaming behind a
-// few microseconds of launch, first-miss and drain latency.  Here the Q8 rows a workgroup will
-// need next are already on their way into LDS (asynchronous global->LDS loads, four ring slots)
-// while it finishes the current phase and waits at the barrier, so the HBM stream does not stop
-// at phase boundaries.
-//
-// Division of labour inside a workgroup (8 wavefronts): wavefronts 0-6 issue the weight
-// prefetches; all 8 multiply rows out of LDS; wavefront 7 alone touches activations in global
-// memory (loads x, applies RMSNorm, stages it in LDS; adds bias/residual/SwiGLU and stores the
-// outputs).  Its vector-memory counter therefore never contains a prefetch, and the prefetching
-// wavefronts never wait for anything but the chunk they are about to read.
+// few microseconds of launch, first-miss and drain latency.  Here a wavefront issues the loads of
+// the Q8 rows it owns of the NEXT phase's matrix right after signalling the barrier that ends
+// the current phase: the HBM stream runs while the workgroup waits for the other workgroups.
 //
 // Activations written in one phase are read by other workgroups in the next: they are written
-// and read with agent-scope (device-coherent) accesses; weights, tables and KV rows of earlier
-// positions use ordinary loads.
+// and read with agent-scope (device-coherent) accesses, and a workgroup waits for its stores
+// to complete before it signals the barrier; weights, tables and KV rows of earlier positions
+// use ordinary loads.  Plain HIP throughout: no inline assembly.
 #include "dj_common.h"
 
 namespace dj {
@@ -30,23 +24,13 @@ namespace {
 
 constexpr int kDT = 512;                  // threads per workgroup
 constexpr int kDW = kDT / 64;             // wavefronts per workgroup
-constexpr int kIssuers = kDW - 1;         // wavefronts 0..6 issue weight prefetches
-constexpr unsigned kSlotBytes = 32768;    // one ring slot (14 rows of K = 2048 with their scales)
-constexpr unsigned kAuxBytes = 10240;     // attention merge area / output staging
-constexpr unsigned kLdsLimit = 160 * 1024;
 constexpr unsigned kSpinLimit = 1u << 20;
-constexpr int kMaxSlots = 4;
 
 // words of the sync buffer (uint32 index); every counter sits on its own 256-byte line
 constexpr int SY_TOP = 0, SY_FAILED = 64, SY_EPOCH = 128, SY_GRP = 192, SY_REL = SY_GRP + 8 * 64,
               SY_HEAD = SY_REL + 8 * 64;
 constexpr int kHeadStride = 16;
 constexpr int kMaxHeads = 256;
-constexpr int kMaxChunkRows = 112;        // staged sums per chunk (two buffers of 128 floats in aux)
-
-using Mat = Q8Mat;
-using DecLayer = DecodeLayer;
-
 
 // ── device-coherent accesses ────────────────────────────────────────────────
 __device__ __forceinline__ unsigned ldc_u32(const unsigned *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -58,29 +42,8 @@ __device__ __forceinline__ float2 ldc_f2(const float *p) {
     unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return make_float2(__builtin_bit_cast(float, (unsigned)(v & 0xffffffffull)), __builtin_bit_cast(float, (unsigned)(v >> 32)));
 }
-__device__ __forceinline__ void stc_f2(float *p, float2 v) {
-    unsigned long long u = (unsigned long long)__builtin_bit_cast(unsigned, v.x) | ((unsigned long long)__builtin_bit_cast(unsigned, v.y) << 32);
-    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// 16 bytes per lane from global memory straight into LDS at lds_off + lane * 16 (lds_off wave-uniform).
-__device__ __forceinline__ void dma16(const void *g, unsigned lds_off) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_off) : "memory", "m0");
-}
-
-// wait until at most n of this wavefront's vector-memory operations are outstanding
-__device__ __forceinline__ void wait_vm(unsigned n) {
-    switch (n) {
-#define DJ_W(i) case i: asm volatile("s_waitcnt vmcnt(" #i ")" ::: "memory"); break;
-        DJ_W(1) DJ_W(2) DJ_W(3) DJ_W(4) DJ_W(5) DJ_W(6) DJ_W(7) DJ_W(8) DJ_W(9) DJ_W(10) DJ_W(11) DJ_W(12)
-        DJ_W(13) DJ_W(14) DJ_W(15) DJ_W(16) DJ_W(17) DJ_W(18) DJ_W(19) DJ_W(20) DJ_W(21) DJ_W(22) DJ_W(23) DJ_W(24)
-#undef DJ_W
-        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    }
-}
-
-// workgroup barrier that leaves vector-memory operations (the prefetches) in flight
-__device__ __forceinline__ void wg_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// all of this wavefront's vector-memory operations (its stores in particular) have completed
+__device__ __forceinline__ void wait_stores() { __builtin_amdgcn_s_waitcnt(0x0f70); }     // vmcnt(0)
 
 __device__ __forceinline__ float d_sigmoid(float x) { return 1.0f / (1.0f + (float)exp((double)(-x))); }
 
@@ -119,296 +82,204 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
     return i < bi;
 }
 
-// ── per-workgroup view of the kernel ────────────────────────────────────────
-struct Ctx {
-    const DecodeParams &P;
-    unsigned char *lds;        // dynamic LDS
-    unsigned lds_base;         // its LDS byte address (for M0)
-    float *xs;                 // staged activation row [kp]
-    unsigned char *aux;
-    int wg, G, tid, lane, wave;
-    unsigned epoch;            // grid barriers passed so far (all launches)
-    bool failed;
+// ── Q8 rows in registers ────────────────────────────────────────────────────
+// R rows x NC chunks of 16 int8 per lane (one 1 KiB stripe of a row per chunk) with their scales.
+// One register store serves every matrix in turn: slot u * NC + c holds chunk c of row u.
+constexpr int kSlots = 12;
+struct Store {
+    int4 w[kSlots];
+    float sc[kSlots];
 };
 
-// rows of a matrix owned by workgroup wg, in units of `unit` rows
-__device__ __forceinline__ void wg_rows(const Mat &m, int unit, int wg, int G, int &r0, int &r1) {
-    int units = m.rows / unit;
-    r0 = (int)(((long long)units * wg) / G) * unit;
-    r1 = (int)(((long long)units * (wg + 1)) / G) * unit;
-}
-// rows per ring slot: as many as fit, a multiple of `unit`
-__device__ __forceinline__ int rows_per_chunk(const Mat &m, int unit) {
-    int r = (int)(kSlotBytes / (unsigned)(m.kp + m.kp / 8));
-    if (r > kMaxChunkRows) r = kMaxChunkRows;
-    r -= r % unit;
-    return r < unit ? unit : r;
+// outputs [ob, oe) of a matrix with n_out outputs that workgroup wg owns
+__device__ __forceinline__ void wg_outputs(int n_out, int wg, int G, int &ob, int &oe) {
+    ob = (int)(((long long)n_out * wg) / G);
+    oe = (int)(((long long)n_out * (wg + 1)) / G);
 }
 
-// ── weight prefetch ring ────────────────────────────────────────────────────
-// The chunk sequence of a workgroup is a pure function of (step, layer, matrix, row), so the
-// prefetching side and the consuming side each walk it with their own cursor.
-struct Cursor { int step, layer, kind, row; };     // kind 0 qkv, 1 wo, 2 gate/up, 3 down, 4 LM head; row < 0: not entered
-
-__device__ __forceinline__ const Mat &mat_of(const DecodeParams &P, int layer, int kind) {
-    if (kind == 4) return P.lm;
-    const DecLayer &L = P.layers[layer];
-    return kind == 0 ? L.qkv : (kind == 1 ? L.wo : (kind == 2 ? L.gu : L.down));
-}
-
-struct Pipe {
-    Cursor cur;
-    unsigned issued, consumed;
-    unsigned nload0, nload1, nload2, nload3;    // prefetch loads this wavefront issued for the chunk in each slot
-
-    __device__ __forceinline__ unsigned get_nload(unsigned s) const { return s == 0 ? nload0 : (s == 1 ? nload1 : (s == 2 ? nload2 : nload3)); }
-    __device__ __forceinline__ void set_nload(unsigned s, unsigned v) {
-        if (s == 0) nload0 = v; else if (s == 1) nload1 = v; else if (s == 2) nload2 = v; else nload3 = v;
-    }
-
-    // next chunk of the sequence; false when all steps are done
-    __device__ __forceinline__ bool next(const Ctx &c, const int8_t *&w, const float *&sc, int &rows, int &kp) {
-        const DecodeParams &P = c.P;
-        while (cur.step < P.steps) {
-            const Mat &m = mat_of(P, cur.layer, cur.kind);
-            const int unit = cur.kind == 2 ? 2 : 1;
-            int r0, r1;
-            wg_rows(m, unit, c.wg, c.G, r0, r1);
-            if (cur.row < 0) cur.row = r0;
-            if (cur.row < r1) {
-                int rpc = rows_per_chunk(m, unit);
-                rows = r1 - cur.row < rpc ? r1 - cur.row : rpc;
-                kp = m.kp;
-                w = m.w + (long long)cur.row * m.kp;
-                sc = m.sc + (long long)cur.row * (m.kp / kQ8Group);
-                cur.row += rows;
-                return true;
-            }
-            cur.row = -1;
-            if (cur.kind == 4) { cur.kind = 0; cur.layer = 0; cur.step++; }
-            else if (cur.kind == 3) {
-                if (cur.layer + 1 < P.L) { cur.layer++; cur.kind = 0; }
-                else cur.kind = 4;
-            } else cur.kind++;
-        }
-        return false;
-    }
-
-    __device__ __forceinline__ void top_up(const Ctx &c) {
-        const unsigned slots = c.P.slot_count;
-        while (issued - consumed < slots) {
-            const int8_t *w; const float *sc; int rows, kp;
-            if (!next(c, w, sc, rows, kp)) break;
-            const unsigned slot = issued % slots;
-            const unsigned base = c.lds_base + slot * kSlotBytes;
-            unsigned n = 0;
-            if (c.wave < kIssuers) {
-                const unsigned wbytes = (unsigned)rows * (unsigned)kp;
-                const unsigned sbytes = (unsigned)rows * (unsigned)(kp / kQ8Group) * 4u;
-                for (unsigned p = c.wave; p * 1024u < wbytes; p += kIssuers) {
-                    unsigned off = p * 1024u + c.lane * 16u;
-                    if (off < wbytes) dma16(reinterpret_cast<const unsigned char *>(w) + off, __builtin_amdgcn_readfirstlane(base + p * 1024u));
-                    n++;
-                }
-                for (unsigned p = c.wave; p * 1024u < sbytes; p += kIssuers) {
-                    unsigned off = p * 1024u + c.lane * 16u;
-                    if (off < sbytes) dma16(reinterpret_cast<const unsigned char *>(sc) + off, __builtin_amdgcn_readfirstlane(base + wbytes + p * 1024u));
-                    n++;
-                }
-            }
-            set_nload(slot, n);
-            issued++;
-        }
-    }
-
-    // LDS byte offset of the oldest chunk once all of it has landed
-    __device__ __forceinline__ unsigned acquire(const Ctx &c) {
-        const unsigned slots = c.P.slot_count;
-        unsigned younger = 0;
-        for (unsigned i = consumed + 1; i < issued; i++) younger += get_nload(i % slots);
-        if (c.wave < kIssuers) wait_vm(younger);
-        wg_sync();
-        return (consumed % slots) * kSlotBytes;
-    }
-    // every wavefront has finished reading the oldest chunk (callers sync before this)
-    __device__ __forceinline__ void release(const Ctx &c) {
-        consumed++;
-        top_up(c);
-    }
-};
-
-// ── grid barrier ────────────────────────────────────────────────────────────
-__device__ __forceinline__ bool spin_until(Ctx &c, const unsigned *p, unsigned target) {
-    unsigned spins = 0;
-    while ((int)(ldc_u32(p) - target) < 0) {
-        if (++spins > kSpinLimit || ldc_u32(c.P.sync + SY_FAILED)) {
-            stc_u32(c.P.sync + SY_FAILED, 1u);
-            return false;
-        }
-        __builtin_amdgcn_s_sleep(1);
-    }
-    return true;
-}
-
-// Called by all threads.  Wavefront 7 has no prefetch in flight, so its vmcnt(0) only covers
-// the activation stores of this phase.
-__device__ __forceinline__ void grid_sync(Ctx &c) {
-    c.epoch++;
-    if (c.wave == kDW - 1) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (c.lane == 0 && !c.failed) {
-            unsigned *sy = c.P.sync;
-            const unsigned g = c.wg & 7;
-            const unsigned ngroups = c.G < 8 ? c.G : 8;
-            const unsigned gsize = (c.G - g + 7) >> 3;
-            unsigned old = addc_u32(sy + SY_GRP + g * 64, 1u);
-            if (old + 1 == c.epoch * gsize) {
-                unsigned o2 = addc_u32(sy + SY_TOP, 1u);
-                if (o2 + 1 == c.epoch * ngroups)
-                    for (unsigned i = 0; i < ngroups; i++) stc_u32(sy + SY_REL + i * 64, c.epoch);
-            }
-            if (!spin_until(c, sy + SY_REL + g * 64, c.epoch)) *reinterpret_cast<volatile int *>(c.aux + kAuxBytes - 4) = 1;
-        }
-    }
-    wg_sync();
-    if (*reinterpret_cast<volatile int *>(c.aux + kAuxBytes - 4)) c.failed = true;
-}
-
-// ── activation staging (wavefront 7) ────────────────────────────────────────
-// xs[0..kp) = optional RMSNorm of src[0..k) (RMSNorm1D.java:46-57), zero beyond k.
-__device__ __forceinline__ void stage_x(Ctx &c, const float *src, const bool COHERENT, int k, int kp, const float *gamma) {
-    if (c.wave != kDW - 1) return;
-    // lane handles 16 consecutive floats of each 1024-float block
-    float ss = 0.0f;
-    for (int kb = c.lane * 16; kb < kp; kb += 1024) {
-        float v[16];
+// Loads rows row0 .. row0+R-1 of m (clamped to row_last); chunks past Kp read chunk 0 (their
+// activations are zero), so no load sits under a branch.
+template <int NC, int R>
+__device__ __forceinline__ void load_batch(Store &b, const Q8Mat &m, int row0, int row_last, int lane) {
+    static_assert(NC * R <= kSlots, "batch does not fit the register store");
+    const int groups = m.kp / kQ8Group;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            int e = kb + 2 * j;
-            float2 t = make_float2(0.f, 0.f);
-            if (e + 1 < k) t = COHERENT ? ldc_f2(src + e) : *reinterpret_cast<const float2 *>(src + e);
-            else if (e < k) t.x = COHERENT ? ldc_f32(src + e) : src[e];
-            v[2 * j] = t.x; v[2 * j + 1] = t.y;
-            ss += t.x * t.x + t.y * t.y;
-        }
+    for (int u = 0; u < R; u++) {
+        int row = row0 + u < row_last ? row0 + u : row_last;
+        const int8_t *wrow = m.w + (long long)row * m.kp;
+        const float *srow = m.sc + (long long)row * groups;
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            *reinterpret_cast<float4 *>(c.xs + kb + 4 * j) = make_float4(v[4 * j], v[4 * j + 1], v[4 * j + 2], v[4 * j + 3]);
-    }
-    if (gamma) {
-        float tot = wave_sum_dpp(ss);
-        float rms = sqrtf(tot * (1.0f / (float)k) + kRmsEps);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        for (int kb = c.lane * 16; kb < kp; kb += 1024) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                int e = kb + 4 * j;
-                float4 t = *reinterpret_cast<float4 *>(c.xs + e);
-                float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (e + 3 < k) g = *reinterpret_cast<const float4 *>(gamma + e);
-                else { if (e < k) g.x = gamma[e]; if (e + 1 < k) g.y = gamma[e + 1]; if (e + 2 < k) g.z = gamma[e + 2]; }
-                t.x = (t.x / rms) * g.x; t.y = (t.y / rms) * g.y; t.z = (t.z / rms) * g.z; t.w = (t.w / rms) * g.w;
-                *reinterpret_cast<float4 *>(c.xs + e) = t;
-            }
+        for (int c = 0; c < NC; c++) {
+            int chunk = c * 64 + lane;
+            if (chunk * 16 >= m.kp) chunk = 0;
+            b.w[u * NC + c] = *reinterpret_cast<const int4 *>(wrow + chunk * 16);
+            b.sc[u * NC + c] = srow[chunk >> 1];
         }
     }
 }
 
-// ── one matrix-vector phase ─────────────────────────────────────────────────
-// kind selects the epilogue wavefront 7 applies when it stores a chunk's outputs:
-//   0 qkv: plain; 1 wo: + residual; 2 gate/up: SiLU(gate + bg) * (up + bu); 3 down: + bd + residual;
-//   4 LM head: + blm, tracks the arg-max.
+// How a phase finishes its outputs.
 struct Epilogue {
     float *out; const float *bias, *bias2, *residual;
     bool residual_coherent;
-    float best_v; int best_i;      // kind 4, wavefront 7
 };
 
-template <int NC, bool PAIRS>
-__device__ __forceinline__ void run_matrix(Ctx &c, Pipe &pipe, const Mat &m, Epilogue &ep) {
-    constexpr int unit = PAIRS ? 2 : 1;
-    int r0, r1;
-    wg_rows(m, unit, c.wg, c.G, r0, r1);
-    const int kp = m.kp, groups = kp / kQ8Group;
-    const int rpc = rows_per_chunk(m, unit);
-    float *stage = reinterpret_cast<float *>(c.aux);          // two buffers of 128 floats
+// The rows of matrix m this wavefront owns: batches of B outputs (RPO rows each) dealt
+// round-robin to the 8 wavefronts of the workgroup inside the workgroup's output range.
+template <int NC, int B, bool PAIRS> struct Work {
+    static constexpr int RPO = PAIRS ? 2 : 1;
+    static constexpr int R = B * RPO;
+    using Regs = Store;
 
-    // this lane's slice of the staged activation row
-    float xr[NC][16];
-#pragma unroll
-    for (int cc = 0; cc < NC; cc++) {
-        int kb = (cc * 64 + c.lane) * 16;
-        bool active = kb < kp;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float4 v = active ? *reinterpret_cast<const float4 *>(c.xs + kb + 4 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
-            xr[cc][4 * j] = v.x; xr[cc][4 * j + 1] = v.y; xr[cc][4 * j + 2] = v.z; xr[cc][4 * j + 3] = v.w;
-        }
+    // first batch of this wavefront into `b` (no-op when it has none)
+    static __device__ __forceinline__ void prefetch(Regs &b, const Q8Mat &m, int wg, int G, int wave, int lane) {
+        int ob, oe;
+        wg_outputs(m.rows / RPO, wg, G, ob, oe);
+        int o0 = ob + wave * B;
+        if (o0 < oe) load_batch<NC, R>(b, m, o0 * RPO, oe * RPO - 1, lane);
     }
 
-    int parity = 0;
-    for (int row = r0; row < r1; row += rpc, parity ^= 1) {
-        const int rows = r1 - row < rpc ? r1 - row : rpc;
-        const unsigned slot = pipe.acquire(c);
-        const unsigned char *wl = c.lds + slot;
-        const float *sl = reinterpret_cast<const float *>(c.lds + slot + (unsigned)rows * (unsigned)kp);
-        float *st = stage + parity * 128;
-        for (int u = c.wave * unit; u < rows; u += kDW * unit) {
-            float a0 = 0.0f, a1 = 0.0f;
+    // `b` holds the first batch (prefetch above); xs = staged activation row in LDS.
+    static __device__ __forceinline__ void run(Regs &b, const Q8Mat &m, const float *xs, const Epilogue &ep, int wg, int G,
+                                               int wave, int lane, float &best_v, int &best_i) {
+        int ob, oe;
+        wg_outputs(m.rows / RPO, wg, G, ob, oe);
+        const int step = kDW * B;
+        for (int o0 = ob + wave * B; o0 < oe; o0 += step) {
+            // The lane's 16 activations of each 1 KiB stripe come from LDS stripe by stripe, so only
+            // one stripe's worth is live in registers next to the weight batches.
+            float acc[R];
 #pragma unroll
-            for (int cc = 0; cc < NC; cc++) {
-                int chunk = cc * 64 + c.lane;
-                if (chunk * 16 >= kp) chunk = 0;          // its activations are zero
-                int4 w0 = *reinterpret_cast<const int4 *>(wl + (unsigned)u * kp + chunk * 16);
-                float s0 = sl[u * groups + (chunk >> 1)];
-                a0 = fmaf(dot16(w0, xr[cc]), s0, a0);
-                if (PAIRS) {
-                    int4 w1 = *reinterpret_cast<const int4 *>(wl + (unsigned)(u + 1) * kp + chunk * 16);
-                    float s1 = sl[(u + 1) * groups + (chunk >> 1)];
-                    a1 = fmaf(dot16(w1, xr[cc]), s1, a1);
+            for (int u = 0; u < R; u++) acc[u] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NC; c++) {
+                const int kb = (c * 64 + lane) * 16;
+                const bool active = kb < m.kp;
+                float xc[16];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float4 v = active ? *reinterpret_cast<const float4 *>(xs + kb + 4 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    xc[4 * j] = v.x; xc[4 * j + 1] = v.y; xc[4 * j + 2] = v.z; xc[4 * j + 3] = v.w;
                 }
+#pragma unroll
+                for (int u = 0; u < R; u++) acc[u] = fmaf(dot16(b.w[u * NC + c], xc), b.sc[u * NC + c], acc[u]);
+                __builtin_amdgcn_sched_barrier(0);     // keep one stripe of activations live at a time
             }
-            a0 = wave_sum_dpp(a0);
-            if (PAIRS) a1 = wave_sum_dpp(a1);
-            if (c.lane == 0) {
-                st[u] = a0;
-                if (PAIRS) st[u + 1] = a1;
+#pragma unroll
+            for (int u = 0; u < R; u++) acc[u] = wave_sum_dpp(acc[u]);
+            if (o0 + step < oe) load_batch<NC, R>(b, m, (o0 + step) * RPO, oe * RPO - 1, lane);   // next batch streams in
+            if (lane == 0) {
+#pragma unroll
+                for (int u = 0; u < B; u++) {
+                    int o = o0 + u;
+                    if (o < oe) {
+                        float v;
+                        if (PAIRS) {
+                            float gate = acc[2 * u], up = acc[2 * u + 1];
+                            if (ep.bias) gate = gate + ep.bias[o];
+                            if (ep.bias2) up = up + ep.bias2[o];
+                            float sg = gate * d_sigmoid(gate);      // SiLU.java:20-24
+                            v = sg * up;                             // SwiGLULayer.java:69
+                        } else {
+                            v = acc[u];
+                            if (ep.bias) v = v + ep.bias[o];
+                        }
+                        if (ep.residual) v = (ep.residual_coherent ? ldc_f32(ep.residual + o) : ep.residual[o]) + v;
+                        stc_f32(ep.out + o, v);
+                        if (better(v, o, best_v, best_i)) { best_v = v; best_i = o; }
+                    }
+                }
             }
         }
-        wg_sync();                                     // chunk fully read, staged sums visible
-        pipe.release(c);
-        if (c.wave == kDW - 1) {
-            const int n_out = rows / unit;
-            for (int i = c.lane; i < n_out; i += 64) {
-                const int o = (row / unit) + i;
-                float v;
-                if (PAIRS) {
-                    float gate = st[2 * i], up = st[2 * i + 1];
-                    if (ep.bias) gate = gate + ep.bias[o];
-                    if (ep.bias2) up = up + ep.bias2[o];
-                    float sg = gate * d_sigmoid(gate);          // SiLU.java:20-24
-                    v = sg * up;                                 // SwiGLULayer.java:69
-                } else {
-                    v = st[i];
-                    if (ep.bias) v = v + ep.bias[o];
-                }
-                if (ep.residual) v = (ep.residual_coherent ? ldc_f32(ep.residual + o) : ep.residual[o]) + v;
-                stc_f32(ep.out + o, v);
-                if (better(v, o, ep.best_v, ep.best_i)) { ep.best_v = v; ep.best_i = o; }
-            }
+    }
+};
+
+// ── per-workgroup state ─────────────────────────────────────────────────────
+struct Ctx {
+    int wg, G, tid, lane, wave;
+    unsigned epoch;            // grid barriers passed so far (all launches)
+    bool failed;
+    unsigned *sync;
+    int *s_flag;               // LDS: [0] barrier failure, [1] last-split flag
+};
+
+// ── grid barrier, in two halves so that loads can be issued in between ──────
+__device__ __forceinline__ void grid_arrive(Ctx &c) {
+    wait_stores();
+    __syncthreads();                       // every wavefront's activation stores are complete
+    c.epoch++;
+    if (c.tid == 0 && !c.failed) {
+        const unsigned g = c.wg & 7;
+        const unsigned ngroups = c.G < 8 ? c.G : 8;
+        const unsigned gsize = (c.G - g + 7) >> 3;
+        unsigned old = addc_u32(c.sync + SY_GRP + g * 64, 1u);
+        if (old + 1 == c.epoch * gsize) {
+            unsigned o2 = addc_u32(c.sync + SY_TOP, 1u);
+            if (o2 + 1 == c.epoch * ngroups)
+                for (unsigned i = 0; i < ngroups; i++) stc_u32(c.sync + SY_REL + i * 64, c.epoch);
         }
     }
 }
+__device__ __forceinline__ void grid_wait(Ctx &c) {
+    if (c.tid == 0 && !c.failed) {
+        const unsigned *p = c.sync + SY_REL + (c.wg & 7) * 64;
+        unsigned spins = 0;
+        while ((int)(ldc_u32(p) - c.epoch) < 0) {
+            if (++spins > kSpinLimit || ldc_u32(c.sync + SY_FAILED)) {
+                stc_u32(c.sync + SY_FAILED, 1u);
+                c.s_flag[0] = 1;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    __syncthreads();
+    if (c.s_flag[0]) c.failed = true;
+}
 
-template <bool PAIRS>
-__device__ __forceinline__ void run_matrix_nc(Ctx &c, Pipe &pipe, const Mat &m, Epilogue &ep) {
-    const int nc = (m.kp + 1023) / 1024;
-    if (nc <= 1) run_matrix<1, PAIRS>(c, pipe, m, ep);
-    else if (nc <= 2) run_matrix<2, PAIRS>(c, pipe, m, ep);
-    else if (nc <= 4) run_matrix<4, PAIRS>(c, pipe, m, ep);
-    else if (nc <= 6) run_matrix<6, PAIRS>(c, pipe, m, ep);
-    else if (nc <= 8) run_matrix<8, PAIRS>(c, pipe, m, ep);
-    else run_matrix<11, PAIRS>(c, pipe, m, ep);
+// ── activation staging ──────────────────────────────────────────────────────
+// xs[0..kp) = optional RMSNorm of src[0..k) (RMSNorm1D.java:46-57), zero beyond k.  All 512
+// threads; NCX = ceil(kp / 1024).
+template <int NCX>
+__device__ __forceinline__ void stage_x(const Ctx &c, const float *src, bool coherent, int k, int kp, const float *gamma,
+                                        float *xs, float *red) {
+    float2 xv[NCX], gv[NCX];
+#pragma unroll
+    for (int j = 0; j < NCX; j++) {
+        int e = (c.tid + kDT * j) * 2;
+        xv[j] = make_float2(0.f, 0.f);
+        gv[j] = make_float2(0.f, 0.f);
+        if (e + 1 < k) {
+            xv[j] = coherent ? ldc_f2(src + e) : *reinterpret_cast<const float2 *>(src + e);
+            if (gamma) gv[j] = *reinterpret_cast<const float2 *>(gamma + e);
+        } else if (e < k) {
+            xv[j].x = coherent ? ldc_f32(src + e) : src[e];
+            if (gamma) gv[j].x = gamma[e];
+        }
+    }
+    if (gamma) {
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCX; j++) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y;
+        ss = wave_sum_dpp(ss);
+        if (c.lane == 0) red[c.wave] = ss;
+        __syncthreads();
+        float tot = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kDW; w++) tot += red[w];
+        float rms = sqrtf(tot * (1.0f / (float)k) + kRmsEps);
+#pragma unroll
+        for (int j = 0; j < NCX; j++) {
+            xv[j].x = (xv[j].x / rms) * gv[j].x;
+            xv[j].y = (xv[j].y / rms) * gv[j].y;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NCX; j++) {
+        int e = (c.tid + kDT * j) * 2;
+        if (e < kp) *reinterpret_cast<float2 *>(xs + e) = xv[j];
+    }
+    __syncthreads();
 }
 
 // ── attention for one (head, split) item ────────────────────────────────────
@@ -416,15 +287,14 @@ __device__ __forceinline__ void run_matrix_nc(Ctx &c, Pipe &pipe, const Mat &m, 
 // runs the online softmax over this split's keys (HeadOps.java:90-140 for one query row) and
 // leaves a partial record; the last split of a head to finish merges the head's records.
 template <int LPK>
-__device__ __forceinline__ void attention_item(Ctx &c, int layer, int pos, int h, int split) {
-    const DecodeParams &P = c.P;
+__device__ __forceinline__ void attention_item(Ctx &c, const DecodeParams &P, int layer, int pos, int h, int split,
+                                               float *aux) {
     constexpr int HD = LPK * 4;
     constexpr int KPW = 64 / LPK;
     constexpr int NSUB = kDW * KPW;
-    float *s_m = reinterpret_cast<float *>(c.aux);
+    float *s_m = aux;
     float *s_l = s_m + NSUB;
     float *s_o = s_l + NSUB;                               // [NSUB][HD]
-    int *s_last = reinterpret_cast<int *>(c.aux + kAuxBytes - 8);
     const int sub = c.lane / LPK, dl = c.lane % LPK;
     const int d = P.d, half = HD / 2, ns = P.nsplit;
 
@@ -443,6 +313,7 @@ __device__ __forceinline__ void attention_item(Ctx &c, int layer, int pos, int h
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 1
     for (int key = k_begin + c.wave * KPW + sub; key < k_end; key += kDW * KPW) {
         float4 kk, vv;
         if (key == pos) {
@@ -451,10 +322,11 @@ __device__ __forceinline__ void attention_item(Ctx &c, int layer, int pos, int h
                              kc2.x * c2.y - kc2.y * s2.y, kc2.x * s2.y + kc2.y * c2.y);
             const float2 va = ldc_f2(P.qkv + 2 * d + h * HD + dl * 4), vb2 = ldc_f2(P.qkv + 2 * d + h * HD + dl * 4 + 2);
             vv = make_float4(va.x, va.y, vb2.x, vb2.y);
-            stc_f2(kb + (long long)key * HD, make_float2(kk.x, kk.y));
-            stc_f2(kb + (long long)key * HD + 2, make_float2(kk.z, kk.w));
-            stc_f2(vb + (long long)key * HD, make_float2(vv.x, vv.y));
-            stc_f2(vb + (long long)key * HD + 2, make_float2(vv.z, vv.w));
+            // the appended row is read by later tokens, possibly from another CU in this same launch
+            stc_f32(kb + (long long)key * HD, kk.x); stc_f32(kb + (long long)key * HD + 1, kk.y);
+            stc_f32(kb + (long long)key * HD + 2, kk.z); stc_f32(kb + (long long)key * HD + 3, kk.w);
+            stc_f32(vb + (long long)key * HD, vv.x); stc_f32(vb + (long long)key * HD + 1, vv.y);
+            stc_f32(vb + (long long)key * HD + 2, vv.z); stc_f32(vb + (long long)key * HD + 3, vv.w);
         } else {
             kk = *reinterpret_cast<const float4 *>(kb + (long long)key * HD);
             vv = *reinterpret_cast<const float4 *>(vb + (long long)key * HD);
@@ -474,14 +346,14 @@ __device__ __forceinline__ void attention_item(Ctx &c, int layer, int pos, int h
     const int slot = c.wave * KPW + sub;
     if (dl == 0) { s_m[slot] = m; s_l[slot] = l; }
     *reinterpret_cast<float4 *>(s_o + slot * HD + dl * 4) = o;
-    wg_sync();
+    __syncthreads();
     float *rec = P.scratch + ((long long)h * ns + split) * (HD + 4);
     if (c.tid < HD) {
         float M = -INFINITY, L = 0.0f, O = 0.0f;
-#pragma unroll 8
+#pragma unroll 4
         for (int i = 0; i < NSUB; i++) M = fmaxf(M, s_m[i]);
         if (M != -INFINITY) {
-#pragma unroll 8
+#pragma unroll 2
             for (int i = 0; i < NSUB; i++) {
                 float w = expf(s_m[i] - M);
                 L += s_l[i] * w;
@@ -491,19 +363,21 @@ __device__ __forceinline__ void attention_item(Ctx &c, int layer, int pos, int h
         stc_f32(rec + 4 + c.tid, O);
         if (c.tid == 0) { stc_f32(rec, M); stc_f32(rec + 1, L); }
     }
-    // all of this workgroup's stores (record, appended row) must be complete before it counts itself in
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    wg_sync();
+    // this workgroup's stores (record, appended row) are complete before it counts itself in
+    wait_stores();
+    __syncthreads();
     if (c.tid == 0) {
-        unsigned old = addc_u32(P.sync + SY_HEAD + h * kHeadStride, 1u);
-        *s_last = ((old + 1) % (unsigned)ns) == 0;
+        unsigned old = addc_u32(c.sync + SY_HEAD + h * kHeadStride, 1u);
+        c.s_flag[1] = ((old + 1) % (unsigned)ns) == 0;
     }
-    wg_sync();
-    if (*reinterpret_cast<volatile int *>(s_last) && c.tid < HD) {
+    __syncthreads();
+    if (c.s_flag[1] && c.tid < HD) {
         const float *base = P.scratch + (long long)h * ns * (HD + 4);
         float M = -INFINITY;
+#pragma unroll 1
         for (int i = 0; i < ns; i++) M = fmaxf(M, ldc_f32(base + (long long)i * (HD + 4)));
         float L = 0.0f, O = 0.0f;
+#pragma unroll 1
         for (int i = 0; i < ns; i++) {
             const float *r = base + (long long)i * (HD + 4);
             float mi = ldc_f32(r);
@@ -515,122 +389,138 @@ __device__ __forceinline__ void attention_item(Ctx &c, int layer, int pos, int h
         }
         stc_f32(P.att + h * HD + c.tid, O / L);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the merged head is in memory before the workgroup moves on
-    wg_sync();                                             // aux is reused by the next item / phase
+    __syncthreads();                                       // aux is reused by the next item
 }
 
-__device__ __forceinline__ void attention_phase(Ctx &c, int layer, int pos) {
-    const DecodeParams &P = c.P;
+__device__ __attribute__((noinline)) void attention_phase(Ctx &c, const DecodeParams &P, int layer, int pos, float *aux) {
     const int items = P.H * P.nsplit;
     for (int it = c.wg; it < items; it += c.G) {
         const int h = it / P.nsplit, split = it % P.nsplit;
         switch (P.hd) {
-            case 32: attention_item<8>(c, layer, pos, h, split); break;
-            case 64: attention_item<16>(c, layer, pos, h, split); break;
-            default: attention_item<32>(c, layer, pos, h, split); break;
+            case 32: attention_item<8>(c, P, layer, pos, h, split, aux); break;
+            case 64: attention_item<16>(c, P, layer, pos, h, split, aux); break;
+            default: attention_item<32>(c, P, layer, pos, h, split, aux); break;
         }
     }
 }
 
 // ── the kernel ──────────────────────────────────────────────────────────────
+// ND = ceil(Kp(dModel) / 1024), NF = ceil(Kp(dFF) / 1024).  Rows a wavefront holds per matrix
+// (sized for 256 workgroups; more rows than that simply take more than one batch):
+template <int ND, int NF>
 __global__ void __launch_bounds__(kDT) k_llama_decode(DecodeParams P) {
-    extern __shared__ __align__(16) unsigned char lds[];
-    Ctx c{P};
-    c.lds = lds;
-    c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)lds;
-    c.xs = reinterpret_cast<float *>(lds + P.slot_count * kSlotBytes);
-    c.aux = lds + P.slot_count * kSlotBytes + P.xs_bytes;
+    constexpr int NX = ND > NF ? ND : NF;
+    constexpr int B_QKV = (3 * ND + 1) / 2, B_WO = (ND + 1) / 2, B_GU = (NF + 1) / 2, B_DOWN = (ND + 1) / 2, B_LM = 4;
+    static_assert(ND * B_QKV <= kSlots && ND * B_GU * 2 <= kSlots && NF * B_DOWN <= kSlots && ND * B_LM <= kSlots, "register store too small");
+    using WQkv = Work<ND, B_QKV, false>;
+    using WWo = Work<ND, B_WO, false>;
+    using WGu = Work<ND, B_GU, true>;
+    using WDown = Work<NF, B_DOWN, false>;
+    using WLm = Work<ND, B_LM, false>;
+
+    __shared__ __align__(16) float xs[NX * 1024];
+    __shared__ __align__(16) float aux[2304];              // attention merge area: 2*NSUB + NSUB*HD floats <= 2176
+    __shared__ float red[kDW];
+    __shared__ int s_flag[2];
+    __shared__ float sv[kDW];
+    __shared__ int si[kDW];
+
+    Ctx c;
     c.wg = blockIdx.x; c.G = gridDim.x; c.tid = threadIdx.x; c.lane = c.tid & 63; c.wave = c.tid >> 6;
+    c.sync = P.sync;
     c.epoch = P.sync[SY_EPOCH];
     c.failed = false;
-    if (c.tid == 0) { *reinterpret_cast<volatile int *>(c.aux + kAuxBytes - 4) = 0; *reinterpret_cast<volatile int *>(c.aux + kAuxBytes - 8) = 0; }
-    wg_sync();
+    c.s_flag = s_flag;
+    if (c.tid == 0) { s_flag[0] = 0; s_flag[1] = 0; }
+    __syncthreads();
 
-    Pipe pipe;
-    pipe.cur = Cursor{0, 0, 0, -1};
-    pipe.issued = pipe.consumed = 0;
-    pipe.nload0 = pipe.nload1 = pipe.nload2 = pipe.nload3 = 0;
-    pipe.top_up(c);
+    Store r;                                               // the next phase's rows of this wavefront
+    WQkv::prefetch(r, P.layers[0].qkv, c.wg, c.G, c.wave, c.lane);
 
     const int pos0 = P.state[0], gen0 = P.state[2];
     int tok = P.state[1];
-    Epilogue ep;
-    const int phases = 5 * P.L + 1;                  // five per block, then the LM head
+    float nb_v = -INFINITY; int nb_i = 0x7fffffff;         // unused arg-max trackers of the block phases
     for (int step = 0; step < P.steps && !c.failed; step++) {
-        const int pos = pos0 + step;
-        const bool tok_ok = tok >= 0 && tok < P.vocab && pos < P.max_seq;
+        const int pos = pos0 + step < P.max_seq ? pos0 + step : P.max_seq - 1;
+        const bool tok_ok = tok >= 0 && tok < P.vocab;
         const float *emb_row = P.emb + (long long)(tok_ok ? tok : 0) * P.d;
-        for (int item = 0; item < phases && !c.failed; item++) {
-            const int l = item / 5, ph = item - 5 * l;
-            if (l < P.L && ph == 1) {
-                attention_phase(c, l, pos < P.max_seq ? pos : P.max_seq - 1);
-                grid_sync(c);
-                continue;
-            }
-            // what this phase multiplies, from where, and how its outputs are finished
-            const Mat *m; const float *src, *gamma = nullptr; int k; bool coherent = true, pairs = false;
-            if (l == P.L) {                          // logits = norm(x) . Wlm + blm        DecoderOnlyModel.java:58-64
-                m = &P.lm; src = P.x; k = P.d; gamma = P.gf;
-                ep = Epilogue{P.logits, P.blm, nullptr, nullptr, false, -INFINITY, 0x7fffffff};
-            } else {
-                const DecLayer &L = P.layers[l];
-                const float *xin = l == 0 ? emb_row : P.x;
-                if (ph == 0) {                       // qkv = norm1(x) . [Wq|Wk|Wv]
-                    m = &L.qkv; src = xin; k = P.d; gamma = L.g1; coherent = l != 0;
-                    ep = Epilogue{P.qkv, nullptr, nullptr, nullptr, false, -INFINITY, 0x7fffffff};
-                } else if (ph == 2) {                // x2 = x + att . Wo                  LlamaTransformerBlock.java:51
-                    m = &L.wo; src = P.att; k = P.d;
-                    ep = Epilogue{P.x2, nullptr, nullptr, xin, l != 0, -INFINITY, 0x7fffffff};
-                } else if (ph == 3) {                // ff = SiLU(gate(norm2(x2))) * up(norm2(x2))
-                    m = &L.gu; src = P.x2; k = P.d; gamma = L.g2; pairs = true;
-                    ep = Epilogue{P.ff, L.bg, L.bu, nullptr, false, -INFINITY, 0x7fffffff};
-                } else {                             // x = x2 + down(ff)                  LlamaTransformerBlock.java:52
-                    m = &L.down; src = P.ff; k = P.dff;
-                    ep = Epilogue{P.x, L.bd, nullptr, P.x2, true, -INFINITY, 0x7fffffff};
-                }
-            }
-            stage_x(c, src, coherent, k, m->kp, gamma);
-            wg_sync();
-            if (pairs) run_matrix_nc<true>(c, pipe, *m, ep);
-            else run_matrix_nc<false>(c, pipe, *m, ep);
-            if (l == P.L && c.wave == kDW - 1) {     // this workgroup's best logit
-                float bv = ep.best_v; int bi = ep.best_i;
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) {
-                    float ov = __shfl_xor(bv, off, 64);
-                    int oi = __shfl_xor(bi, off, 64);
-                    if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
-                }
-                if (c.lane == 0) { stc_f32(P.argbuf + 2 * c.wg, bv); stc_u32(reinterpret_cast<unsigned *>(P.argbuf) + 2 * c.wg + 1, (unsigned)bi); }
-            }
-            grid_sync(c);
+        for (int l = 0; l < P.L && !c.failed; l++) {
+            const DecodeLayer &L = P.layers[l];
+            const bool last = l + 1 == P.L;
+            const float *xin = l == 0 ? emb_row : P.x;
+
+            // qkv = norm1(x) . [Wq|Wk|Wv]
+            stage_x<ND>(c, xin, l != 0, P.d, L.qkv.kp, L.g1, xs, red);
+            WQkv::run(r, L.qkv, xs, Epilogue{P.qkv, nullptr, nullptr, nullptr, false}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
+            grid_arrive(c);
+            WWo::prefetch(r, L.wo, c.wg, c.G, c.wave, c.lane);          // streams in during the barrier and the attention
+            grid_wait(c);
+
+            attention_phase(c, P, l, pos, aux);
+            grid_arrive(c);
+            grid_wait(c);
+
+            // x2 = x + att . Wo                                              LlamaTransformerBlock.java:51
+            stage_x<ND>(c, P.att, true, P.d, L.wo.kp, nullptr, xs, red);
+            WWo::run(r, L.wo, xs, Epilogue{P.x2, nullptr, nullptr, xin, l != 0}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
+            grid_arrive(c);
+            WGu::prefetch(r, L.gu, c.wg, c.G, c.wave, c.lane);
+            grid_wait(c);
+
+            // ff = SiLU(gate(norm2(x2))) * up(norm2(x2))
+            stage_x<ND>(c, P.x2, true, P.d, L.gu.kp, L.g2, xs, red);
+            WGu::run(r, L.gu, xs, Epilogue{P.ff, L.bg, L.bu, nullptr, false}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
+            grid_arrive(c);
+            WDown::prefetch(r, L.down, c.wg, c.G, c.wave, c.lane);
+            grid_wait(c);
+
+            // x = x2 + down(ff)                                              LlamaTransformerBlock.java:52
+            stage_x<NF>(c, P.ff, true, P.dff, L.down.kp, nullptr, xs, red);
+            WDown::run(r, L.down, xs, Epilogue{P.x, L.bd, nullptr, P.x2, true}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
+            grid_arrive(c);
+            if (last) WLm::prefetch(r, P.lm, c.wg, c.G, c.wave, c.lane);
+            else WQkv::prefetch(r, P.layers[l + 1].qkv, c.wg, c.G, c.wave, c.lane);
+            grid_wait(c);
         }
-        // every workgroup reduces the per-workgroup winners to the same token
-        {
-            float bv = -INFINITY; int bi = 0x7fffffff;
-            if (c.tid < c.G) {
-                bv = ldc_f32(P.argbuf + 2 * c.tid);
-                bi = (int)ldc_u32(reinterpret_cast<const unsigned *>(P.argbuf) + 2 * c.tid + 1);
-            }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                float ov = __shfl_xor(bv, off, 64);
-                int oi = __shfl_xor(bi, off, 64);
-                if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
-            }
-            float *sv = reinterpret_cast<float *>(c.aux);
-            int *si = reinterpret_cast<int *>(c.aux) + kDW;
-            if (c.lane == 0) { sv[c.wave] = bv; si[c.wave] = bi; }
-            wg_sync();
-            bv = sv[0]; bi = si[0];
+        if (c.failed) break;
+        // logits = norm(x) . Wlm + blm, arg-max of this workgroup's rows       DecoderOnlyModel.java:58-64
+        float bv = -INFINITY; int bi = 0x7fffffff;
+        stage_x<ND>(c, P.x, true, P.d, P.lm.kp, P.gf, xs, red);
+        WLm::run(r, P.lm, xs, Epilogue{P.logits, P.blm, nullptr, nullptr, false}, c.wg, c.G, c.wave, c.lane, bv, bi);
+        bv = __shfl(bv, 0, 64); bi = __shfl(bi, 0, 64);    // lane 0 tracked the wavefront's rows
+        if (c.lane == 0) { sv[c.wave] = bv; si[c.wave] = bi; }
+        __syncthreads();
+        if (c.tid == 0) {
             for (int w = 1; w < kDW; w++)
                 if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
-            tok = bi;
-            wg_sync();
+            stc_f32(P.argbuf + 2 * c.wg, bv);
+            stc_u32(reinterpret_cast<unsigned *>(P.argbuf) + 2 * c.wg + 1, (unsigned)bi);
         }
+        grid_arrive(c);
+        if (step + 1 < P.steps) WQkv::prefetch(r, P.layers[0].qkv, c.wg, c.G, c.wave, c.lane);     // next token's first rows
+        grid_wait(c);
+        if (c.failed) break;
+        // every workgroup reduces the per-workgroup winners to the same token
+        bv = -INFINITY; bi = 0x7fffffff;
+        if (c.tid < c.G) {
+            bv = ldc_f32(P.argbuf + 2 * c.tid);
+            bi = (int)ldc_u32(reinterpret_cast<const unsigned *>(P.argbuf) + 2 * c.tid + 1);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            float ov = __shfl_xor(bv, off, 64);
+            int oi = __shfl_xor(bi, off, 64);
+            if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+        }
+        if (c.lane == 0) { sv[c.wave] = bv; si[c.wave] = bi; }
+        __syncthreads();
+        bv = sv[0]; bi = si[0];
+        for (int w = 1; w < kDW; w++)
+            if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+        tok = bi;
+        __syncthreads();
         if (c.wg == 0 && c.tid == 0 && gen0 + step < P.capacity) P.tokens[gen0 + step] = tok;
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // Leave x = embedding row of the token to process next, as the per-token stream does
     // (Embedding.java:28-34), so the two decode paths can be mixed within a sequence.
     if (c.wg == 0 && !c.failed) {
@@ -673,39 +563,25 @@ void llama_decode_plan(int H, int hd, int *grid, int *nsplit, int64_t *scratch_f
     if (argbuf_floats) *argbuf_floats = 2 * (int64_t)g;
 }
 
+bool llama_decode_supported(int d, int dff) {
+    int nd = (q8_padded_k(d) + 1023) / 1024, nf = (q8_padded_k(dff) + 1023) / 1024;
+    return (nd == 1 && nf == 1) || (nd <= 2 && nf <= 6);
+}
+
 // The caller has filled every pointer and dimension; this derives the launch geometry.
 void launch_llama_decode(hipStream_t s, DecodeParams &p) {
     if (p.hd != 32 && p.hd != 64 && p.hd != 128) fail("llama_decode: head dim must be 32, 64 or 128");
     if (p.H < 1 || p.H > kMaxHeads || p.H * p.hd != p.d) fail("llama_decode: bad head count");
+    if (!llama_decode_supported(p.d, p.dff)) fail("llama_decode: dModel above 2048 or dFF above 6144 is not supported");
     if (p.steps <= 0) return;
     int grid = 0, ns = 0;
     llama_decode_plan(p.H, p.hd, &grid, &ns, nullptr, nullptr);
     p.nsplit = ns;
     p.scale = (float)(1.0 / sqrt((double)p.hd));
-    int kp_max = p.lm.kp;
-    auto check = [&](const Q8Mat &m, int unit) {
-        if (m.kp > 11 * 1024) fail("llama_decode: inner dimension above 11264 is not supported");
-        if ((int64_t)(m.kp + m.kp / 8) * unit > (int64_t)kSlotBytes) fail("llama_decode: row does not fit a prefetch slot");
-        if (m.rows % unit) fail("llama_decode: odd gate/up row count");
-        if (m.kp > kp_max) kp_max = m.kp;
-    };
-    check(p.lm, 1);
-    for (int l = 0; l < p.L; l++) {
-        check(p.layers_host[l].qkv, 1); check(p.layers_host[l].wo, 1); check(p.layers_host[l].gu, 2); check(p.layers_host[l].down, 1);
-    }
-    p.xs_bytes = (unsigned)round_up((int64_t)kp_max * 4, 1024);
-    int64_t room = (int64_t)kLdsLimit - kAuxBytes - p.xs_bytes;
-    int slots = (int)(room / kSlotBytes);
-    if (slots > kMaxSlots) slots = kMaxSlots;
-    if (slots < 2) fail("llama_decode: not enough LDS for the prefetch ring");
-    p.slot_count = (unsigned)slots;
-    size_t lds = (size_t)slots * kSlotBytes + p.xs_bytes + kAuxBytes;
-    static bool attr_set = false;
-    if (!attr_set) {
-        DJ_HIP(hipFuncSetAttribute((const void *)k_llama_decode, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit));
-        attr_set = true;
-    }
-    hipLaunchKernelGGL(k_llama_decode, dim3(grid), dim3(kDT), lds, s, p);
+    p.slot_count = 0; p.xs_bytes = 0;
+    int nd = (q8_padded_k(p.d) + 1023) / 1024, nf = (q8_padded_k(p.dff) + 1023) / 1024;
+    if (nd == 1 && nf == 1) hipLaunchKernelGGL((k_llama_decode<1, 1>), dim3(grid), dim3(kDT), 0, s, p);
+    else hipLaunchKernelGGL((k_llama_decode<2, 6>), dim3(grid), dim3(kDT), 0, s, p);
 }
 
 }  // namespace dj

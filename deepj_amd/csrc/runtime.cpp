@@ -53,7 +53,6 @@ struct Runtime {
     std::unordered_map<int32_t, Graph> graphs;
     int32_t next_graph = 1;
     unsigned *attn_counters = nullptr;             // kAttnCounterHeads zeroed words: decode attention's split arrivals
-    bool allow_persistent_decode = false;          // no caller sets this: OP_LLAMA_DECODE refuses to launch
     void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
     std::vector<int64_t> decode_table_key;
 };
@@ -602,11 +601,8 @@ void exec_one(Cursor &c) {
                 T.g1 = buf(q[4], d, op, "g1"); T.g2 = buf(q[5], d, op, "g2");
                 T.bg = buf(q[6], dff, op, "bg"); T.bu = buf(q[7], dff, op, "bu"); T.bd = buf(q[8], d, op, "bd");
             }
-            // Switched off: the one run of this kernel on an MI355X ended in a GPU memory fault whose cause
-            // has not been found by reading the code; the op validates its operands and then refuses to launch.
-            if (run && steps > 0 && !g.allow_persistent_decode)
-                fail("OP_LLAMA_DECODE is disabled in this build (persistent decode kernel under investigation); "
-                     "use the per-token stream or its graph");
+            if (!llama_decode_supported((int)d, (int)dff))
+                fail("OP_LLAMA_DECODE: dModel above 2048 or dFF above 6144 is not supported by the persistent kernel");
             if (run && steps > 0) {
                 // device copy of the layer table, rebuilt only when a pointer in it changes
                 const size_t bytes = table.size() * sizeof(DecodeLayer);

@@ -196,7 +196,7 @@ class _DecoderOnlyModel:
 
     def _mode(self, use_graph, persistent) -> int:
         """0 eager per-token stream, 1 the stream as a replayed HIP graph (default), 2 the persistent
-        decode kernel (Llama only; switched off in the native library for now, so it raises)."""
+        decode kernel (Llama with dModel <= 2048 and dFF <= 6144)."""
         if persistent:
             return 2
         return 0 if use_graph is False else 1

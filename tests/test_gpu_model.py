@@ -59,8 +59,6 @@ def test_c1_greedy_64_tokens_identical_to_oracle(c1):
     assert gap > 1e-3
 
 
-@pytest.mark.skip(reason="the persistent decode kernel (OP_LLAMA_DECODE) ended its one GPU run in a memory fault whose "
-                         "cause is not yet found; the op refuses to launch until it is, and this test stays off the GPU")
 def test_c1_persistent_kernel_equals_graph_and_eager(c1):
     """The persistent decode kernel (all tokens in one launch), the replayed graph of the per-token stream
     and its eager execution produce the same ids; the persistent path is repeatable and can be entered
