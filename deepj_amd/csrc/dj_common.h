@@ -135,6 +135,7 @@ struct DecodeParams {
     int32_t *state, *tokens;
     unsigned *sync;
     float scale;
+    unsigned long long *timing;            // debug: phase time stamps of workgroup 0 (null = off)
 };
 int64_t llama_decode_sync_words();
 void llama_decode_plan(int H, int hd, int *grid, int *nsplit, int64_t *scratch_floats, int64_t *argbuf_floats);

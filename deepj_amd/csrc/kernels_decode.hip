@@ -17,6 +17,9 @@
 // and read with agent-scope (device-coherent) accesses, and a workgroup waits for its stores
 // to complete before it signals the barrier; weights, tables and KV rows of earlier positions
 // use ordinary loads.  Plain HIP throughout: no inline assembly.
+#include <cstdio>
+#include <cstdlib>
+
 #include "dj_common.h"
 
 namespace dj {
@@ -148,6 +151,15 @@ template <int NC, int B, bool PAIRS> struct Work {
         for (int o0 = ob + wave * B; o0 < oe; o0 += step) {
             // The lane's 16 activations of each 1 KiB stripe come from LDS stripe by stripe, so only
             // one stripe's worth is live in registers next to the weight batches.
+            // bias / residual of this batch's outputs: requested now, used after the reduction
+            float pb[B], pb2[B], pr[B];
+#pragma unroll
+            for (int u = 0; u < B; u++) {
+                const int o = o0 + u < oe ? o0 + u : oe - 1;
+                pb[u] = ep.bias ? ep.bias[o] : 0.0f;
+                pb2[u] = (PAIRS && ep.bias2) ? ep.bias2[o] : 0.0f;
+                pr[u] = ep.residual ? (ep.residual_coherent ? ldc_f32(ep.residual + o) : ep.residual[o]) : 0.0f;
+            }
             float acc[R];
 #pragma unroll
             for (int u = 0; u < R; u++) acc[u] = 0.0f;
@@ -176,15 +188,15 @@ template <int NC, int B, bool PAIRS> struct Work {
                         float v;
                         if (PAIRS) {
                             float gate = acc[2 * u], up = acc[2 * u + 1];
-                            if (ep.bias) gate = gate + ep.bias[o];
-                            if (ep.bias2) up = up + ep.bias2[o];
+                            if (ep.bias) gate = gate + pb[u];
+                            if (ep.bias2) up = up + pb2[u];
                             float sg = gate * d_sigmoid(gate);      // SiLU.java:20-24
                             v = sg * up;                             // SwiGLULayer.java:69
                         } else {
                             v = acc[u];
-                            if (ep.bias) v = v + ep.bias[o];
+                            if (ep.bias) v = v + pb[u];
                         }
-                        if (ep.residual) v = (ep.residual_coherent ? ldc_f32(ep.residual + o) : ep.residual[o]) + v;
+                        if (ep.residual) v = pr[u] + v;
                         stc_f32(ep.out + o, v);
                         if (better(v, o, best_v, best_i)) { best_v = v; best_i = o; }
                     }
@@ -240,24 +252,31 @@ __device__ __forceinline__ void grid_wait(Ctx &c) {
 // ── activation staging ──────────────────────────────────────────────────────
 // xs[0..kp) = optional RMSNorm of src[0..k) (RMSNorm1D.java:46-57), zero beyond k.  All 512
 // threads; NCX = ceil(kp / 1024).
+// This thread's share of a gain vector, requested ahead of the phase that uses it.
 template <int NCX>
-__device__ __forceinline__ void stage_x(const Ctx &c, const float *src, bool coherent, int k, int kp, const float *gamma,
+__device__ __forceinline__ void load_gain(float2 (&gv)[NCX], const float *gamma, int k, int tid) {
+#pragma unroll
+    for (int j = 0; j < NCX; j++) {
+        int e = (tid + kDT * j) * 2;
+        gv[j] = make_float2(0.f, 0.f);
+        if (e + 1 < k) gv[j] = *reinterpret_cast<const float2 *>(gamma + e);
+        else if (e < k) gv[j].x = gamma[e];
+    }
+}
+
+// gv = null: no RMSNorm.
+template <int NCX>
+__device__ __forceinline__ void stage_x(const Ctx &c, const float *src, bool coherent, int k, int kp, const float2 *gv,
                                         float *xs, float *red) {
-    float2 xv[NCX], gv[NCX];
+    float2 xv[NCX];
 #pragma unroll
     for (int j = 0; j < NCX; j++) {
         int e = (c.tid + kDT * j) * 2;
         xv[j] = make_float2(0.f, 0.f);
-        gv[j] = make_float2(0.f, 0.f);
-        if (e + 1 < k) {
-            xv[j] = coherent ? ldc_f2(src + e) : *reinterpret_cast<const float2 *>(src + e);
-            if (gamma) gv[j] = *reinterpret_cast<const float2 *>(gamma + e);
-        } else if (e < k) {
-            xv[j].x = coherent ? ldc_f32(src + e) : src[e];
-            if (gamma) gv[j].x = gamma[e];
-        }
+        if (e + 1 < k) xv[j] = coherent ? ldc_f2(src + e) : *reinterpret_cast<const float2 *>(src + e);
+        else if (e < k) xv[j].x = coherent ? ldc_f32(src + e) : src[e];
     }
-    if (gamma) {
+    if (gv) {
         float ss = 0.0f;
 #pragma unroll
         for (int j = 0; j < NCX; j++) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y;
@@ -313,7 +332,7 @@ __device__ __forceinline__ void attention_item(Ctx &c, const DecodeParams &P, in
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 1
+#pragma unroll 4
     for (int key = k_begin + c.wave * KPW + sub; key < k_end; key += kDW * KPW) {
         float4 kk, vv;
         if (key == pos) {
@@ -372,19 +391,24 @@ __device__ __forceinline__ void attention_item(Ctx &c, const DecodeParams &P, in
     }
     __syncthreads();
     if (c.s_flag[1] && c.tid < HD) {
+        // all record loads are issued before the first use: one memory round trip (ns <= 16)
         const float *base = P.scratch + (long long)h * ns * (HD + 4);
+        float rm[16], rl[16], ro[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float *r = base + (long long)(i < ns ? i : 0) * (HD + 4);
+            rm[i] = ldc_f32(r); rl[i] = ldc_f32(r + 1); ro[i] = ldc_f32(r + 4 + c.tid);
+        }
         float M = -INFINITY;
-#pragma unroll 1
-        for (int i = 0; i < ns; i++) M = fmaxf(M, ldc_f32(base + (long long)i * (HD + 4)));
+#pragma unroll
+        for (int i = 0; i < 16; i++) if (i < ns) M = fmaxf(M, rm[i]);
         float L = 0.0f, O = 0.0f;
-#pragma unroll 1
-        for (int i = 0; i < ns; i++) {
-            const float *r = base + (long long)i * (HD + 4);
-            float mi = ldc_f32(r);
-            if (mi != -INFINITY) {
-                float w = expf(mi - M);
-                L += ldc_f32(r + 1) * w;
-                O += ldc_f32(r + 4 + c.tid) * w;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (i < ns && rm[i] != -INFINITY) {
+                float w = expf(rm[i] - M);
+                L += rl[i] * w;
+                O += ro[i] * w;
             }
         }
         stc_f32(P.att + h * HD + c.tid, O / L);
@@ -435,11 +459,15 @@ __global__ void __launch_bounds__(kDT) k_llama_decode(DecodeParams P) {
     __syncthreads();
 
     Store r;                                               // the next phase's rows of this wavefront
+    float2 gain[ND];                                       // the next normalising phase's gain, this thread's share
+    load_gain<ND>(gain, P.layers[0].g1, P.d, c.tid);
     WQkv::prefetch(r, P.layers[0].qkv, c.wg, c.G, c.wave, c.lane);
 
     const int pos0 = P.state[0], gen0 = P.state[2];
     int tok = P.state[1];
     float nb_v = -INFINITY; int nb_i = 0x7fffffff;         // unused arg-max trackers of the block phases
+    int tix = 0;
+#define DJ_STAMP() do { if (P.timing && c.wg == 0 && c.tid == 0 && step == P.steps - 1 && l == 1 && tix < 60) P.timing[tix++] = wall_clock64(); } while (0)
     for (int step = 0; step < P.steps && !c.failed; step++) {
         const int pos = pos0 + step < P.max_seq ? pos0 + step : P.max_seq - 1;
         const bool tok_ok = tok >= 0 && tok < P.vocab;
@@ -450,42 +478,43 @@ __global__ void __launch_bounds__(kDT) k_llama_decode(DecodeParams P) {
             const float *xin = l == 0 ? emb_row : P.x;
 
             // qkv = norm1(x) . [Wq|Wk|Wv]
-            stage_x<ND>(c, xin, l != 0, P.d, L.qkv.kp, L.g1, xs, red);
-            WQkv::run(r, L.qkv, xs, Epilogue{P.qkv, nullptr, nullptr, nullptr, false}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
-            grid_arrive(c);
+            stage_x<ND>(c, xin, l != 0, P.d, L.qkv.kp, gain, xs, red); DJ_STAMP();
+            WQkv::run(r, L.qkv, xs, Epilogue{P.qkv, nullptr, nullptr, nullptr, false}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i); DJ_STAMP();
+            grid_arrive(c); DJ_STAMP();
             WWo::prefetch(r, L.wo, c.wg, c.G, c.wave, c.lane);          // streams in during the barrier and the attention
-            grid_wait(c);
+            load_gain<ND>(gain, L.g2, P.d, c.tid);
+            grid_wait(c); DJ_STAMP();
 
-            attention_phase(c, P, l, pos, aux);
-            grid_arrive(c);
-            grid_wait(c);
+            attention_phase(c, P, l, pos, aux); DJ_STAMP();
+            grid_arrive(c); DJ_STAMP();
+            grid_wait(c); DJ_STAMP();
 
             // x2 = x + att . Wo                                              LlamaTransformerBlock.java:51
-            stage_x<ND>(c, P.att, true, P.d, L.wo.kp, nullptr, xs, red);
-            WWo::run(r, L.wo, xs, Epilogue{P.x2, nullptr, nullptr, xin, l != 0}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
-            grid_arrive(c);
+            stage_x<ND>(c, P.att, true, P.d, L.wo.kp, nullptr, xs, red); DJ_STAMP();
+            WWo::run(r, L.wo, xs, Epilogue{P.x2, nullptr, nullptr, xin, l != 0}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i); DJ_STAMP();
+            grid_arrive(c); DJ_STAMP();
             WGu::prefetch(r, L.gu, c.wg, c.G, c.wave, c.lane);
-            grid_wait(c);
+            grid_wait(c); DJ_STAMP();
 
             // ff = SiLU(gate(norm2(x2))) * up(norm2(x2))
-            stage_x<ND>(c, P.x2, true, P.d, L.gu.kp, L.g2, xs, red);
-            WGu::run(r, L.gu, xs, Epilogue{P.ff, L.bg, L.bu, nullptr, false}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
-            grid_arrive(c);
+            stage_x<ND>(c, P.x2, true, P.d, L.gu.kp, gain, xs, red); DJ_STAMP();
+            WGu::run(r, L.gu, xs, Epilogue{P.ff, L.bg, L.bu, nullptr, false}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i); DJ_STAMP();
+            grid_arrive(c); DJ_STAMP();
             WDown::prefetch(r, L.down, c.wg, c.G, c.wave, c.lane);
-            grid_wait(c);
+            grid_wait(c); DJ_STAMP();
 
             // x = x2 + down(ff)                                              LlamaTransformerBlock.java:52
-            stage_x<NF>(c, P.ff, true, P.dff, L.down.kp, nullptr, xs, red);
-            WDown::run(r, L.down, xs, Epilogue{P.x, L.bd, nullptr, P.x2, true}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i);
-            grid_arrive(c);
-            if (last) WLm::prefetch(r, P.lm, c.wg, c.G, c.wave, c.lane);
-            else WQkv::prefetch(r, P.layers[l + 1].qkv, c.wg, c.G, c.wave, c.lane);
-            grid_wait(c);
+            stage_x<NF>(c, P.ff, true, P.dff, L.down.kp, nullptr, xs, red); DJ_STAMP();
+            WDown::run(r, L.down, xs, Epilogue{P.x, L.bd, nullptr, P.x2, true}, c.wg, c.G, c.wave, c.lane, nb_v, nb_i); DJ_STAMP();
+            grid_arrive(c); DJ_STAMP();
+            if (last) { WLm::prefetch(r, P.lm, c.wg, c.G, c.wave, c.lane); load_gain<ND>(gain, P.gf, P.d, c.tid); }
+            else { WQkv::prefetch(r, P.layers[l + 1].qkv, c.wg, c.G, c.wave, c.lane); load_gain<ND>(gain, P.layers[l + 1].g1, P.d, c.tid); }
+            grid_wait(c); DJ_STAMP();
         }
         if (c.failed) break;
         // logits = norm(x) . Wlm + blm, arg-max of this workgroup's rows       DecoderOnlyModel.java:58-64
         float bv = -INFINITY; int bi = 0x7fffffff;
-        stage_x<ND>(c, P.x, true, P.d, P.lm.kp, P.gf, xs, red);
+        stage_x<ND>(c, P.x, true, P.d, P.lm.kp, gain, xs, red);
         WLm::run(r, P.lm, xs, Epilogue{P.logits, P.blm, nullptr, nullptr, false}, c.wg, c.G, c.wave, c.lane, bv, bi);
         bv = __shfl(bv, 0, 64); bi = __shfl(bi, 0, 64);    // lane 0 tracked the wavefront's rows
         if (c.lane == 0) { sv[c.wave] = bv; si[c.wave] = bi; }
@@ -497,7 +526,10 @@ __global__ void __launch_bounds__(kDT) k_llama_decode(DecodeParams P) {
             stc_u32(reinterpret_cast<unsigned *>(P.argbuf) + 2 * c.wg + 1, (unsigned)bi);
         }
         grid_arrive(c);
-        if (step + 1 < P.steps) WQkv::prefetch(r, P.layers[0].qkv, c.wg, c.G, c.wave, c.lane);     // next token's first rows
+        if (step + 1 < P.steps) {                          // next token's first rows
+            WQkv::prefetch(r, P.layers[0].qkv, c.wg, c.G, c.wave, c.lane);
+            load_gain<ND>(gain, P.layers[0].g1, P.d, c.tid);
+        }
         grid_wait(c);
         if (c.failed) break;
         // every workgroup reduces the per-workgroup winners to the same token
@@ -579,9 +611,22 @@ void launch_llama_decode(hipStream_t s, DecodeParams &p) {
     p.nsplit = ns;
     p.scale = (float)(1.0 / sqrt((double)p.hd));
     p.slot_count = 0; p.xs_bytes = 0;
+    static unsigned long long *timing = nullptr;
+    const bool want_timing = getenv("DJ_DECODE_TIMING") != nullptr;
+    if (want_timing && !timing) { DJ_HIP(hipMalloc((void **)&timing, 64 * 8)); }
+    if (want_timing) DJ_HIP(hipMemsetAsync(timing, 0, 64 * 8, s));
+    p.timing = want_timing ? timing : nullptr;
     int nd = (q8_padded_k(p.d) + 1023) / 1024, nf = (q8_padded_k(p.dff) + 1023) / 1024;
     if (nd == 1 && nf == 1) hipLaunchKernelGGL((k_llama_decode<1, 1>), dim3(grid), dim3(kDT), 0, s, p);
     else hipLaunchKernelGGL((k_llama_decode<2, 6>), dim3(grid), dim3(kDT), 0, s, p);
+    if (want_timing) {
+        unsigned long long h[64];
+        DJ_HIP(hipStreamSynchronize(s));
+        DJ_HIP(hipMemcpy(h, timing, sizeof(h), hipMemcpyDeviceToHost));
+        fprintf(stderr, "decode phase stamps (us since first):");
+        for (int i = 0; i < 64 && h[i]; i++) fprintf(stderr, " %.2f", (double)(h[i] - h[0]) / 100.0);
+        fprintf(stderr, "\n");
+    }
 }
 
 }  // namespace dj
