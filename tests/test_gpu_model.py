@@ -219,3 +219,29 @@ def test_deepseek_config_validation():
         DeepSeekModel(DeepSeekConfig(256, 16, 128, 4, 1, 64, 0, 8), None)
     with pytest.raises(ValueError, match="kvRank must be > 0"):
         DeepSeekModel(DeepSeekConfig(256, 16, 128, 4, 1, 64, 8, 0), None)
+
+
+def test_llama_one_block_at_7b_width_matches_oracle():
+    """One block at the baseline's prefill configuration width (dModel 4096, 32 heads of 128, SwiGLU hidden
+    11008: inner dimensions that take the 4- and 11-stripe matvec paths and the K = 11008 GEMM), small
+    vocabulary, oracle run live: prompt logits through the GEMM path, then decode rows through the matvec
+    path against the full-context forward."""
+    cfg = LlamaConfig(vocabSize=512, maxSeqLen=128, dModel=4096, nHeads=32, nLayers=1, dFF=11008)
+    ref.set_threads(ref.default_threads())
+    gpu = LlamaModel(cfg, 42)
+    cpu = oracle_model(cfg, 42)
+    try:
+        ids = ref.JavaRandom(4).ints(72, 512)
+        exp = cpu.forward(ids)
+        got = gpu.forward(ids[:64])
+        err = float(np.max(np.abs(got - exp[:64])))
+        assert err <= 1e-3, f"prefill logits max-abs error {err}"
+        gpu.reset()
+        gpu.prefill(ids[:64], choose_next=False)
+        for t in range(64, 72):
+            gpu.step(int(ids[t]))
+            assert float(np.max(np.abs(gpu.lastLogits() - exp[t]))) <= 1e-3, t
+    finally:
+        gpu.close()
+        cpu.close()
+        ref.set_threads(1)

@@ -91,7 +91,7 @@ def linear_case(dev, m, k, n, *, norm=False, bias=False, residual=False, seed=0)
     return exp, dev.download(ob, (m, n))
 
 
-@pytest.mark.parametrize("k,n", [(2048, 2048), (2048, 5632), (5632, 2048), (4096, 1100), (11008, 512),
+@pytest.mark.parametrize("k,n", [(2048, 2048), (2048, 5632), (5632, 2048), (4096, 1100), (11008, 512), (4096, 11008),
                                  (688, 256), (256, 688), (32, 1), (1024, 5)])
 def test_q8_matvec_matches_oracle(dev, k, n):
     exp, got = linear_case(dev, 1, k, n)
@@ -128,7 +128,8 @@ def test_q8_swiglu_gate_up(dev, m):
     assert_close(exp, dev.download(ob, (m, n)), atol=2e-6, rtol=1e-4, what=f"swiglu m={m}")
 
 
-@pytest.mark.parametrize("m,k,n", [(64, 2048, 512), (512, 2048, 256), (64, 688, 256), (7, 96, 33), (130, 5632, 128)])
+@pytest.mark.parametrize("m,k,n", [(64, 2048, 512), (512, 2048, 256), (64, 688, 256), (7, 96, 33), (130, 5632, 128),
+                                   (64, 4096, 344), (96, 11008, 128)])
 def test_q8_gemm_matches_oracle(dev, m, k, n):
     exp, got = linear_case(dev, m, k, n, norm=True, bias=True, residual=True, seed=30)
     scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
