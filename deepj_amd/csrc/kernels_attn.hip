@@ -200,30 +200,50 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int key = k_begin + wave * KPW + sub; key < k_end; key += kWaves * KPW) {
-        float4 kk, vv;
-        if (FUSED && key == pos) {                          // the new token: rotate, use, append
-            const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
-            kk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
-                             k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
-            vv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
-            *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = kk;
-            *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = vv;
-        } else {
-            kk = *reinterpret_cast<const float4 *>(kb + (int64_t)key * a.tok_stride);
-            vv = *reinterpret_cast<const float4 *>(vb + (int64_t)key * a.tok_stride);
-        }
-        float s = qv.x * kk.x + qv.y * kk.y + qv.z * kk.z + qv.w * kk.w;
+    // Four keys per lane group per round: their rows are requested together (clamped, never under a
+    // branch), so a split of up to 4 * 64 / LPK * 4 keys costs one memory round trip.  The new token's
+    // row is not in memory yet: it is rotated in registers, used, and appended.
+    constexpr int U = 4;
+    constexpr int STRIDE = kWaves * KPW;
+    float4 nk = make_float4(0.f, 0.f, 0.f, 0.f), nv = nk;
+    if (FUSED) {
+        const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
+        nk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
+                         k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
+        nv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
+    }
+    for (int base = k_begin + wave * KPW + sub; base < k_end; base += U * STRIDE) {
+        float4 kk[U], vv[U];
 #pragma unroll
-        for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-        s *= a.scale;
-        float mn = fmaxf(m, s);
-        float corr = expf(m - mn);
-        float p = expf(s - mn);
-        l = l * corr + p;
-        o.x = o.x * corr + p * vv.x; o.y = o.y * corr + p * vv.y;
-        o.z = o.z * corr + p * vv.z; o.w = o.w * corr + p * vv.w;
-        m = mn;
+        for (int u = 0; u < U; u++) {
+            int key = base + u * STRIDE;
+            int row = (key < k_end && !(FUSED && key == pos)) ? key : k_begin;     // any row of the cache is readable
+            kk[u] = *reinterpret_cast<const float4 *>(kb + (int64_t)row * a.tok_stride);
+            vv[u] = *reinterpret_cast<const float4 *>(vb + (int64_t)row * a.tok_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int key = base + u * STRIDE;
+            bool valid = key < k_end;                       // uniform over the LPK lanes of a key
+            if (FUSED && valid && key == pos) {
+                kk[u] = nk; vv[u] = nv;
+                *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = nk;
+                *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = nv;
+            }
+            float s = qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w;
+#pragma unroll
+            for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+            if (valid) {
+                s *= a.scale;
+                float mn = fmaxf(m, s);
+                float corr = expf(m - mn);
+                float p = expf(s - mn);
+                l = l * corr + p;
+                o.x = o.x * corr + p * vv[u].x; o.y = o.y * corr + p * vv[u].y;
+                o.z = o.z * corr + p * vv[u].z; o.w = o.w * corr + p * vv[u].w;
+                m = mn;
+            }
+        }
     }
     const int slot = wave * KPW + sub;
     if (dl == 0) { s_m[slot] = m; s_l[slot] = l; }
