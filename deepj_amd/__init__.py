@@ -8,6 +8,7 @@ from .compute_graph import ComputeGraph, GpuBuffer
 from .hip_backend import HipBackend, HipGpuRuntime
 from .tensor import Tensor
 from .models import DeepSeekConfig, DeepSeekModel, JavaRandom, LlamaConfig, LlamaModel, TextGenerator
+from .persistence import ModelSerializer, parameter_names, parameter_shapes
 
-__all__ = ["opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor",
+__all__ = ["ModelSerializer", "parameter_names", "parameter_shapes", "opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor",
            "LlamaConfig", "LlamaModel", "DeepSeekConfig", "DeepSeekModel", "TextGenerator", "JavaRandom"]

@@ -245,3 +245,21 @@ def test_llama_one_block_at_7b_width_matches_oracle():
         gpu.close()
         cpu.close()
         ref.set_threads(1)
+
+
+def test_checkpoint_in_the_reference_format_loads_into_the_runner(tmp_path):
+    """A checkpoint written in ModelSerializer's format from the oracle's seeded parameters, loaded through
+    ModelSerializer.load, gives the same logits as the model initialised from the seed."""
+    from deepj_amd import ModelSerializer, parameter_names
+    cfg = LlamaConfig(vocabSize=64, maxSeqLen=32, dModel=64, nHeads=2, nLayers=2, dFF=96)
+    cpu = ref.Model(vocab=64, max_seq=32, d=64, heads=2, layers=2, dff=96, seed=5)
+    assert parameter_names(cfg) == cpu.weight_names()
+    path = tmp_path / "llama.bin"
+    ModelSerializer.save([cpu.weight(n) for n in cpu.weight_names()], path)
+    a, b = LlamaModel(cfg, 5), LlamaModel(cfg, None)
+    try:
+        ModelSerializer.load(b, path)
+        ids = [3, 9, 27, 1, 60]
+        assert np.array_equal(a.forward(ids), b.forward(ids))
+    finally:
+        a.close(); b.close(); cpu.close()
