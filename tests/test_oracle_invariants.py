@@ -233,7 +233,7 @@ TINY = dict(vocab=256, max_seq=16, d=32, heads=4, layers=2, dff=88)   # LlamaMod
 
 def test_llama_init_order_and_forward_matches_layers():
     m = ref.Model(seed=42, **TINY)
-    # §RNG wiring (LlamaModel.java:27-42): embedding and layer-0 Wq start with the same Gaussians
+    # RNG wiring (LlamaModel.java:27-42): embedding and layer-0 Wq start with the same Gaussians
     assert np.array_equal(m.weight("emb").reshape(-1)[:32 * 32], m.weight("L0.wq").reshape(-1))
     r = ref.JavaRandom(42)
     for name, shape in [("L0.wq", (32, 32)), ("L0.wk", (32, 32)), ("L0.wv", (32, 32)), ("L0.wo", (32, 32)),
