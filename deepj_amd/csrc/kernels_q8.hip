@@ -131,7 +131,21 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 template <int NC, int R> struct RowBatch {
     int4 w[R][NC];
     float sc[R][NC];
+    float eb[R], eb2[R], er[R];       // bias, second bias and residual of the batch's outputs (index = output)
 };
+
+// The epilogue operands of outputs o0 .. o0+B-1 are requested together with the weight rows, so the
+// finished sums never wait for a bias or residual that is still in memory.
+template <int NC, int R, int B, bool SWIGLU>
+__device__ __forceinline__ void load_epilogue(RowBatch<NC, R> &b, const MatvecArgs &p, int o0) {
+#pragma unroll
+    for (int u = 0; u < B; u++) {
+        int o = o0 + u < p.n_out ? o0 + u : p.n_out - 1;
+        b.eb[u] = p.bias ? p.bias[o] : 0.0f;
+        b.eb2[u] = (SWIGLU && p.bias2) ? p.bias2[o] : 0.0f;
+        b.er[u] = p.residual ? p.residual[o] : 0.0f;
+    }
+}
 
 // Loads are unconditional: rows past the wave's range are clamped to its last row and
 // chunks past Kp to chunk 0 (their activations are zero), so no load sits under a branch.
@@ -155,7 +169,7 @@ __device__ __forceinline__ void load_batch(RowBatch<NC, R> &b, const MatvecArgs 
 
 template <int NC, int B, bool SWIGLU>
 __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 : 1)> &b, const float (&xr)[NC][16],
-                                             const MatvecArgs &p, int o0, int o_end, int lane) {
+                                             const MatvecArgs &p, int o0, int o_end, int lane, float rms) {
     constexpr int R = B * (SWIGLU ? 2 : 1);
     float acc[R];
 #pragma unroll
@@ -163,7 +177,7 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
         float a = 0.0f;
 #pragma unroll
         for (int c = 0; c < NC; c++) a = fmaf(dot16(b.w[u][c], xr[c]), b.sc[u][c], a);
-        acc[u] = wave_sum_dpp(a);
+        acc[u] = wave_sum_dpp(a) / rms;        // rms = 1 unless the RMSNorm scale was deferred to here
     }
     if (lane == 0) {
 #pragma unroll
@@ -173,15 +187,15 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
                 float v;
                 if constexpr (SWIGLU) {
                     float gate = acc[2 * u], up = acc[2 * u + 1];
-                    if (p.bias) gate = gate + p.bias[o];
-                    if (p.bias2) up = up + p.bias2[o];
+                    if (p.bias) gate = gate + b.eb[u];
+                    if (p.bias2) up = up + b.eb2[u];
                     float sg = gate * d_sigmoid(gate);     // SiLU.java:20-24
                     v = sg * up;                            // SwiGLULayer.java:69
                 } else {
                     v = acc[u];
-                    if (p.bias) v = v + p.bias[o];
+                    if (p.bias) v = v + b.eb[u];
                 }
-                if (p.residual) v = p.residual[o] + v;
+                if (p.residual) v = b.er[u] + v;
                 p.out[o] = v;
             }
         }
@@ -215,6 +229,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     const int o_step = wave_count * B;
 
     RowBatch<NC, R> ba, bb;
+    bool deferred_norm = false;
     const bool vec = (p.k & 3) == 0;              // kernel-uniform
     float4 xv[NC], gv[NC];
     if (vec) {
@@ -228,25 +243,26 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             gv[j] = (ok && p.gamma) ? *reinterpret_cast<const float4 *>(p.gamma + e) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
-    if (has_work) load_batch<NC, R>(ba, p, o_begin * RPO, row_last, lane, groups);
+    if (has_work) { load_batch<NC, R>(ba, p, o_begin * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(ba, p, o_begin); }
 
     // Stage the activation row through LDS (zero beyond K so padded weights meet zeros).
     // All global loads of the prologue - x and, for the RMSNorm prologue, gamma - were
     // issued together, so it costs one memory round trip, not one per element.
     if (vec) {
-        if (p.gamma) {                            // RMSNorm prologue, fp32 like the reference
+        if (p.gamma) {
+            // RMSNorm prologue (RMSNorm1D.java:46-57).  W.(g * x / rms) = (W.(g * x)) / rms: the staged row is
+            // g * x, which needs no reduction, and the division by rms is applied to the finished sums, so the
+            // sum of squares is reduced while the weight rows are still streaming in.
             float ss = 0.0f;
 #pragma unroll
             for (int j = 0; j < NC; j++) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
             ss = wave_sum_dpp(ss);
             if (lane == 0) red[wave] = ss;
-            __syncthreads();
-            float tot = red[0] + red[1] + red[2] + red[3];
-            float rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
+            deferred_norm = true;
 #pragma unroll
             for (int j = 0; j < NC; j++) {
-                xv[j].x = (xv[j].x / rms) * gv[j].x; xv[j].y = (xv[j].y / rms) * gv[j].y;
-                xv[j].z = (xv[j].z / rms) * gv[j].z; xv[j].w = (xv[j].w / rms) * gv[j].w;
+                xv[j].x = xv[j].x * gv[j].x; xv[j].y = xv[j].y * gv[j].y;
+                xv[j].z = xv[j].z * gv[j].z; xv[j].w = xv[j].w * gv[j].w;
             }
         }
 #pragma unroll
@@ -272,6 +288,11 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     }
     __syncthreads();
     if (!has_work) return;
+    float rms = 1.0f;
+    if (deferred_norm) {
+        float tot = red[0] + red[1] + red[2] + red[3];
+        rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
+    }
 
     // this lane's activation slice: 16 consecutive k of each 1 KiB chunk
     float xr[NC][16];
@@ -287,18 +308,16 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     }
 
     for (int o0 = o_begin; o0 < o_end; o0 += 2 * o_step) {
-        if (o0 + o_step < o_end) load_batch<NC, R>(bb, p, (o0 + o_step) * RPO, row_last, lane, groups);
-        finish_batch<NC, B, SWIGLU>(ba, xr, p, o0, o_end, lane);
+        if (o0 + o_step < o_end) { load_batch<NC, R>(bb, p, (o0 + o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(bb, p, o0 + o_step); }
+        finish_batch<NC, B, SWIGLU>(ba, xr, p, o0, o_end, lane, rms);
         if (o0 + o_step >= o_end) break;
-        if (o0 + 2 * o_step < o_end) load_batch<NC, R>(ba, p, (o0 + 2 * o_step) * RPO, row_last, lane, groups);
-        finish_batch<NC, B, SWIGLU>(bb, xr, p, o0 + o_step, o_end, lane);
+        if (o0 + 2 * o_step < o_end) { load_batch<NC, R>(ba, p, (o0 + 2 * o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(ba, p, o0 + 2 * o_step); }
+        finish_batch<NC, B, SWIGLU>(bb, xr, p, o0 + o_step, o_end, lane, rms);
     }
 }
 
-inline int mv_grid_cap() {
-    static int cap = [] { const char *e = getenv("DJ_MV_GRID"); return e ? atoi(e) : 768; }();
-    return cap;
-}
+constexpr int kMvGridCap = 768;          // three workgroups per CU
+inline int mv_grid_cap() { return kMvGridCap; }
 
 template <int NC, int B, bool SW>
 void launch_mv(hipStream_t s, const MatvecArgs &a) {
@@ -316,10 +335,7 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
 // row gets its own wavefront, so the whole matrix is requested at once and the serial work
 // after the data arrives is one row.  Large matrices want deeper batches (about eight 128-bit
 // loads per lane in flight per buffer) so ~3000 resident wavefronts keep the HBM queues full.
-inline int mv_target_waves() {
-    static int t = [] { const char *e = getenv("DJ_MV_WAVES"); return e ? atoi(e) : 3072; }();
-    return t;
-}
+inline int mv_target_waves() { return 3072; }
 
 template <int NC>
 void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu) {
