@@ -263,3 +263,39 @@ def test_checkpoint_in_the_reference_format_loads_into_the_runner(tmp_path):
         assert np.array_equal(a.forward(ids), b.forward(ids))
     finally:
         a.close(); b.close(); cpu.close()
+
+
+def test_edge_shapes_single_head_odd_vocab_ragged_dff():
+    """Shapes off the beaten path: one head of 32, vocabulary not a multiple of 4, SwiGLU hidden size that is
+    neither a multiple of 32 (padded Q8 rows) nor of 4 (scalar activation staging), a one-token prompt."""
+    cfg = LlamaConfig(vocabSize=251, maxSeqLen=24, dModel=32, nHeads=1, nLayers=2, dFF=50)
+    gpu = LlamaModel(cfg, 9)
+    cpu = oracle_model(cfg, 9)
+    try:
+        ids = ref.JavaRandom(2).ints(9, 251)
+        assert float(np.max(np.abs(gpu.forward(ids) - cpu.forward(ids)))) <= 1e-3
+        one = [int(ids[0])]
+        assert float(np.max(np.abs(gpu.forward(one) - cpu.forward(one)))) <= 1e-3
+        exp = cpu.generate(one, 12, top_k=1, use_cache=True)
+        assert np.array_equal(TextGenerator.generate(gpu, one, 12, top_k=1), exp)
+        assert np.array_equal(TextGenerator.generate(gpu, one, 12, top_k=1, use_graph=False), exp)
+        assert np.array_equal(TextGenerator.generate(gpu, one, 12, top_k=1, persistent=True), exp)
+    finally:
+        gpu.close(); cpu.close()
+
+
+def test_cache_filled_to_the_last_position_and_not_beyond(c1):
+    """Decoding up to position maxSeqLen - 1 works and matches the oracle; one more step is refused on the host
+    before anything is launched (the cached driver has no sliding window)."""
+    gpu, cpu = c1
+    prompt = ref.JavaRandom(13).ints(200, 256)
+    new = 256 - 200 + 1                      # the last generated token is chosen at position 255 and never fed back
+    exp = cpu.generate(prompt, new, top_k=1, use_cache=False)      # the literal full-context path; no window slides yet
+    got = TextGenerator.generate(gpu, prompt, new, top_k=1)
+    assert np.array_equal(got, exp)
+    with pytest.raises(ValueError, match="exceeds maxSeqLen"):
+        gpu.decode(1)
+    with pytest.raises(ValueError, match="exceeds maxSeqLen"):
+        gpu.decode(1, persistent=True)
+    with pytest.raises(ValueError, match="exceeds maxSeqLen"):
+        gpu.step(3)
