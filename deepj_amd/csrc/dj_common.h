@@ -104,7 +104,8 @@ void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *
                           const int32_t *state, const float *cos_t, const float *sin_t, int S, int H, int hd,
                           int max_seq);
 void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *state, const float *cos_t,
-                      const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row);
+                      const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row, int row_stride,
+                      int live_extra);
 void launch_attention(hipStream_t s, const AttnArgs &a);
 void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *out,
                         const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,

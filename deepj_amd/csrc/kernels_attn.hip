@@ -63,9 +63,13 @@ __global__ void __launch_bounds__(kThreads) k_rope_rows(const float *x, float *o
                                                         const int32_t *__restrict__ state,
                                                         const float *__restrict__ cos_t,
                                                         const float *__restrict__ sin_t, int rows, int H, int hd,
-                                                        int max_seq, int pos_from_row) {
-    const int half = hd >> 1, d = H * hd;
+                                                        int max_seq, int pos_from_row, int row_stride, int live_extra) {
+    const int half = hd >> 1, d = row_stride;
     const int pos0 = pos_from_row ? 0 : state[0];
+    if (live_extra >= 0) {                        // only the rows a growing cache holds so far
+        int live = state[0] + live_extra;
+        rows = rows < live ? rows : live;
+    }
     int64_t total = (int64_t)rows * H * half;
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
@@ -329,13 +333,14 @@ void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *
 }
 
 void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *state, const float *cos_t,
-                      const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row) {
+                      const float *sin_t, int rows, int H, int hd, int max_seq, int pos_from_row, int row_stride,
+                      int live_extra) {
     int64_t total = (int64_t)rows * H * (hd / 2);
     if (total <= 0) return;
     int64_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(k_rope_rows, dim3((int)blocks), dim3(kThreads), 0, s, x, out, state, cos_t, sin_t, rows, H, hd,
-                       max_seq, pos_from_row);
+                       max_seq, pos_from_row, row_stride > 0 ? row_stride : H * hd, live_extra);
 }
 
 // S = 1 uses the split kernels (scratch: attn_decode_scratch_floats); S > 1 needs no scratch.

@@ -153,8 +153,9 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
         else if (c.kind == 1 && w == "wdq") { expect_shape(name, rows, cols, d, c.q_rank); quantize_into(r, L.wdq, data, d, c.q_rank, 0, 1, c.q_rank); }
         else if (c.kind == 1 && w == "wuq") { expect_shape(name, rows, cols, c.q_rank, d); quantize_into(r, L.wuq, data, c.q_rank, d, 0, 1, d); }
         else if (c.kind == 1 && w == "wdkv") { expect_shape(name, rows, cols, d, c.kv_rank); quantize_into(r, L.wdkv, data, d, c.kv_rank, 0, 1, c.kv_rank); }
-        else if (c.kind == 1 && w == "wuk") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuk, data, c.kv_rank, d, 0, 1, d); }
-        else if (c.kind == 1 && w == "wuv") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuv, data, c.kv_rank, d, 0, 1, d); }
+        // Wuk and Wuv share one Q8 buffer (K rows first, then V rows): one GEMM re-expands both from the latent rows
+        else if (c.kind == 1 && w == "wuk") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuk, data, c.kv_rank, d, 0, 1, 2 * d); }
+        else if (c.kind == 1 && w == "wuv") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuk, data, c.kv_rank, d, d, 1, 2 * d); }
         else throw Error("unknown weight " + name);
     } else throw Error("unknown weight " + name);
     r.have[name] = true;
@@ -262,8 +263,7 @@ void finalize(Runner &r) {
         // position are re-expanded from them - and K re-rotated - for each layer of each step,
         // into these two scratch tensors (token-major [maxSeq x d]).
         r.latent = r.alloc((int64_t)c.layers * c.max_seq * c.kv_rank);
-        r.kc = r.alloc(per_layer);
-        r.vc = r.alloc(per_layer);
+        r.kc = r.alloc(2 * per_layer);           // row t = [K_t | V_t]
     }
     r.state = r.alloc(4);
     r.tok = r.alloc(4);
@@ -316,11 +316,10 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
         q8_linear(s, a.cq, L.wuq, a.qkv, S, qr, d, 0);                               // Q  = cQ.Wuq
         q8_linear(s, a.x, L.wdkv, a.ckv, S, d, kvr, DJ_LIN_RMSNORM, L.g1);          // cKV = norm1(x).Wdkv
         emit(s, DJ_OP_APPEND_ROWS, a.ckv, r.latent, r.state, S, kvr, c.max_seq, lat_off);
-        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wuk, r.kc, c.max_seq, kvr, d, r.state, S, lat_off);   // K = cKV.Wuk, all rows
-        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wuv, r.vc, c.max_seq, kvr, d, r.state, S, lat_off);   // V = cKV.Wuv
-        emit(s, DJ_OP_ROPE_ROWS, r.kc, r.kc, r.state, r.cos_t, r.sin_t, c.max_seq, H, hd, c.max_seq, 1);  // row = position
-        emit(s, DJ_OP_ROPE_ROWS, a.qkv, a.q, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, 0);
-        emit(s, DJ_OP_ATTENTION_KV, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0);
+        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wuk, r.kc, c.max_seq, kvr, 2 * d, r.state, S, lat_off);   // [K | V] = cKV.[Wuk | Wuv], all rows
+        emit(s, DJ_OP_ROPE_ROWS, r.kc, r.kc, r.state, r.cos_t, r.sin_t, c.max_seq, H, hd, c.max_seq, 1, 2 * d, S);  // K part, row = position
+        emit(s, DJ_OP_ROPE_ROWS, a.qkv, a.q, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, 0, 0, -1);
+        emit(s, DJ_OP_ATTENTION_KV, a.q, r.kc, r.kc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0, 2 * d, d);
     }
     q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
     // x = x2 + down(SiLU(gate(norm2(x2))) * up(norm2(x2)))                  LlamaTransformerBlock.java:52

@@ -184,8 +184,8 @@ int stride_of(int op) {
         case DJ_OP_DECODE_ADVANCE: return 6;
         case DJ_OP_COPY: return 6;
         case DJ_OP_FILL: return 4;
-        case DJ_OP_ROPE_ROWS: return 11;
-        case DJ_OP_ATTENTION_KV: return 12;
+        case DJ_OP_ROPE_ROWS: return 13;
+        case DJ_OP_ATTENTION_KV: return 14;
         case DJ_OP_DECODE_NEXT: return 10;
         case DJ_OP_ATTN_DECODE: return 13;
         case DJ_OP_APPEND_ROWS: return 8;
@@ -438,22 +438,24 @@ void exec_one(Cursor &c) {
             break;
         }
         case DJ_OP_ROPE_ROWS: {
-            // [op, x, out, state, cos, sin, rows, H, hd, maxSeq, posFromRow]
-            int64_t rows = w[6], H = w[7], hd = w[8], max_seq = w[9];
+            // [op, x, out, state, cos, sin, rows, H, hd, maxSeq, posFromRow, rowStride, liveExtra]
+            int64_t rows = w[6], H = w[7], hd = w[8], max_seq = w[9], stride = w[11], live_extra = w[12];
             if (rows <= 0 || H <= 0 || hd <= 0 || (hd & 1) || max_seq <= 0) fail("OP_ROPE_ROWS: bad shape");
             if (w[10] && rows > max_seq) fail("OP_ROPE_ROWS: more rows than RoPE table positions");
-            const float *x = buf(w[1], rows * H * hd, op, "x");
-            float *o = buf(w[2], rows * H * hd, op, "out");
+            if (stride == 0) stride = H * hd;
+            if (stride < H * hd || (stride & 1) || live_extra < -1) fail("OP_ROPE_ROWS: bad row stride or live-row count");
+            const float *x = buf(w[1], (rows - 1) * stride + H * hd, op, "x");
+            float *o = buf(w[2], (rows - 1) * stride + H * hd, op, "out");
             const float *st = buf(w[3], 4, op, "state");
             const float *ct = buf(w[4], max_seq * (hd / 2), op, "cos"), *sn = buf(w[5], max_seq * (hd / 2), op, "sin");
             if (run)
                 launch_rope_rows(s, x, o, reinterpret_cast<const int32_t *>(st), ct, sn, (int)rows, (int)H, (int)hd,
-                                 (int)max_seq, w[10]);
+                                 (int)max_seq, w[10], (int)stride, (int)live_extra);
             break;
         }
         case DJ_OP_ATTENTION: case DJ_OP_ATTENTION_KV: {
             // ATTENTION    [op, q, kCache, vCache, out, state, scratch, S, H, hd, maxSeq, layer]  head-major cache
-            // ATTENTION_KV [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0]  k,v token-major [maxSeq x H*hd]
+            // ATTENTION_KV [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0, tokStride, vOff]  k,v token-major rows
             int64_t S = w[7], H = w[8], hd = w[9], max_seq = w[10], layer = w[11];
             if (S <= 0 || H <= 0 || max_seq <= 0 || layer < 0) fail(std::string(op_name(op)) + ": bad shape");
             if (hd != 32 && hd != 64 && hd != 128) fail(std::string(op_name(op)) + ": head dim must be 32, 64 or 128");
@@ -462,10 +464,17 @@ void exec_one(Cursor &c) {
             a.q = buf(w[1], S * d, op, "q");
             bool cache = op == DJ_OP_ATTENTION;
             if (!cache && layer != 0) fail("OP_ATTENTION_KV: layer must be 0");
-            const float *kc = buf(w[2], (layer + 1) * per_layer, op, "k");
-            const float *vc = buf(w[3], (layer + 1) * per_layer, op, "v");
+            int64_t tok = d, voff = 0;
+            if (!cache) {
+                tok = w[12] == 0 ? d : w[12];
+                voff = w[13];
+                if (tok < d || (tok & 3) || voff < 0 || (voff & 3)) fail("OP_ATTENTION_KV: bad token stride or value offset");
+            }
+            const float *kc = cache ? buf(w[2], (layer + 1) * per_layer, op, "k") : buf(w[2], (max_seq - 1) * tok + d, op, "k");
+            const float *vc = cache ? buf(w[3], (layer + 1) * per_layer, op, "v")
+                                    : buf(w[3], voff + (max_seq - 1) * tok + d, op, "v") + voff;
             a.k = kc + layer * per_layer; a.v = vc + layer * per_layer;
-            a.k_tok_stride = cache ? hd : d;
+            a.k_tok_stride = cache ? hd : tok;
             a.k_head_stride = cache ? max_seq * hd : hd;
             a.out = buf(w[4], S * d, op, "out");
             a.state = reinterpret_cast<const int32_t *>(buf(w[5], 4, op, "state"));

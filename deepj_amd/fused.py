@@ -92,14 +92,15 @@ class Stream:
     def rope_kv_store(self, qkv, q_out, k_cache, v_cache, state, cos, sin, S, H, hd, max_seq, layer):
         return self.emit(op.OP_ROPE_KV_STORE, qkv, q_out, k_cache, v_cache, state, cos, sin, S, H, hd, max_seq, layer)
 
-    def rope_rows(self, x, out, state, cos, sin, rows, H, hd, max_seq, pos_from_row):
-        return self.emit(op.OP_ROPE_ROWS, x, out, state, cos, sin, rows, H, hd, max_seq, 1 if pos_from_row else 0)
+    def rope_rows(self, x, out, state, cos, sin, rows, H, hd, max_seq, pos_from_row, row_stride=0, live_extra=-1):
+        return self.emit(op.OP_ROPE_ROWS, x, out, state, cos, sin, rows, H, hd, max_seq, 1 if pos_from_row else 0,
+                         row_stride, live_extra)
 
     def attention(self, q, k_cache, v_cache, out, state, scratch, S, H, hd, max_seq, layer):
         return self.emit(op.OP_ATTENTION, q, k_cache, v_cache, out, state, scratch, S, H, hd, max_seq, layer)
 
-    def attention_kv(self, q, k, v, out, state, scratch, S, H, hd, max_seq):
-        return self.emit(op.OP_ATTENTION_KV, q, k, v, out, state, scratch, S, H, hd, max_seq, 0)
+    def attention_kv(self, q, k, v, out, state, scratch, S, H, hd, max_seq, tok_stride=0, v_off=0):
+        return self.emit(op.OP_ATTENTION_KV, q, k, v, out, state, scratch, S, H, hd, max_seq, 0, tok_stride, v_off)
 
     def argmax_rows(self, logits, out, rows, cols): return self.emit(op.OP_ARGMAX_ROWS, logits, out, rows, cols)
 

@@ -124,8 +124,11 @@ enum {
      *     tokens[state[2]++] = token[0]; state[1] = token[0]; state[0] += nPos
      * COPY          [op, src, dst, n, srcOff, dstOff]
      * FILL          [op, dst, bits, n]
-     * ROPE_ROWS     [op, x, out, state, cosT, sinT, rows, H, hd, maxSeq, posFromRow]  token-major rows
-     * ATTENTION_KV  [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0]  k, v token-major [maxSeq x H*hd]
+     * ROPE_ROWS     [op, x, out, state, cosT, sinT, rows, H, hd, maxSeq, posFromRow, rowStride, liveExtra]
+     *     token-major rows rowStride floats apart (0 = H*hd); posFromRow: row i sits at position i, else at
+     *     state[0]+i; liveExtra >= 0: only rows below state[0]+liveExtra are touched (-1 = all rows)
+     * ATTENTION_KV  [op, q, k, v, out, state, scratch, S, H, hd, maxSeq, 0, tokStride, vOff]
+     *     k, v token-major rows tokStride floats apart (0 = H*hd); values start vOff floats into buffer v
      * DECODE_NEXT   [op, logits, state, tokens, capacity, table, x, vocab, d, nPos]
      *     argmax + DECODE_ADVANCE + EMBED_GATHER of the chosen token into x, one launch
      * ATTN_DECODE   [op, qkv, kCache, vCache, out, state, scratch, cosT, sinT, H, hd, maxSeq, layer]
