@@ -58,64 +58,79 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
     const int a_k = (t & 3) * 8;         // 0,8,16,24
     const bool a_vec = (K & 3) == 0;
 
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        // ── stage A: 64 rows x 32 k ────────────────────────────────────────
+    // Register-staged software pipeline: the global loads of K-step i+1 are issued before the MFMAs of
+    // step i, so their latency hides behind the matrix work instead of adding to every step.
+    float va[8];                 // A: 8 consecutive k of one row
+    float wb[8];                 // B fp32: 8 consecutive columns of one k
+    int2 qraw = make_int2(0, 0); // B Q8: 8 consecutive k of one column
+    float qsc = 0.0f;
+    auto fetch = [&](int k0) {
         {
             int gr = m0 + a_row;
-            float v[8];
             if (gr < M && a_vec && k0 + a_k + 8 <= K) {
                 const float4 *p = reinterpret_cast<const float4 *>(A + (int64_t)gr * K + k0 + a_k);
                 float4 x = p[0], y = p[1];
-                v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w; v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+                va[0] = x.x; va[1] = x.y; va[2] = x.z; va[3] = x.w; va[4] = y.x; va[5] = y.y; va[6] = y.z; va[7] = y.w;
             } else {
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     int gk = k0 + a_k + j;
-                    v[j] = (gr < M && gk < K) ? A[(int64_t)gr * K + gk] : 0.0f;
+                    va[j] = (gr < M && gk < K) ? A[(int64_t)gr * K + gk] : 0.0f;
                 }
             }
-#pragma unroll
-            for (int j = 0; j < 8; j++) As[a_k + j][a_row] = v[j];
         }
-        // ── stage B: 32 k x 64 cols ────────────────────────────────────────
         if constexpr (Q8) {
             int col = t >> 2, part = t & 3;          // 8 int8 per thread
             int gn = n0 + col;
-            float w[8];
             if (gn < N) {
                 const int8_t *p = Bq + (int64_t)gn * kp + k0 + part * 8;   // kp is a multiple of 32: in bounds
-                int2 raw = *reinterpret_cast<const int2 *>(p);
-                float sc = Bs[(int64_t)gn * (kp / kQ8Group) + k0 / kQ8Group];
-                int r0 = raw.x, r1 = raw.y;
-                w[0] = (float)(int8_t)(r0 & 0xff) * sc;         w[1] = (float)(int8_t)((r0 >> 8) & 0xff) * sc;
-                w[2] = (float)(int8_t)((r0 >> 16) & 0xff) * sc; w[3] = (float)(int8_t)((r0 >> 24) & 0xff) * sc;
-                w[4] = (float)(int8_t)(r1 & 0xff) * sc;         w[5] = (float)(int8_t)((r1 >> 8) & 0xff) * sc;
-                w[6] = (float)(int8_t)((r1 >> 16) & 0xff) * sc; w[7] = (float)(int8_t)((r1 >> 24) & 0xff) * sc;
+                qraw = *reinterpret_cast<const int2 *>(p);
+                qsc = Bs[(int64_t)gn * (kp / kQ8Group) + k0 / kQ8Group];
             } else {
-#pragma unroll
-                for (int j = 0; j < 8; j++) w[j] = 0.0f;
+                qraw = make_int2(0, 0);
+                qsc = 0.0f;
             }
-#pragma unroll
-            for (int j = 0; j < 8; j++) Bl[part * 8 + j][col] = w[j];
         } else {
             int bk = t >> 3, bn = (t & 7) * 8;       // 8 consecutive columns per thread
             int gk = k0 + bk;
-            float w[8];
             if (gk < K && (N & 3) == 0 && n0 + bn + 8 <= N) {
                 const float4 *p = reinterpret_cast<const float4 *>(Bf + (int64_t)gk * N + n0 + bn);
                 float4 x = p[0], y = p[1];
-                w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w; w[4] = y.x; w[5] = y.y; w[6] = y.z; w[7] = y.w;
+                wb[0] = x.x; wb[1] = x.y; wb[2] = x.z; wb[3] = x.w; wb[4] = y.x; wb[5] = y.y; wb[6] = y.z; wb[7] = y.w;
             } else {
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     int gn = n0 + bn + j;
-                    w[j] = (gk < K && gn < N) ? Bf[(int64_t)gk * N + gn] : 0.0f;
+                    wb[j] = (gk < K && gn < N) ? Bf[(int64_t)gk * N + gn] : 0.0f;
                 }
             }
-#pragma unroll
-            for (int j = 0; j < 8; j++) Bl[bk][bn + j] = w[j];
         }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int j = 0; j < 8; j++) As[a_k + j][a_row] = va[j];
+        if constexpr (Q8) {
+            int col = t >> 2, part = t & 3;
+            int r0 = qraw.x, r1 = qraw.y;
+            float w[8];
+            w[0] = (float)(int8_t)(r0 & 0xff) * qsc;         w[1] = (float)(int8_t)((r0 >> 8) & 0xff) * qsc;
+            w[2] = (float)(int8_t)((r0 >> 16) & 0xff) * qsc; w[3] = (float)(int8_t)((r0 >> 24) & 0xff) * qsc;
+            w[4] = (float)(int8_t)(r1 & 0xff) * qsc;         w[5] = (float)(int8_t)((r1 >> 8) & 0xff) * qsc;
+            w[6] = (float)(int8_t)((r1 >> 16) & 0xff) * qsc; w[7] = (float)(int8_t)((r1 >> 24) & 0xff) * qsc;
+#pragma unroll
+            for (int j = 0; j < 8; j++) Bl[part * 8 + j][col] = w[j];
+        } else {
+            int bk = t >> 3, bn = (t & 7) * 8;
+#pragma unroll
+            for (int j = 0; j < 8; j++) Bl[bk][bn + j] = wb[j];
+        }
+    };
+
+    if (K > 0) fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        stage();
         __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);
 
         // ── 16 MFMA steps of K = 2 ─────────────────────────────────────────
         const int half = lane >> 5, l32 = lane & 31;
