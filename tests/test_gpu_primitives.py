@@ -24,7 +24,8 @@ def test_small_matmul_matches_expected_values():                      # :46-68
         assert_close([[58, 64], [139, 154]], c, atol=1e-6, rtol=0)
 
 
-@pytest.mark.parametrize("m,k,n", [(128, 192, 64), (1, 2048, 513), (65, 33, 127), (200, 513, 70), (3, 1, 5)])
+@pytest.mark.parametrize("m,k,n", [(128, 192, 64), (1, 2048, 513), (65, 33, 127), (200, 513, 70), (3, 1, 5),
+                                   (1100, 257, 2050), (1536, 64, 1537)])       # large enough for the 128 x 128 tile, ragged
 def test_matmul_matches_cpu(m, k, n):                                 # :70-78 (+ ragged shapes)
     a, b = rnd(m, k, 1), rnd(k, n, 2)
     with backend() as be:

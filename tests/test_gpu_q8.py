@@ -129,7 +129,8 @@ def test_q8_swiglu_gate_up(dev, m):
 
 
 @pytest.mark.parametrize("m,k,n", [(64, 2048, 512), (512, 2048, 256), (64, 688, 256), (7, 96, 33), (130, 5632, 128),
-                                   (64, 4096, 344), (96, 11008, 128)])
+                                   (64, 4096, 344), (96, 11008, 128),
+                                   (1300, 688, 1400), (1024, 2048, 2100)])     # 128 x 128 tile, ragged edges
 def test_q8_gemm_matches_oracle(dev, m, k, n):
     exp, got = linear_case(dev, m, k, n, norm=True, bias=True, residual=True, seed=30)
     scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
