@@ -152,6 +152,131 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
     }
 }
 
+// ── attention, many query rows: tiled on the matrix cores ────────────────────
+// grid (H, ceil(S / 128)): a workgroup takes one head and 128 query rows, 32 per wavefront, and walks the
+// keys in tiles of 32 that all four wavefronts share through LDS (K transposed, V as is).  Per tile and
+// wavefront two products run on v_mfma_f32_32x32x2_f32:
+//     S^T = K . Q^T      32 keys x 32 queries; a lane ends up with ONE query column and 16 of its keys, so
+//                        the running soft-max state (max, sum) is one scalar pair per lane
+//     O^T += V^T . P     P is consumed straight from the accumulator registers of the first product: the
+//                        key order of the contraction is chosen to be the order in which a lane holds them
+// Causal masking (HeadOps.java:105-126) excludes key j for query position p when j > p; a tile that lies
+// beyond every query of a wavefront is skipped by it.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int HD>
+__global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
+    constexpr int KT = 32, NT = HD / 32;
+    __shared__ float Kt[HD][KT + 1];
+    __shared__ __align__(16) float Vs[KT][HD];
+
+    const int h = blockIdx.x, qt = blockIdx.y;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, half = lane >> 5, l32 = lane & 31;
+    const int d = a.H * HD;
+    int pos0 = a.state[0];
+    if (pos0 < 0) pos0 = 0;
+    const int q_wave0 = qt * 128 + wave * 32;
+    const int qi = q_wave0 + l32;                           // this lane's query row
+    const bool q_ok = qi < a.S;
+    int qpos = pos0 + qi;                                   // its position: keys 0 .. qpos
+    if (qpos >= a.max_seq) qpos = a.max_seq - 1;
+    const int q_end_wg = a.S < qt * 128 + 128 ? a.S : qt * 128 + 128;
+    const int q_end_wave = a.S < q_wave0 + 32 ? a.S : q_wave0 + 32;
+    int wg_last = pos0 + q_end_wg - 1;                      // last key any query of the workgroup sees
+    if (wg_last >= a.max_seq) wg_last = a.max_seq - 1;
+    const int wave_last = q_end_wave > q_wave0 ? pos0 + q_end_wave - 1 : -1;
+
+    // this lane's query row: the elements of parity `half`
+    float qreg[HD / 2];
+    {
+        const float *qrow = a.q + (int64_t)(q_ok ? qi : 0) * d + h * HD;
+#pragma unroll
+        for (int kk = 0; kk < HD / 2; kk++) {
+            float2 v = *reinterpret_cast<const float2 *>(qrow + 2 * kk);
+            qreg[kk] = half ? v.y : v.x;
+        }
+    }
+    floatx16 acc[NT];
+#pragma unroll
+    for (int i = 0; i < NT; i++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[i][e] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+
+    const float *kbase = a.k + (int64_t)h * a.head_stride;
+    const float *vbase = a.v + (int64_t)h * a.head_stride;
+    for (int k0 = 0; k0 <= wg_last; k0 += KT) {
+        {   // stage the key tile transposed and the value tile; rows past the last key repeat it (masked below)
+            constexpr int PART = HD / 8;
+            int key = k0 + (t & 31);
+            if (key > wg_last) key = wg_last;
+            const float *kr = kbase + (int64_t)key * a.tok_stride + (t >> 5) * PART;
+#pragma unroll
+            for (int j = 0; j < PART; j += 4) {
+                float4 v = *reinterpret_cast<const float4 *>(kr + j);
+                int c = (t >> 5) * PART + j;
+                Kt[c][t & 31] = v.x; Kt[c + 1][t & 31] = v.y; Kt[c + 2][t & 31] = v.z; Kt[c + 3][t & 31] = v.w;
+            }
+            int vkey = k0 + (t >> 3);
+            if (vkey > wg_last) vkey = wg_last;
+            const float *vr = vbase + (int64_t)vkey * a.tok_stride + (t & 7) * PART;
+#pragma unroll
+            for (int j = 0; j < PART; j += 4)
+                *reinterpret_cast<float4 *>(&Vs[t >> 3][(t & 7) * PART + j]) = *reinterpret_cast<const float4 *>(vr + j);
+        }
+        __syncthreads();
+        if (k0 <= wave_last) {                              // wave-uniform
+            floatx16 st;
+#pragma unroll
+            for (int e = 0; e < 16; e++) st[e] = 0.0f;
+#pragma unroll
+            for (int kk = 0; kk < HD / 2; kk++)
+                st = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[2 * kk + half][l32], qreg[kk], st, 0, 0, 0);
+            // st[e] = q . k for key k0 + 8*(e/4) + 4*half + e%4 and this lane's query
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                int key = k0 + 8 * (e >> 2) + 4 * half + (e & 3);
+                float sv = (q_ok && key <= qpos) ? st[e] * a.scale : -INFINITY;      // scale after the product
+                st[e] = sv;
+                tmax = fmaxf(tmax, sv);
+            }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float mn = fmaxf(m, tmax);
+            const float corr = (mn == -INFINITY) ? 1.0f : expf(m - mn);
+            float psum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                float p = (st[e] == -INFINITY) ? 0.0f : expf(st[e] - mn);
+                st[e] = p;
+                psum += p;
+            }
+            l = l * corr + psum;
+            m = mn;
+#pragma unroll
+            for (int i = 0; i < NT; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][e] *= corr;
+#pragma unroll
+            for (int kk = 0; kk < 16; kk++) {
+                const int key = 8 * (kk >> 2) + 4 * half + (kk & 3);
+#pragma unroll
+                for (int i = 0; i < NT; i++)
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[key][32 * i + l32], st[kk], acc[i], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    l += __shfl_xor(l, 32, 64);
+    if (q_ok) {
+        float *orow = a.out + (int64_t)qi * d + h * HD;
+#pragma unroll
+        for (int i = 0; i < NT; i++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) orow[32 * i + 8 * (e >> 2) + 4 * half + (e & 3)] = acc[i][e] / l;
+    }
+}
+
 // ── fused decode attention ──────────────────────────────────────────────────
 // Record layout in scratch, per (head, split): [max, sum, pad, pad, o[hd]].
 struct DecodeArgs {
@@ -394,6 +519,16 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
     a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
     a.S = p.s; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
     a.scale = (float)(1.0 / sqrt((double)p.hd));
+    if (p.s >= 16) {                     // enough rows to share key tiles: matrix-core kernel
+        dim3 tg(p.h, (p.s + 127) / 128);
+        switch (p.hd) {
+            case 32: hipLaunchKernelGGL(k_attention_tiled<32>, tg, dim3(256), 0, s, a); break;
+            case 64: hipLaunchKernelGGL(k_attention_tiled<64>, tg, dim3(256), 0, s, a); break;
+            case 128: hipLaunchKernelGGL(k_attention_tiled<128>, tg, dim3(256), 0, s, a); break;
+            default: fail("attention: head dim must be 32, 64 or 128");
+        }
+        return;
+    }
     dim3 grid(p.h, p.s);
     switch (p.hd) {
         case 32: hipLaunchKernelGGL(k_attention<8>, grid, dim3(kThreads), 0, s, a); break;
