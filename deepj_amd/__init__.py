@@ -7,8 +7,9 @@ from ._native import HipNative, LIB_PATH
 from .compute_graph import ComputeGraph, GpuBuffer
 from .hip_backend import HipBackend, HipGpuRuntime
 from .tensor import Tensor
-from .models import DeepSeekConfig, DeepSeekModel, JavaRandom, LlamaConfig, LlamaModel, TextGenerator
+from .models import (DeepSeekConfig, DeepSeekModel, GPTConfig, GPTModel, JavaRandom, LlamaConfig, LlamaModel,
+                     TextGenerator)
 from .persistence import ModelSerializer, parameter_names, parameter_shapes
 
 __all__ = ["ModelSerializer", "parameter_names", "parameter_shapes", "opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor",
-           "LlamaConfig", "LlamaModel", "DeepSeekConfig", "DeepSeekModel", "TextGenerator", "JavaRandom"]
+           "LlamaConfig", "LlamaModel", "GPTConfig", "GPTModel", "DeepSeekConfig", "DeepSeekModel", "TextGenerator", "JavaRandom"]

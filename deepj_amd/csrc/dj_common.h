@@ -14,6 +14,7 @@ namespace dj {
 
 constexpr int kQ8Group = 32;          // weights per fp32 scale, along the input (K) axis
 constexpr float kRmsEps = 1e-6f;      // RMSNorm1D.java:30 in the reference
+constexpr float kLayerNormEps = 1e-5f;  // LayerNorm1D.java:15
 
 struct Error : std::runtime_error {
     using std::runtime_error::runtime_error;
@@ -68,6 +69,10 @@ void launch_layernorm_backward(hipStream_t s, const float *dxhat, const float *x
 void launch_cross_entropy(hipStream_t s, bool gradient, const float *logits, const float *targets, float *out,
                           int rows, int cols);
 void launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int rows, int cols);
+void launch_layernorm(hipStream_t s, const float *x, const float *gamma, const float *beta, float *out, int rows,
+                      int cols);
+void launch_add_positions(hipStream_t s, float *x, const float *table, const int32_t *state, int rows, int d,
+                          int max_seq);
 void launch_argmax_rows(hipStream_t s, const float *a, int32_t *out, int rows, int cols);
 
 // kernels_matmul.hip
@@ -78,6 +83,7 @@ struct Q8Linear {
     const float *x; const int8_t *wq; const float *scales; float *out;
     int m, k, n, flags;
     const float *gamma, *bias, *bias2, *residual;
+    const float *beta = nullptr;      // LayerNorm prologue only
     const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
     int m_extra = 0;
 };

@@ -30,7 +30,15 @@ struct GemmEpilogue {
     int interleaved_bias;
     const int32_t *m_dev;   // when set, only rows < min(M, m_dev[0] + m_extra) exist (row count kept on the device)
     int m_extra;
+    int gelu;               // GELU (tanh form, tensor/cpu/CpuBackend.java:338, used by activations/GELU.java:15-18) on acc + bias, before the residual
 };
+
+__device__ __forceinline__ float gemm_gelu(float x) {
+    float c = sqrtf(2.0f / 3.14159265358979323846f);
+    float x3 = x * x * x;
+    float t = c * (x + 0.044715f * x3);
+    return 0.5f * x * (1.0f + (float)tanh((double)t));
+}
 
 template <bool Q8>
 __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const float *__restrict__ Bf,
@@ -154,6 +162,7 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
             if (row < M) {
                 float v = acc[j];
                 if (ep.bias) v = v + badd;
+                if (ep.gelu) v = gemm_gelu(v);
                 if (ep.residual) v = ep.residual[(int64_t)row * N + col] + v;
                 C[(int64_t)row * N + col] = v;
             }
@@ -302,6 +311,7 @@ __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, co
                 if (row < M) {
                     float v = acc[i][jn][e];
                     if (ep.bias) v = v + badd;
+                    if (ep.gelu) v = gemm_gelu(v);
                     if (ep.residual) v = ep.residual[(int64_t)row * N + col] + v;
                     C[(int64_t)row * N + col] = v;
                 }
@@ -320,7 +330,7 @@ inline bool use_big_tile(int m, int n) {
 void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out, int m, int n, int k) {
     if (m <= 0 || n <= 0) return;
     if (k <= 0) { launch_fill(s, reinterpret_cast<uint32_t *>(out), 0u, (int64_t)m * n); return; }
-    GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0};
+    GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0, 0};
     if (use_big_tile(m, n)) {
         dim3 grid2((n + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
         hipLaunchKernelGGL(k_gemm128<false>, grid2, dim3(256), 0, s, a, b, (const int8_t *)nullptr, (const float *)nullptr,
@@ -336,9 +346,9 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
 // (= output columns of this launch; 2N for an interleaved gate/up weight).
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias, const int32_t *m_dev, int m_extra) {
+                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu) {
     if (m <= 0 || n_rows <= 0) return;
-    GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra};
+    GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu};
     if (!m_dev && use_big_tile(m, n_rows)) {       // a device-side row count is usually far below m: keep small tiles
         dim3 grid2((n_rows + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
         hipLaunchKernelGGL(k_gemm128<true>, grid2, dim3(256), 0, s, x, (const float *)nullptr, wq, scales, out, m,

@@ -24,7 +24,7 @@ namespace dj {
 
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias, const int32_t *m_dev, int m_extra);
+                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu);
 
 namespace {
 
@@ -38,6 +38,13 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 __device__ __forceinline__ float d_sigmoid(float x) { return 1.0f / (1.0f + (float)exp((double)(-x))); }
+// tensor/cpu/CpuBackend.java:338 (tanh form)
+__device__ __forceinline__ float d_gelu(float x) {
+    float c = sqrtf(2.0f / 3.14159265358979323846f);
+    float x3 = x * x * x;
+    float t = c * (x + 0.044715f * x3);
+    return 0.5f * x * (1.0f + (float)tanh((double)t));
+}
 
 // ── quantise: grid (ceil(N/64), Kp/32); a workgroup takes 64 columns x one group ──
 __global__ void __launch_bounds__(kThreads) k_q8_quantize(const float *__restrict__ w, int8_t *__restrict__ q,
@@ -95,6 +102,7 @@ struct MatvecArgs {
     const float *x; const int8_t *wq; const float *scales; float *out;
     int k, kp, n_out;                 // n_out outputs; SwiGLU: output o uses rows 2o, 2o+1
     const float *gamma, *bias, *bias2, *residual;
+    const float *beta;                // set: LayerNorm prologue with gamma and beta (otherwise gamma alone = RMSNorm)
 };
 
 __device__ __forceinline__ float dot16(const int4 &w, const float *xr) {
@@ -167,7 +175,7 @@ __device__ __forceinline__ void load_batch(RowBatch<NC, R> &b, const MatvecArgs 
     }
 }
 
-template <int NC, int B, bool SWIGLU>
+template <int NC, int B, bool SWIGLU, bool GELU>
 __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 : 1)> &b, const float (&xr)[NC][16],
                                              const MatvecArgs &p, int o0, int o_end, int lane, float rms) {
     constexpr int R = B * (SWIGLU ? 2 : 1);
@@ -194,6 +202,7 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
                 } else {
                     v = acc[u];
                     if (p.bias) v = v + b.eb[u];
+                    if constexpr (GELU) v = d_gelu(v);
                 }
                 if (p.residual) v = b.er[u] + v;
                 p.out[o] = v;
@@ -209,10 +218,12 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
 // the HBM stream is already running while the workgroup stages x through LDS and
 // applies the RMSNorm prologue; after that the next batch is always in flight while
 // the current one is multiplied (two register buffers used in turn).
-template <int NC, int B, bool SWIGLU>
+// GELU (compile time: its double-precision tanh would cost every other variant some forty registers)
+// applies the activation to the biased sum.
+template <int NC, int B, bool SWIGLU, bool GELU>
 __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     extern __shared__ __align__(16) float xs[];   // Kp floats
-    __shared__ float red[kWaves];
+    __shared__ float red[kWaves], red2[kWaves];
     constexpr int RPO = SWIGLU ? 2 : 1;           // Q8 rows per output
     constexpr int R = B * RPO;                    // rows per batch
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -248,7 +259,44 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     // Stage the activation row through LDS (zero beyond K so padded weights meet zeros).
     // All global loads of the prologue - x and, for the RMSNorm prologue, gamma - were
     // issued together, so it costs one memory round trip, not one per element.
-    if (vec) {
+    if (vec && p.beta) {
+        // LayerNorm prologue (LayerNorm1D.java:34-66): mean, then the population variance about it, then
+        // ((x - mean) / sqrt(var + 1e-5)) * gamma + beta goes to LDS.
+        float4 bv[NC];
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            int e = (tid + kThreads * j) * 4;
+            bv[j] = e < p.k ? *reinterpret_cast<const float4 *>(p.beta + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        const float inv_k = 1.0f / (float)p.k;
+        float sm = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NC; j++) sm += (xv[j].x + xv[j].y) + (xv[j].z + xv[j].w);
+        sm = wave_sum_dpp(sm);
+        if (lane == 0) red[wave] = sm;
+        __syncthreads();
+        const float mean = (red[0] + red[1] + red[2] + red[3]) * inv_k;
+        float sv = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            bool ok = (tid + kThreads * j) * 4 < p.k;
+            float a = xv[j].x - mean, b = xv[j].y - mean, c = xv[j].z - mean, d = xv[j].w - mean;
+            xv[j] = ok ? make_float4(a, b, c, d) : make_float4(0.f, 0.f, 0.f, 0.f);
+            sv += ok ? (a * a + b * b) + (c * c + d * d) : 0.0f;
+        }
+        sv = wave_sum_dpp(sv);
+        if (lane == 0) red2[wave] = sv;
+        __syncthreads();
+        const float sd = sqrtf((red2[0] + red2[1] + red2[2] + red2[3]) * inv_k + kLayerNormEps);
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            int e = (tid + kThreads * j) * 4;
+            float4 y;
+            y.x = (xv[j].x / sd) * gv[j].x + bv[j].x; y.y = (xv[j].y / sd) * gv[j].y + bv[j].y;
+            y.z = (xv[j].z / sd) * gv[j].z + bv[j].z; y.w = (xv[j].w / sd) * gv[j].w + bv[j].w;
+            if (e < p.kp) *reinterpret_cast<float4 *>(xs + e) = y;      // e >= k: x, gamma and beta are all zero
+        }
+    } else if (vec) {
         if (p.gamma) {
             // RMSNorm prologue (RMSNorm1D.java:46-57).  W.(g * x / rms) = (W.(g * x)) / rms: the staged row is
             // g * x, which needs no reduction, and the division by rms is applied to the finished sums, so the
@@ -277,7 +325,21 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             xs[i] = v;
             ss += v * v;
         }
-        if (p.gamma) {
+        if (p.beta) {
+            float sm = 0.0f;
+            for (int i = tid; i < p.k; i += kThreads) sm += p.x[i];
+            sm = wave_sum_dpp(sm);
+            if (lane == 0) red[wave] = sm;
+            __syncthreads();
+            float mean = (red[0] + red[1] + red[2] + red[3]) * (1.0f / (float)p.k);
+            float sv = 0.0f;
+            for (int i = tid; i < p.k; i += kThreads) { float c = xs[i] - mean; sv += c * c; }
+            sv = wave_sum_dpp(sv);
+            if (lane == 0) red2[wave] = sv;
+            __syncthreads();
+            float sd = sqrtf((red2[0] + red2[1] + red2[2] + red2[3]) * (1.0f / (float)p.k) + kLayerNormEps);
+            for (int i = tid; i < p.k; i += kThreads) xs[i] = ((xs[i] - mean) / sd) * p.gamma[i] + p.beta[i];
+        } else if (p.gamma) {
             ss = wave_sum_dpp(ss);
             if (lane == 0) red[wave] = ss;
             __syncthreads();
@@ -309,17 +371,17 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
 
     for (int o0 = o_begin; o0 < o_end; o0 += 2 * o_step) {
         if (o0 + o_step < o_end) { load_batch<NC, R>(bb, p, (o0 + o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(bb, p, o0 + o_step); }
-        finish_batch<NC, B, SWIGLU>(ba, xr, p, o0, o_end, lane, rms);
+        finish_batch<NC, B, SWIGLU, GELU>(ba, xr, p, o0, o_end, lane, rms);
         if (o0 + o_step >= o_end) break;
         if (o0 + 2 * o_step < o_end) { load_batch<NC, R>(ba, p, (o0 + 2 * o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(ba, p, o0 + 2 * o_step); }
-        finish_batch<NC, B, SWIGLU>(bb, xr, p, o0 + o_step, o_end, lane, rms);
+        finish_batch<NC, B, SWIGLU, GELU>(bb, xr, p, o0 + o_step, o_end, lane, rms);
     }
 }
 
 constexpr int kMvGridCap = 768;          // three workgroups per CU
 inline int mv_grid_cap() { return kMvGridCap; }
 
-template <int NC, int B, bool SW>
+template <int NC, int B, bool SW, bool GELU = false>
 void launch_mv(hipStream_t s, const MatvecArgs &a) {
     // Three workgroups (12 wavefronts) per CU when there are outputs for them; never
     // more wavefronts than outputs.
@@ -328,7 +390,7 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     if (grid > mv_grid_cap()) grid = mv_grid_cap();
     if (grid < 1) grid = 1;
     size_t lds = (size_t)a.kp * sizeof(float);
-    hipLaunchKernelGGL((k_q8_matvec<NC, B, SW>), dim3(grid), dim3(kThreads), lds, s, a);
+    hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, GELU>), dim3(grid), dim3(kThreads), lds, s, a);
 }
 
 // Batch depth B (outputs a wavefront multiplies per step).  Small matrices want B = 1: every
@@ -338,7 +400,7 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
 inline int mv_target_waves() { return 3072; }
 
 template <int NC>
-void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu) {
+void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu, bool gelu) {
     constexpr int BMAX = NC == 1 ? 8 : (NC == 2 ? 4 : (NC <= 4 ? 2 : 1));
     int rows = swiglu ? 2 * a.n_out : a.n_out;
     int want = (rows + mv_target_waves() - 1) / mv_target_waves();      // rows per wavefront per step
@@ -347,6 +409,10 @@ void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu) {
         if (BS >= 4 && want >= 8) launch_mv<NC, (BS >= 4 ? 4 : 1), true>(s, a);
         else if (BS >= 2 && want >= 4) launch_mv<NC, (BS >= 2 ? 2 : 1), true>(s, a);
         else launch_mv<NC, 1, true>(s, a);
+    } else if (gelu) {
+        if (BMAX >= 4 && want >= 4) launch_mv<NC, (BMAX >= 4 ? 4 : 1), false, true>(s, a);
+        else if (BMAX >= 2 && want >= 2) launch_mv<NC, (BMAX >= 2 ? 2 : 1), false, true>(s, a);
+        else launch_mv<NC, 1, false, true>(s, a);
     } else {
         if (BMAX >= 8 && want >= 8) launch_mv<NC, (BMAX >= 8 ? 8 : 1), false>(s, a);
         else if (BMAX >= 4 && want >= 4) launch_mv<NC, (BMAX >= 4 ? 4 : 1), false>(s, a);
@@ -392,7 +458,7 @@ int64_t q8_linear_workspace_floats(int m, int k, int n, int flags) {
     bool mv = (m == 1) && matvec_supported(k);
     int64_t ws = 0;
     if (!mv) {
-        if (flags & DJ_LIN_RMSNORM) ws += (int64_t)m * k;            // normalised activations
+        if (flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM)) ws += (int64_t)m * k;   // normalised activations
         if (flags & DJ_LIN_SWIGLU) ws += (int64_t)m * 2 * n;         // interleaved gate/up before the gate
     }
     return ws;
@@ -401,27 +467,30 @@ int64_t q8_linear_workspace_floats(int m, int k, int n, int flags) {
 void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_t workspace_floats) {
     if (p.m <= 0 || p.n <= 0) return;
     const bool swiglu = (p.flags & DJ_LIN_SWIGLU) != 0;
-    const float *gamma = (p.flags & DJ_LIN_RMSNORM) ? p.gamma : nullptr;
+    const bool layernorm = (p.flags & DJ_LIN_LAYERNORM) != 0;
+    const int gelu = (p.flags & DJ_LIN_GELU) ? 1 : 0;
+    const float *gamma = (p.flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM)) ? p.gamma : nullptr;
+    const float *beta = layernorm ? p.beta : nullptr;
     const float *bias = (p.flags & DJ_LIN_BIAS) ? p.bias : nullptr;
     const float *bias2 = (p.flags & DJ_LIN_BIAS) && swiglu ? p.bias2 : nullptr;
     const float *residual = (p.flags & DJ_LIN_RESIDUAL) ? p.residual : nullptr;
     const int kp = q8_padded_k(p.k);
 
     if (p.m == 1 && !p.m_dev && matvec_supported(p.k)) {
-        MatvecArgs a{p.x, p.wq, p.scales, p.out, p.k, kp, p.n, gamma, bias, bias2, residual};
+        MatvecArgs a{p.x, p.wq, p.scales, p.out, p.k, kp, p.n, gamma, bias, bias2, residual, beta};
         int nc = (kp + 1023) / 1024;
         switch (nc) {
-            case 1: dispatch_mv<1>(s, a, swiglu); break;
-            case 2: dispatch_mv<2>(s, a, swiglu); break;
-            case 3: dispatch_mv<3>(s, a, swiglu); break;
-            case 4: dispatch_mv<4>(s, a, swiglu); break;
-            case 5: dispatch_mv<5>(s, a, swiglu); break;
-            case 6: dispatch_mv<6>(s, a, swiglu); break;
-            case 7: dispatch_mv<7>(s, a, swiglu); break;
-            case 8: dispatch_mv<8>(s, a, swiglu); break;
-            case 9: dispatch_mv<9>(s, a, swiglu); break;
-            case 10: dispatch_mv<10>(s, a, swiglu); break;
-            default: dispatch_mv<11>(s, a, swiglu); break;
+            case 1: dispatch_mv<1>(s, a, swiglu, gelu != 0); break;
+            case 2: dispatch_mv<2>(s, a, swiglu, gelu != 0); break;
+            case 3: dispatch_mv<3>(s, a, swiglu, gelu != 0); break;
+            case 4: dispatch_mv<4>(s, a, swiglu, gelu != 0); break;
+            case 5: dispatch_mv<5>(s, a, swiglu, gelu != 0); break;
+            case 6: dispatch_mv<6>(s, a, swiglu, gelu != 0); break;
+            case 7: dispatch_mv<7>(s, a, swiglu, gelu != 0); break;
+            case 8: dispatch_mv<8>(s, a, swiglu, gelu != 0); break;
+            case 9: dispatch_mv<9>(s, a, swiglu, gelu != 0); break;
+            case 10: dispatch_mv<10>(s, a, swiglu, gelu != 0); break;
+            default: dispatch_mv<11>(s, a, swiglu, gelu != 0); break;
         }
         return;
     }
@@ -431,12 +500,13 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     const float *x = p.x;
     float *ws = workspace;
     if (gamma) {
-        launch_rmsnorm(s, p.x, gamma, ws, p.m, p.k);
+        if (layernorm) launch_layernorm(s, p.x, gamma, beta, ws, p.m, p.k);
+        else launch_rmsnorm(s, p.x, gamma, ws, p.m, p.k);
         x = ws;
         ws += (int64_t)p.m * p.k;
     }
     if (swiglu) {
-        launch_q8_gemm(s, x, p.wq, p.scales, ws, p.m, p.k, 2 * p.n, bias, bias2, nullptr, 1, nullptr, 0);
+        launch_q8_gemm(s, x, p.wq, p.scales, ws, p.m, p.k, 2 * p.n, bias, bias2, nullptr, 1, nullptr, 0, 0);
         int64_t n_out = (int64_t)p.m * p.n;
         int64_t blocks = (n_out + kThreads - 1) / kThreads;
         if (blocks > 8192) blocks = 8192;
@@ -444,7 +514,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
         if (residual) fail("q8_linear: SWIGLU with RESIDUAL is not supported");
         hipLaunchKernelGGL(k_swiglu_combine, dim3((int)blocks), dim3(kThreads), 0, s, ws, p.out, n_out);
     } else {
-        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0, p.m_dev, p.m_extra);
+        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0, p.m_dev, p.m_extra, gelu);
     }
 }
 

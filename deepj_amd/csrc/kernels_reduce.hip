@@ -219,6 +219,42 @@ __global__ void __launch_bounds__(kThreads) k_rmsnorm(const float *__restrict__ 
     }
 }
 
+// out = ((x - mean) / sqrt(var + 1e-5)) * gamma + beta, population variance about the mean
+// (LayerNorm1D.java:34-66 composes this from eight primitive ops).
+__global__ void __launch_bounds__(kThreads) k_layernorm(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta, float *__restrict__ out,
+                                                        int rows, int cols) {
+    __shared__ float lds[kWaves];
+    const float inv = 1.0f / (float)cols;
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float *row = x + (int64_t)r * cols;
+        float *orow = out + (int64_t)r * cols;
+        float s = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) s += row[c];
+        float mean = block_sum(s, lds) * inv;
+        float v = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += kThreads) { float t = row[c] - mean; v += t * t; }
+        float sd = sqrtf(block_sum(v, lds) * inv + kLayerNormEps);
+        for (int c = threadIdx.x; c < cols; c += kThreads) orow[c] = ((row[c] - mean) / sd) * gamma[c] + beta[c];
+    }
+}
+
+// x[i, :] += table[state[0] + i, :]: learned positions of rows that sit at state[0].. (GPTModel.java:52-54,
+// PositionalEmbedding.java:26-33).  Rows whose position falls outside the table become NaN.
+__global__ void __launch_bounds__(kThreads) k_add_positions(float *__restrict__ x, const float *__restrict__ table,
+                                                            const int32_t *__restrict__ state, int rows, int d,
+                                                            int max_seq) {
+    const int p0 = state[0];
+    const int64_t total = (int64_t)rows * d;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        int r = (int)(i / d);
+        int c = (int)(i - (int64_t)r * d);
+        int pos = p0 + r;
+        x[i] = (pos >= 0 && pos < max_seq) ? x[i] + table[(int64_t)pos * d + c] : __builtin_nanf("");
+    }
+}
+
 // Index of the row maximum, lowest index on ties: what topK=1 sampling reduces to
 // (TextGenerator.java:110-114,163-170: stable descending sort, first element).
 // NaN ranks above everything, as Float.compare orders it.
@@ -378,6 +414,21 @@ void launch_cross_entropy(hipStream_t s, bool gradient, const float *logits, con
 void launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int rows, int cols) {
     if (rows <= 0) return;
     hipLaunchKernelGGL(k_rmsnorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, out, rows, cols);
+}
+
+void launch_layernorm(hipStream_t s, const float *x, const float *gamma, const float *beta, float *out, int rows,
+                      int cols) {
+    if (rows <= 0) return;
+    hipLaunchKernelGGL(k_layernorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, beta, out, rows, cols);
+}
+
+void launch_add_positions(hipStream_t s, float *x, const float *table, const int32_t *state, int rows, int d,
+                          int max_seq) {
+    int64_t total = (int64_t)rows * d;
+    if (total <= 0) return;
+    int64_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(k_add_positions, dim3((int)blocks), dim3(kThreads), 0, s, x, table, state, rows, d, max_seq);
 }
 
 void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,

@@ -1,7 +1,7 @@
 // Native decode driver: the caller on the host side of the C ABI.  It plays the part of
-// the reference's LlamaModel / DeepSeekModel + TextGenerator
+// the reference's LlamaModel / DeepSeekModel / GPTModel + TextGenerator
 //   (src/main/java/io/github/kirstenali/deepj/models/{DecoderOnlyModel,TextGenerator}.java,
-//    models/llama/LlamaModel.java, models/deepseek/DeepSeekModel.java)
+//    models/llama/LlamaModel.java, models/deepseek/DeepSeekModel.java, models/gpt/GPTModel.java)
 // for inference, but instead of re-running the whole context for every token
 // (TextGenerator.java:91-100) it keeps a KV cache in HBM, records ONE fused command
 // stream per token and replays it as a HIP graph.  Position, current token and the
@@ -15,6 +15,8 @@
 //   g1 g2 wq wk wv wo           (Llama;  MultiHeadSelfAttention.java:47-50)
 //   g1 g2 wdq wuq wdkv wuk wuv wo (DeepSeek; MultiHeadLatentAttention.java:81-86)
 //   wg bg wu bu wd bd           (SwiGLULayer.java:56-58)
+// GPT (GPTTransformerBlock.java:52-57): g1 be1 g2 be2 (LayerNorm gamma/beta), wq wk wv wo, and the FNN's two
+//   Linears as wg bg (dModel -> dFF) and wd bd (dFF -> dModel); model level adds "pos" and "bf".
 // Matrices are given in the reference's orientation, fp32 [dIn x dOut] row-major.
 #include <algorithm>
 #include <cmath>
@@ -35,7 +37,7 @@ float deepj_host_random_next_float(void *h);
 namespace {
 
 struct Config {
-    int32_t kind;       // 0 Llama, 1 DeepSeek (MLA)
+    int32_t kind;       // 0 Llama, 1 DeepSeek (MLA), 2 GPT
     int32_t vocab, max_seq, d, heads, layers, dff, q_rank, kv_rank;
 };
 
@@ -46,7 +48,7 @@ void hip(int rc) {
 }
 
 struct Layer {
-    int32_t g1 = -1, g2 = -1;
+    int32_t g1 = -1, g2 = -1, be1 = -1, be2 = -1;     // be*: LayerNorm betas (GPT)
     int32_t wqkv = -1, wo = -1;                       // Llama: fused [3d x d]
     int32_t wdq = -1, wuq = -1, wdkv = -1, wuk = -1, wuv = -1;   // MLA
     int32_t wgu = -1, bg = -1, bu = -1, wd = -1, bd = -1;
@@ -64,6 +66,7 @@ struct Runner {
     std::map<std::string, bool> have;
     std::vector<Layer> layers;
     int32_t emb = -1, gf = -1, wlm = -1, blm = -1;
+    int32_t pos_table = -1, bf = -1;                       // GPT: learned positions, final LayerNorm beta
     int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
     int32_t state = -1, tok = -1, tokens = -1, scratch = -1, scratch_dec = -1, logits = -1, last_x = -1;
     int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
@@ -127,6 +130,8 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
     if (r.finalized) throw Error("set_weight after finalize");
     if (name == "emb") { expect_shape(name, rows, cols, c.vocab, d); r.emb = r.upload_new(data, (int64_t)rows * cols); }
     else if (name == "gf") { expect_shape(name, rows, cols, 1, d); r.gf = r.upload_new(data, d); }
+    else if (c.kind == 2 && name == "bf") { expect_shape(name, rows, cols, 1, d); r.bf = r.upload_new(data, d); }
+    else if (c.kind == 2 && name == "pos") { expect_shape(name, rows, cols, c.max_seq, d); r.pos_table = r.upload_new(data, (int64_t)rows * cols); }
     else if (name == "blm") { expect_shape(name, rows, cols, 1, c.vocab); r.blm = r.upload_new(data, c.vocab); }
     else if (name == "wlm") { expect_shape(name, rows, cols, d, c.vocab); quantize_into(r, r.wlm, data, d, c.vocab, 0, 1, c.vocab); }
     else if (name.size() > 2 && name[0] == 'L') {
@@ -138,6 +143,10 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
         std::string w = name.substr(dot + 1);
         if (w == "g1") { expect_shape(name, rows, cols, 1, d); L.g1 = r.upload_new(data, d); }
         else if (w == "g2") { expect_shape(name, rows, cols, 1, d); L.g2 = r.upload_new(data, d); }
+        else if (c.kind == 2 && w == "be1") { expect_shape(name, rows, cols, 1, d); L.be1 = r.upload_new(data, d); }
+        else if (c.kind == 2 && w == "be2") { expect_shape(name, rows, cols, 1, d); L.be2 = r.upload_new(data, d); }
+        else if (c.kind == 2 && w == "wg") { expect_shape(name, rows, cols, d, c.dff); quantize_into(r, L.wgu, data, d, c.dff, 0, 1, c.dff); }
+        else if (c.kind == 2 && (w == "wu" || w == "bu")) throw Error("unknown weight " + name);
         else if (w == "bg") { expect_shape(name, rows, cols, 1, c.dff); L.bg = r.upload_new(data, c.dff); }
         else if (w == "bu") { expect_shape(name, rows, cols, 1, c.dff); L.bu = r.upload_new(data, c.dff); }
         else if (w == "bd") { expect_shape(name, rows, cols, 1, d); L.bd = r.upload_new(data, d); }
@@ -145,7 +154,7 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
         else if (w == "wu") { expect_shape(name, rows, cols, d, c.dff); quantize_into(r, L.wgu, data, d, c.dff, 1, 2, 2 * c.dff); }
         else if (w == "wd") { expect_shape(name, rows, cols, c.dff, d); quantize_into(r, L.wd, data, c.dff, d, 0, 1, d); }
         else if (w == "wo") { expect_shape(name, rows, cols, d, d); quantize_into(r, L.wo, data, d, d, 0, 1, d); }
-        else if (c.kind == 0 && (w == "wq" || w == "wk" || w == "wv")) {
+        else if (c.kind != 1 && (w == "wq" || w == "wk" || w == "wv")) {
             expect_shape(name, rows, cols, d, d);
             int part = w == "wq" ? 0 : (w == "wk" ? 1 : 2);
             quantize_into(r, L.wqkv, data, d, d, part * d, 1, 3 * d);
@@ -163,6 +172,15 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
 
 std::vector<std::string> weight_names(const Config &c) {
     std::vector<std::string> names{"emb"};
+    if (c.kind == 2) {
+        names.push_back("pos");
+        for (int l = 0; l < c.layers; l++) {
+            std::string p = "L" + std::to_string(l) + ".";
+            for (const char *w : {"g1", "be1", "g2", "be2", "wq", "wk", "wv", "wo", "wg", "bg", "wd", "bd"}) names.push_back(p + w);
+        }
+        names.insert(names.end(), {"gf", "bf", "wlm", "blm"});
+        return names;
+    }
     for (int l = 0; l < c.layers; l++) {
         std::string p = "L" + std::to_string(l) + ".";
         for (const char *w : {"g1", "g2"}) names.push_back(p + w);
@@ -176,28 +194,42 @@ std::vector<std::string> weight_names(const Config &c) {
 
 // new LlamaModel(cfg, seed) / new DeepSeekModel(cfg, seed): same RNG wiring and draw order
 // (LlamaModel.java:27-42, LlamaTransformerBuilder.java:45-55, DeepSeekTransformerBuilder.java:56-68).
-void init_seeded(Runner &r, int64_t seed, int threads) {
+// GPT: new GPTModel(cfg, seed) - Random(seed) for the token table, a second Random(seed) shared by the
+// blocks, Random(seed + 1) for the head, Random(seed + 2) for the positions, then every parameter times
+// initScale (GPTModel.java:27-46,76-81; GPTTransformerBlock.java:52-57; FNN draws its Linears in order).
+void init_seeded(Runner &r, int64_t seed, int threads, float init_scale) {
     const Config &c = r.cfg;
     const int d = c.d;
     std::vector<float> buf;
     auto draw = [&](void *rng, const std::string &name, int rows, int cols) {
         buf.resize((size_t)rows * cols);
         deepj_host_random_fill(rng, buf.data(), (int64_t)rows * cols, 0.1, threads);
+        if (init_scale != 1.0f) for (float &v : buf) v *= init_scale;
         set_weight(r, name, buf.data(), rows, cols);
     };
     auto constant = [&](const std::string &name, int cols, float v) {
-        buf.assign((size_t)cols, v);
+        buf.assign((size_t)cols, init_scale != 1.0f ? v * init_scale : v);
         set_weight(r, name, buf.data(), 1, cols);
     };
     void *emb_rng = deepj_host_random_create(seed);
     void *stack_rng = deepj_host_random_create(seed);
     void *head_rng = deepj_host_random_create(seed + 1);
+    void *pos_rng = deepj_host_random_create(seed + 2);
     try {
         draw(emb_rng, "emb", c.vocab, d);
+        if (c.kind == 2) draw(pos_rng, "pos", c.max_seq, d);
         for (int l = 0; l < c.layers; l++) {
             std::string p = "L" + std::to_string(l) + ".";
             constant(p + "g1", d, 1.0f);
             constant(p + "g2", d, 1.0f);
+            if (c.kind == 2) {
+                constant(p + "be1", d, 0.0f);
+                constant(p + "be2", d, 0.0f);
+                for (const char *w : {"wq", "wk", "wv", "wo"}) draw(stack_rng, p + w, d, d);
+                draw(stack_rng, p + "wg", d, c.dff);  constant(p + "bg", c.dff, 0.0f);
+                draw(stack_rng, p + "wd", c.dff, d);  constant(p + "bd", d, 0.0f);
+                continue;
+            }
             if (c.kind == 0) {
                 for (const char *w : {"wq", "wk", "wv", "wo"}) draw(stack_rng, p + w, d, d);
             } else {
@@ -213,13 +245,16 @@ void init_seeded(Runner &r, int64_t seed, int threads) {
             draw(stack_rng, p + "wd", c.dff, d);  constant(p + "bd", d, 0.0f);
         }
         constant("gf", d, 1.0f);
+        if (c.kind == 2) constant("bf", d, 0.0f);
         draw(head_rng, "wlm", d, c.vocab);
         constant("blm", c.vocab, 0.0f);
     } catch (...) {
         deepj_host_random_destroy(emb_rng); deepj_host_random_destroy(stack_rng); deepj_host_random_destroy(head_rng);
+        deepj_host_random_destroy(pos_rng);
         throw;
     }
     deepj_host_random_destroy(emb_rng); deepj_host_random_destroy(stack_rng); deepj_host_random_destroy(head_rng);
+    deepj_host_random_destroy(pos_rng);
 }
 
 // ── buffers ────────────────────────────────────────────────────────────────
@@ -231,7 +266,7 @@ void alloc_acts(Runner &r, Acts &a, int rows) {
     int64_t S = rows, d = c.d;
     a.x = r.alloc(S * d); a.x2 = r.alloc(S * d); a.q = r.alloc(S * d); a.att = r.alloc(S * d);
     a.ff = r.alloc(S * c.dff); a.ids = r.alloc(std::max<int64_t>(S, 4));
-    if (c.kind == 0) a.qkv = r.alloc(S * 3 * d);
+    if (c.kind != 1) a.qkv = r.alloc(S * 3 * d);
     else { a.cq = r.alloc(S * c.q_rank); a.ckv = r.alloc(S * c.kv_rank); a.qkv = r.alloc(S * d); }
     a.rows = rows;
 }
@@ -248,13 +283,15 @@ void finalize(Runner &r) {
         for (int i = 0; i < half; i++) {
             float expo = (2.0f * (float)i) / (float)hd;
             float theta = (float)((double)pos / std::pow((double)10000.0f, (double)expo));
-            ct[(size_t)pos * half + i] = (float)std::cos((double)theta);
-            st[(size_t)pos * half + i] = (float)std::sin((double)theta);
+            // GPT attends without rotation (MultiHeadSelfAttention.java:60-86): the identity tables turn the
+            // rotation inside the attention kernels into x * 1 - y * 0 = x.
+            ct[(size_t)pos * half + i] = c.kind == 2 ? 1.0f : (float)std::cos((double)theta);
+            st[(size_t)pos * half + i] = c.kind == 2 ? 0.0f : (float)std::sin((double)theta);
         }
     r.cos_t = r.upload_new(ct.data(), (int64_t)ct.size());
     r.sin_t = r.upload_new(st.data(), (int64_t)st.size());
     int64_t per_layer = (int64_t)c.max_seq * c.d;
-    if (c.kind == 0) {
+    if (c.kind != 1) {
         r.kc = r.alloc(per_layer * c.layers);
         r.vc = r.alloc(per_layer * c.layers);
     } else {
@@ -298,9 +335,11 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     const Config &c = r.cfg;
     const Layer &L = r.layers[l];
     const int d = c.d, H = c.heads, hd = r.hd();
-    if (c.kind == 0) {
+    if (c.kind != 1) {
         // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
-        q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
+        // GPT: LayerNorm instead of RMSNorm and no rotation                  GPTTransformerBlock.java:66-68
+        if (c.kind == 2) q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1);
+        else q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
         if (S == 1 && &a == &r.dec) {
             emit(s, DJ_OP_ATTN_DECODE, a.qkv, r.kc, r.vc, a.att, r.state, r.scratch_dec, r.cos_t, r.sin_t, H, hd,
                  c.max_seq, l);
@@ -322,14 +361,30 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
         emit(s, DJ_OP_ATTENTION_KV, a.q, r.kc, r.kc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0, 2 * d, d);
     }
     q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
+    if (c.kind == 2) {
+        // x = x2 + W2 . GELU(W1 . ln2(x2) + b1) + b2                        GPTTransformerBlock.java:70-72, FNN.java:57-73
+        q8_linear(s, a.x2, L.wgu, a.ff, S, d, c.dff, DJ_LIN_LAYERNORM | DJ_LIN_BIAS | DJ_LIN_GELU, L.g2, L.bg, L.be2);
+        q8_linear(s, a.ff, L.wd, a.x, S, c.dff, d, DJ_LIN_BIAS | DJ_LIN_RESIDUAL, -1, L.bd, -1, a.x2);
+        return;
+    }
     // x = x2 + down(SiLU(gate(norm2(x2))) * up(norm2(x2)))                  LlamaTransformerBlock.java:52
     q8_linear(s, a.x2, L.wgu, a.ff, S, d, c.dff, DJ_LIN_RMSNORM | DJ_LIN_BIAS | DJ_LIN_SWIGLU, L.g2, L.bg, L.bu);
     q8_linear(s, a.ff, L.wd, a.x, S, c.dff, d, DJ_LIN_BIAS | DJ_LIN_RESIDUAL, -1, L.bd, -1, a.x2);
 }
 
-void head_stream(Runner &r, Stream &s, int32_t x_row) {
+// logits = lmHead(normF(x)) on `rows` rows                                   DecoderOnlyModel.java:62-63
+void head_rows(Runner &r, Stream &s, int32_t x, int32_t out, int rows) {
     const Config &c = r.cfg;
-    q8_linear(s, x_row, r.wlm, r.logits, 1, c.d, c.vocab, DJ_LIN_RMSNORM | DJ_LIN_BIAS, r.gf, r.blm);
+    if (c.kind == 2) q8_linear(s, x, r.wlm, out, rows, c.d, c.vocab, DJ_LIN_LAYERNORM | DJ_LIN_BIAS, r.gf, r.blm, r.bf);
+    else q8_linear(s, x, r.wlm, out, rows, c.d, c.vocab, DJ_LIN_RMSNORM | DJ_LIN_BIAS, r.gf, r.blm);
+}
+void head_stream(Runner &r, Stream &s, int32_t x_row) { head_rows(r, s, x_row, r.logits, 1); }
+
+// GPT: the token rows in x (first one at position state[0]) get their learned position rows added
+// (GPTModel.java:52-54).
+void positions(Runner &r, Stream &s, int32_t x, int rows) {
+    const Config &c = r.cfg;
+    if (c.kind == 2) emit(s, DJ_OP_ADD_POSITIONS, x, r.pos_table, r.state, rows, c.d, c.max_seq);
 }
 
 Stream decode_stream(Runner &r, bool sample_on_device) {
@@ -337,11 +392,16 @@ Stream decode_stream(Runner &r, bool sample_on_device) {
     Stream s;
     // Greedy on the device: the previous step (or the prefill) already left the embedding of
     // the token to process in dec.x.  Host sampling: gather it from state[1] first.
-    if (!sample_on_device) emit(s, DJ_OP_EMBED_GATHER, r.emb, r.state, r.dec.x, 1, c.d, c.vocab, 1);
+    if (!sample_on_device) {
+        emit(s, DJ_OP_EMBED_GATHER, r.emb, r.state, r.dec.x, 1, c.d, c.vocab, 1);
+        positions(r, s, r.dec.x, 1);
+    }
     for (int l = 0; l < c.layers; l++) block_stream(r, s, r.dec, l, 1);
     head_stream(r, s, r.dec.x);
-    if (sample_on_device)
+    if (sample_on_device) {
         emit(s, DJ_OP_DECODE_NEXT, r.logits, r.state, r.tokens, c.max_seq, r.emb, r.dec.x, c.vocab, c.d, 1);
+        positions(r, s, r.dec.x, 1);        // state[0] is already the position of the token just chosen
+    }
     return s;
 }
 
@@ -363,16 +423,20 @@ void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choos
     hip(deepj_hip_upload(r.pre.ids, reinterpret_cast<const float *>(ids), n));
     Stream s;
     emit(s, DJ_OP_EMBED_GATHER, r.emb, r.pre.ids, r.pre.x, n, c.d, c.vocab, 0);
+    positions(r, s, r.pre.x, n);
     for (int l = 0; l < c.layers; l++) block_stream(r, s, r.pre, l, n);
     emit(s, DJ_OP_COPY, r.pre.x, r.last_x, c.d, (int64_t)(n - 1) * c.d, 0);
     head_stream(r, s, r.last_x);
-    if (choose) emit(s, DJ_OP_DECODE_NEXT, r.logits, r.state, r.tokens, c.max_seq, r.emb, r.dec.x, c.vocab, c.d, n);
+    if (choose) {
+        emit(s, DJ_OP_DECODE_NEXT, r.logits, r.state, r.tokens, c.max_seq, r.emb, r.dec.x, c.vocab, c.d, n);
+        if (r.pos + n < c.max_seq) positions(r, s, r.dec.x, 1);     // a full cache takes no further token
+    }
     r.run(s);
     if (all_logits) {
         // DecoderOnlyModel.forward returns logits for every row; only parity tests ask for them.
         int32_t full = r.alloc((int64_t)n * c.vocab);
         Stream t;
-        q8_linear(t, r.pre.x, r.wlm, full, n, c.d, c.vocab, DJ_LIN_RMSNORM | DJ_LIN_BIAS, r.gf, r.blm);
+        head_rows(r, t, r.pre.x, full, n);
         r.run(t);
         hip(deepj_hip_download(full, all_logits, (int64_t)n * c.vocab));
         r.release(full);
@@ -572,7 +636,7 @@ void *deepj_runner_create(const int32_t cfg[9], int32_t id_base) {
     if (c.vocab <= 0 || c.max_seq <= 0 || c.d <= 0 || c.heads <= 0 || c.layers <= 0 || c.dff <= 0) return nullptr;
     if (c.d % c.heads != 0) return nullptr;
     if (c.kind == 1 && (c.q_rank <= 0 || c.kv_rank <= 0)) return nullptr;
-    if (c.kind != 0 && c.kind != 1) return nullptr;
+    if (c.kind < 0 || c.kind > 2) return nullptr;
     int hd = c.d / c.heads;
     if (hd != 32 && hd != 64 && hd != 128) return nullptr;
     auto *r = new Runner;
@@ -591,9 +655,10 @@ void deepj_runner_destroy(void *h) {
     std::vector<int32_t> ids;
     auto add = [&](int32_t id) { if (id >= 0) ids.push_back(id); };
     for (auto &L : r->layers)
-        for (int32_t id : {L.g1, L.g2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wuk, L.wuv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
+        for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wuk, L.wuv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
     for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state, r->tok,
-                       r->tokens, r->scratch, r->scratch_dec, r->logits, r->last_x})
+                       r->tokens, r->scratch, r->scratch_dec, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
+                       r->pos_table, r->bf})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
         for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv, a->kfull, a->vfull, a->kvexp}) add(id);
@@ -610,7 +675,19 @@ int deepj_runner_set_weight(void *h, const char *name, const float *data, int32_
 
 int deepj_runner_init_seeded(void *h, int64_t seed, int32_t threads) {
     auto *r = static_cast<Runner *>(h);
-    return guarded(r, [&] { init_seeded(*r, seed, threads); });
+    return guarded(r, [&] {
+        if (r->cfg.kind == 2) throw Error("a GPT model is seeded through deepj_runner_init_seeded_gpt (it needs initScale)");
+        init_seeded(*r, seed, threads, 1.0f);
+    });
+}
+
+int deepj_runner_init_seeded_gpt(void *h, int64_t seed, float init_scale, int32_t threads) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] {
+        if (r->cfg.kind != 2) throw Error("deepj_runner_init_seeded_gpt: not a GPT model");
+        if (!std::isfinite(init_scale) || init_scale <= 0.0f) throw Error("initScale must be finite and > 0");   // GPTConfig.java:22-23
+        init_seeded(*r, seed, threads, init_scale);
+    });
 }
 
 int deepj_runner_finalize(void *h) {

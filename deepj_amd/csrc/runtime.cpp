@@ -191,6 +191,8 @@ int stride_of(int op) {
         case DJ_OP_APPEND_ROWS: return 8;
         case DJ_OP_Q8_LINEAR_DYN: return 10;
         case DJ_OP_LLAMA_DECODE: return 0;      // variable: word 1
+        case DJ_OP_LAYERNORM: return 7;
+        case DJ_OP_ADD_POSITIONS: return 7;
         default: return -1;
     }
 }
@@ -376,9 +378,12 @@ void exec_one(Cursor &c) {
             int64_t m = w[4], k = w[5], n = w[6];
             int flags = w[7];
             if (m <= 0 || k <= 0 || n <= 0) fail("OP_Q8_LINEAR: bad shape");
-            if (flags & ~15) fail("OP_Q8_LINEAR: unknown flag bits");
+            if (flags & ~63) fail("OP_Q8_LINEAR: unknown flag bits");
             bool sw = flags & DJ_LIN_SWIGLU;
+            bool ln = flags & DJ_LIN_LAYERNORM;
             if (sw && (flags & DJ_LIN_RESIDUAL)) fail("OP_Q8_LINEAR: SWIGLU cannot be combined with RESIDUAL");
+            if (sw && (flags & (DJ_LIN_LAYERNORM | DJ_LIN_GELU))) fail("OP_Q8_LINEAR: SWIGLU cannot be combined with LAYERNORM or GELU");
+            if (ln && (flags & DJ_LIN_RMSNORM)) fail("OP_Q8_LINEAR: RMSNORM and LAYERNORM are exclusive");
             int64_t rows = sw ? 2 * n : n;
             Q8Linear p;
             p.x = buf(w[1], m * k, op, "x");
@@ -387,7 +392,8 @@ void exec_one(Cursor &c) {
             p.scales = reinterpret_cast<const float *>(p.wq + q8_scale_offset_bytes((int)k, (int)rows));
             p.out = buf(w[3], m * n, op, "out");
             p.m = (int)m; p.k = (int)k; p.n = (int)n; p.flags = flags;
-            p.gamma = (flags & DJ_LIN_RMSNORM) ? buf(w[8], k, op, "gamma") : nullptr;
+            p.gamma = (flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM)) ? buf(w[8], k, op, "gamma") : nullptr;
+            p.beta = ln ? buf(w[10], k, op, "beta") : nullptr;
             p.bias = (flags & DJ_LIN_BIAS) ? buf(w[9], n, op, "bias") : nullptr;
             p.bias2 = ((flags & DJ_LIN_BIAS) && sw) ? buf(w[10], n, op, "bias2") : nullptr;
             p.residual = (flags & DJ_LIN_RESIDUAL) ? buf(w[11], m * n, op, "residual") : nullptr;
@@ -401,6 +407,26 @@ void exec_one(Cursor &c) {
             const float *x = buf(w[1], rows * cols, op, "x"), *gm = buf(w[2], cols, op, "gamma");
             float *o = buf(w[3], rows * cols, op, "out");
             if (run) launch_rmsnorm(s, x, gm, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_LAYERNORM: {
+            // [op, x, gamma, beta, out, rows, cols]
+            int64_t rows = w[5], cols = w[6]; need_positive(op, "rows", rows);
+            if (cols <= 0) fail("OP_LAYERNORM: bad shape");
+            const float *x = buf(w[1], rows * cols, op, "x"), *gm = buf(w[2], cols, op, "gamma");
+            const float *bt = buf(w[3], cols, op, "beta");
+            float *o = buf(w[4], rows * cols, op, "out");
+            if (run) launch_layernorm(s, x, gm, bt, o, (int)rows, (int)cols);
+            break;
+        }
+        case DJ_OP_ADD_POSITIONS: {
+            // [op, x, table, state, rows, d, maxSeq]
+            int64_t rows = w[4], d = w[5], max_seq = w[6]; need_positive(op, "rows", rows);
+            if (d <= 0 || max_seq <= 0) fail("OP_ADD_POSITIONS: bad shape");
+            float *x = buf(w[1], rows * d, op, "x");
+            const float *tb = buf(w[2], max_seq * d, op, "table");
+            const float *st = buf(w[3], 4, op, "state");
+            if (run) launch_add_positions(s, x, tb, reinterpret_cast<const int32_t *>(st), (int)rows, (int)d, (int)max_seq);
             break;
         }
         case DJ_OP_SILU_MUL: {
@@ -702,6 +728,8 @@ const char *op_name(int op) {
         case DJ_OP_Q8_DEQUANTIZE: return "OP_Q8_DEQUANTIZE";
         case DJ_OP_Q8_LINEAR: return "OP_Q8_LINEAR";
         case DJ_OP_RMSNORM: return "OP_RMSNORM";
+        case DJ_OP_LAYERNORM: return "OP_LAYERNORM";
+        case DJ_OP_ADD_POSITIONS: return "OP_ADD_POSITIONS";
         case DJ_OP_SILU_MUL: return "OP_SILU_MUL";
         case DJ_OP_EMBED_GATHER: return "OP_EMBED_GATHER";
         case DJ_OP_ROPE_KV_STORE: return "OP_ROPE_KV_STORE";

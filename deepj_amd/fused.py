@@ -78,10 +78,22 @@ class Stream:
     def q8_dequantize(self, src, dst, k, n, row_off=0, row_step=1, total_rows=None):
         return self.emit(op.OP_Q8_DEQUANTIZE, src, dst, k, n, row_off, row_step, n if total_rows is None else total_rows)
 
-    def q8_linear(self, x, w, out, m, k, n, *, gamma=-1, bias=-1, bias2=-1, residual=-1, swiglu=False):
-        flags = ((op.LIN_RMSNORM if gamma >= 0 else 0) | (op.LIN_BIAS if bias >= 0 else 0) |
-                 (op.LIN_RESIDUAL if residual >= 0 else 0) | (op.LIN_SWIGLU if swiglu else 0))
-        return self.emit(op.OP_Q8_LINEAR, x, w, out, m, k, n, flags, gamma, bias, bias2, residual)
+    def q8_linear(self, x, w, out, m, k, n, *, gamma=-1, bias=-1, bias2=-1, residual=-1, swiglu=False, beta=-1,
+                  gelu=False):
+        """beta >= 0 turns the gamma prologue into LayerNorm (beta travels in the bias2 word)."""
+        layernorm = beta >= 0
+        if layernorm and swiglu:
+            raise ValueError("LayerNorm prologue and SwiGLU share the bias2 word")
+        flags = ((op.LIN_LAYERNORM if layernorm else (op.LIN_RMSNORM if gamma >= 0 else 0)) |
+                 (op.LIN_BIAS if bias >= 0 else 0) | (op.LIN_RESIDUAL if residual >= 0 else 0) |
+                 (op.LIN_SWIGLU if swiglu else 0) | (op.LIN_GELU if gelu else 0))
+        return self.emit(op.OP_Q8_LINEAR, x, w, out, m, k, n, flags, gamma, bias, beta if layernorm else bias2, residual)
+
+    def layernorm(self, x, gamma, beta, out, rows, cols):
+        return self.emit(op.OP_LAYERNORM, x, gamma, beta, out, rows, cols)
+
+    def add_positions(self, x, table, state, rows, d, max_seq):
+        return self.emit(op.OP_ADD_POSITIONS, x, table, state, rows, d, max_seq)
 
     def rmsnorm(self, x, gamma, out, rows, cols): return self.emit(op.OP_RMSNORM, x, gamma, out, rows, cols)
     def silu_mul(self, gate, up, out, n): return self.emit(op.OP_SILU_MUL, gate, up, out, n)

@@ -1,5 +1,5 @@
 """Inference models on the native decode driver: Python faces of the reference's
-LlamaConfig/LlamaModel, DeepSeekConfig/DeepSeekModel and TextGenerator
+LlamaConfig/LlamaModel, DeepSeekConfig/DeepSeekModel, GPTConfig/GPTModel and TextGenerator
 (src/main/java/io/github/kirstenali/deepj/models/...) for the forward/generate path.
 
 `forward(ids)` returns logits for every row like DecoderOnlyModel.forward
@@ -33,6 +33,7 @@ def _lib():
         lib.deepj_runner_last_error.restype = C.c_char_p
         lib.deepj_runner_set_weight.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_int32, C.c_int32]
         lib.deepj_runner_init_seeded.argtypes = [C.c_void_p, C.c_int64, C.c_int32]
+        lib.deepj_runner_init_seeded_gpt.argtypes = [C.c_void_p, C.c_int64, C.c_float, C.c_int32]
         lib.deepj_runner_finalize.argtypes = [C.c_void_p]
         lib.deepj_runner_reset.argtypes = [C.c_void_p]
         lib.deepj_runner_prefill.argtypes = [C.c_void_p, _i32p, C.c_int32, C.c_void_p, C.c_int32]
@@ -114,7 +115,27 @@ class DeepSeekConfig:
     kvRank: int
 
 
-def _validate(cfg) -> None:
+@dataclass(frozen=True)
+class GPTConfig:
+    """GPTConfig.java:8-27: initScale multiplies every parameter after init, gradClipNorm is a training knob."""
+    vocabSize: int
+    maxSeqLen: int
+    dModel: int
+    nHeads: int
+    nLayers: int
+    dFF: int
+    initScale: float = 0.2
+    gradClipNorm: float = 1.0
+
+    def __post_init__(self):
+        _validate(self, head_dims=False)
+        if not np.isfinite(self.initScale) or self.initScale <= 0.0:
+            raise ValueError("initScale must be finite and > 0")
+        if not np.isfinite(self.gradClipNorm) or self.gradClipNorm <= 0.0:
+            raise ValueError("gradClipNorm must be finite and > 0")
+
+
+def _validate(cfg, head_dims: bool = True) -> None:
     # TransformerConfig.validateCommon (TransformerConfig.java:19-31)
     for name in ("vocabSize", "maxSeqLen", "dModel", "nHeads", "nLayers", "dFF"):
         if getattr(cfg, name) <= 0:
@@ -126,7 +147,7 @@ def _validate(cfg) -> None:
             raise ValueError("qRank must be > 0")
         if cfg.kvRank <= 0:
             raise ValueError("kvRank must be > 0")
-    if cfg.dModel // cfg.nHeads not in (32, 64, 128):
+    if head_dims and cfg.dModel // cfg.nHeads not in (32, 64, 128):
         raise ValueError("this backend supports head dims 32, 64 and 128")
 
 
@@ -137,7 +158,7 @@ class _DecoderOnlyModel:
     def __init__(self, cfg, seed: int | None, threads: int = 0):
         _validate(cfg)
         self.cfg = cfg
-        kind = 1 if isinstance(cfg, DeepSeekConfig) else 0
+        kind = 1 if isinstance(cfg, DeepSeekConfig) else (2 if isinstance(cfg, GPTConfig) else 0)
         arr = (C.c_int32 * 9)(kind, cfg.vocabSize, cfg.maxSeqLen, cfg.dModel, cfg.nHeads, cfg.nLayers, cfg.dFF,
                               getattr(cfg, "qRank", 0), getattr(cfg, "kvRank", 0))
         base = _next_id_base[0]
@@ -146,7 +167,10 @@ class _DecoderOnlyModel:
         if not self._h:
             raise ValueError("invalid model configuration")
         if seed is not None:
-            self._check(_lib().deepj_runner_init_seeded(self._h, seed, threads))
+            if kind == 2:
+                self._check(_lib().deepj_runner_init_seeded_gpt(self._h, seed, cfg.initScale, threads))
+            else:
+                self._check(_lib().deepj_runner_init_seeded(self._h, seed, threads))
             self._check(_lib().deepj_runner_finalize(self._h))
 
     def _check(self, rc: int) -> None:
@@ -239,6 +263,17 @@ class DeepSeekModel(_DecoderOnlyModel):
 
     def __init__(self, cfg: DeepSeekConfig, seed: int | None = 42, threads: int = 0):
         super().__init__(cfg, seed, threads)
+
+
+class GPTModel(_DecoderOnlyModel):
+    """new GPTModel(cfg, seed) (GPTModel.java:27-46): LayerNorm blocks with a GELU feed-forward, learned
+    positions, every parameter scaled by cfg.initScale."""
+
+    def __init__(self, cfg: GPTConfig, seed: int | None = 42, threads: int = 0):
+        super().__init__(cfg, seed, threads)
+
+    def gradClipNorm(self) -> float:
+        return self.cfg.gradClipNorm
 
 
 class TextGenerator:

@@ -6,6 +6,8 @@ For the decoder-only models that order is (DecoderOnlyModel.java:79-85, Abstract
 sub-layers {ln1, ln2, attn, mlp}; Linear.java:54-56 = W then b):
     emb, per block [g1, g2, attention matrices, wg, bg, wu, bu, wd, bd], gf, wlm, blm
 i.e. 12 parameters per Llama block and 14 per DeepSeek block - the names `parameter_names` returns.
+GPTModel (GPTModel.java:64-69, LayerNorm1D.java:80-82 = gamma then beta, FNN = its Linears in order):
+    emb, pos, per block [g1, be1, g2, be2, wq, wk, wv, wo, wg, bg, wd, bd], gf, bf, wlm, blm
 """
 from __future__ import annotations
 
@@ -14,10 +16,16 @@ import struct
 
 import numpy as np
 
-from .models import DeepSeekConfig, LlamaConfig
+from .models import DeepSeekConfig, GPTConfig, LlamaConfig
 
 
 def parameter_names(cfg) -> list[str]:
+    if isinstance(cfg, GPTConfig):
+        per = ["g1", "be1", "g2", "be2", "wq", "wk", "wv", "wo", "wg", "bg", "wd", "bd"]
+        names = ["emb", "pos"]
+        for l in range(cfg.nLayers):
+            names += [f"L{l}.{w}" for w in per]
+        return names + ["gf", "bf", "wlm", "blm"]
     attn = ["wdq", "wuq", "wdkv", "wuk", "wuv", "wo"] if isinstance(cfg, DeepSeekConfig) else ["wq", "wk", "wv", "wo"]
     per = ["g1", "g2"] + attn + ["wg", "bg", "wu", "bu", "wd", "bd"]
     names = ["emb"]
@@ -29,6 +37,9 @@ def parameter_names(cfg) -> list[str]:
 def parameter_shapes(cfg) -> list[tuple[int, int]]:
     """(rows, cols) of every parameter, reference orientation (weights [dIn x dOut], vectors [1 x n])."""
     d, f, v = cfg.dModel, cfg.dFF, cfg.vocabSize
+    if isinstance(cfg, GPTConfig):
+        per = [(1, d)] * 4 + [(d, d)] * 4 + [(d, f), (1, f), (f, d), (1, d)]
+        return [(v, d), (cfg.maxSeqLen, d)] + per * cfg.nLayers + [(1, d), (1, d), (d, v), (1, v)]
     if isinstance(cfg, DeepSeekConfig):
         q, k = cfg.qRank, cfg.kvRank
         attn = [(d, q), (q, d), (d, k), (k, d), (k, d), (d, d)]

@@ -111,6 +111,10 @@ enum {
      *           bit1: add bias[N]          bit2: add residual[M x N]
      *           bit3: SwiGLU: w has 2N rows (gate n at row 2n, up n at 2n+1),
      *                 out = SiLU(gate + bias) * (up + bias2)
+     *           bit4: LayerNorm prologue, f(x) = (x - mean) / sqrt(var + 1e-5) * gamma + beta with the beta
+     *                 buffer in the bias2 word (J/layers/transformer/norm/LayerNorm1D.java:34-66)
+     *           bit5: GELU (tanh form) on x.W + bias, before the residual (J/activations/GELU.java:15-18)
+     *           bit3 excludes bits 2, 4 and 5; bit0 excludes bit4
      * RMSNORM       [op, x, gamma, out, rows, cols]
      * SILU_MUL      [op, gate, up, out, n]            out = gate*sigmoid(gate)*up
      * EMBED_GATHER  [op, table, ids, out, nIds, d, vocab, idsOff]  ids are int32 words
@@ -150,15 +154,21 @@ enum {
      *     wqkv [3d x d], wgu interleaved [2 dFF x d], all weights Q8.  scratch >= H*nsplit*(hd+4) floats, argbuf >=
      *     2*grid floats (deepj_hip_llama_decode_plan), sync = deepj_hip_llama_decode_sync_floats() floats, zero-filled
      *     once.  Not capturable into a graph; calls that overlap on one device are not supported.
+     * LAYERNORM     [op, x, gamma, beta, out, rows, cols]      J/layers/transformer/norm/LayerNorm1D.java:34-66
+     * ADD_POSITIONS [op, x, table, state, rows, d, maxSeq]
+     *     x[i, :] += table[state[0] + i, :]: the learned positional rows of J/models/gpt/GPTModel.java:52-54 for
+     *     rows that sit at positions state[0].. of the sequence
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
-    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82
+    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82, DJ_OP_LAYERNORM = 83,
+    DJ_OP_ADD_POSITIONS = 84
 };
 
-enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8 };
+enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8, DJ_LIN_LAYERNORM = 16,
+       DJ_LIN_GELU = 32 };
 
 /* Buffer sizes LLAMA_DECODE needs on this device: workgroups launched, key splits per head, floats of
  * `scratch` and `argbuf`; and the floats of its `sync` buffer. */
@@ -185,15 +195,20 @@ float   deepj_host_random_next_float(void *rng);
  * TextGenerator of the reference (J/models/DecoderOnlyModel.java:58-64,
  * J/models/TextGenerator.java:66-181) with a device-resident KV cache, Q8 weights and one
  * fused command stream per token replayed as a HIP graph.  It uses only the functions
- * above.  cfg = {kind (0 Llama, 1 DeepSeek), vocab, maxSeq, dModel, nHeads, nLayers, dFF,
+ * above.  cfg = {kind (0 Llama, 1 DeepSeek, 2 GPT), vocab, maxSeq, dModel, nHeads, nLayers, dFF,
  * qRank, kvRank}; id_base = first buffer id the runner may use.  Weight names: "emb",
  * "gf", "wlm", "blm", "L<i>.g1|g2|wq|wk|wv|wo|wdq|wuq|wdkv|wuk|wuv|wg|bg|wu|bu|wd|bd";
- * matrices in the reference's [dIn x dOut] fp32 orientation. */
+ * GPT (J/models/gpt/GPTModel.java:27-45, J/layers/transformer/blocks/GPTTransformerBlock.java:52-73) adds
+ * "pos" [maxSeq x dModel], "bf" and "L<i>.be1|be2" (LayerNorm betas; g1, g2, gf are the gammas), names its
+ * FNN's two Linears wg,bg (dModel -> dFF) and wd,bd (dFF -> dModel) and has no wu,bu.
+ * Matrices in the reference's [dIn x dOut] fp32 orientation. */
 void       *deepj_runner_create(const int32_t cfg[9], int32_t id_base);   /* NULL: invalid config */
 void        deepj_runner_destroy(void *runner);
 const char *deepj_runner_last_error(void *runner);
 int deepj_runner_set_weight(void *runner, const char *name, const float *data, int32_t rows, int32_t cols);
 int deepj_runner_init_seeded(void *runner, int64_t seed, int32_t threads);  /* new LlamaModel(cfg, seed) */
+/* new GPTModel(cfg, seed) with GPTConfig.initScale = init_scale (J/models/gpt/GPTModel.java:27-46,76-81) */
+int deepj_runner_init_seeded_gpt(void *runner, int64_t seed, float init_scale, int32_t threads);
 int deepj_runner_finalize(void *runner);
 int deepj_runner_reset(void *runner);
 int deepj_runner_prefill(void *runner, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next);

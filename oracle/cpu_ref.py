@@ -351,6 +351,7 @@ def slice_rows(t, idx):
 # ── layers ──────────────────────────────────────────────────────────────────
 _sig("ref_linear", f32p, f32p, f32p, f32p, _I, _I, _I)
 _sig("ref_rmsnorm", f32p, f32p, f32p, _I, _I)
+_sig("ref_layernorm", f32p, f32p, f32p, f32p, _I, _I)
 _sig("ref_swiglu", f32p, f32p, f32p, f32p, f32p, f32p, f32p, f32p, _I, _I, _I)
 _sig("ref_rope_tables", _I, _I, f32p, f32p)
 _sig("ref_rope_apply", f32p, f32p, _I, _I, _I, f32p, f32p, _I)
@@ -378,6 +379,13 @@ def rmsnorm(x, gamma):
     x, gamma = f32(x), f32(gamma).reshape(1, -1)
     out = np.empty_like(x)
     lib.ref_rmsnorm(_fp(x), _fp(gamma), _fp(out), x.shape[0], x.shape[1])
+    return out
+
+
+def layernorm(x, gamma, beta):
+    x, gamma, beta = f32(x), f32(gamma).reshape(1, -1), f32(beta).reshape(1, -1)
+    out = np.empty_like(x)
+    lib.ref_layernorm(_fp(x), _fp(gamma), _fp(beta), _fp(out), x.shape[0], x.shape[1])
     return out
 
 
@@ -471,7 +479,7 @@ def q8_roundtrip(w):
 
 class _Cfg(C.Structure):
     _fields_ = [("kind", _I), ("vocab", _I), ("max_seq", _I), ("d", _I), ("heads", _I), ("layers", _I),
-                ("dff", _I), ("q_rank", _I), ("kv_rank", _I)]
+                ("dff", _I), ("q_rank", _I), ("kv_rank", _I), ("init_scale", _F)]
 
 
 lib.ref_set_fast_fill.argtypes = [_I]
@@ -494,17 +502,23 @@ lib.ref_generate.restype = _I
 
 
 class Model:
-    """LlamaModel / DeepSeekModel of the reference, seeded init included."""
+    """LlamaModel / DeepSeekModel / GPTModel of the reference, seeded init included."""
 
-    def __init__(self, *, vocab, max_seq, d, heads, layers, dff, seed, q_rank=0, kv_rank=0, timing_only_fill=False):
+    def __init__(self, *, vocab, max_seq, d, heads, layers, dff, seed, q_rank=0, kv_rank=0, timing_only_fill=False,
+                 gpt=False, init_scale=0.2):
         """timing_only_fill: weights from a cheap hash instead of the seeded Gaussian stream - same
-        sizes and arithmetic, different values; only for measuring the CPU path's speed."""
-        self.kind = 1 if q_rank else 0
+        sizes and arithmetic, different values; only for measuring the CPU path's speed.
+        gpt: GPTModel (LayerNorm, GELU FNN, learned positions), every parameter times init_scale
+        (GPTConfig.java default 0.2)."""
+        self.kind = 2 if gpt else (1 if q_rank else 0)
+        if gpt and q_rank:
+            raise ValueError("a GPT model has no latent ranks")
         if vocab <= 0 or max_seq <= 0 or d <= 0 or heads <= 0 or layers <= 0 or dff <= 0:
             raise ValueError("config values must be > 0")
         if d % heads != 0:
             raise ValueError("dModel must be divisible by nHeads")
-        self.cfg = _Cfg(self.kind, vocab, max_seq, d, heads, layers, dff, q_rank, kv_rank)
+        self.cfg = _Cfg(self.kind, vocab, max_seq, d, heads, layers, dff, q_rank, kv_rank, init_scale)
+        self.init_scale = init_scale
         self.vocab, self.max_seq, self.d, self.heads, self.layers, self.dff = vocab, max_seq, d, heads, layers, dff
         self.q_rank, self.kv_rank = q_rank, kv_rank
         lib.ref_set_fast_fill(1 if timing_only_fill else 0)
@@ -533,17 +547,26 @@ class Model:
         return np.ctypeslib.as_array(p, shape=(r.value, c.value))
 
     def weight_names(self):
-        names = ["emb"]
-        per = (["g1", "g2", "wq", "wk", "wv", "wo"] if self.kind == 0 else
-               ["g1", "g2", "wdq", "wuq", "wdkv", "wuk", "wuv", "wo"]) + ["wg", "bg", "wu", "bu", "wd", "bd"]
+        if self.kind == 2:      # GPTModel parameter order: tokEmb, posEmb, blocks {ln1, ln2, attn, mlp}, normF, lmHead
+            names = ["emb", "pos"]
+            per = ["g1", "be1", "g2", "be2", "wq", "wk", "wv", "wo", "wg", "bg", "wd", "bd"]
+            tail = ["gf", "bf", "wlm", "blm"]
+        else:
+            names = ["emb"]
+            per = (["g1", "g2", "wq", "wk", "wv", "wo"] if self.kind == 0 else
+                   ["g1", "g2", "wdq", "wuq", "wdkv", "wuk", "wuv", "wo"]) + ["wg", "bg", "wu", "bu", "wd", "bd"]
+            tail = ["gf", "wlm", "blm"]
         for l in range(self.layers):
             names += [f"L{l}.{w}" for w in per]
-        return names + ["gf", "wlm", "blm"]
+        return names + tail
 
     def forward(self, ids) -> np.ndarray:
         ids = i32(ids)
         out = np.empty((len(ids), self.vocab), dtype=np.float32)
-        if lib.ref_model_forward(self._h, _ip(ids), len(ids), _fp(out)) != 0:
+        rc = lib.ref_model_forward(self._h, _ip(ids), len(ids), _fp(out))
+        if rc == -2:
+            raise ValueError(f"seqLen {len(ids)} exceeds maxSeq {self.max_seq}")
+        if rc != 0:
             raise ValueError("Token id out of range")
         return out
 

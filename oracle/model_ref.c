@@ -39,6 +39,32 @@ void ref_rmsnorm(const float *x, const float *gamma, float *out, int rows, int d
     free(sq); free(mean); free(rms); free(xhat);
 }
 
+/* LayerNorm1D.java:34-66: mean = meanAlongRows, var = varianceAlongRows (population), std = sqrt(var + EPS),
+ * xHat = (x - mean) / std, out = xHat * gamma + beta; EPS = 1e-5f (LayerNorm1D.java:15). */
+void ref_layernorm(const float *x, const float *gamma, const float *beta, float *out, int rows, int dim) {
+    int64_t n = (int64_t)rows * dim;
+    float *mean = falloc(rows), *var = falloc(rows), *std = falloc(rows), *c = falloc(n), *xhat = falloc(n), *sc = falloc(n);
+    ref_mean_along_rows(x, mean, rows, dim);
+    ref_variance_along_rows(x, var, rows, dim);
+    ref_add_scalar(var, 1e-5f, std, rows, 1);
+    ref_sqrt(std, std, rows, 1);
+    ref_subtract_broadcast_cols(x, mean, c, rows, dim);
+    ref_divide_broadcast_cols(c, std, xhat, rows, dim);
+    ref_multiply_broadcast_rows(xhat, gamma, sc, rows, dim);
+    ref_add_row_vector(sc, beta, out, rows, dim);
+    free(mean); free(var); free(std); free(c); free(xhat); free(sc);
+}
+
+/* FNN.java:57-73 with one hidden layer and GELU: Linear -> GELU -> Linear */
+static void gpt_fnn(const float *x, const float *w1, const float *b1, const float *w2, const float *b2,
+                    float *out, int rows, int d, int dff) {
+    float *z = falloc((int64_t)rows * dff), *hh = falloc((int64_t)rows * dff);
+    ref_linear(x, w1, b1, z, rows, d, dff);
+    ref_gelu(z, hh, rows, dff);
+    ref_linear(hh, w2, b2, out, rows, dff, d);
+    free(z); free(hh);
+}
+
 /* SiLU.java:20-24: input.multiply(input.sigmoidActivation()) */
 void ref_silu(const float *x, float *out, int rows, int cols) {
     float *s = falloc((int64_t)rows * cols);
@@ -287,6 +313,16 @@ ref_model *ref_model_create(const ref_config *cfg, int64_t seed) {
     for (int l = 0; l < cfg->layers; l++) {
         ref_layer *L = &m->layer[l];
         L->g1 = ones(d); L->g2 = ones(d);
+        if (cfg->kind == 2) {       /* GPTTransformerBlock.java:45-50: ln1, ln2, attention, then the FNN's two Linears */
+            L->be1 = falloc(d); L->be2 = falloc(d);
+            L->wq = rand_tensor(d, d, &stack_r);
+            L->wk = rand_tensor(d, d, &stack_r);
+            L->wv = rand_tensor(d, d, &stack_r);
+            L->wo = rand_tensor(d, d, &stack_r);
+            L->wg = rand_tensor(d, dff, &stack_r);  L->bg = falloc(dff);
+            L->wd = rand_tensor(dff, d, &stack_r);  L->bd = falloc(d);
+            continue;
+        }
         if (cfg->kind == 0) {       /* MultiHeadSelfAttention.java:47-50 */
             L->wq = rand_tensor(d, d, &stack_r);
             L->wk = rand_tensor(d, d, &stack_r);
@@ -311,6 +347,27 @@ ref_model *ref_model_create(const ref_config *cfg, int64_t seed) {
     m->cos_t = falloc((int64_t)cfg->max_seq * (hd / 2));
     m->sin_t = falloc((int64_t)cfg->max_seq * (hd / 2));
     ref_rope_tables(hd, cfg->max_seq, m->cos_t, m->sin_t);
+    if (cfg->kind == 2) {
+        /* GPTModel.java:27-45: final LayerNorm, positional table from Random(seed + 2); no rotary embedding:
+         * the incremental path keeps its rotation code and gets the identity (cos 1, sin 0: x*1 - y*0 == x). */
+        jrandom pos_r; jr_init(&pos_r, seed + 2);
+        m->bf = falloc(d);
+        m->pos = rand_tensor(cfg->max_seq, d, &pos_r);
+        for (int64_t i = 0; i < (int64_t)cfg->max_seq * (hd / 2); i++) { m->cos_t[i] = 1.0f; m->sin_t[i] = 0.0f; }
+        float f = cfg->init_scale;
+        if (f != 1.0f) {            /* applyInitScale: every parameter, gains and biases included */
+            #define SCALE(p, n) do { for (int64_t i_ = 0; i_ < (int64_t)(n); i_++) (p)[i_] *= f; } while (0)
+            SCALE(m->emb, (int64_t)cfg->vocab * d); SCALE(m->pos, (int64_t)cfg->max_seq * d);
+            for (int l = 0; l < cfg->layers; l++) {
+                ref_layer *L = &m->layer[l];
+                SCALE(L->g1, d); SCALE(L->be1, d); SCALE(L->g2, d); SCALE(L->be2, d);
+                SCALE(L->wq, (int64_t)d * d); SCALE(L->wk, (int64_t)d * d); SCALE(L->wv, (int64_t)d * d); SCALE(L->wo, (int64_t)d * d);
+                SCALE(L->wg, (int64_t)d * dff); SCALE(L->bg, dff); SCALE(L->wd, (int64_t)dff * d); SCALE(L->bd, d);
+            }
+            SCALE(m->gf, d); SCALE(m->bf, d); SCALE(m->wlm, (int64_t)d * cfg->vocab); SCALE(m->blm, cfg->vocab);
+            #undef SCALE
+        }
+    }
     return m;
 }
 
@@ -321,7 +378,9 @@ void ref_model_free(ref_model *m) {
         free(L->g1); free(L->g2); free(L->wq); free(L->wk); free(L->wv); free(L->wo);
         free(L->wdq); free(L->wuq); free(L->wdkv); free(L->wuk); free(L->wuv);
         free(L->wg); free(L->bg); free(L->wu); free(L->bu); free(L->wd); free(L->bd);
+        free(L->be1); free(L->be2);
     }
+    free(m->bf); free(m->pos);
     free(m->layer); free(m->emb); free(m->gf); free(m->wlm); free(m->blm);
     free(m->cos_t); free(m->sin_t); free(m->kcache); free(m->vcache);
     free(m);
@@ -331,6 +390,12 @@ void ref_model_q8_roundtrip(ref_model *m) {
     const ref_config *c = &m->cfg;
     for (int l = 0; l < c->layers; l++) {
         ref_layer *L = &m->layer[l];
+        if (c->kind == 2) {
+            q8_roundtrip(L->wq, c->d, c->d); q8_roundtrip(L->wk, c->d, c->d);
+            q8_roundtrip(L->wv, c->d, c->d); q8_roundtrip(L->wo, c->d, c->d);
+            q8_roundtrip(L->wg, c->d, c->dff); q8_roundtrip(L->wd, c->dff, c->d);
+            continue;
+        }
         if (c->kind == 0) {
             q8_roundtrip(L->wq, c->d, c->d); q8_roundtrip(L->wk, c->d, c->d);
             q8_roundtrip(L->wv, c->d, c->d);
@@ -351,6 +416,8 @@ float *ref_model_weight(ref_model *m, const char *name, int *rows, int *cols) {
     int r = 0, k = 0; float *p = NULL;
     if (!strcmp(name, "emb")) { p = m->emb; r = c->vocab; k = c->d; }
     else if (!strcmp(name, "gf")) { p = m->gf; r = 1; k = c->d; }
+    else if (!strcmp(name, "bf") && m->bf) { p = m->bf; r = 1; k = c->d; }
+    else if (!strcmp(name, "pos") && m->pos) { p = m->pos; r = c->max_seq; k = c->d; }
     else if (!strcmp(name, "wlm")) { p = m->wlm; r = c->d; k = c->vocab; }
     else if (!strcmp(name, "blm")) { p = m->blm; r = 1; k = c->vocab; }
     else if (name[0] == 'L') {
@@ -359,7 +426,9 @@ float *ref_model_weight(ref_model *m, const char *name, int *rows, int *cols) {
         if (!dot || l < 0 || l >= c->layers) return NULL;
         const char *w = dot + 1;
         ref_layer *L = &m->layer[l];
-        if (!strcmp(w, "g1")) { p = L->g1; r = 1; k = c->d; }
+        if (!strcmp(w, "be1")) { p = L->be1; r = 1; k = c->d; }
+        else if (!strcmp(w, "be2")) { p = L->be2; r = 1; k = c->d; }
+        else if (!strcmp(w, "g1")) { p = L->g1; r = 1; k = c->d; }
         else if (!strcmp(w, "g2")) { p = L->g2; r = 1; k = c->d; }
         else if (!strcmp(w, "wq")) { p = L->wq; r = c->d; k = c->d; }
         else if (!strcmp(w, "wk")) { p = L->wk; r = c->d; k = c->d; }
@@ -390,6 +459,34 @@ static int embed(const ref_model *m, const int32_t *ids, int n, float *x) {
     return 0;
 }
 
+/* GPTModel.java:52-54: token rows plus position rows 0..n-1 (PositionalEmbedding slices the first n rows);
+ * pos0 is the position of the first row for the incremental path. */
+static void add_positions(const ref_model *m, float *x, int n, int pos0) {
+    int d = m->cfg.d;
+    float *t = falloc((int64_t)n * d);
+    ref_add(x, m->pos + (int64_t)pos0 * d, t, n, d);
+    memcpy(x, t, (size_t)n * d * sizeof(float));
+    free(t);
+}
+
+/* DecoderOnlyModel.java:58-64 with GPT blocks (GPTTransformerBlock.java:65-73) */
+static void gpt_forward(ref_model *m, float *x, float *h, float *a, float *x2, int n, float *logits) {
+    const ref_config *c = &m->cfg;
+    int d = c->d;
+    add_positions(m, x, n, 0);
+    for (int l = 0; l < c->layers; l++) {
+        const ref_layer *L = &m->layer[l];
+        ref_layernorm(x, L->g1, L->be1, h, n, d);
+        ref_mhsa_forward(h, L->wq, L->wk, L->wv, L->wo, a, n, d, c->heads, NULL, NULL, 1);
+        ref_add(x, a, x2, n, d);
+        ref_layernorm(x2, L->g2, L->be2, h, n, d);
+        gpt_fnn(h, L->wg, L->bg, L->wd, L->bd, a, n, d, c->dff);
+        ref_add(x2, a, x, n, d);
+    }
+    ref_layernorm(x, m->gf, m->bf, h, n, d);
+    ref_linear(h, m->wlm, m->blm, logits, n, d, c->vocab);
+}
+
 /* DecoderOnlyModel.java:58-64 with Llama/DeepSeek blocks */
 int ref_model_forward(ref_model *m, const int32_t *ids, int n, float *logits) {
     const ref_config *c = &m->cfg;
@@ -397,6 +494,12 @@ int ref_model_forward(ref_model *m, const int32_t *ids, int n, float *logits) {
     int64_t nd = (int64_t)n * d;
     float *x = falloc(nd), *h = falloc(nd), *a = falloc(nd), *x2 = falloc(nd);
     if (embed(m, ids, n, x) != 0) { free(x); free(h); free(a); free(x2); return -1; }
+    if (c->kind == 2) {
+        if (n > c->max_seq) { free(x); free(h); free(a); free(x2); return -2; }   /* PositionalEmbedding.java: seqLen > maxSeqLen throws */
+        gpt_forward(m, x, h, a, x2, n, logits);
+        free(x); free(h); free(a); free(x2);
+        return 0;
+    }
     for (int l = 0; l < c->layers; l++) {
         const ref_layer *L = &m->layer[l];
         ref_rmsnorm(x, L->g1, h, n, d);
@@ -492,10 +595,13 @@ int ref_model_forward_cached(ref_model *m, const int32_t *ids, int n, float *log
     float *q = falloc(nd), *k = falloc(nd), *v = falloc(nd), *mg = falloc(nd);
     int rc = embed(m, ids, n, x);
     if (rc == 0) {
+        int gpt = c->kind == 2;
+        if (gpt) add_positions(m, x, n, m->cached);
         for (int l = 0; l < c->layers; l++) {
             const ref_layer *L = &m->layer[l];
-            ref_rmsnorm(x, L->g1, h, n, d);
-            if (c->kind == 0) {
+            if (gpt) ref_layernorm(x, L->g1, L->be1, h, n, d);
+            else ref_rmsnorm(x, L->g1, h, n, d);
+            if (c->kind != 1) {
                 ref_matmul(h, L->wq, q, n, d, d);
                 ref_matmul(h, L->wk, k, n, d, d);
                 ref_matmul(h, L->wv, v, n, d, d);
@@ -511,18 +617,21 @@ int ref_model_forward_cached(ref_model *m, const int32_t *ids, int n, float *log
             cached_attention(m, l, q, k, v, mg, n);
             ref_matmul(mg, L->wo, a, n, d, d);
             ref_add(x, a, x2, n, d);
-            ref_rmsnorm(x2, L->g2, h, n, d);
-            ref_swiglu(h, L->wg, L->bg, L->wu, L->bu, L->wd, L->bd, a, n, d, c->dff);
+            if (gpt) {
+                ref_layernorm(x2, L->g2, L->be2, h, n, d);
+                gpt_fnn(h, L->wg, L->bg, L->wd, L->bd, a, n, d, c->dff);
+            } else {
+                ref_rmsnorm(x2, L->g2, h, n, d);
+                ref_swiglu(h, L->wg, L->bg, L->wu, L->bu, L->wd, L->bd, a, n, d, c->dff);
+            }
             ref_add(x2, a, x, n, d);
         }
         m->cached += n;
-        if (last_only) {
-            ref_rmsnorm(x + (int64_t)(n - 1) * d, m->gf, h, 1, d);
-            ref_linear(h, m->wlm, m->blm, logits, 1, d, c->vocab);
-        } else {
-            ref_rmsnorm(x, m->gf, h, n, d);
-            ref_linear(h, m->wlm, m->blm, logits, n, d, c->vocab);
-        }
+        int rows = last_only ? 1 : n;
+        const float *xr = last_only ? x + (int64_t)(n - 1) * d : x;
+        if (gpt) ref_layernorm(xr, m->gf, m->bf, h, rows, d);
+        else ref_rmsnorm(xr, m->gf, h, rows, d);
+        ref_linear(h, m->wlm, m->blm, logits, rows, d, c->vocab);
     }
     free(x); free(h); free(a); free(x2); free(q); free(k); free(v); free(mg);
     return rc;

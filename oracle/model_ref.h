@@ -59,6 +59,9 @@ void ref_mla_forward(const float *x, const float *wdq, const float *wuq, const f
                      int seq, int d, int n_heads, int q_rank, int kv_rank,
                      const float *cos_t, const float *sin_t);
 
+/* LayerNorm1D.java:34-66: (x - mean) / sqrt(var + 1e-5) * gamma + beta, population variance */
+void ref_layernorm(const float *x, const float *gamma, const float *beta, float *out, int rows, int dim);
+
 /* ── Q8 (this build's format; see header comment) ───────────────────── */
 /* w is [K x N] row-major fp32 (the reference's weight orientation, Linear.java:13).
  * q is [N x Kp] int8 with Kp = K rounded up to 32 (zero padded), scales [N x Kp/32]. */
@@ -68,16 +71,18 @@ void ref_q8_dequantize(const int8_t *q, const float *scales, int k, int n, float
 
 /* ── models ─────────────────────────────────────────────────────────── */
 typedef struct {
-    int kind;          /* 0 = Llama, 1 = DeepSeek (MLA) */
+    int kind;          /* 0 = Llama, 1 = DeepSeek (MLA), 2 = GPT (LayerNorm, GELU FNN, learned positions) */
     int vocab, max_seq, d, heads, layers, dff;
     int q_rank, kv_rank;   /* DeepSeek only */
+    float init_scale;      /* GPT only: every parameter is multiplied by it after init (GPTModel.java:76-81) */
 } ref_config;
 
 typedef struct {
     float *g1, *g2;
     float *wq, *wk, *wv, *wo;                 /* Llama */
     float *wdq, *wuq, *wdkv, *wuk, *wuv;      /* DeepSeek (wo shared above) */
-    float *wg, *bg, *wu, *bu, *wd, *bd;
+    float *wg, *bg, *wu, *bu, *wd, *bd;       /* GPT: wg,bg = first FNN linear, wd,bd = second; wu,bu unused */
+    float *be1, *be2;                         /* GPT: LayerNorm betas (g1, g2 are the gammas) */
 } ref_layer;
 
 typedef struct {
@@ -85,6 +90,8 @@ typedef struct {
     float *emb;            /* [vocab x d] */
     ref_layer *layer;
     float *gf;             /* final norm gain */
+    float *bf;             /* GPT: final LayerNorm beta */
+    float *pos;            /* GPT: positional embedding [max_seq x d] */
     float *wlm, *blm;      /* [d x vocab], [vocab] */
     float *cos_t, *sin_t;  /* [max_seq x hd/2] */
     /* incremental state (not in the reference) */

@@ -318,3 +318,135 @@ def test_threading_never_changes_results():
     ref.set_column_parallel(True); y5c = ref.matmul(a[:2], b); ref.set_column_parallel(False)
     ref.set_threads(1)
     assert np.array_equal(y1, y5) and np.array_equal(s1, s5) and np.array_equal(y1[:2], y5c)
+
+
+# ── GPT path: LayerNorm, GELU feed-forward, learned positions ────────────────
+# The reference's tests hold no forward known answers for these layers (LayerNorm1DTest.java and FNNTest.java
+# check gradients and loss decrease only), so they are pinned by closed forms and fp64 brute force.
+
+def test_layernorm_closed_forms_and_fp64():
+    g = np.array([[2.0, -1.0, 0.5, 3.0]], np.float32)
+    b = np.array([[0.1, 0.2, -0.3, 0.4]], np.float32)
+    # a constant row has xHat = 0: the output is beta whatever gamma is
+    assert np.array_equal(ref.layernorm(np.full((1, 4), 7.5, np.float32), g, b), b)
+    # two columns (a, c): mean (a+c)/2, population variance ((a-c)/2)^2, xHat = +-h/sqrt(h^2 + 1e-5)
+    a, c = 3.0, 1.0
+    h = (a - c) / 2
+    xh = h / np.sqrt(h * h + 1e-5)
+    close(ref.layernorm([[a, c]], [[1.0, 1.0]], [[0.0, 0.0]]), [[xh, -xh]], atol=1e-7)
+    # a spread of the size of sqrt(eps) separates sqrt(var + eps) from sqrt(var) + eps
+    x = (np.float32(0.03) * rnd(5, 4, 90)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    mu = x64.mean(1, keepdims=True)
+    var = ((x64 - mu) ** 2).sum(1, keepdims=True) / x.shape[1]
+    close(ref.layernorm(x, g, b), (x64 - mu) / np.sqrt(var + 1e-5) * g + b, atol=1e-5, rtol=1e-5)
+    wrong_eps = (x64 - mu) / (np.sqrt(var) + 1e-5) * g + b
+    assert np.abs(ref.layernorm(x, g, b) - wrong_eps).max() > 1e-2
+    x = rnd(6, 24, 91)
+    x64 = x.astype(np.float64)
+    g, b = rnd(1, 24, 92) * 10, rnd(1, 24, 93)
+    mu = x64.mean(1, keepdims=True)
+    var = x64.var(1, keepdims=True)
+    close(ref.layernorm(x, g, b), (x64 - mu) / np.sqrt(var + 1e-5) * g + b, atol=1e-5)
+    assert np.abs(ref.layernorm(x, g, b) - ((x64 - mu) / np.sqrt(var * 24 / 23 + 1e-5) * g + b)).max() > 1e-3
+    # gamma = 1, beta = 0: rows have mean 0 and variance var / (var + eps); shifting a row changes nothing
+    y = ref.layernorm(x, np.ones((1, 24)), np.zeros((1, 24))).astype(np.float64)
+    close(y.mean(1), np.zeros(6), atol=1e-6)
+    close(y.var(1), (var / (var + 1e-5)).reshape(-1), atol=1e-5)
+    close(ref.layernorm(x + np.float32(0.5), g, b), ref.layernorm(x, g, b), atol=2e-5)
+
+
+GPT_TINY = dict(vocab=11, max_seq=8, d=4, heads=2, layers=1, dff=8)    # GPTModelTest.java:64-82
+
+
+def test_gpt_init_wiring_scale_and_parameter_count():
+    base = ref.Model(seed=1234, gpt=True, init_scale=1.0, **GPT_TINY)
+    scaled = ref.Model(seed=1234, gpt=True, **GPT_TINY)                # GPTConfig default initScale 0.2
+    # GPTModelTest.java:21-33: first parameter's sumAbs ratio is the init scale
+    ratio = float(np.abs(scaled.weight("emb")).astype(np.float64).sum() / np.abs(base.weight("emb")).astype(np.float64).sum())
+    assert abs(ratio - 0.2) < 1e-6
+    # GPTModelTest.java:85-97: 1 + 1 + 12 per block + 2 + 2 parameters
+    assert len(base.weight_names()) == 1 + 1 + 12 * 1 + 2 + 2
+    m = ref.Model(seed=5, gpt=True, init_scale=1.0, vocab=50, max_seq=16, d=32, heads=4, layers=2, dff=48)
+    assert len(m.weight_names()) == 1 + 1 + 12 * 2 + 2 + 2
+    # RNG wiring (GPTModel.java:27-45): token table Random(seed), blocks a second Random(seed) drawn in
+    # construction order (attention, then the FNN's Linears), head Random(seed + 1), positions Random(seed + 2)
+    assert np.array_equal(m.weight("emb"), ref.JavaRandom(5).tensor(50, 32))
+    r = ref.JavaRandom(5)
+    for name, shape in [("L0.wq", (32, 32)), ("L0.wk", (32, 32)), ("L0.wv", (32, 32)), ("L0.wo", (32, 32)),
+                        ("L0.wg", (32, 48)), ("L0.wd", (48, 32)), ("L1.wq", (32, 32))]:
+        assert np.array_equal(m.weight(name), r.tensor(*shape)), name
+    assert np.array_equal(m.weight("wlm"), ref.JavaRandom(6).tensor(32, 50))
+    assert np.array_equal(m.weight("pos"), ref.JavaRandom(7).tensor(16, 32))
+    # every parameter is scaled, gains and biases included (GPTModel.java:76-81)
+    s = ref.Model(seed=5, gpt=True, init_scale=0.2, vocab=50, max_seq=16, d=32, heads=4, layers=2, dff=48)
+    f = np.float32(0.2)
+    for name in s.weight_names():
+        assert np.array_equal(s.weight(name), m.weight(name) * f), name
+    assert np.all(s.weight("L1.g2") == f) and np.all(s.weight("gf") == f) and np.all(s.weight("L0.be1") == 0)
+
+
+def brute_gpt_forward(m, ids):
+    """GPTModel.forward in fp64 numpy, written from the layer definitions."""
+    w = lambda n: m.weight(n).astype(np.float64)
+    def ln(x, g, b):
+        mu = x.mean(1, keepdims=True)
+        return (x - mu) / np.sqrt(((x - mu) ** 2).mean(1, keepdims=True) + 1e-5) * g + b
+    def gelu(x):
+        return 0.5 * x * (1 + np.tanh(np.sqrt(2 / np.pi) * (x + 0.044715 * x ** 3)))
+    x = w("emb")[ids] + w("pos")[:len(ids)]
+    for l in range(m.layers):
+        p = lambda n: m.weight(f"L{l}.{n}")
+        h = ln(x, w(f"L{l}.g1"), w(f"L{l}.be1"))
+        x = x + brute_attention(h, p("wq"), p("wk"), p("wv"), p("wo"), m.heads)
+        h = ln(x, w(f"L{l}.g2"), w(f"L{l}.be2"))
+        x = x + gelu(h @ w(f"L{l}.wg") + w(f"L{l}.bg")) @ w(f"L{l}.wd") + w(f"L{l}.bd")
+    return ln(x, w("gf"), w("bf")) @ w("wlm") + w("blm")
+
+
+def test_gpt_forward_matches_layers_and_fp64_brute_force():
+    cfg = dict(vocab=50, max_seq=16, d=32, heads=4, layers=2, dff=48)
+    m = ref.Model(seed=5, gpt=True, init_scale=0.2, **cfg)
+    # make betas and biases non-trivial so that a dropped one shows
+    for i, name in enumerate(n for n in m.weight_names() if n.split(".")[-1] in ("be1", "be2", "bg", "bd", "bf", "blm")):
+        v = m.weight(name)
+        v[:] = rnd(1, v.shape[1], 300 + i)
+    ids = ref.JavaRandom(7).ints(9, 50)
+    got = m.forward(ids)
+    assert got.shape == (9, 50)                                          # GPTModelTest.java:64-82
+    close(got, brute_gpt_forward(m, ids), atol=2e-5, rtol=1e-4)
+    # composition of the oracle's own layer functions, bit for bit (GPTTransformerBlock.java:65-73)
+    x = ref.add(ref.slice_rows(m.weight("emb"), ids), m.weight("pos")[:9])
+    for l in range(2):
+        w = lambda n: m.weight(f"L{l}.{n}")
+        x2 = ref.add(x, ref.mhsa_forward(ref.layernorm(x, w("g1"), w("be1")), w("wq"), w("wk"), w("wv"), w("wo"), 4))
+        hid = ref.gelu(ref.linear(ref.layernorm(x2, w("g2"), w("be2")), w("wg"), w("bg")))
+        x = ref.add(x2, ref.linear(hid, w("wd"), w("bd")))
+    exp = ref.linear(ref.layernorm(x, m.weight("gf"), m.weight("bf")), m.weight("wlm"), m.weight("blm"))
+    assert np.array_equal(got, exp)
+    # the position rows matter: the same token at two positions gives different logits
+    two = m.forward([3, 3])
+    assert np.abs(two[0] - m.forward([3])[0]).max() == 0 and np.abs(two[1] - two[0]).max() > 1e-4
+    with pytest.raises(ValueError, match="exceeds maxSeq"):             # PositionalEmbeddingTest.java:49-53
+        m.forward(np.zeros(17, np.int32))
+    with pytest.raises(ValueError, match="out of range"):
+        m.forward([0, 50])
+
+
+def test_gpt_cached_forward_and_generate_equivalence():
+    m = ref.Model(seed=9, gpt=True, vocab=64, max_seq=16, d=32, heads=4, layers=2, dff=48)
+    ids = ref.JavaRandom(3).ints(12, 64)
+    full = m.forward(ids)
+    m.reset_cache()
+    got = [m.forward_cached(ids[:5]), m.forward_cached(ids[5:6]), m.forward_cached(ids[6:12])]
+    assert np.array_equal(np.vstack(got), full)
+    prompt = ids[:4]
+    a = m.generate(prompt, 8, top_k=1)
+    c, logits = m.generate(prompt, 8, top_k=1, use_cache=True, return_logits=True)
+    assert np.array_equal(a, c) and np.array_equal(np.argmax(logits, axis=1), c[4:])
+    # Q8 round trip touches the six matrices of a block and the head, nothing else
+    before = {n: m.weight(n).copy() for n in m.weight_names()}
+    m.q8_roundtrip()
+    for n, v in before.items():
+        changed = not np.array_equal(v, m.weight(n))
+        assert changed == (n.split(".")[-1] in ("wq", "wk", "wv", "wo", "wg", "wd", "wlm")), n
