@@ -569,48 +569,62 @@ int32_t sample_from_logits(const std::vector<float> &logits, float temperature, 
 }
 
 // TextGenerator.generate on token ids (TextGenerator.java:66-87).  out holds n_prompt + max_new ids.
+//
+// Token t is drawn from the logits of the last row of forward(last(ids, maxSeqLen)) (TextGenerator.java:91-100,
+// 172-175).  While the whole sequence fits the window its rows keep their positions, so the KV cache serves them;
+// once it is longer the window slides by one per token and every row's position changes, so each further token is
+// a fresh forward of the maxSeqLen-row window - what the reference does for every token.
 void generate(Runner &r, const int32_t *prompt, int n_prompt, int max_new, float temperature, int top_k,
               int64_t seed, int32_t *out, int mode) {
     const Config &c = r.cfg;
     if (max_new < 0) throw Error("maxNewTokens must be >= 0");
     if (!(temperature > 0.0f)) throw Error("temperature must be > 0");
     if (top_k < 0) throw Error("topK must be >= 0");
-    if (max_new > 0 && n_prompt + max_new - 1 > c.max_seq)
-        throw Error("context of " + std::to_string(n_prompt + max_new - 1) + " tokens exceeds maxSeqLen " +
-                    std::to_string(c.max_seq) + " (the sliding window of TextGenerator is not cached)");
+    if (n_prompt <= 0 && max_new > 0) throw Error("prefill: empty prompt");
+    check_ids(c, prompt, n_prompt);
     std::memcpy(out, prompt, (size_t)n_prompt * sizeof(int32_t));
     if (max_new == 0) return;
-    reset(r);
-    if (top_k == 1) {
-        // argmax needs no random draw to pick, and greedy output is seed independent
-        prefill(r, prompt, n_prompt, nullptr, true);
-        decode_greedy(r, max_new - 1, mode);
-        check_persistent(r);
-        hip(deepj_hip_download(r.tokens, reinterpret_cast<float *>(out + n_prompt), max_new));
-        return;
-    }
-    void *rng = deepj_host_random_create(seed);
+    // tokens 0 .. cached-1 see a context that fits the window (n_prompt + t <= maxSeqLen)
+    const int cached = n_prompt > c.max_seq ? 0 : std::min(max_new, c.max_seq - n_prompt + 1);
+    const bool greedy = top_k == 1;       // argmax needs no random draw to pick, and greedy output is seed independent
+    void *rng = greedy ? nullptr : deepj_host_random_create(seed);
     try {
-        std::vector<float> logits((size_t)c.vocab);
-        Stream fwd = decode_stream(r, false);
-        prefill(r, prompt, n_prompt, nullptr, false);
-        for (int t = 0; t < max_new; t++) {
-            if (t > 0) {
-                r.run(fwd);          // consumes the token in state[1] at position state[0]
-                r.pos += 1;
-            }
+        std::vector<float> logits(greedy ? 0 : (size_t)c.vocab);
+        auto sample = [&](int t) {
             hip(deepj_hip_download(r.logits, logits.data(), c.vocab));
-            int32_t next = sample_from_logits(logits, temperature, top_k, rng);
-            out[n_prompt + t] = next;
-            int32_t st[4] = {r.pos, next, t + 1, 0};
-            hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
-            r.generated = t + 1;
+            out[n_prompt + t] = sample_from_logits(logits, temperature, top_k, rng);
+        };
+        reset(r);
+        if (cached > 0 && greedy) {
+            prefill(r, prompt, n_prompt, nullptr, true);
+            decode_greedy(r, cached - 1, mode);
+            check_persistent(r);
+            hip(deepj_hip_download(r.tokens, reinterpret_cast<float *>(out + n_prompt), cached));
+        } else if (cached > 0) {
+            Stream fwd = decode_stream(r, false);
+            prefill(r, prompt, n_prompt, nullptr, false);
+            for (int t = 0; t < cached; t++) {
+                if (t > 0) {
+                    r.run(fwd);          // consumes the token in state[1] at position state[0]
+                    r.pos += 1;
+                }
+                sample(t);
+                int32_t st[4] = {r.pos, out[n_prompt + t], t + 1, 0};
+                hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
+                r.generated = t + 1;
+            }
+        }
+        for (int t = cached; t < max_new; t++) {
+            reset(r);
+            prefill(r, out + n_prompt + t - c.max_seq, c.max_seq, nullptr, greedy);
+            if (greedy) hip(deepj_hip_download(r.tokens, reinterpret_cast<float *>(out + n_prompt + t), 1));
+            else sample(t);
         }
     } catch (...) {
-        deepj_host_random_destroy(rng);
+        if (rng) deepj_host_random_destroy(rng);
         throw;
     }
-    deepj_host_random_destroy(rng);
+    if (rng) deepj_host_random_destroy(rng);
 }
 
 template <class F> int guarded(Runner *r, F &&f) {

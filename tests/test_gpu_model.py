@@ -121,8 +121,10 @@ def test_generator_and_model_argument_errors(c1):
         gpu.forward([0, 256])
     with pytest.raises(ValueError, match="temperature must be > 0"):        # TextGenerator.java:155-159
         TextGenerator.generate(gpu, [1, 2], 3, temperature=0.0)
-    with pytest.raises(ValueError, match="exceeds maxSeqLen"):
-        TextGenerator.generate(gpu, list(range(200)), 100)
+    with pytest.raises(ValueError, match="topK must be >= 0"):              # TextGenerator.java:155-159
+        TextGenerator.generate(gpu, [1, 2], 3, top_k=-1)
+    with pytest.raises(ValueError, match="exceeds maxSeqLen"):               # forward() itself has no window
+        gpu.forward(list(range(200)) + list(range(100)))
     with pytest.raises(ValueError, match="divisible"):                       # TransformerConfig.java:27-28
         LlamaModel(LlamaConfig(256, 16, 100, 3, 1, 64), None)
     out = TextGenerator.generate(gpu, [5, 6, 7], 0)
@@ -285,8 +287,8 @@ def test_edge_shapes_single_head_odd_vocab_ragged_dff():
 
 
 def test_cache_filled_to_the_last_position_and_not_beyond(c1):
-    """Decoding up to position maxSeqLen - 1 works and matches the oracle; one more step is refused on the host
-    before anything is launched (the cached driver has no sliding window)."""
+    """Decoding up to position maxSeqLen - 1 works and matches the oracle; one more cached step is refused on the
+    host before anything is launched (generate() slides the window instead, see the next test)."""
     gpu, cpu = c1
     prompt = ref.JavaRandom(13).ints(200, 256)
     new = 256 - 200 + 1                      # the last generated token is chosen at position 255 and never fed back
@@ -299,3 +301,28 @@ def test_cache_filled_to_the_last_position_and_not_beyond(c1):
         gpu.decode(1, persistent=True)
     with pytest.raises(ValueError, match="exceeds maxSeqLen"):
         gpu.step(3)
+
+
+def test_generate_slides_the_window_past_max_seq_len():
+    """TextGenerator.java:91-100,172-175: the context is the last maxSeqLen ids, so generation never stops at the
+    window: past it every token is a fresh forward of the window (positions restart at 0).  Greedy and sampled,
+    prompt shorter and longer than the window, all three model families, against the oracle's literal path."""
+    from deepj_amd import GPTConfig, GPTModel
+    cases = [(LlamaModel, LlamaConfig(vocabSize=64, maxSeqLen=16, dModel=64, nHeads=2, nLayers=2, dFF=96), {}),
+             (DeepSeekModel, DeepSeekConfig(vocabSize=64, maxSeqLen=16, dModel=64, nHeads=2, nLayers=2, dFF=96, qRank=32, kvRank=16),
+              dict(q_rank=32, kv_rank=16)),
+             (GPTModel, GPTConfig(vocabSize=64, maxSeqLen=16, dModel=64, nHeads=2, nLayers=2, dFF=96, initScale=1.0),
+              dict(gpt=True, init_scale=1.0))]
+    for cls, cfg, extra in cases:
+        gpu, cpu = cls(cfg, 21), oracle_model(cfg, 21, **extra)
+        try:
+            prompt = ref.JavaRandom(4).ints(20, 64)
+            for n_prompt, new in ((4, 20), (16, 3), (20, 4), (12, 5)):
+                exp = cpu.generate(prompt[:n_prompt], new, top_k=1, use_cache=False)
+                got = TextGenerator.generate(gpu, prompt[:n_prompt], new, top_k=1)
+                assert np.array_equal(got, exp), (cls.__name__, n_prompt, new, got, exp)
+            exp = cpu.generate(prompt[:10], 12, temperature=0.9, top_k=4, seed=77, use_cache=False)
+            got = TextGenerator.generate(gpu, prompt[:10], 12, temperature=0.9, top_k=4, seed=77)
+            assert np.array_equal(got, exp), cls.__name__
+        finally:
+            gpu.close(); cpu.close()
