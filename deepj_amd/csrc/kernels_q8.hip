@@ -37,7 +37,9 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-__device__ __forceinline__ float d_sigmoid(float x) { return 1.0f / (1.0f + (float)exp((double)(-x))); }
+// The epilogue sits on the critical path of every wavefront: single precision exp (about 1 ulp) instead of the
+// double precision one the element-wise SIGMOID opcode uses; the difference is far inside the 1e-4 per-op bound.
+__device__ __forceinline__ float d_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 // tensor/cpu/CpuBackend.java:338 (tanh form)
 __device__ __forceinline__ float d_gelu(float x) {
     float c = sqrtf(2.0f / 3.14159265358979323846f);
@@ -97,6 +99,15 @@ __global__ void __launch_bounds__(kThreads) k_q8_dequantize(const int8_t *__rest
     }
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global
+// load (its workgroup-scope fence needs vmcnt(0)), which here would park the workgroup until the weight rows
+// already requested from HBM have arrived; the staged activations only need the LDS writes to be complete.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // ── decode matvec ──────────────────────────────────────────────────────────
 struct MatvecArgs {
     const float *x; const int8_t *wq; const float *scales; float *out;
@@ -146,12 +157,18 @@ template <int NC, int R> struct RowBatch {
 // finished sums never wait for a bias or residual that is still in memory.
 template <int NC, int R, int B, bool SWIGLU>
 __device__ __forceinline__ void load_epilogue(RowBatch<NC, R> &b, const MatvecArgs &p, int o0) {
+    // No load sits under a branch: an absent operand reads a valid dummy address instead (the value is never
+    // used).  A conditional load would leave the number of loads in flight unknown at compile time, and every
+    // later wait for an EARLIER load would have to be a wait for all of them.
+    const float *bias = p.bias ? p.bias : p.scales, *bias2 = (SWIGLU && p.bias2) ? p.bias2 : p.scales;
+    const float *residual = p.residual ? p.residual : p.scales;
 #pragma unroll
     for (int u = 0; u < B; u++) {
         int o = o0 + u < p.n_out ? o0 + u : p.n_out - 1;
-        b.eb[u] = p.bias ? p.bias[o] : 0.0f;
-        b.eb2[u] = (SWIGLU && p.bias2) ? p.bias2[o] : 0.0f;
-        b.er[u] = p.residual ? p.residual[o] : 0.0f;
+        o = o < 0 ? 0 : o;
+        b.eb[u] = bias[o];
+        if constexpr (SWIGLU) b.eb2[u] = bias2[o]; else b.eb2[u] = 0.0f;
+        b.er[u] = residual[o];
     }
 }
 
@@ -242,19 +259,44 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     RowBatch<NC, R> ba, bb;
     bool deferred_norm = false;
     const bool vec = (p.k & 3) == 0;              // kernel-uniform
-    float4 xv[NC], gv[NC];
+    float4 xv[NC], gv[NC], bv[NC];
     if (vec) {
-        // The activation (and gain) loads go out first: they hit in L2 and come back while
-        // the weight loads issued right behind them are still on their way from HBM.
+        // The activation, gain and beta loads go out first: they hit in L2 and come back while the weight loads
+        // issued right behind them are still on their way from HBM.  All of them are unconditional (clamped
+        // address, dummy pointer for an absent operand), so the wait for them is a counted one that leaves the
+        // weight loads in flight.
+        const float *gp = p.gamma ? p.gamma : p.x, *bp = p.beta ? p.beta : p.x;
 #pragma unroll
         for (int j = 0; j < NC; j++) {
-            int e = (tid + kThreads * j) * 4;
-            bool ok = e < p.k;
-            xv[j] = ok ? *reinterpret_cast<const float4 *>(p.x + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-            gv[j] = (ok && p.gamma) ? *reinterpret_cast<const float4 *>(p.gamma + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const int e = (tid + kThreads * j) * 4;
+            const int ec = e < p.k ? e : 0;
+            xv[j] = *reinterpret_cast<const float4 *>(p.x + ec);
+            gv[j] = *reinterpret_cast<const float4 *>(gp + ec);
+            bv[j] = *reinterpret_cast<const float4 *>(bp + ec);
         }
     }
-    if (has_work) { load_batch<NC, R>(ba, p, o_begin * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(ba, p, o_begin); }
+    asm volatile("" ::: "memory");      // the loads above are issued before the ones below ...
+    {
+        // waves without a batch load their (clamped) last row too: cheaper than a branch around the loads
+        const int first = has_work ? o_begin : 0;
+        load_batch<NC, R>(ba, p, first * RPO, row_last, lane, groups);
+        load_epilogue<NC, R, B, SWIGLU>(ba, p, first);
+    }
+    asm volatile("" ::: "memory");
+    if (vec) {
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            // ... and nothing consumes them before the weight loads are out (the scheduler would otherwise park
+            // the wavefront on the activations first and request the weights one L2 round trip later)
+            float x0 = xv[j].x, x1 = xv[j].y, x2 = xv[j].z, x3 = xv[j].w;
+            asm volatile("" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
+            const bool ok = (tid + kThreads * j) * 4 < p.k;
+            const bool okg = ok && p.gamma;
+            xv[j] = make_float4(ok ? x0 : 0.f, ok ? x1 : 0.f, ok ? x2 : 0.f, ok ? x3 : 0.f);
+            gv[j] = make_float4(okg ? gv[j].x : 0.f, okg ? gv[j].y : 0.f, okg ? gv[j].z : 0.f, okg ? gv[j].w : 0.f);
+            bv[j] = make_float4(ok ? bv[j].x : 0.f, ok ? bv[j].y : 0.f, ok ? bv[j].z : 0.f, ok ? bv[j].w : 0.f);
+        }
+    }
 
     // Stage the activation row through LDS (zero beyond K so padded weights meet zeros).
     // All global loads of the prologue - x and, for the RMSNorm prologue, gamma - were
@@ -262,19 +304,13 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     if (vec && p.beta) {
         // LayerNorm prologue (LayerNorm1D.java:34-66): mean, then the population variance about it, then
         // ((x - mean) / sqrt(var + 1e-5)) * gamma + beta goes to LDS.
-        float4 bv[NC];
-#pragma unroll
-        for (int j = 0; j < NC; j++) {
-            int e = (tid + kThreads * j) * 4;
-            bv[j] = e < p.k ? *reinterpret_cast<const float4 *>(p.beta + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
         const float inv_k = 1.0f / (float)p.k;
         float sm = 0.0f;
 #pragma unroll
         for (int j = 0; j < NC; j++) sm += (xv[j].x + xv[j].y) + (xv[j].z + xv[j].w);
         sm = wave_sum_dpp(sm);
         if (lane == 0) red[wave] = sm;
-        __syncthreads();
+        lds_barrier();
         const float mean = (red[0] + red[1] + red[2] + red[3]) * inv_k;
         float sv = 0.0f;
 #pragma unroll
@@ -286,7 +322,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
         }
         sv = wave_sum_dpp(sv);
         if (lane == 0) red2[wave] = sv;
-        __syncthreads();
+        lds_barrier();
         const float sd = sqrtf((red2[0] + red2[1] + red2[2] + red2[3]) * inv_k + kLayerNormEps);
 #pragma unroll
         for (int j = 0; j < NC; j++) {
@@ -330,25 +366,25 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             for (int i = tid; i < p.k; i += kThreads) sm += p.x[i];
             sm = wave_sum_dpp(sm);
             if (lane == 0) red[wave] = sm;
-            __syncthreads();
+            lds_barrier();
             float mean = (red[0] + red[1] + red[2] + red[3]) * (1.0f / (float)p.k);
             float sv = 0.0f;
             for (int i = tid; i < p.k; i += kThreads) { float c = xs[i] - mean; sv += c * c; }
             sv = wave_sum_dpp(sv);
             if (lane == 0) red2[wave] = sv;
-            __syncthreads();
+            lds_barrier();
             float sd = sqrtf((red2[0] + red2[1] + red2[2] + red2[3]) * (1.0f / (float)p.k) + kLayerNormEps);
             for (int i = tid; i < p.k; i += kThreads) xs[i] = ((xs[i] - mean) / sd) * p.gamma[i] + p.beta[i];
         } else if (p.gamma) {
             ss = wave_sum_dpp(ss);
             if (lane == 0) red[wave] = ss;
-            __syncthreads();
+            lds_barrier();
             float tot = red[0] + red[1] + red[2] + red[3];
             float rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
             for (int i = tid; i < p.k; i += kThreads) xs[i] = (xs[i] / rms) * p.gamma[i];
         }
     }
-    __syncthreads();
+    lds_barrier();
     if (!has_work) return;
     float rms = 1.0f;
     if (deferred_norm) {
