@@ -84,6 +84,7 @@ struct Q8Linear {
     int m, k, n, flags;
     const float *gamma, *bias, *bias2, *residual;
     const float *beta = nullptr;      // LayerNorm prologue only
+    int rec_hd = 0;                   // ATTN_MERGE prologue only: head width of the records in x
     const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
     int m_extra = 0;
 };
@@ -117,6 +118,12 @@ void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *
                         const int32_t *state, float *scratch, const float *cos_t, const float *sin_t, int H, int hd,
                         int max_seq, unsigned *counters);
 int64_t attn_decode_scratch_floats(int H, int hd);
+// Decode attention that stops at per-split records [H][kAttnRecordSplits][hd + 4] = {max, sum, -, -, o[hd]};
+// the consumer (Q8 matvec with the ATTN_MERGE prologue) merges them.
+constexpr int kAttnRecordSplits = 4;
+void launch_attn_decode_records(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *records,
+                                const int32_t *state, const float *cos_t, const float *sin_t, int H, int hd,
+                                int max_seq);
 void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
                         const float *table, float *x, int vocab, int d, int n_positions);
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq);

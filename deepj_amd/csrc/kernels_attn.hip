@@ -437,6 +437,119 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
 }
 
 // Splits per head for the fused decode op: about two workgroups per CU in total.
+// ── decode attention that leaves the split merge to its consumer ───────────
+// Same work as the fused kernel above (rotate q and the new key, append the new row, online softmax over this
+// split's keys) with kRecSplits splits per head and 1024 threads per workgroup, but it stops at the per-split
+// record [max, sum, -, -, o[hd]]: merging records across workgroups inside one kernel costs a store
+// acknowledgement, an atomic and a reload - three trips to memory in a row - while the next kernel reads them
+// across the kernel boundary for free (the Q8 matvec's ATTN_MERGE prologue does the merge while its weight rows
+// are in flight).
+constexpr int kRecThreads = 1024;
+constexpr int kRecWaves = kRecThreads / 64;
+
+template <int LPK>
+__global__ void __launch_bounds__(kRecThreads) k_attn_decode_records(DecodeArgs a) {
+    constexpr int HD = LPK * 4;
+    constexpr int KPW = 64 / LPK;                  // keys a wavefront handles at a time
+    constexpr int STRIDE = kRecWaves * KPW;        // keys per workgroup round
+    constexpr int U = 4;
+    __shared__ float s_m[kRecWaves], s_l[kRecWaves];
+    __shared__ __align__(16) float s_o[kRecWaves][HD];
+
+    const int h = blockIdx.x, split = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane / LPK, dl = lane % LPK;
+    const int d = a.H * HD, half = HD / 2;
+
+    int pos = a.state[0];
+    if (pos < 0) pos = 0;
+    if (pos >= a.max_seq) pos = a.max_seq - 1;             // the host never lets this happen; stay in bounds
+    const int n_keys = pos + 1;
+    const int per = (n_keys + a.nsplit - 1) / a.nsplit;
+    const int k_begin = split * per;
+    const int k_end = k_begin + per < n_keys ? k_begin + per : n_keys;
+
+    const float2 c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
+    const float2 s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
+    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
+    const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
+    const float4 nv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
+    const float4 qv = make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
+                                  q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y);
+    const float4 nk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
+                                  k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
+    float *kb = a.k_cache + (int64_t)h * a.head_stride + dl * 4;
+    float *vb = a.v_cache + (int64_t)h * a.head_stride + dl * 4;
+
+    float m = -INFINITY, l = 0.0f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int base = k_begin + wave * KPW + sub; base < k_end; base += U * STRIDE) {
+        float4 kk[U], vv[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int key = base + u * STRIDE;
+            int row = (key < k_end && key != pos) ? key : k_begin;      // k_begin < n_keys: a row that exists
+            kk[u] = *reinterpret_cast<const float4 *>(kb + (int64_t)row * a.tok_stride);
+            vv[u] = *reinterpret_cast<const float4 *>(vb + (int64_t)row * a.tok_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int key = base + u * STRIDE;
+            bool valid = key < k_end;                       // uniform over the LPK lanes of a key
+            if (valid && key == pos) {
+                kk[u] = nk; vv[u] = nv;
+                *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = nk;
+                *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = nv;
+            }
+            float s = qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w;
+#pragma unroll
+            for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+            if (valid) {
+                s *= a.scale;
+                float mn = fmaxf(m, s);
+                float corr = expf(m - mn);
+                float p = expf(s - mn);
+                l = l * corr + p;
+                o.x = o.x * corr + p * vv[u].x; o.y = o.y * corr + p * vv[u].y;
+                o.z = o.z * corr + p * vv[u].z; o.w = o.w * corr + p * vv[u].w;
+                m = mn;
+            }
+        }
+    }
+    // the KPW lane groups of a wavefront first (shuffles), then the wavefronts (LDS)
+#pragma unroll
+    for (int off = LPK; off < 64; off <<= 1) {
+        float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
+        float4 o2 = make_float4(__shfl_xor(o.x, off, 64), __shfl_xor(o.y, off, 64), __shfl_xor(o.z, off, 64),
+                                __shfl_xor(o.w, off, 64));
+        float mn = fmaxf(m, m2);
+        float w1 = m == -INFINITY ? 0.0f : expf(m - mn), w2 = m2 == -INFINITY ? 0.0f : expf(m2 - mn);
+        l = l * w1 + l2 * w2;
+        o.x = o.x * w1 + o2.x * w2; o.y = o.y * w1 + o2.y * w2; o.z = o.z * w1 + o2.z * w2; o.w = o.w * w1 + o2.w * w2;
+        m = mn;
+    }
+    if (lane == 0) { s_m[wave] = m; s_l[wave] = l; }
+    if (sub == 0) *reinterpret_cast<float4 *>(&s_o[wave][dl * 4]) = o;
+    __syncthreads();
+    if (tid < HD) {
+        float M = -INFINITY, L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRecWaves; i++) M = fmaxf(M, s_m[i]);
+        if (M != -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < kRecWaves; i++) {
+                float w = expf(s_m[i] - M);
+                L += s_l[i] * w;
+                O += s_o[i][tid] * w;
+            }
+        }
+        float *rec = a.scratch + ((int64_t)h * a.nsplit + split) * (HD + 4);
+        rec[4 + tid] = O;
+        if (tid == 0) { rec[0] = M; rec[1] = L; }
+    }
+}
+
+
 inline int fused_decode_splits(int H) {
     int ns = 512 / H;
     if (ns < 1) ns = 1;
@@ -499,6 +612,25 @@ void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *
     a.tok_stride = hd; a.head_stride = (int64_t)max_seq * hd;
     a.cos_t = cos_t; a.sin_t = sin_t; a.H = H; a.hd = hd; a.max_seq = max_seq;
     launch_decode_kernels<true>(s, a);
+}
+
+void launch_attn_decode_records(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *records,
+                                const int32_t *state, const float *cos_t, const float *sin_t, int H, int hd,
+                                int max_seq) {
+    DecodeArgs a;
+    a.counters = nullptr;
+    a.qkv = qkv; a.k_cache = k_cache; a.v_cache = v_cache; a.out = nullptr; a.state = state; a.scratch = records;
+    a.tok_stride = hd; a.head_stride = (int64_t)max_seq * hd;
+    a.cos_t = cos_t; a.sin_t = sin_t; a.H = H; a.hd = hd; a.max_seq = max_seq;
+    a.nsplit = kAttnRecordSplits;
+    a.scale = (float)(1.0 / sqrt((double)hd));
+    dim3 grid(H, kAttnRecordSplits);
+    switch (hd) {
+        case 32: hipLaunchKernelGGL((k_attn_decode_records<8>), grid, dim3(kRecThreads), 0, s, a); break;
+        case 64: hipLaunchKernelGGL((k_attn_decode_records<16>), grid, dim3(kRecThreads), 0, s, a); break;
+        case 128: hipLaunchKernelGGL((k_attn_decode_records<32>), grid, dim3(kRecThreads), 0, s, a); break;
+        default: fail("attention: head dim must be 32, 64 or 128");
+    }
 }
 
 void launch_attention(hipStream_t s, const AttnArgs &p) {

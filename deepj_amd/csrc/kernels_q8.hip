@@ -114,6 +114,7 @@ struct MatvecArgs {
     int k, kp, n_out;                 // n_out outputs; SwiGLU: output o uses rows 2o, 2o+1
     const float *gamma, *bias, *bias2, *residual;
     const float *beta;                // set: LayerNorm prologue with gamma and beta (otherwise gamma alone = RMSNorm)
+    int rec_hd;                       // ATTN_MERGE prologue: x holds attention records of heads this wide
 };
 
 __device__ __forceinline__ float dot16(const int4 &w, const float *xr) {
@@ -235,10 +236,15 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
 // the HBM stream is already running while the workgroup stages x through LDS and
 // applies the RMSNorm prologue; after that the next batch is always in flight while
 // the current one is multiplied (two register buffers used in turn).
-// GELU (compile time: its double-precision tanh would cost every other variant some forty registers)
-// applies the activation to the biased sum.
-template <int NC, int B, bool SWIGLU, bool GELU>
+// MODE (compile time, so that the other variants do not pay for its registers): 1 = GELU on the biased sum
+// (its double-precision tanh costs some forty registers); 2 = ATTN_MERGE prologue: x is not the activation row
+// but the per-split records [head][kAttnRecordSplits][hd + 4] = {max, sum, -, -, o[hd]} the decode attention
+// kernel left, and the row is their merge  x[h*hd + j] = sum_s w_s o_s[j] / sum_s w_s l_s,  w_s = exp(max_s - max).
+template <int NC, int B, bool SWIGLU, int MODE>
 __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
+    constexpr bool GELU = MODE == 1;
+    constexpr bool MERGE = MODE == 2;
+    constexpr int NS = kAttnRecordSplits;
     extern __shared__ __align__(16) float xs[];   // Kp floats
     __shared__ float red[kWaves], red2[kWaves];
     constexpr int RPO = SWIGLU ? 2 : 1;           // Q8 rows per output
@@ -260,7 +266,24 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     bool deferred_norm = false;
     const bool vec = (p.k & 3) == 0;              // kernel-uniform
     float4 xv[NC], gv[NC], bv[NC];
-    if (vec) {
+    float2 rml[MERGE ? NC : 1][NS];
+    float4 rov[MERGE ? NC : 1][NS];
+    if constexpr (MERGE) {
+        // the records of the head each float4 of the row belongs to: unconditional, issued before the weights
+        const int rstride = p.rec_hd + 4;
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            const int e = (tid + kThreads * j) * 4;
+            const int ec = e < p.k ? e : 0;
+            const int head = ec / p.rec_hd, off = ec - head * p.rec_hd;
+            const float *r = p.x + (int64_t)head * NS * rstride;
+#pragma unroll
+            for (int sp = 0; sp < NS; sp++) {
+                rml[j][sp] = *reinterpret_cast<const float2 *>(r + sp * rstride);
+                rov[j][sp] = *reinterpret_cast<const float4 *>(r + sp * rstride + 4 + off);
+            }
+        }
+    } else if (vec) {
         // The activation, gain and beta loads go out first: they hit in L2 and come back while the weight loads
         // issued right behind them are still on their way from HBM.  All of them are unconditional (clamped
         // address, dummy pointer for an absent operand), so the wait for them is a counted one that leaves the
@@ -283,7 +306,29 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
         load_epilogue<NC, R, B, SWIGLU>(ba, p, first);
     }
     asm volatile("" ::: "memory");
-    if (vec) {
+    if constexpr (MERGE) {
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            float m0 = rml[j][0].x;
+            asm volatile("" : "+v"(m0));        // nothing consumes the records before the weight loads are out
+            float mx = m0;
+#pragma unroll
+            for (int sp = 1; sp < NS; sp++) mx = fmaxf(mx, rml[j][sp].x);
+            float lsum = 0.0f;
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int sp = 0; sp < NS; sp++) {
+                const float ms = sp == 0 ? m0 : rml[j][sp].x;
+                const float w = ms == -INFINITY ? 0.0f : expf(ms - mx);     // a split without keys
+                lsum += rml[j][sp].y * w;
+                acc.x += rov[j][sp].x * w; acc.y += rov[j][sp].y * w; acc.z += rov[j][sp].z * w; acc.w += rov[j][sp].w * w;
+            }
+            const bool ok = (tid + kThreads * j) * 4 < p.k;
+            const float inv = 1.0f / lsum;
+            xv[j] = ok ? make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv) : make_float4(0.f, 0.f, 0.f, 0.f);
+            gv[j] = bv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    } else if (vec) {
 #pragma unroll
         for (int j = 0; j < NC; j++) {
             // ... and nothing consumes them before the weight loads are out (the scheduler would otherwise park
@@ -417,7 +462,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
 constexpr int kMvGridCap = 768;          // three workgroups per CU
 inline int mv_grid_cap() { return kMvGridCap; }
 
-template <int NC, int B, bool SW, bool GELU = false>
+template <int NC, int B, bool SW, int MODE = 0>
 void launch_mv(hipStream_t s, const MatvecArgs &a) {
     // Three workgroups (12 wavefronts) per CU when there are outputs for them; never
     // more wavefronts than outputs.
@@ -426,7 +471,7 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     if (grid > mv_grid_cap()) grid = mv_grid_cap();
     if (grid < 1) grid = 1;
     size_t lds = (size_t)a.kp * sizeof(float);
-    hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, GELU>), dim3(grid), dim3(kThreads), lds, s, a);
+    hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE>), dim3(grid), dim3(kThreads), lds, s, a);
 }
 
 // Batch depth B (outputs a wavefront multiplies per step).  Small matrices want B = 1: every
@@ -437,6 +482,14 @@ inline int mv_target_waves() { return 3072; }
 
 template <int NC>
 void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu, bool gelu) {
+    if (a.rec_hd > 0) {           // ATTN_MERGE prologue (never with SwiGLU or GELU)
+        // Every workgroup merges the whole row for itself, so fewer, deeper workgroups: two outputs per
+        // wavefront even when that leaves wavefronts to spare (measured: +0.2 us over the plain kernel at
+        // 2048 x 2048, +0.9 us with one output per wavefront).
+        constexpr int BM = NC <= 4 ? 2 : 1;
+        launch_mv<NC, BM, false, 2>(s, a);
+        return;
+    }
     constexpr int BMAX = NC == 1 ? 8 : (NC == 2 ? 4 : (NC <= 4 ? 2 : 1));
     int rows = swiglu ? 2 * a.n_out : a.n_out;
     int want = (rows + mv_target_waves() - 1) / mv_target_waves();      // rows per wavefront per step
@@ -446,9 +499,9 @@ void dispatch_mv(hipStream_t s, const MatvecArgs &a, bool swiglu, bool gelu) {
         else if (BS >= 2 && want >= 4) launch_mv<NC, (BS >= 2 ? 2 : 1), true>(s, a);
         else launch_mv<NC, 1, true>(s, a);
     } else if (gelu) {
-        if (BMAX >= 4 && want >= 4) launch_mv<NC, (BMAX >= 4 ? 4 : 1), false, true>(s, a);
-        else if (BMAX >= 2 && want >= 2) launch_mv<NC, (BMAX >= 2 ? 2 : 1), false, true>(s, a);
-        else launch_mv<NC, 1, false, true>(s, a);
+        if (BMAX >= 4 && want >= 4) launch_mv<NC, (BMAX >= 4 ? 4 : 1), false, 1>(s, a);
+        else if (BMAX >= 2 && want >= 2) launch_mv<NC, (BMAX >= 2 ? 2 : 1), false, 1>(s, a);
+        else launch_mv<NC, 1, false, 1>(s, a);
     } else {
         if (BMAX >= 8 && want >= 8) launch_mv<NC, (BMAX >= 8 ? 8 : 1), false>(s, a);
         else if (BMAX >= 4 && want >= 4) launch_mv<NC, (BMAX >= 4 ? 4 : 1), false>(s, a);
@@ -513,7 +566,8 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     const int kp = q8_padded_k(p.k);
 
     if (p.m == 1 && !p.m_dev && matvec_supported(p.k)) {
-        MatvecArgs a{p.x, p.wq, p.scales, p.out, p.k, kp, p.n, gamma, bias, bias2, residual, beta};
+        const int rec_hd = (p.flags & DJ_LIN_ATTN_MERGE) ? p.rec_hd : 0;
+        MatvecArgs a{p.x, p.wq, p.scales, p.out, p.k, kp, p.n, gamma, bias, bias2, residual, beta, rec_hd};
         int nc = (kp + 1023) / 1024;
         switch (nc) {
             case 1: dispatch_mv<1>(s, a, swiglu, gelu != 0); break;
@@ -532,6 +586,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     }
 
     // GEMM path
+    if (p.flags & DJ_LIN_ATTN_MERGE) fail("q8_linear: the ATTN_MERGE prologue exists for M = 1 only");
     if (workspace_floats < q8_linear_workspace_floats(p.m, p.k, p.n, p.flags)) fail("q8_linear: workspace too small");
     const float *x = p.x;
     float *ws = workspace;

@@ -69,6 +69,7 @@ struct Runner {
     int32_t pos_table = -1, bf = -1;                       // GPT: learned positions, final LayerNorm beta
     int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
     int32_t state = -1, tok = -1, tokens = -1, scratch = -1, scratch_dec = -1, logits = -1, last_x = -1;
+    int32_t records = -1;                                  // decode attention records (merged by the Wo matvec)
     int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
     int64_t p_sync_floats = 0;
     bool p_pending = false;                                // a persistent launch has not been checked yet
@@ -311,6 +312,7 @@ void finalize(Runner &r) {
     int64_t sf = (int64_t)c.heads * ns * (hd + 4);           // split-attention records (S = 1 paths)
     r.scratch = r.alloc(sf);
     r.scratch_dec = r.alloc(sf);
+    r.records = r.alloc((int64_t)c.heads * 4 * (hd + 4));
     Stream s;
     emit(s, DJ_OP_FILL, r.state, 0, 4);
     emit(s, DJ_OP_FILL, r.tok, 0, 4);
@@ -335,14 +337,17 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     const Config &c = r.cfg;
     const Layer &L = r.layers[l];
     const int d = c.d, H = c.heads, hd = r.hd();
+    bool wo_done = false;
     if (c.kind != 1) {
         // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
         // GPT: LayerNorm instead of RMSNorm and no rotation                  GPTTransformerBlock.java:66-68
         if (c.kind == 2) q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1);
         else q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
         if (S == 1 && &a == &r.dec) {
-            emit(s, DJ_OP_ATTN_DECODE, a.qkv, r.kc, r.vc, a.att, r.state, r.scratch_dec, r.cos_t, r.sin_t, H, hd,
-                 c.max_seq, l);
+            // the key splits' records go straight to the Wo matvec, whose prologue merges them
+            emit(s, DJ_OP_ATTN_DECODE_RECORDS, a.qkv, r.kc, r.vc, r.records, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
+            emit(s, DJ_OP_Q8_LINEAR, r.records, L.wo, a.x2, 1, d, d, DJ_LIN_RESIDUAL | DJ_LIN_ATTN_MERGE, hd, -1, -1, a.x);
+            wo_done = true;
         } else {
             emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
             emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
@@ -360,7 +365,7 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
         emit(s, DJ_OP_ROPE_ROWS, a.qkv, a.q, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, 0, 0, -1);
         emit(s, DJ_OP_ATTENTION_KV, a.q, r.kc, r.kc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0, 2 * d, d);
     }
-    q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
+    if (!wo_done) q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
     if (c.kind == 2) {
         // x = x2 + W2 . GELU(W1 . ln2(x2) + b1) + b2                        GPTTransformerBlock.java:70-72, FNN.java:57-73
         q8_linear(s, a.x2, L.wgu, a.ff, S, d, c.dff, DJ_LIN_LAYERNORM | DJ_LIN_BIAS | DJ_LIN_GELU, L.g2, L.bg, L.be2);
@@ -671,7 +676,7 @@ void deepj_runner_destroy(void *h) {
     for (auto &L : r->layers)
         for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wuk, L.wuv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
     for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state, r->tok,
-                       r->tokens, r->scratch, r->scratch_dec, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
+                       r->tokens, r->scratch, r->scratch_dec, r->records, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
                        r->pos_table, r->bf})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})

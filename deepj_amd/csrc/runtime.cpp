@@ -192,6 +192,7 @@ int stride_of(int op) {
         case DJ_OP_Q8_LINEAR_DYN: return 10;
         case DJ_OP_LLAMA_DECODE: return 0;      // variable: word 1
         case DJ_OP_LAYERNORM: return 7;
+        case DJ_OP_ATTN_DECODE_RECORDS: return 12;
         case DJ_OP_ADD_POSITIONS: return 7;
         default: return -1;
     }
@@ -378,7 +379,18 @@ void exec_one(Cursor &c) {
             int64_t m = w[4], k = w[5], n = w[6];
             int flags = w[7];
             if (m <= 0 || k <= 0 || n <= 0) fail("OP_Q8_LINEAR: bad shape");
-            if (flags & ~63) fail("OP_Q8_LINEAR: unknown flag bits");
+            if (flags & ~127) fail("OP_Q8_LINEAR: unknown flag bits");
+            const bool merge = flags & DJ_LIN_ATTN_MERGE;
+            int64_t rec_hd = 0;
+            if (merge) {
+                // x holds decode-attention records [K / hd][kAttnRecordSplits][hd + 4]; hd travels in the gamma word
+                rec_hd = w[8];
+                if (flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM | DJ_LIN_SWIGLU | DJ_LIN_GELU))
+                    fail("OP_Q8_LINEAR: ATTN_MERGE cannot be combined with a norm prologue, SWIGLU or GELU");
+                if (rec_hd != 32 && rec_hd != 64 && rec_hd != 128) fail("OP_Q8_LINEAR: ATTN_MERGE head dim must be 32, 64 or 128");
+                if (m != 1 || k % rec_hd != 0) fail("OP_Q8_LINEAR: ATTN_MERGE needs M = 1 and K a multiple of the head dim");
+                if (q8_linear_workspace_floats(1, (int)k, (int)n, 0) != 0 || k > 11 * 1024) fail("OP_Q8_LINEAR: ATTN_MERGE: K too large");
+            }
             bool sw = flags & DJ_LIN_SWIGLU;
             bool ln = flags & DJ_LIN_LAYERNORM;
             if (sw && (flags & DJ_LIN_RESIDUAL)) fail("OP_Q8_LINEAR: SWIGLU cannot be combined with RESIDUAL");
@@ -386,13 +398,14 @@ void exec_one(Cursor &c) {
             if (ln && (flags & DJ_LIN_RMSNORM)) fail("OP_Q8_LINEAR: RMSNORM and LAYERNORM are exclusive");
             int64_t rows = sw ? 2 * n : n;
             Q8Linear p;
-            p.x = buf(w[1], m * k, op, "x");
+            p.x = merge ? buf(w[1], (k / rec_hd) * kAttnRecordSplits * (rec_hd + 4), op, "attention records") : buf(w[1], m * k, op, "x");
+            p.rec_hd = (int)rec_hd;
             const float *wq = buf(w[2], (q8_bytes((int)k, (int)rows) + 3) / 4, op, "weight");
             p.wq = reinterpret_cast<const int8_t *>(wq);
             p.scales = reinterpret_cast<const float *>(p.wq + q8_scale_offset_bytes((int)k, (int)rows));
             p.out = buf(w[3], m * n, op, "out");
             p.m = (int)m; p.k = (int)k; p.n = (int)n; p.flags = flags;
-            p.gamma = (flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM)) ? buf(w[8], k, op, "gamma") : nullptr;
+            p.gamma = (flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM)) ? buf(w[8], k, op, "gamma") : nullptr;   // (ATTN_MERGE: w[8] = hd)
             p.beta = ln ? buf(w[10], k, op, "beta") : nullptr;
             p.bias = (flags & DJ_LIN_BIAS) ? buf(w[9], n, op, "bias") : nullptr;
             p.bias2 = ((flags & DJ_LIN_BIAS) && sw) ? buf(w[10], n, op, "bias2") : nullptr;
@@ -565,6 +578,24 @@ void exec_one(Cursor &c) {
                                    g.attn_counters);
             break;
         }
+        case DJ_OP_ATTN_DECODE_RECORDS: {
+            // [op, qkv, kCache, vCache, records, state, cos, sin, H, hd, maxSeq, layer]
+            int64_t H = w[8], hd = w[9], max_seq = w[10], layer = w[11];
+            if (H <= 0 || max_seq <= 0 || layer < 0) fail("OP_ATTN_DECODE_RECORDS: bad shape");
+            if (hd != 32 && hd != 64 && hd != 128) fail("OP_ATTN_DECODE_RECORDS: head dim must be 32, 64 or 128");
+            if (H > 65535) fail("OP_ATTN_DECODE_RECORDS: too many heads");
+            int64_t d = H * hd, per_layer = H * max_seq * hd;
+            const float *qkv = buf(w[1], 3 * d, op, "qkv");
+            float *kc = buf(w[2], (layer + 1) * per_layer, op, "kCache");
+            float *vc = buf(w[3], (layer + 1) * per_layer, op, "vCache");
+            float *rec = buf(w[4], H * kAttnRecordSplits * (hd + 4), op, "records");
+            const float *st = buf(w[5], 4, op, "state");
+            const float *ct = buf(w[6], max_seq * (hd / 2), op, "cos"), *sn = buf(w[7], max_seq * (hd / 2), op, "sin");
+            if (run)
+                launch_attn_decode_records(s, qkv, kc + layer * per_layer, vc + layer * per_layer, rec,
+                                           reinterpret_cast<const int32_t *>(st), ct, sn, (int)H, (int)hd, (int)max_seq);
+            break;
+        }
         case DJ_OP_APPEND_ROWS: {
             // [op, src, dst, state, rows, rowFloats, maxRows, dstOff]: dst[dstOff + (state[0]+i)*rowFloats ..] = src row i
             int64_t rows = w[4], rf = w[5], max_rows = w[6], off = w[7];
@@ -729,6 +760,7 @@ const char *op_name(int op) {
         case DJ_OP_Q8_LINEAR: return "OP_Q8_LINEAR";
         case DJ_OP_RMSNORM: return "OP_RMSNORM";
         case DJ_OP_LAYERNORM: return "OP_LAYERNORM";
+        case DJ_OP_ATTN_DECODE_RECORDS: return "OP_ATTN_DECODE_RECORDS";
         case DJ_OP_ADD_POSITIONS: return "OP_ADD_POSITIONS";
         case DJ_OP_SILU_MUL: return "OP_SILU_MUL";
         case DJ_OP_EMBED_GATHER: return "OP_EMBED_GATHER";

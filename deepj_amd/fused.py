@@ -79,8 +79,12 @@ class Stream:
         return self.emit(op.OP_Q8_DEQUANTIZE, src, dst, k, n, row_off, row_step, n if total_rows is None else total_rows)
 
     def q8_linear(self, x, w, out, m, k, n, *, gamma=-1, bias=-1, bias2=-1, residual=-1, swiglu=False, beta=-1,
-                  gelu=False):
-        """beta >= 0 turns the gamma prologue into LayerNorm (beta travels in the bias2 word)."""
+                  gelu=False, attn_merge_hd=0):
+        """beta >= 0 turns the gamma prologue into LayerNorm (beta travels in the bias2 word); attn_merge_hd > 0:
+        x is the records buffer of attn_decode_records and the prologue merges it (head dim in the gamma word)."""
+        if attn_merge_hd:
+            flags = op.LIN_ATTN_MERGE | (op.LIN_BIAS if bias >= 0 else 0) | (op.LIN_RESIDUAL if residual >= 0 else 0)
+            return self.emit(op.OP_Q8_LINEAR, x, w, out, m, k, n, flags, attn_merge_hd, bias, -1, residual)
         layernorm = beta >= 0
         if layernorm and swiglu:
             raise ValueError("LayerNorm prologue and SwiGLU share the bias2 word")
@@ -125,6 +129,9 @@ class Stream:
     def attn_decode(self, qkv, k_cache, v_cache, out, state, scratch, cos, sin, H, hd, max_seq, layer):
         return self.emit(op.OP_ATTN_DECODE, qkv, k_cache, v_cache, out, state, scratch, cos, sin, H, hd, max_seq, layer)
 
+    def attn_decode_records(self, qkv, k_cache, v_cache, records, state, cos, sin, H, hd, max_seq, layer):
+        return self.emit(op.OP_ATTN_DECODE_RECORDS, qkv, k_cache, v_cache, records, state, cos, sin, H, hd, max_seq, layer)
+
     def append_rows(self, src, dst, state, rows, row_floats, max_rows, dst_off=0):
         return self.emit(op.OP_APPEND_ROWS, src, dst, state, rows, row_floats, max_rows, dst_off)
 
@@ -151,6 +158,11 @@ class Stream:
 def attn_decode_scratch_floats(H: int, hd: int) -> int:
     """Floats of the scratch buffer the fused ATTN_DECODE op needs (no initialisation required)."""
     return H * max(1, min(16, 512 // H)) * (hd + 4)
+
+
+def attn_record_floats(H: int, hd: int) -> int:
+    """Floats of the records buffer ATTN_DECODE_RECORDS writes and the ATTN_MERGE prologue reads."""
+    return H * op.ATTN_RECORD_SPLITS * (hd + 4)
 
 
 def attention_scratch_floats(H: int, hd: int, max_seq: int = 0) -> int:

@@ -114,7 +114,9 @@ enum {
      *           bit4: LayerNorm prologue, f(x) = (x - mean) / sqrt(var + 1e-5) * gamma + beta with the beta
      *                 buffer in the bias2 word (J/layers/transformer/norm/LayerNorm1D.java:34-66)
      *           bit5: GELU (tanh form) on x.W + bias, before the residual (J/activations/GELU.java:15-18)
-     *           bit3 excludes bits 2, 4 and 5; bit0 excludes bit4
+     *           bit6: ATTN_MERGE prologue (M = 1): x is the records buffer ATTN_DECODE_RECORDS wrote, the gamma
+     *                 word holds the head dim, K = H * hd; f(x) = the merged attention row
+     *           bit3 excludes bits 2, 4, 5 and 6; bit0 excludes bit4; bit6 excludes bits 0, 4 and 5
      * RMSNORM       [op, x, gamma, out, rows, cols]
      * SILU_MUL      [op, gate, up, out, n]            out = gate*sigmoid(gate)*up
      * EMBED_GATHER  [op, table, ids, out, nIds, d, vocab, idsOff]  ids are int32 words
@@ -154,6 +156,11 @@ enum {
      *     wqkv [3d x d], wgu interleaved [2 dFF x d], all weights Q8.  scratch >= H*nsplit*(hd+4) floats, argbuf >=
      *     2*grid floats (deepj_hip_llama_decode_plan), sync = deepj_hip_llama_decode_sync_floats() floats, zero-filled
      *     once.  Not capturable into a graph; calls that overlap on one device are not supported.
+     * ATTN_DECODE_RECORDS [op, qkv, kCache, vCache, records, state, cosT, sinT, H, hd, maxSeq, layer]
+     *     ATTN_DECODE that stops before the merge of its key splits: records holds H * 4 * (hd + 4) floats,
+     *     per (head, split) {max, sum, -, -, o[hd]}; a Q8_LINEAR with the ATTN_MERGE prologue consumes them.
+     *     (Merging across workgroups inside one kernel costs three dependent trips to memory; across the
+     *     kernel boundary it is free.)
      * LAYERNORM     [op, x, gamma, beta, out, rows, cols]      J/layers/transformer/norm/LayerNorm1D.java:34-66
      * ADD_POSITIONS [op, x, table, state, rows, d, maxSeq]
      *     x[i, :] += table[state[0] + i, :]: the learned positional rows of J/models/gpt/GPTModel.java:52-54 for
@@ -164,11 +171,11 @@ enum {
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
     DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82, DJ_OP_LAYERNORM = 83,
-    DJ_OP_ADD_POSITIONS = 84
+    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8, DJ_LIN_LAYERNORM = 16,
-       DJ_LIN_GELU = 32 };
+       DJ_LIN_GELU = 32, DJ_LIN_ATTN_MERGE = 64 };
 
 /* Buffer sizes LLAMA_DECODE needs on this device: workgroups launched, key splits per head, floats of
  * `scratch` and `argbuf`; and the floats of its `sync` buffer. */

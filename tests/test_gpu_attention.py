@@ -5,7 +5,8 @@ cache (split-K path), for head dims 32/64/128."""
 import numpy as np
 import pytest
 
-from deepj_amd.fused import DeviceBuffers, Stream, attention_scratch_floats, attn_decode_scratch_floats
+from deepj_amd.fused import (DeviceBuffers, Stream, attention_scratch_floats, attn_decode_scratch_floats,
+                             attn_record_floats)
 from oracle import cpu_ref as ref
 from gpu_util import assert_close
 
@@ -104,6 +105,73 @@ def test_fused_decode_attention_and_decode_next(H, hd, max_seq, prefill, steps):
         qr = ref.merge_heads(ref.rope_apply(ref.split_heads(q, H), total, H, cos, sin), H)[total - 1:]
         (Stream().attention(dev.upload(qr), kc, vc, o_b, state, scratch, 1, H, hd, max_seq, 0).run())
         assert_close(exp[total - 1:], dev.download(o_b, (1, d)), atol=2e-5, rtol=1e-4)
+    finally:
+        dev.release_all()
+
+
+@pytest.mark.parametrize("H,hd,max_seq,start,steps", [(8, 32, 256, 0, 6), (32, 64, 2048, 515, 3), (4, 128, 96, 55, 41),
+                                                      (2, 64, 1, 0, 1), (5, 32, 700, 509, 5)])
+def test_decode_attention_records_merged_by_the_q8_linear_prologue(H, hd, max_seq, start, steps):
+    """ATTN_DECODE_RECORDS leaves one record per (head, key split); the ATTN_MERGE prologue of the following
+    Q8_LINEAR merges them.  With an identity-like projection out of reach (Q8), the check is against the oracle's
+    attention row pushed through the dequantised weight, plus a residual; positions from an empty cache (three
+    of the four splits have no key) to the last row of the cache."""
+    from deepj_amd import HipNative
+    d = H * hd
+    total = start + steps
+    q, k, v = (gaussian(total, d, 60 + i) for i in range(3))
+    cos, sin = ref.rope_tables(hd, max_seq)
+    exp_att = oracle_attention(q, k, v, H, cos, sin)
+    n_out = 48
+    w = gaussian(d, n_out, 70, 0.05)
+    res = gaussian(1, n_out, 71)
+    wdq = ref.q8_roundtrip(w)
+    dev = DeviceBuffers()
+    try:
+        kc, vc = dev.alloc(max_seq * d), dev.alloc(max_seq * d)
+        state = dev.upload(np.zeros(4, np.int32))
+        cos_b, sin_b = dev.upload(cos), dev.upload(sin)
+        if start:
+            sf = attention_scratch_floats(H, hd, max_seq)
+            scratch = dev.alloc(sf)
+            qkv0 = np.concatenate([q[:start], k[:start], v[:start]], axis=1)
+            qkv_b, q_b = dev.upload(qkv0), dev.alloc(start * d)
+            Stream().rope_kv_store(qkv_b, q_b, kc, vc, state, cos_b, sin_b, start, H, hd, max_seq, 0).run()
+        wsrc, wq = dev.upload(w), dev.alloc(HipNative.q8Floats(d, n_out))
+        Stream().q8_quantize(wsrc, wq, d, n_out).run()
+        rec = dev.alloc(attn_record_floats(H, hd))
+        row_b, out_b, res_b, att_b = dev.alloc(3 * d), dev.alloc(n_out), dev.upload(res), dev.alloc(d)
+        scratch_dec = dev.alloc(attn_decode_scratch_floats(H, hd))
+        for i in range(steps):
+            p = start + i
+            dev.write(state, np.array([p, 0, 0, 0], np.int32))
+            dev.write(row_b, np.concatenate([q[p], k[p], v[p]]))
+            (Stream().attn_decode_records(row_b, kc, vc, rec, state, cos_b, sin_b, H, hd, max_seq, 0)
+             .q8_linear(rec, wq, out_b, 1, d, n_out, residual=res_b, attn_merge_hd=hd).run())
+            exp = ref.add(res, ref.matmul(exp_att[p:p + 1], wdq))
+            scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+            assert_close(exp, dev.download(out_b, (1, n_out)), atol=1e-4 * scale, rtol=1e-4, what=f"step {i} at position {p}")
+            # the merging path and the self-merging ATTN_DECODE agree on the attention row itself (the row was
+            # appended by the first of them; the second rewrites the same values)
+            Stream().attn_decode(row_b, kc, vc, att_b, state, scratch_dec, cos_b, sin_b, H, hd, max_seq, 0).run()
+            assert_close(exp_att[p:p + 1], dev.download(att_b, (1, d)), atol=2e-5, rtol=1e-4, what=f"row {p}")
+    finally:
+        dev.release_all()
+
+
+def test_attn_merge_prologue_rejects_bad_combinations():
+    from deepj_amd import opcodes as op
+    dev = DeviceBuffers()
+    try:
+        rec, w, out, g = dev.alloc(attn_record_floats(2, 32)), dev.alloc(4096), dev.alloc(64), dev.alloc(64)
+        for flags, m, hd in ((op.LIN_ATTN_MERGE | op.LIN_RMSNORM, 1, 32), (op.LIN_ATTN_MERGE | op.LIN_GELU, 1, 32),
+                             (op.LIN_ATTN_MERGE, 2, 32), (op.LIN_ATTN_MERGE, 1, 48), (op.LIN_ATTN_MERGE, 1, 128)):
+            with pytest.raises(RuntimeError, match="OP_Q8_LINEAR"):
+                Stream().emit(op.OP_Q8_LINEAR, rec, w, out, m, 64, 4, flags, hd, -1, -1, -1).run()
+        small = dev.alloc(8)
+        with pytest.raises(RuntimeError, match="op needs"):
+            Stream().emit(op.OP_Q8_LINEAR, small, w, out, 1, 64, 4, op.LIN_ATTN_MERGE, 32, -1, -1, -1).run()
+        del g
     finally:
         dev.release_all()
 
