@@ -13,8 +13,9 @@
 // loads (1 KiB per wave-load, fully coalesced), convert int8 -> fp32 in registers,
 // multiply with the activation slice the lane keeps in VGPRs for the whole kernel,
 // and reduce across the wavefront with shuffles.  The activation vector is staged
-// once per workgroup through LDS, where the optional RMSNorm prologue is applied,
-// so norm + projection (+ bias, + residual, or the SwiGLU gate) is one launch.
+// once per workgroup through LDS, where the optional prologue is applied (RMSNorm,
+// LayerNorm, or the merge of the decode attention's per-split records), so norm +
+// projection (+ bias, + GELU, + residual, or the SwiGLU gate) is one launch.
 // M > 1 goes to the MFMA GEMM in kernels_matmul.hip.
 #include <cstdlib>
 
