@@ -277,6 +277,22 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     }
 }
 
+// Sum over the LPK (8, 16 or 32) consecutive lanes that share a key; every lane of the group gets the total.
+// DPP row operations instead of shuffles: a shuffle is an LDS-crossbar round trip with a wait behind it, and the
+// score of every key needs log2(LPK) of them in a row.
+template <int LPK>
+__device__ __forceinline__ float group_sum(float v) {
+#define DJ_DPP_ADD(ctrl) \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
+    DJ_DPP_ADD(0xB1);                             // quad_perm [1,0,3,2]
+    DJ_DPP_ADD(0x4E);                             // quad_perm [2,3,0,1]: quad sums
+    if constexpr (LPK >= 8) DJ_DPP_ADD(0x141);    // row_half_mirror: 8 lanes
+    if constexpr (LPK >= 16) DJ_DPP_ADD(0x140);   // row_mirror: 16 lanes
+#undef DJ_DPP_ADD
+    if constexpr (LPK == 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
 // ── fused decode attention ──────────────────────────────────────────────────
 // Record layout in scratch, per (head, split): [max, sum, pad, pad, o[hd]].
 struct DecodeArgs {
@@ -359,9 +375,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
                 *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = nk;
                 *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = nv;
             }
-            float s = qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w;
-#pragma unroll
-            for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+            float s = group_sum<LPK>(qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w);
             if (valid) {
                 s *= a.scale;
                 float mn = fmaxf(m, s);
@@ -469,29 +483,39 @@ __global__ void __launch_bounds__(kRecThreads) k_attn_decode_records(DecodeArgs 
     const int k_begin = split * per;
     const int k_end = k_begin + per < n_keys ? k_begin + per : n_keys;
 
+    float *kb = a.k_cache + (int64_t)h * a.head_stride + dl * 4;
+    float *vb = a.v_cache + (int64_t)h * a.head_stride + dl * 4;
+    float4 kk[U], vv[U];
+    auto load_tile = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int key = base + u * STRIDE;
+            const int row = (key < k_end && key != pos) ? key : 0;      // row 0 always exists; unused rows are masked
+            kk[u] = *reinterpret_cast<const float4 *>(kb + (int64_t)row * a.tok_stride);
+            vv[u] = *reinterpret_cast<const float4 *>(vb + (int64_t)row * a.tok_stride);
+        }
+    };
+    // The small operands (L2 hits) go out first and the first round of keys and values right behind them, all
+    // unconditional: the rotation below then waits for the small ones only (a counted wait) while the key/value
+    // rows are on their way from HBM.
     const float2 c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
     const float2 s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
-    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
+    float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
     const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
     const float4 nv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
+    const int base0 = k_begin + wave * KPW + sub;
+    load_tile(base0);
+    asm volatile("" ::: "memory");
+    asm volatile("" : "+v"(q0.x), "+v"(q0.y), "+v"(q0.z), "+v"(q0.w));
     const float4 qv = make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
                                   q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y);
     const float4 nk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
                                   k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
-    float *kb = a.k_cache + (int64_t)h * a.head_stride + dl * 4;
-    float *vb = a.v_cache + (int64_t)h * a.head_stride + dl * 4;
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int base = k_begin + wave * KPW + sub; base < k_end; base += U * STRIDE) {
-        float4 kk[U], vv[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            int key = base + u * STRIDE;
-            int row = (key < k_end && key != pos) ? key : k_begin;      // k_begin < n_keys: a row that exists
-            kk[u] = *reinterpret_cast<const float4 *>(kb + (int64_t)row * a.tok_stride);
-            vv[u] = *reinterpret_cast<const float4 *>(vb + (int64_t)row * a.tok_stride);
-        }
+    for (int off = 0;; ) {                                  // every lane runs the same number of rounds
+        const int base = base0 + off;
 #pragma unroll
         for (int u = 0; u < U; u++) {
             int key = base + u * STRIDE;
@@ -501,9 +525,7 @@ __global__ void __launch_bounds__(kRecThreads) k_attn_decode_records(DecodeArgs 
                 *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = nk;
                 *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = nv;
             }
-            float s = qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w;
-#pragma unroll
-            for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+            float s = group_sum<LPK>(qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w);
             if (valid) {
                 s *= a.scale;
                 float mn = fmaxf(m, s);
@@ -515,6 +537,9 @@ __global__ void __launch_bounds__(kRecThreads) k_attn_decode_records(DecodeArgs 
                 m = mn;
             }
         }
+        off += U * STRIDE;
+        if (off >= per) break;                              // workgroup-uniform
+        load_tile(base0 + off);
     }
     // the KPW lane groups of a wavefront first (shuffles), then the wavefronts (LDS)
 #pragma unroll
