@@ -43,6 +43,8 @@ struct Config {
 
 struct Error : std::runtime_error { using std::runtime_error::runtime_error; };
 
+constexpr int kGraphUnroll = 4;     // tokens per replay of the unrolled decode graph
+
 void hip(int rc) {
     if (rc != 0) throw Error(deepj_hip_last_error());
 }
@@ -74,7 +76,7 @@ struct Runner {
     int64_t p_sync_floats = 0;
     bool p_pending = false;                                // a persistent launch has not been checked yet
     Acts dec, pre;
-    int32_t graph = 0;
+    int32_t graph = 0, graph_unrolled = 0;                 // one token per replay / kGraphUnroll tokens per replay
     bool finalized = false;
     int32_t pos = 0;          // host mirror of state[0]
     int32_t generated = 0;    // host mirror of state[2]
@@ -505,11 +507,24 @@ void decode_greedy(Runner &r, int steps, int mode) {
         r.run(persistent_stream(r, steps));
         r.p_pending = true;
     } else if (use_graph) {
-        if (!r.graph) {
-            Stream s = decode_stream(r, true);
-            hip(deepj_hip_graph_capture(s.data(), (int32_t)s.size(), &r.graph));
+        // A replay costs a few microseconds of its own on top of its kernels: long runs go through a graph
+        // that holds kGraphUnroll consecutive tokens, the remainder through the one-token graph.
+        const int runs = steps / kGraphUnroll, rest = steps % kGraphUnroll;
+        if (runs > 0) {
+            if (!r.graph_unrolled) {
+                Stream one = decode_stream(r, true), s;
+                for (int i = 0; i < kGraphUnroll; i++) s.insert(s.end(), one.begin(), one.end());
+                hip(deepj_hip_graph_capture(s.data(), (int32_t)s.size(), &r.graph_unrolled));
+            }
+            hip(deepj_hip_graph_launch(r.graph_unrolled, runs));
         }
-        hip(deepj_hip_graph_launch(r.graph, steps));
+        if (rest > 0) {
+            if (!r.graph) {
+                Stream s = decode_stream(r, true);
+                hip(deepj_hip_graph_capture(s.data(), (int32_t)s.size(), &r.graph));
+            }
+            hip(deepj_hip_graph_launch(r.graph, rest));
+        }
     } else {
         Stream s = decode_stream(r, true);
         for (int i = 0; i < steps; i++) r.run(s);
@@ -669,6 +684,7 @@ void deepj_runner_destroy(void *h) {
     auto *r = static_cast<Runner *>(h);
     if (!r) return;
     if (r->graph) deepj_hip_graph_destroy(r->graph);
+    if (r->graph_unrolled) deepj_hip_graph_destroy(r->graph_unrolled);
     deepj_hip_synchronize();
     // every id in [id_base, next_id) that is still live belongs to this runner
     std::vector<int32_t> ids;
