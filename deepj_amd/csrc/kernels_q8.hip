@@ -134,8 +134,6 @@ __device__ __forceinline__ float dot16(const int4 &w, const float *xr) {
 
 // Sum over the 64 lanes with DPP row operations (no LDS traffic); every lane gets the total.
 __device__ __forceinline__ float wave_sum_dpp(float v) {
-    auto dpp = [](float x, int ctrl_unused) { return x; };
-    (void)dpp;
 #define DJ_DPP_ADD(ctrl, row_mask)                                                                        \
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, false))
     DJ_DPP_ADD(0xB1, 0xf);    // quad_perm [1,0,3,2]
