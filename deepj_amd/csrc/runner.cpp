@@ -59,7 +59,7 @@ struct Layer {
 struct Acts {          // activation buffers for S rows
     int32_t rows = 0;
     int32_t x = -1, x2 = -1, qkv = -1, q = -1, att = -1, ff = -1, ids = -1;
-    int32_t cq = -1, ckv = -1, kfull = -1, vfull = -1, kvexp = -1;   // MLA
+    int32_t cq = -1, ckv = -1;                                       // MLA
 };
 
 struct Runner {
@@ -70,7 +70,7 @@ struct Runner {
     int32_t emb = -1, gf = -1, wlm = -1, blm = -1;
     int32_t pos_table = -1, bf = -1;                       // GPT: learned positions, final LayerNorm beta
     int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
-    int32_t state = -1, tok = -1, tokens = -1, scratch = -1, scratch_dec = -1, logits = -1, last_x = -1;
+    int32_t state = -1, tokens = -1, scratch = -1, logits = -1, last_x = -1;
     int32_t records = -1;                                  // decode attention records (merged by the Wo matvec)
     int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
     int64_t p_sync_floats = 0;
@@ -306,18 +306,15 @@ void finalize(Runner &r) {
         r.kc = r.alloc(2 * per_layer);           // row t = [K_t | V_t]
     }
     r.state = r.alloc(4);
-    r.tok = r.alloc(4);
     r.tokens = r.alloc(c.max_seq);
     r.logits = r.alloc(c.vocab);
     r.last_x = r.alloc(c.d);
     int ns = std::max(1, std::min(16, 512 / c.heads));
     int64_t sf = (int64_t)c.heads * ns * (hd + 4);           // split-attention records (S = 1 paths)
     r.scratch = r.alloc(sf);
-    r.scratch_dec = r.alloc(sf);
     r.records = r.alloc((int64_t)c.heads * 4 * (hd + 4));
     Stream s;
     emit(s, DJ_OP_FILL, r.state, 0, 4);
-    emit(s, DJ_OP_FILL, r.tok, 0, 4);
     if (c.kind == 0) {
         int64_t psf = 0, paf = 0;
         hip(deepj_hip_llama_decode_plan(c.heads, hd, nullptr, nullptr, &psf, &paf));
@@ -691,12 +688,12 @@ void deepj_runner_destroy(void *h) {
     auto add = [&](int32_t id) { if (id >= 0) ids.push_back(id); };
     for (auto &L : r->layers)
         for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wuk, L.wuv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
-    for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state, r->tok,
-                       r->tokens, r->scratch, r->scratch_dec, r->records, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
+    for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state,
+                       r->tokens, r->scratch, r->records, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
                        r->pos_table, r->bf})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
-        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv, a->kfull, a->vfull, a->kvexp}) add(id);
+        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv}) add(id);
     if (!ids.empty()) deepj_hip_release(ids.data(), (int32_t)ids.size());
     delete r;
 }
