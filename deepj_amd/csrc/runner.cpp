@@ -14,6 +14,9 @@
 // Weight names: "emb", "gf", "wlm", "blm" and per layer "L<i>.<w>" with w in
 //   g1 g2 wq wk wv wo           (Llama;  MultiHeadSelfAttention.java:47-50)
 //   g1 g2 wdq wuq wdkv wuk wuv wo (DeepSeek; MultiHeadLatentAttention.java:81-86)
+//     kept as two Q8 matrices: the down-projections stacked by output row, [Wdq | pad | Wdkv], and the
+//     up-projections as one block matrix that maps [cQ | pad | cKV] to [Q | K | V] (zero blocks elsewhere),
+//     so MLA costs two projections and then shares the Llama attention path and its rotated K/V cache
 //   wg bg wu bu wd bd           (SwiGLULayer.java:56-58)
 // GPT (GPTTransformerBlock.java:52-57): g1 be1 g2 be2 (LayerNorm gamma/beta), wq wk wv wo, and the FNN's two
 //   Linears as wg bg (dModel -> dFF) and wd bd (dFF -> dModel); model level adds "pos" and "bf".
@@ -52,14 +55,14 @@ void hip(int rc) {
 struct Layer {
     int32_t g1 = -1, g2 = -1, be1 = -1, be2 = -1;     // be*: LayerNorm betas (GPT)
     int32_t wqkv = -1, wo = -1;                       // Llama: fused [3d x d]
-    int32_t wdq = -1, wuq = -1, wdkv = -1, wuk = -1, wuv = -1;   // MLA
+    int32_t wdown = -1, wup = -1;                     // MLA: stacked down-projections, block up-projection
     int32_t wgu = -1, bg = -1, bu = -1, wd = -1, bd = -1;
 };
 
 struct Acts {          // activation buffers for S rows
     int32_t rows = 0;
     int32_t x = -1, x2 = -1, qkv = -1, q = -1, att = -1, ff = -1, ids = -1;
-    int32_t cq = -1, ckv = -1;                                       // MLA
+    int32_t cq = -1;                                                 // MLA: [cQ | pad | cKV] rows
 };
 
 struct Runner {
@@ -69,7 +72,7 @@ struct Runner {
     std::vector<Layer> layers;
     int32_t emb = -1, gf = -1, wlm = -1, blm = -1;
     int32_t pos_table = -1, bf = -1;                       // GPT: learned positions, final LayerNorm beta
-    int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1, latent = -1;
+    int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1;
     int32_t state = -1, tokens = -1, scratch = -1, logits = -1, last_x = -1;
     int32_t records = -1;                                  // decode attention records (merged by the Wo matvec)
     int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
@@ -83,6 +86,10 @@ struct Runner {
     std::string error;
 
     int hd() const { return cfg.d / cfg.heads; }
+    // MLA: width of [cQ | pad | cKV]; cKV starts at a multiple of 32 so that the Q8 groups of Wuk and Wuv
+    // (32 consecutive inputs) are the ones each matrix would get on its own
+    int q_rank_padded() const { return (cfg.q_rank + 31) / 32 * 32; }
+    int latent_width() const { return q_rank_padded() + cfg.kv_rank; }
 
     int32_t alloc(int64_t floats) {
         if (floats > 0x7fffffffLL) throw Error("buffer too large for an int32 float count");
@@ -162,12 +169,28 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
             int part = w == "wq" ? 0 : (w == "wk" ? 1 : 2);
             quantize_into(r, L.wqkv, data, d, d, part * d, 1, 3 * d);
         }
-        else if (c.kind == 1 && w == "wdq") { expect_shape(name, rows, cols, d, c.q_rank); quantize_into(r, L.wdq, data, d, c.q_rank, 0, 1, c.q_rank); }
-        else if (c.kind == 1 && w == "wuq") { expect_shape(name, rows, cols, c.q_rank, d); quantize_into(r, L.wuq, data, c.q_rank, d, 0, 1, d); }
-        else if (c.kind == 1 && w == "wdkv") { expect_shape(name, rows, cols, d, c.kv_rank); quantize_into(r, L.wdkv, data, d, c.kv_rank, 0, 1, c.kv_rank); }
-        // Wuk and Wuv share one Q8 buffer (K rows first, then V rows): one GEMM re-expands both from the latent rows
-        else if (c.kind == 1 && w == "wuk") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuk, data, c.kv_rank, d, 0, 1, 2 * d); }
-        else if (c.kind == 1 && w == "wuv") { expect_shape(name, rows, cols, c.kv_rank, d); quantize_into(r, L.wuk, data, c.kv_rank, d, d, 1, 2 * d); }
+        else if (c.kind == 1 && (w == "wdq" || w == "wdkv")) {
+            // output rows [0, qRank) = Wdq, [qRankPadded, +kvRank) = Wdkv; the pad rows stay zero (the buffer is
+            // zero-filled when it is created) and so produce zeros
+            const bool q = w == "wdq";
+            expect_shape(name, rows, cols, d, q ? c.q_rank : c.kv_rank);
+            if (L.wdown < 0) {
+                L.wdown = r.alloc(deepj_hip_q8_floats(d, r.latent_width()));
+                Stream z; emit(z, DJ_OP_FILL, L.wdown, 0, deepj_hip_q8_floats(d, r.latent_width())); r.run(z);
+            }
+            quantize_into(r, L.wdown, data, d, cols, q ? 0 : r.q_rank_padded(), 1, r.latent_width());
+        }
+        else if (c.kind == 1 && (w == "wuq" || w == "wuk" || w == "wuv")) {
+            // block matrix over the inputs [cQ | pad | cKV]: the matrix is widened with zero rows to the full
+            // input width on the host, then its columns become Q8 rows [0,d) / [d,2d) / [2d,3d)
+            const bool q = w == "wuq";
+            const int in = q ? c.q_rank : c.kv_rank, k2 = r.latent_width(), off = q ? 0 : r.q_rank_padded();
+            expect_shape(name, rows, cols, in, d);
+            std::vector<float> wide((size_t)k2 * d, 0.0f);
+            std::memcpy(wide.data() + (size_t)off * d, data, (size_t)in * d * sizeof(float));
+            if (L.wup < 0) L.wup = r.alloc(deepj_hip_q8_floats(k2, 3 * d));
+            quantize_into(r, L.wup, wide.data(), k2, d, (q ? 0 : (w == "wuk" ? 1 : 2)) * d, 1, 3 * d);
+        }
         else throw Error("unknown weight " + name);
     } else throw Error("unknown weight " + name);
     r.have[name] = true;
@@ -265,12 +288,12 @@ void init_seeded(Runner &r, int64_t seed, int threads, float init_scale) {
 void alloc_acts(Runner &r, Acts &a, int rows) {
     const Config &c = r.cfg;
     if (a.rows == rows) return;
-    for (int32_t *id : {&a.x, &a.x2, &a.qkv, &a.q, &a.att, &a.ff, &a.ids, &a.cq, &a.ckv}) r.release(*id);
+    for (int32_t *id : {&a.x, &a.x2, &a.qkv, &a.q, &a.att, &a.ff, &a.ids, &a.cq}) r.release(*id);
     int64_t S = rows, d = c.d;
     a.x = r.alloc(S * d); a.x2 = r.alloc(S * d); a.q = r.alloc(S * d); a.att = r.alloc(S * d);
     a.ff = r.alloc(S * c.dff); a.ids = r.alloc(std::max<int64_t>(S, 4));
-    if (c.kind != 1) a.qkv = r.alloc(S * 3 * d);
-    else { a.cq = r.alloc(S * c.q_rank); a.ckv = r.alloc(S * c.kv_rank); a.qkv = r.alloc(S * d); }
+    a.qkv = r.alloc(S * 3 * d);
+    if (c.kind == 1) a.cq = r.alloc(S * r.latent_width());
     a.rows = rows;
 }
 
@@ -294,17 +317,12 @@ void finalize(Runner &r) {
     r.cos_t = r.upload_new(ct.data(), (int64_t)ct.size());
     r.sin_t = r.upload_new(st.data(), (int64_t)st.size());
     int64_t per_layer = (int64_t)c.max_seq * c.d;
-    if (c.kind != 1) {
-        r.kc = r.alloc(per_layer * c.layers);
-        r.vc = r.alloc(per_layer * c.layers);
-    } else {
-        // The latent rows cKV = norm1(x).Wdkv are the only per-token state that is kept
-        // (kvRank floats per token per layer instead of 2*dModel); K and V of every cached
-        // position are re-expanded from them - and K re-rotated - for each layer of each step,
-        // into these two scratch tensors (token-major [maxSeq x d]).
-        r.latent = r.alloc((int64_t)c.layers * c.max_seq * c.kv_rank);
-        r.kc = r.alloc(2 * per_layer);           // row t = [K_t | V_t]
-    }
+    // K (after RoPE) and V of every position, per layer [H][maxSeq][hd].  DeepSeek too: its latent rows could
+    // be cached instead (kvRank floats per token rather than 2*dModel), but the reference rotates K after the
+    // up-projection (MultiHeadLatentAttention.java:108-112), so the up-projection cannot be folded into the query
+    // and every step would have to re-expand and re-rotate all cached positions.
+    r.kc = r.alloc(per_layer * c.layers);
+    r.vc = r.alloc(per_layer * c.layers);
     r.state = r.alloc(4);
     r.tokens = r.alloc(c.max_seq);
     r.logits = r.alloc(c.vocab);
@@ -337,32 +355,26 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     const Layer &L = r.layers[l];
     const int d = c.d, H = c.heads, hd = r.hd();
     bool wo_done = false;
-    if (c.kind != 1) {
-        // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
-        // GPT: LayerNorm instead of RMSNorm and no rotation                  GPTTransformerBlock.java:66-68
-        if (c.kind == 2) q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1);
-        else q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
-        if (S == 1 && &a == &r.dec) {
-            // the key splits' records go straight to the Wo matvec, whose prologue merges them
-            emit(s, DJ_OP_ATTN_DECODE_RECORDS, a.qkv, r.kc, r.vc, r.records, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
-            emit(s, DJ_OP_Q8_LINEAR, r.records, L.wo, a.x2, 1, d, d, DJ_LIN_RESIDUAL | DJ_LIN_ATTN_MERGE, hd, -1, -1, a.x);
-            wo_done = true;
-        } else {
-            emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
-            emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
-        }
+    // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
+    // GPT: LayerNorm instead of RMSNorm and no rotation                  GPTTransformerBlock.java:66-68
+    // DeepSeek: [Q|K|V] = ([cQ|cKV] = norm1(x).[Wdq|Wdkv]) . blockdiag(Wuq, [Wuk|Wuv])   MultiHeadLatentAttention.java:92-123
+    if (c.kind == 1) {
+        const int k2 = r.latent_width();
+        q8_linear(s, a.x, L.wdown, a.cq, S, d, k2, DJ_LIN_RMSNORM, L.g1);
+        q8_linear(s, a.cq, L.wup, a.qkv, S, k2, 3 * d, 0);
+    } else if (c.kind == 2) {
+        q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1);
     } else {
-        // MultiHeadLatentAttention.java:92-123 with a latent cache
-        const int qr = c.q_rank, kvr = c.kv_rank;
-        const int64_t lat_off = (int64_t)l * c.max_seq * kvr;
-        q8_linear(s, a.x, L.wdq, a.cq, S, d, qr, DJ_LIN_RMSNORM, L.g1);            // cQ = norm1(x).Wdq
-        q8_linear(s, a.cq, L.wuq, a.qkv, S, qr, d, 0);                               // Q  = cQ.Wuq
-        q8_linear(s, a.x, L.wdkv, a.ckv, S, d, kvr, DJ_LIN_RMSNORM, L.g1);          // cKV = norm1(x).Wdkv
-        emit(s, DJ_OP_APPEND_ROWS, a.ckv, r.latent, r.state, S, kvr, c.max_seq, lat_off);
-        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wuk, r.kc, c.max_seq, kvr, 2 * d, r.state, S, lat_off);   // [K | V] = cKV.[Wuk | Wuv], all rows
-        emit(s, DJ_OP_ROPE_ROWS, r.kc, r.kc, r.state, r.cos_t, r.sin_t, c.max_seq, H, hd, c.max_seq, 1, 2 * d, S);  // K part, row = position
-        emit(s, DJ_OP_ROPE_ROWS, a.qkv, a.q, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, 0, 0, -1);
-        emit(s, DJ_OP_ATTENTION_KV, a.q, r.kc, r.kc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0, 2 * d, d);
+        q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
+    }
+    if (S == 1 && &a == &r.dec) {
+        // the key splits' records go straight to the Wo matvec, whose prologue merges them
+        emit(s, DJ_OP_ATTN_DECODE_RECORDS, a.qkv, r.kc, r.vc, r.records, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
+        emit(s, DJ_OP_Q8_LINEAR, r.records, L.wo, a.x2, 1, d, d, DJ_LIN_RESIDUAL | DJ_LIN_ATTN_MERGE, hd, -1, -1, a.x);
+        wo_done = true;
+    } else {
+        emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
+        emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
     }
     if (!wo_done) q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
     if (c.kind == 2) {
@@ -687,13 +699,13 @@ void deepj_runner_destroy(void *h) {
     std::vector<int32_t> ids;
     auto add = [&](int32_t id) { if (id >= 0) ids.push_back(id); };
     for (auto &L : r->layers)
-        for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdq, L.wuq, L.wdkv, L.wuk, L.wuv, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
-    for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->latent, r->state,
+        for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdown, L.wup, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
+    for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->state,
                        r->tokens, r->scratch, r->records, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
                        r->pos_table, r->bf})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
-        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv}) add(id);
+        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq}) add(id);
     if (!ids.empty()) deepj_hip_release(ids.data(), (int32_t)ids.size());
     delete r;
 }

@@ -148,7 +148,7 @@ def test_external_weights_path_matches_seeded_init():
     a.close(); b.close()
 
 
-# ── DeepSeek-style MLA model (latent KV cache) ───────────────────────────────
+# ── DeepSeek-style MLA model ────────────────────────────────────────────────
 
 DS = DeepSeekConfig(vocabSize=256, maxSeqLen=96, dModel=128, nHeads=4, nLayers=2, dFF=176, qRank=64, kvRank=32)
 
@@ -181,8 +181,8 @@ def test_deepseek_greedy_tokens_identical_and_graph_replay(ds):
     assert np.array_equal(eager, exp)
 
 
-def test_deepseek_latent_decode_row_equals_prefill_row(ds):
-    """The latent cache (cKV rows re-expanded every step) reproduces the full-context forward."""
+def test_deepseek_decode_row_equals_prefill_row(ds):
+    """The cached single-row path reproduces the full-context forward."""
     gpu, _ = ds
     ids = ref.JavaRandom(12).ints(30, 256)
     full = gpu.forward(ids)
