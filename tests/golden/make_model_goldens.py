@@ -3,12 +3,12 @@
 the baseline's full-size model configurations, which are too slow to run inside the test suite.
 
 The numbers come from this repository's oracle (oracle/, a C restatement of the reference's
-CpuBackend, layers, LlamaModel/DeepSeekModel and TextGenerator) run on the Q8-dequantised seeded
+CpuBackend, layers, LlamaModel/DeepSeekModel/GPTModel and TextGenerator) run on the Q8-dequantised seeded
 weights; nothing from the reference tree is imported or executed.  The reference's own tests hold
 no logits or token values for any model, so these fixtures pin the GPU path to the oracle, not to
 a JVM run.
 
-    python tests/golden/make_model_goldens.py c3 [c5]      # minutes per config on 8 cores
+    python tests/golden/make_model_goldens.py c3 [c5] [g2]      # minutes per config on 8 cores
 """
 import json
 import os
@@ -35,6 +35,13 @@ CONFIGS = {
     # seeded reference initialisation.
     "c5": dict(model=dict(vocab=32000, max_seq=512, d=2048, heads=16, layers=16, dff=5632, q_rank=1024, kv_rank=512),
                seed=42, prompt_seed=5, prompt_len=256, new_tokens=64, mla_weight_scale=0.25),
+    # GPT path at the size of GPT-2 small (GPTModel.java; not a BASELINE config): LayerNorm, GELU feed-forward,
+    # learned positions, an odd vocabulary, dModel = 768 (a Q8 row shorter than one 1 KiB chunk).  initScale 1:
+    # with GPTConfig's default 0.2 every LayerNorm gain is 0.2 too and the logits of a random model shrink to a
+    # few 1e-4, where the top-1/top-2 gap is no longer far above fp32 noise.  Prompt seed 8: the smallest
+    # top-1/top-2 gap over the 64 steps is 0.029 (seed 6 has a step with 5e-4, which no fp32 reordering is bound to keep).
+    "g2": dict(model=dict(vocab=50257, max_seq=1024, d=768, heads=12, layers=12, dff=3072, gpt=True, init_scale=1.0),
+               seed=42, prompt_seed=8, prompt_len=128, new_tokens=64),
 }
 OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "model_greedy.json")
 

@@ -10,7 +10,8 @@ path's (x1.25), and GPU-vs-oracle <= FULL_SIZE_LOGIT_ATOL.  (The 1e-3 gate is as
 small models in test_gpu_model.py.)  The DeepSeek fixture scales the MLA projections by 0.25: with the
 reference's initialiser at this width the attention softmax is a hard arg-max (scores with a standard
 deviation near 150) and two correct fp32 implementations diverge by O(1) within a few layers (see
-tests/golden/make_model_goldens.py).  Also size-independent properties at full size: graph
+tests/golden/make_model_goldens.py).  "g2" is the GPT path (LayerNorm, GELU, learned positions) at the size
+of GPT-2 small.  Also size-independent properties at full size: graph
 replay == eager, decode row == prefill row (KV-cache causality)."""
 import json
 import os
@@ -18,7 +19,8 @@ import os
 import numpy as np
 import pytest
 
-from deepj_amd import DeepSeekConfig, DeepSeekModel, JavaRandom, LlamaConfig, LlamaModel, TextGenerator
+from deepj_amd import (DeepSeekConfig, DeepSeekModel, GPTConfig, GPTModel, JavaRandom, LlamaConfig, LlamaModel,
+                       TextGenerator)
 
 pytestmark = pytest.mark.gpu
 
@@ -63,11 +65,14 @@ def build(name):
         if "mla_weight_scale" in c:
             return seeded_deepseek_with_scaled_mla(cfg, c["seed"], c["mla_weight_scale"]), c
         return DeepSeekModel(cfg, c["seed"]), c
+    if m.get("gpt"):
+        cfg = GPTConfig(m["vocab"], m["max_seq"], m["d"], m["heads"], m["layers"], m["dff"], initScale=m["init_scale"])
+        return GPTModel(cfg, c["seed"]), c
     cfg = LlamaConfig(m["vocab"], m["max_seq"], m["d"], m["heads"], m["layers"], m["dff"])
     return LlamaModel(cfg, c["seed"]), c
 
 
-@pytest.mark.parametrize("name", ["c3", "c5"])
+@pytest.mark.parametrize("name", ["c3", "c5", "g2"])
 def test_full_size_greedy_tokens_and_logits_match_oracle_fixture(name):
     if name not in GOLD:
         pytest.skip(f"no fixture for {name} (run tests/golden/make_model_goldens.py {name})")
