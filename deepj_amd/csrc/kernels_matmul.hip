@@ -1,17 +1,18 @@
-// Dense contractions on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+// Dense contractions on the matrix cores.
 //
 //   C[M x N] = A[M x K] . B      A fp32 row-major, fp32 accumulate
 //
-// B is either fp32 [K x N] row-major (OP_MATMUL; CpuBackend.java:168-188 in the
-// reference) or a Q8 weight [N x Kp] int8 + one fp32 scale per 32-group, which is
-// dequantised while it is staged into LDS (prefill-time Q8 GEMM: a dense
-// contraction, so it belongs on MFMA; the M = 1 decode case is a separate
-// HBM-bound kernel in kernels_q8.hip).
+// fp32 B [K x N] row-major (OP_MATMUL; CpuBackend.java:168-188 in the reference): v_mfma_f32_32x32x2_f32.
+// 256 threads = 4 wavefronts; workgroup tile 64 x 64 (one 32 x 32 accumulator per wavefront) or 128 x 128 (four),
+// K advances 32 per step.  Both operand tiles sit k-major in LDS so the 64 lanes of an MFMA operand read 32
+// consecutive floats per half-wave (no bank conflicts).
 //
-// Tiling: 256 threads = 4 wavefronts, workgroup tile 64 x 64, each wavefront owns
-// one 32 x 32 accumulator (16 VGPRs), K advances 32 per step = one Q8 group.
-// Both operand tiles sit k-major in LDS so the 64 lanes of an MFMA operand read
-// 32 consecutive floats per half-wave (no bank conflicts).
+// Q8 B [N x Kp] int8 + one fp32 scale per 32-group (prefill-time Q8 GEMM; the M = 1 decode case is the HBM-bound
+// kernel in kernels_q8.hip): v_mfma_f32_32x32x16_bf16 at full fp32 accuracy.  An int8 weight is exact in bf16,
+// and an fp32 activation is the exact sum of three bf16 numbers (its top, middle and bottom 8 significant bits,
+// taken by truncation), so x . q = hi . q + mid . q + lo . q with every product exact and fp32 accumulation: three
+// bf16 MFMAs of K = 16 replace eight fp32 MFMAs of K = 2 at four times the rate.  The group scale multiplies the
+// finished 32-k partial sums (one scale per accumulator column per step).
 #include "dj_common.h"
 
 namespace dj {
@@ -40,10 +41,8 @@ __device__ __forceinline__ float gemm_gelu(float x) {
     return 0.5f * x * (1.0f + (float)tanh((double)t));
 }
 
-template <bool Q8>
 __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const float *__restrict__ Bf,
-                                              const int8_t *__restrict__ Bq, const float *__restrict__ Bs,
-                                              float *__restrict__ C, int M, const int N, const int K, const int kp,
+                                              float *__restrict__ C, int M, const int N, const int K,
                                               GemmEpilogue ep) {
     __shared__ float As[BK][BM + PAD];
     __shared__ float Bl[BK][BN + PAD];
@@ -69,9 +68,7 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
     // Register-staged software pipeline: the global loads of K-step i+1 are issued before the MFMAs of
     // step i, so their latency hides behind the matrix work instead of adding to every step.
     float va[8];                 // A: 8 consecutive k of one row
-    float wb[8];                 // B fp32: 8 consecutive columns of one k
-    int2 qraw = make_int2(0, 0); // B Q8: 8 consecutive k of one column
-    float qsc = 0.0f;
+    float wb[8];                 // B: 8 consecutive columns of one k
     auto fetch = [&](int k0) {
         {
             int gr = m0 + a_row;
@@ -87,18 +84,7 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
                 }
             }
         }
-        if constexpr (Q8) {
-            int col = t >> 2, part = t & 3;          // 8 int8 per thread
-            int gn = n0 + col;
-            if (gn < N) {
-                const int8_t *p = Bq + (int64_t)gn * kp + k0 + part * 8;   // kp is a multiple of 32: in bounds
-                qraw = *reinterpret_cast<const int2 *>(p);
-                qsc = Bs[(int64_t)gn * (kp / kQ8Group) + k0 / kQ8Group];
-            } else {
-                qraw = make_int2(0, 0);
-                qsc = 0.0f;
-            }
-        } else {
+        {
             int bk = t >> 3, bn = (t & 7) * 8;       // 8 consecutive columns per thread
             int gk = k0 + bk;
             if (gk < K && (N & 3) == 0 && n0 + bn + 8 <= N) {
@@ -117,17 +103,7 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
     auto stage = [&]() {
 #pragma unroll
         for (int j = 0; j < 8; j++) As[a_k + j][a_row] = va[j];
-        if constexpr (Q8) {
-            int col = t >> 2, part = t & 3;
-            int r0 = qraw.x, r1 = qraw.y;
-            float w[8];
-            w[0] = (float)(int8_t)(r0 & 0xff) * qsc;         w[1] = (float)(int8_t)((r0 >> 8) & 0xff) * qsc;
-            w[2] = (float)(int8_t)((r0 >> 16) & 0xff) * qsc; w[3] = (float)(int8_t)((r0 >> 24) & 0xff) * qsc;
-            w[4] = (float)(int8_t)(r1 & 0xff) * qsc;         w[5] = (float)(int8_t)((r1 >> 8) & 0xff) * qsc;
-            w[6] = (float)(int8_t)((r1 >> 16) & 0xff) * qsc; w[7] = (float)(int8_t)((r1 >> 24) & 0xff) * qsc;
-#pragma unroll
-            for (int j = 0; j < 8; j++) Bl[part * 8 + j][col] = w[j];
-        } else {
+        {
             int bk = t >> 3, bn = (t & 7) * 8;
 #pragma unroll
             for (int j = 0; j < 8; j++) Bl[bk][bn + j] = wb[j];
@@ -175,10 +151,8 @@ __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const
 // value read from LDS feeds two MFMAs instead of one, which is what the 64 x 64 kernel is bound by.
 constexpr int BM2 = 128, BN2 = 128;
 
-template <bool Q8>
 __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, const float *__restrict__ Bf,
-                                                 const int8_t *__restrict__ Bq, const float *__restrict__ Bs,
-                                                 float *__restrict__ C, int M, const int N, const int K, const int kp,
+                                                 float *__restrict__ C, int M, const int N, const int K,
                                                  GemmEpilogue ep) {
     __shared__ float As[BK][BM2 + PAD];
     __shared__ float Bl[BK][BN2 + PAD];
@@ -206,9 +180,7 @@ __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, co
     const bool a_vec = (K & 3) == 0;
 
     float va[16];                // A: 16 consecutive k of one row
-    float wb[16];                // B fp32: 16 consecutive columns of one k
-    int4 qraw = make_int4(0, 0, 0, 0);   // B Q8: 16 consecutive k of one column (half a scale group)
-    float qsc = 0.0f;
+    float wb[16];                // B: 16 consecutive columns of one k
     auto fetch = [&](int k0) {
         {
             int gr = m0 + a_row;
@@ -227,18 +199,7 @@ __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, co
                 }
             }
         }
-        if constexpr (Q8) {
-            int col = t >> 1, part = t & 1;
-            int gn = n0 + col;
-            if (gn < N) {
-                const int8_t *p = Bq + (int64_t)gn * kp + k0 + part * 16;  // kp is a multiple of 32: in bounds
-                qraw = *reinterpret_cast<const int4 *>(p);
-                qsc = Bs[(int64_t)gn * (kp / kQ8Group) + k0 / kQ8Group];
-            } else {
-                qraw = make_int4(0, 0, 0, 0);
-                qsc = 0.0f;
-            }
-        } else {
+        {
             int bk = t >> 3, bn = (t & 7) * 16;      // 16 consecutive columns per thread
             int gk = k0 + bk;
             if (gk < K && (N & 3) == 0 && n0 + bn + 16 <= N) {
@@ -260,18 +221,7 @@ __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, co
     auto stage = [&]() {
 #pragma unroll
         for (int j = 0; j < 16; j++) As[a_k + j][a_row] = va[j];
-        if constexpr (Q8) {
-            int col = t >> 1, part = t & 1;
-            const int words[4] = {qraw.x, qraw.y, qraw.z, qraw.w};
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                int r = words[q];
-                Bl[part * 16 + 4 * q + 0][col] = (float)(int8_t)(r & 0xff) * qsc;
-                Bl[part * 16 + 4 * q + 1][col] = (float)(int8_t)((r >> 8) & 0xff) * qsc;
-                Bl[part * 16 + 4 * q + 2][col] = (float)(int8_t)((r >> 16) & 0xff) * qsc;
-                Bl[part * 16 + 4 * q + 3][col] = (float)(int8_t)((r >> 24) & 0xff) * qsc;
-            }
-        } else {
+        {
             int bk = t >> 3, bn = (t & 7) * 16;
 #pragma unroll
             for (int j = 0; j < 16; j++) Bl[bk][bn + j] = wb[j];
@@ -320,6 +270,179 @@ __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, co
     }
 }
 
+// ── Q8 weights: three-way bf16 split of the activations ────────────────────
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int LDK = 40;      // LDS row: 32 bf16 of payload + 8 of padding (80 bytes: 16-byte aligned, spreads banks)
+
+// bf16(a) | bf16(b) << 16, both by truncation
+__device__ __forceinline__ uint32_t pack_bf16_hi(float a, float b) {
+    return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, b), __builtin_bit_cast(uint32_t, a), 0x07060302);
+}
+__device__ __forceinline__ float top_bits(float x) {      // the leading 8 significant bits of x: a bf16 value
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & 0xffff0000u);
+}
+
+// WT = 1: workgroup tile 64 x 64, one 32 x 32 accumulator per wavefront; WT = 2: 128 x 128, four.
+// Operand element j of lane l is k = 16*step + 8*(l / 32) + j for A and B alike, so the pairing of the MFMA's
+// k slots does not depend on how the hardware numbers them.
+template <int WT>
+__global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, const int8_t *__restrict__ Bq,
+                                                 const float *__restrict__ Bs, float *__restrict__ C, int M,
+                                                 const int N, const int K, const int kp, GemmEpilogue ep) {
+    constexpr int TM = 64 * WT, TN = 64 * WT;
+    constexpr int EL = TM * BK / 256;        // activation floats (and weight bytes) a thread stages per step: 8 or 16
+    constexpr int TPR = BK / EL;             // threads per tile row
+    __shared__ __align__(16) uint16_t Xs[3][TM][LDK];     // hi / mid / lo pieces, row-major, k contiguous
+    __shared__ __align__(16) uint16_t Wl[TN][LDK];        // weights as bf16, one row per output column
+    __shared__ float Ss[TN];                               // this step's group scale per output column
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    if (ep.m_dev) {
+        int live = ep.m_dev[0] + ep.m_extra;
+        if (live < M) M = live;
+        if (m0 >= M) return;                 // workgroup-uniform
+    }
+    const int groups = kp / kQ8Group;
+
+    floatx16 acc[WT][WT];
+#pragma unroll
+    for (int i = 0; i < WT; i++)
+#pragma unroll
+        for (int j = 0; j < WT; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    const int s_row = t / TPR;               // tile row (A) and tile column (B) this thread stages
+    const int s_k = (t % TPR) * EL;
+    const bool a_vec = (K & 3) == 0;
+
+    float va[EL];
+    int qraw[EL / 4];
+    float qsc = 0.0f;
+    auto fetch = [&](int k0) {
+        const int gr = m0 + s_row;
+        if (gr < M && a_vec && k0 + s_k + EL <= K) {
+            const float4 *p = reinterpret_cast<const float4 *>(A + (int64_t)gr * K + k0 + s_k);
+#pragma unroll
+            for (int q = 0; q < EL / 4; q++) {
+                float4 x = p[q];
+                va[4 * q] = x.x; va[4 * q + 1] = x.y; va[4 * q + 2] = x.z; va[4 * q + 3] = x.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < EL; j++) {
+                int gk = k0 + s_k + j;
+                va[j] = (gr < M && gk < K) ? A[(int64_t)gr * K + gk] : 0.0f;
+            }
+        }
+        const int gn = n0 + s_row;
+        if (gn < N) {
+            const int *p = reinterpret_cast<const int *>(Bq + (int64_t)gn * kp + k0 + s_k);   // kp is a multiple of 32: in bounds
+#pragma unroll
+            for (int q = 0; q < EL / 4; q++) qraw[q] = p[q];
+            qsc = Bs[(int64_t)gn * groups + k0 / kQ8Group];
+        } else {
+#pragma unroll
+            for (int q = 0; q < EL / 4; q++) qraw[q] = 0;
+            qsc = 0.0f;
+        }
+    };
+    auto stage = [&]() {
+        uint32_t ph[EL / 2], pm[EL / 2], pl[EL / 2], pw[EL / 2];
+#pragma unroll
+        for (int j = 0; j < EL / 2; j++) {
+            const float x0 = va[2 * j], x1 = va[2 * j + 1];
+            const float h0 = top_bits(x0), h1 = top_bits(x1);
+            const float r0 = x0 - h0, r1 = x1 - h1;              // exact: h is a prefix of x
+            const float c0 = top_bits(r0), c1 = top_bits(r1);
+            const float l0 = r0 - c0, l1 = r1 - c1;              // at most 8 significant bits left: a bf16 value
+            ph[j] = pack_bf16_hi(h0, h1); pm[j] = pack_bf16_hi(c0, c1); pl[j] = pack_bf16_hi(l0, l1);
+        }
+#pragma unroll
+        for (int q = 0; q < EL / 4; q++) {
+            const int r = qraw[q];
+            pw[2 * q] = pack_bf16_hi((float)(int8_t)(r & 0xff), (float)(int8_t)((r >> 8) & 0xff));
+            pw[2 * q + 1] = pack_bf16_hi((float)(int8_t)((r >> 16) & 0xff), (float)(int8_t)((r >> 24) & 0xff));
+        }
+#pragma unroll
+        for (int q = 0; q < EL / 8; q++) {
+            reinterpret_cast<uint4 *>(&Xs[0][s_row][s_k])[q] = make_uint4(ph[4 * q], ph[4 * q + 1], ph[4 * q + 2], ph[4 * q + 3]);
+            reinterpret_cast<uint4 *>(&Xs[1][s_row][s_k])[q] = make_uint4(pm[4 * q], pm[4 * q + 1], pm[4 * q + 2], pm[4 * q + 3]);
+            reinterpret_cast<uint4 *>(&Xs[2][s_row][s_k])[q] = make_uint4(pl[4 * q], pl[4 * q + 1], pl[4 * q + 2], pl[4 * q + 3]);
+            reinterpret_cast<uint4 *>(&Wl[s_row][s_k])[q] = make_uint4(pw[4 * q], pw[4 * q + 1], pw[4 * q + 2], pw[4 * q + 3]);
+        }
+        if ((t % TPR) == 0) Ss[s_row] = qsc;
+    };
+
+    if (K > 0) fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        stage();
+        __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);       // next step's global loads fly while this step multiplies
+
+        floatx16 g[WT][WT];                    // this group's unscaled partial sums
+#pragma unroll
+        for (int i = 0; i < WT; i++)
+#pragma unroll
+            for (int j = 0; j < WT; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) g[i][j][e] = 0.0f;
+#pragma unroll
+        for (int step = 0; step < BK / 16; step++) {
+            const int kofs = step * 16 + half * 8;
+            bf16x8 b[WT];
+#pragma unroll
+            for (int tn = 0; tn < WT; tn++) b[tn] = *reinterpret_cast<const bf16x8 *>(&Wl[wn * 32 * WT + 32 * tn + l32][kofs]);
+#pragma unroll
+            for (int piece = 0; piece < 3; piece++) {
+#pragma unroll
+                for (int tm = 0; tm < WT; tm++) {
+                    const bf16x8 a = *reinterpret_cast<const bf16x8 *>(&Xs[piece][wm * 32 * WT + 32 * tm + l32][kofs]);
+#pragma unroll
+                    for (int tn = 0; tn < WT; tn++) g[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[tn], g[tm][tn], 0, 0, 0);
+                }
+            }
+        }
+        // every accumulator entry of a lane belongs to one output column: one scale per lane and tile column
+#pragma unroll
+        for (int tn = 0; tn < WT; tn++) {
+            const float sc = Ss[wn * 32 * WT + 32 * tn + l32];
+#pragma unroll
+            for (int tm = 0; tm < WT; tm++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[tm][tn][e] = fmaf(g[tm][tn][e], sc, acc[tm][tn][e]);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: acc[i][jn][e] is C[32*i + 8*(e/4) + 4*(lane/32) + e%4][32*jn + lane%32] of the wavefront's block
+#pragma unroll
+    for (int jn = 0; jn < WT; jn++) {
+        const int col = n0 + wn * 32 * WT + 32 * jn + l32;
+        if (col >= N) continue;
+        float badd = 0.0f;
+        if (ep.bias) badd = ep.interleaved_bias ? ((col & 1) ? ep.bias2[col >> 1] : ep.bias[col >> 1]) : ep.bias[col];
+#pragma unroll
+        for (int i = 0; i < WT; i++) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = m0 + wm * 32 * WT + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                if (row < M) {
+                    float v = acc[i][jn][e];
+                    if (ep.bias) v = v + badd;
+                    if (ep.gelu) v = gemm_gelu(v);
+                    if (ep.residual) v = ep.residual[(int64_t)row * N + col] + v;
+                    C[(int64_t)row * N + col] = v;
+                }
+            }
+        }
+    }
+}
+
 // The large tile needs enough workgroups to fill the chip; small problems keep the 64 x 64 tile.
 inline bool use_big_tile(int m, int n) {
     return m >= 128 && n >= 128 && (int64_t)((m + BM2 - 1) / BM2) * ((n + BN2 - 1) / BN2) >= 256;
@@ -333,13 +456,11 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
     GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0, 0};
     if (use_big_tile(m, n)) {
         dim3 grid2((n + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
-        hipLaunchKernelGGL(k_gemm128<false>, grid2, dim3(256), 0, s, a, b, (const int8_t *)nullptr, (const float *)nullptr,
-                           out, m, n, k, 0, ep);
+        hipLaunchKernelGGL(k_gemm128, grid2, dim3(256), 0, s, a, b, out, m, n, k, ep);
         return;
     }
     dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM);
-    hipLaunchKernelGGL(k_gemm<false>, grid, dim3(256), 0, s, a, b, (const int8_t *)nullptr, (const float *)nullptr,
-                       out, m, n, k, 0, ep);
+    hipLaunchKernelGGL(k_gemm, grid, dim3(256), 0, s, a, b, out, m, n, k, ep);
 }
 
 // Q8 GEMM used by launch_q8_linear for M > 1.  n_rows is the number of Q8 rows
@@ -351,13 +472,11 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
     GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu};
     if (!m_dev && use_big_tile(m, n_rows)) {       // a device-side row count is usually far below m: keep small tiles
         dim3 grid2((n_rows + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
-        hipLaunchKernelGGL(k_gemm128<true>, grid2, dim3(256), 0, s, x, (const float *)nullptr, wq, scales, out, m,
-                           n_rows, k, q8_padded_k(k), ep);
+        hipLaunchKernelGGL(k_gemm_q8<2>, grid2, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
         return;
     }
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
-    hipLaunchKernelGGL(k_gemm<true>, grid, dim3(256), 0, s, x, (const float *)nullptr, wq, scales, out, m, n_rows, k,
-                       q8_padded_k(k), ep);
+    hipLaunchKernelGGL(k_gemm_q8<1>, grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
 }
 
 }  // namespace dj
