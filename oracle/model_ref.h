@@ -15,7 +15,15 @@
  *   layers/transformer/blocks/LlamaTransformerBlock.java:50-53, DeepSeekTransformerBlock.java:54-57
  *   transformer/TransformerStack.java:28-35, models/DecoderOnlyModel.java:58-64
  *   models/llama/LlamaModel.java:27-42, models/deepseek/DeepSeekModel.java:29-46 (seeded init order)
+ *   layers/transformer/norm/LayerNorm1D.java:34-66       ref_layernorm
+ *   layers/FNN.java:57-73 + activations/GELU.java:15-18   the GPT feed-forward (Linear, GELU, Linear)
+ *   transformer/embeddings/PositionalEmbedding.java:26-33, models/gpt/GPTModel.java:27-81,
+ *   layers/transformer/blocks/GPTTransformerBlock.java:52-73   GPT model: learned positions, init order, initScale
  *   models/TextGenerator.java:66-181 (sliding window, stable argsort, top-k, temperature, categorical draw)
+ *
+ * The reference's tests hold no forward known answers for LayerNorm1D, FNN or GPTModel (gradient checks and
+ * shapes only): those functions are pinned by closed forms and fp64 brute force (tests/test_oracle_invariants.py),
+ * plus GPTModelTest's parameter count and init-scale ratio.
  *
  * The Q8 weight format and the incremental (KV-cached) forward have no
  * counterpart in the reference: parity unpinned by the reference.  They are
