@@ -18,9 +18,11 @@
 // HBM-bound KV read is spread over all CUs, and a second tiny kernel merges the
 // per-split (max, sum, weighted V) records.
 #include "dj_common.h"
+#include "dj_device.h"
 
 namespace dj {
 namespace {
+using namespace dev;
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
@@ -275,22 +277,6 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; e++) orow[32 * i + 8 * (e >> 2) + 4 * half + (e & 3)] = acc[i][e] / l;
     }
-}
-
-// Sum over the LPK (8, 16 or 32) consecutive lanes that share a key; every lane of the group gets the total.
-// DPP row operations instead of shuffles: a shuffle is an LDS-crossbar round trip with a wait behind it, and the
-// score of every key needs log2(LPK) of them in a row.
-template <int LPK>
-__device__ __forceinline__ float group_sum(float v) {
-#define DJ_DPP_ADD(ctrl) \
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
-    DJ_DPP_ADD(0xB1);                             // quad_perm [1,0,3,2]
-    DJ_DPP_ADD(0x4E);                             // quad_perm [2,3,0,1]: quad sums
-    if constexpr (LPK >= 8) DJ_DPP_ADD(0x141);    // row_half_mirror: 8 lanes
-    if constexpr (LPK >= 16) DJ_DPP_ADD(0x140);   // row_mirror: 16 lanes
-#undef DJ_DPP_ADD
-    if constexpr (LPK == 32) v += __shfl_xor(v, 16, 64);
-    return v;
 }
 
 // ── fused decode attention ──────────────────────────────────────────────────

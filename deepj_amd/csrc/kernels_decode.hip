@@ -21,9 +21,11 @@
 #include <cstdlib>
 
 #include "dj_common.h"
+#include "dj_device.h"
 
 namespace dj {
 namespace {
+using namespace dev;
 
 constexpr int kDT = 512;                  // threads per workgroup
 constexpr int kDW = kDT / 64;             // wavefronts per workgroup
@@ -49,33 +51,6 @@ __device__ __forceinline__ float2 ldc_f2(const float *p) {
 __device__ __forceinline__ void wait_stores() { __builtin_amdgcn_s_waitcnt(0x0f70); }     // vmcnt(0)
 
 __device__ __forceinline__ float d_sigmoid(float x) { return 1.0f / (1.0f + (float)exp((double)(-x))); }
-
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-#define DJ_DPP_ADD(ctrl, row_mask) \
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, false))
-    DJ_DPP_ADD(0xB1, 0xf);
-    DJ_DPP_ADD(0x4E, 0xf);
-    DJ_DPP_ADD(0x141, 0xf);
-    DJ_DPP_ADD(0x140, 0xf);
-    DJ_DPP_ADD(0x142, 0xa);
-    DJ_DPP_ADD(0x143, 0xc);
-#undef DJ_DPP_ADD
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
-}
-
-__device__ __forceinline__ float dot16(const int4 &w, const float *xr) {
-    float d = 0.0f;
-    const int words[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        int v = words[i];
-        d = fmaf(xr[4 * i + 0], (float)(int8_t)(v & 0xff), d);
-        d = fmaf(xr[4 * i + 1], (float)(int8_t)((v >> 8) & 0xff), d);
-        d = fmaf(xr[4 * i + 2], (float)(int8_t)((v >> 16) & 0xff), d);
-        d = fmaf(xr[4 * i + 3], (float)(v >> 24), d);
-    }
-    return d;
-}
 
 // Float.compare order, ties to the lower index (TextGenerator.java:163-170)
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {

@@ -20,6 +20,7 @@
 #include <cstdlib>
 
 #include "dj_common.h"
+#include "dj_device.h"
 
 namespace dj {
 
@@ -28,6 +29,7 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
                     int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu);
 
 namespace {
+using namespace dev;
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
@@ -100,15 +102,6 @@ __global__ void __launch_bounds__(kThreads) k_q8_dequantize(const int8_t *__rest
     }
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global
-// load (its workgroup-scope fence needs vmcnt(0)), which here would park the workgroup until the weight rows
-// already requested from HBM have arrived; the staged activations only need the LDS writes to be complete.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
 // ── decode matvec ──────────────────────────────────────────────────────────
 struct MatvecArgs {
     const float *x; const int8_t *wq; const float *scales; float *out;
@@ -117,34 +110,6 @@ struct MatvecArgs {
     const float *beta;                // set: LayerNorm prologue with gamma and beta (otherwise gamma alone = RMSNorm)
     int rec_hd;                       // ATTN_MERGE prologue: x holds attention records of heads this wide
 };
-
-__device__ __forceinline__ float dot16(const int4 &w, const float *xr) {
-    float d = 0.0f;
-    const int words[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        int v = words[i];
-        d = fmaf(xr[4 * i + 0], (float)(int8_t)(v & 0xff), d);
-        d = fmaf(xr[4 * i + 1], (float)(int8_t)((v >> 8) & 0xff), d);
-        d = fmaf(xr[4 * i + 2], (float)(int8_t)((v >> 16) & 0xff), d);
-        d = fmaf(xr[4 * i + 3], (float)(v >> 24), d);
-    }
-    return d;
-}
-
-// Sum over the 64 lanes with DPP row operations (no LDS traffic); every lane gets the total.
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-#define DJ_DPP_ADD(ctrl, row_mask)                                                                        \
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, false))
-    DJ_DPP_ADD(0xB1, 0xf);    // quad_perm [1,0,3,2]
-    DJ_DPP_ADD(0x4E, 0xf);    // quad_perm [2,3,0,1]
-    DJ_DPP_ADD(0x141, 0xf);   // row_half_mirror
-    DJ_DPP_ADD(0x140, 0xf);   // row_mirror: every lane of a 16-lane row holds the row sum
-    DJ_DPP_ADD(0x142, 0xa);   // row_bcast:15 into rows 1 and 3
-    DJ_DPP_ADD(0x143, 0xc);   // row_bcast:31 into rows 2 and 3: lane 63 holds the total
-#undef DJ_DPP_ADD
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
-}
 
 // One batch of Q8 rows held in registers by a wavefront: R rows x NC chunks.
 template <int NC, int R> struct RowBatch {
