@@ -27,9 +27,11 @@ SOURCES = {
     "runtime.cpp": [],
     "kernels_elementwise.hip": ["-ffp-contract=off"],
     "kernels_reduce.hip": ["-ffp-contract=off"],
-    "kernels_matmul.hip": [],
+    # matrix-core accumulators in ordinary vector registers: the kernels rescale or mask them with vector
+    # instructions after every few products, and each trip through the accumulator file costs a move per value
+    "kernels_matmul.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "kernels_q8.hip": [],
-    "kernels_attn.hip": [],
+    "kernels_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "kernels_decode.hip": [],
     "runner.cpp": [],
     "host_random.cpp": [],
