@@ -272,7 +272,6 @@ __global__ void __launch_bounds__(256) k_gemm128(const float *__restrict__ A, co
 
 // ── Q8 weights: three-way bf16 split of the activations ────────────────────
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-constexpr int LDK = 40;      // LDS row: 32 bf16 of payload + 8 of padding (80 bytes: 16-byte aligned, spreads banks)
 
 // bf16(a) | bf16(b) << 16, both by truncation
 __device__ __forceinline__ uint32_t pack_bf16_hi(float a, float b) {
@@ -283,18 +282,23 @@ __device__ __forceinline__ float top_bits(float x) {      // the leading 8 signi
 }
 
 // WT = 1: workgroup tile 64 x 64, one 32 x 32 accumulator per wavefront; WT = 2: 128 x 128, four.
+// G: scale groups (of 32 k) per step.  A step costs two barriers and an LDS round trip whatever its size, and a
+// 64 x 64 tile has only six products per wavefront and group to set against that, so it takes several groups a step.
 // Operand element j of lane l is k = 16*step + 8*(l / 32) + j for A and B alike, so the pairing of the MFMA's
 // k slots does not depend on how the hardware numbers them.
-template <int WT>
+template <int WT, int G>
 __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, const int8_t *__restrict__ Bq,
                                                  const float *__restrict__ Bs, float *__restrict__ C, int M,
                                                  const int N, const int K, const int kp, GemmEpilogue ep) {
     constexpr int TM = 64 * WT, TN = 64 * WT;
-    constexpr int EL = TM * BK / 256;        // activation floats (and weight bytes) a thread stages per step: 8 or 16
-    constexpr int TPR = BK / EL;             // threads per tile row
+    constexpr int QBK = kQ8Group * G;        // k per step
+    constexpr int LDK = QBK + 8;             // LDS row: the step's bf16 payload + 8 of padding (16-byte aligned, spreads banks)
+    constexpr int EL = TM * QBK / 256;       // activation floats (and weight bytes) a thread stages per step
+    constexpr int TPR = QBK / EL;            // threads per tile row
+    static_assert(EL >= 8 && EL <= kQ8Group && kQ8Group % EL == 0, "a thread's share of a row lies inside one scale group");
     __shared__ __align__(16) uint16_t Xs[3][TM][LDK];     // hi / mid / lo pieces, row-major, k contiguous
     __shared__ __align__(16) uint16_t Wl[TN][LDK];        // weights as bf16, one row per output column
-    __shared__ float Ss[TN];                               // this step's group scale per output column
+    __shared__ float Ss[G][TN];                            // this step's group scales per output column
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
@@ -340,11 +344,11 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
             }
         }
         const int gn = n0 + s_row;
-        if (gn < N) {
+        if (gn < N && k0 + s_k < kp) {
             const int *p = reinterpret_cast<const int *>(Bq + (int64_t)gn * kp + k0 + s_k);   // kp is a multiple of 32: in bounds
 #pragma unroll
             for (int q = 0; q < EL / 4; q++) qraw[q] = p[q];
-            qsc = Bs[(int64_t)gn * groups + k0 / kQ8Group];
+            qsc = Bs[(int64_t)gn * groups + (k0 + s_k) / kQ8Group];
         } else {
 #pragma unroll
             for (int q = 0; q < EL / 4; q++) qraw[q] = 0;
@@ -375,15 +379,17 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
             reinterpret_cast<uint4 *>(&Xs[2][s_row][s_k])[q] = make_uint4(pl[4 * q], pl[4 * q + 1], pl[4 * q + 2], pl[4 * q + 3]);
             reinterpret_cast<uint4 *>(&Wl[s_row][s_k])[q] = make_uint4(pw[4 * q], pw[4 * q + 1], pw[4 * q + 2], pw[4 * q + 3]);
         }
-        if ((t % TPR) == 0) Ss[s_row] = qsc;
+        if (s_k % kQ8Group == 0) Ss[s_k / kQ8Group][s_row] = qsc;
     };
 
     if (K > 0) fetch(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
+    for (int k0 = 0; k0 < K; k0 += QBK) {
         stage();
         __syncthreads();
-        if (k0 + BK < K) fetch(k0 + BK);       // next step's global loads fly while this step multiplies
+        if (k0 + QBK < K) fetch(k0 + QBK);     // next step's global loads fly while this step multiplies
 
+#pragma unroll
+        for (int grp = 0; grp < G; grp++) {
         floatx16 g[WT][WT];                    // this group's unscaled partial sums
 #pragma unroll
         for (int i = 0; i < WT; i++)
@@ -392,8 +398,8 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
 #pragma unroll
                 for (int e = 0; e < 16; e++) g[i][j][e] = 0.0f;
 #pragma unroll
-        for (int step = 0; step < BK / 16; step++) {
-            const int kofs = step * 16 + half * 8;
+        for (int step = 0; step < kQ8Group / 16; step++) {
+            const int kofs = grp * kQ8Group + step * 16 + half * 8;
             bf16x8 b[WT];
 #pragma unroll
             for (int tn = 0; tn < WT; tn++) b[tn] = *reinterpret_cast<const bf16x8 *>(&Wl[wn * 32 * WT + 32 * tn + l32][kofs]);
@@ -410,11 +416,12 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
         // every accumulator entry of a lane belongs to one output column: one scale per lane and tile column
 #pragma unroll
         for (int tn = 0; tn < WT; tn++) {
-            const float sc = Ss[wn * 32 * WT + 32 * tn + l32];
+            const float sc = Ss[grp][wn * 32 * WT + 32 * tn + l32];
 #pragma unroll
             for (int tm = 0; tm < WT; tm++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[tm][tn][e] = fmaf(g[tm][tn][e], sc, acc[tm][tn][e]);
+        }
         }
         __syncthreads();
     }
@@ -442,6 +449,8 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
         }
     }
 }
+
+constexpr int kGroupsSmall = 2, kGroupsBig = 1;    // measured: 4 and 2 are slower (LDS per workgroup, registers)
 
 // The large tile needs enough workgroups to fill the chip; small problems keep the 64 x 64 tile.
 inline bool use_big_tile(int m, int n) {
@@ -472,11 +481,11 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
     GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu};
     if (!m_dev && use_big_tile(m, n_rows)) {       // a device-side row count is usually far below m: keep small tiles
         dim3 grid2((n_rows + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
-        hipLaunchKernelGGL(k_gemm_q8<2>, grid2, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        hipLaunchKernelGGL((k_gemm_q8<2, kGroupsBig>), grid2, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
         return;
     }
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
-    hipLaunchKernelGGL(k_gemm_q8<1>, grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+    hipLaunchKernelGGL((k_gemm_q8<1, kGroupsSmall>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
 }
 
 }  // namespace dj
