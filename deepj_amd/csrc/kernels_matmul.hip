@@ -286,22 +286,32 @@ __device__ __forceinline__ float top_bits(float x) {      // the leading 8 signi
 // 64 x 64 tile has only six products per wavefront and group to set against that, so it takes several groups a step.
 // Operand element j of lane l is k = 16*step + 8*(l / 32) + j for A and B alike, so the pairing of the MFMA's
 // k slots does not depend on how the hardware numbers them.
-template <int WT, int G>
-__global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, const int8_t *__restrict__ Bq,
+// KS: wavefront sets per workgroup (256 threads each).  Set s multiplies the groups s, s + KS, ... of every step
+// into accumulators of its own and the sets are added through LDS at the end: with a grid of one small tile per
+// CU this is what puts a second wavefront on every SIMD, so one set's conversions overlap the other's products.
+template <int WT, int G, int KS>
+__global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ A, const int8_t *__restrict__ Bq,
                                                  const float *__restrict__ Bs, float *__restrict__ C, int M,
                                                  const int N, const int K, const int kp, GemmEpilogue ep) {
     constexpr int TM = 64 * WT, TN = 64 * WT;
     constexpr int QBK = kQ8Group * G;        // k per step
     constexpr int LDK = QBK + 8;             // LDS row: the step's bf16 payload + 8 of padding (16-byte aligned, spreads banks)
-    constexpr int EL = TM * QBK / 256;       // activation floats (and weight bytes) a thread stages per step
+    constexpr int NT = 256 * KS;
+    constexpr int EL = TM * QBK / NT;        // activation floats (and weight bytes) a thread stages per step
     constexpr int TPR = QBK / EL;            // threads per tile row
     static_assert(EL >= 8 && EL <= kQ8Group && kQ8Group % EL == 0, "a thread's share of a row lies inside one scale group");
-    __shared__ __align__(16) uint16_t Xs[3][TM][LDK];     // hi / mid / lo pieces, row-major, k contiguous
-    __shared__ __align__(16) uint16_t Wl[TN][LDK];        // weights as bf16, one row per output column
-    __shared__ float Ss[G][TN];                            // this step's group scales per output column
+    static_assert(G % KS == 0, "the step's groups divide over the sets");
+    // One LDS block: the step's operands, and after the last step the sums the sets exchange.
+    constexpr int kXsBytes = 3 * TM * LDK * 2, kWlBytes = TN * LDK * 2, kSsBytes = G * TN * 4;
+    constexpr int kRedBytes = (KS - 1) * 4 * WT * WT * 16 * 64 * 4;
+    constexpr int kOperandBytes = kXsBytes + kWlBytes + kSsBytes;
+    __shared__ __align__(16) unsigned char lds[kOperandBytes > kRedBytes ? kOperandBytes : kRedBytes];
+    uint16_t(*Xs)[TM][LDK] = reinterpret_cast<uint16_t(*)[TM][LDK]>(lds);             // hi / mid / lo pieces, k contiguous
+    uint16_t(*Wl)[LDK] = reinterpret_cast<uint16_t(*)[LDK]>(lds + kXsBytes);          // weights as bf16, a row per output column
+    float(*Ss)[TN] = reinterpret_cast<float(*)[TN]>(lds + kXsBytes + kWlBytes);       // the step's group scales per output column
 
     const int t = threadIdx.x;
-    const int lane = t & 63, wave = t >> 6;
+    const int lane = t & 63, wave = (t >> 6) & 3, kset = t >> 8;
     const int wm = wave >> 1, wn = wave & 1;
     const int half = lane >> 5, l32 = lane & 31;
     const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
@@ -389,7 +399,7 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
         if (k0 + QBK < K) fetch(k0 + QBK);     // next step's global loads fly while this step multiplies
 
 #pragma unroll
-        for (int grp = 0; grp < G; grp++) {
+        for (int grp = kset; grp < G; grp += KS) {
         floatx16 g[WT][WT];                    // this group's unscaled partial sums
 #pragma unroll
         for (int i = 0; i < WT; i++)
@@ -426,6 +436,31 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
         __syncthreads();
     }
 
+    if constexpr (KS > 1) {
+        // add the sets' sums: every set but the first parks its accumulators in the (no longer read) piece buffers
+        float *red = reinterpret_cast<float *>(lds);                // [KS - 1][4 wavefronts][WT*WT*16][64 lanes]
+        if (kset > 0) {
+#pragma unroll
+            for (int i = 0; i < WT; i++)
+#pragma unroll
+                for (int j = 0; j < WT; j++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        red[((((kset - 1) * 4 + wave) * WT * WT + i * WT + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+        }
+        __syncthreads();
+        if (kset > 0) return;
+#pragma unroll
+        for (int ks = 1; ks < KS; ks++)
+#pragma unroll
+            for (int i = 0; i < WT; i++)
+#pragma unroll
+                for (int j = 0; j < WT; j++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        acc[i][j][e] += red[((((ks - 1) * 4 + wave) * WT * WT + i * WT + j) * 16 + e) * 64 + lane];
+    }
+
     // epilogue: acc[i][jn][e] is C[32*i + 8*(e/4) + 4*(lane/32) + e%4][32*jn + lane%32] of the wavefront's block
 #pragma unroll
     for (int jn = 0; jn < WT; jn++) {
@@ -450,6 +485,8 @@ __global__ void __launch_bounds__(256) k_gemm_q8(const float *__restrict__ A, co
     }
 }
 
+constexpr int kFewTiles = 512, kGroupsFew = 4, kSetsFew = 4;
+constexpr int kSetsBig = 1;
 constexpr int kGroupsSmall = 2, kGroupsBig = 1;    // measured: 4 and 2 are slower (LDS per workgroup, registers)
 
 // The large tile needs enough workgroups to fill the chip; small problems keep the 64 x 64 tile.
@@ -481,11 +518,15 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
     GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu};
     if (!m_dev && use_big_tile(m, n_rows)) {       // a device-side row count is usually far below m: keep small tiles
         dim3 grid2((n_rows + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
-        hipLaunchKernelGGL((k_gemm_q8<2, kGroupsBig>), grid2, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        hipLaunchKernelGGL((k_gemm_q8<2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
         return;
     }
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
-    hipLaunchKernelGGL((k_gemm_q8<1, kGroupsSmall>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+    // few tiles (about one per CU): a workgroup brings its own second wavefront per SIMD
+    if ((int64_t)grid.x * grid.y <= kFewTiles)
+        hipLaunchKernelGGL((k_gemm_q8<1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+    else
+        hipLaunchKernelGGL((k_gemm_q8<1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
 }
 
 }  // namespace dj
