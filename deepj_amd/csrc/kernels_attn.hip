@@ -26,6 +26,7 @@ using namespace dev;
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
+constexpr int kAttnFullGrid = 256;        // workgroups that give every CU one
 
 // ── RoPE on the fused projection + cache append ─────────────────────────────
 // qkv [S x 3d]: Q | K | V.  Row i sits at position state[0] + i.
@@ -166,23 +167,32 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 // beyond every query of a wavefront is skipped by it.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int HD>
+// KSETS = 2 (for grids that would leave CUs idle): a workgroup takes 64 query rows; its wavefronts 0, 1 walk the
+// even key tiles and 2, 3 the odd ones for the SAME queries, two tiles are staged per round, and the two partial
+// soft-max states are merged through LDS at the end - twice the workgroups and half the rounds.
+template <int HD, int KSETS>
 __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     constexpr int KT = 32, NT = HD / 32;
-    __shared__ float Kt[HD][KT + 1];
-    __shared__ __align__(16) float Vs[KT][HD];
+    constexpr int QW = 4 / KSETS;                           // wavefronts that hold distinct query rows
+    constexpr int QWG = 32 * QW;                            // query rows per workgroup
+    constexpr int kKtFloats = KSETS * HD * (KT + 1), kVsFloats = KSETS * KT * HD;
+    constexpr int kMergeFloats = KSETS > 1 ? QW * 64 * (NT * 16 + 2) : 0;
+    __shared__ __align__(16) float lds[kKtFloats + kVsFloats > kMergeFloats ? kKtFloats + kVsFloats : kMergeFloats];
+    float(*Kt)[HD][KT + 1] = reinterpret_cast<float(*)[HD][KT + 1]>(lds);              // [set][j][key]: transposed
+    float(*Vs)[KT][HD] = reinterpret_cast<float(*)[KT][HD]>(lds + kKtFloats);          // [set][key][j]
 
     const int h = blockIdx.x, qt = blockIdx.y;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, half = lane >> 5, l32 = lane & 31;
+    const int qw = wave % QW, kset = wave / QW;
     const int d = a.H * HD;
     int pos0 = a.state[0];
     if (pos0 < 0) pos0 = 0;
-    const int q_wave0 = qt * 128 + wave * 32;
+    const int q_wave0 = qt * QWG + qw * 32;
     const int qi = q_wave0 + l32;                           // this lane's query row
     const bool q_ok = qi < a.S;
     int qpos = pos0 + qi;                                   // its position: keys 0 .. qpos
     if (qpos >= a.max_seq) qpos = a.max_seq - 1;
-    const int q_end_wg = a.S < qt * 128 + 128 ? a.S : qt * 128 + 128;
+    const int q_end_wg = a.S < qt * QWG + QWG ? a.S : qt * QWG + QWG;
     const int q_end_wave = a.S < q_wave0 + 32 ? a.S : q_wave0 + 32;
     int wg_last = pos0 + q_end_wg - 1;                      // last key any query of the workgroup sees
     if (wg_last >= a.max_seq) wg_last = a.max_seq - 1;
@@ -207,38 +217,41 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 
     const float *kbase = a.k + (int64_t)h * a.head_stride;
     const float *vbase = a.v + (int64_t)h * a.head_stride;
-    for (int k0 = 0; k0 <= wg_last; k0 += KT) {
-        {   // stage the key tile transposed and the value tile; rows past the last key repeat it (masked below)
+    for (int k0 = 0; k0 <= wg_last; k0 += KT * KSETS) {
+#pragma unroll
+        for (int ks = 0; ks < KSETS; ks++) {
+            // stage the key tile transposed and the value tile; rows past the last key repeat it (masked below)
             constexpr int PART = HD / 8;
-            int key = k0 + (t & 31);
+            int key = k0 + ks * KT + (t & 31);
             if (key > wg_last) key = wg_last;
             const float *kr = kbase + (int64_t)key * a.tok_stride + (t >> 5) * PART;
 #pragma unroll
             for (int j = 0; j < PART; j += 4) {
                 float4 v = *reinterpret_cast<const float4 *>(kr + j);
                 int c = (t >> 5) * PART + j;
-                Kt[c][t & 31] = v.x; Kt[c + 1][t & 31] = v.y; Kt[c + 2][t & 31] = v.z; Kt[c + 3][t & 31] = v.w;
+                Kt[ks][c][t & 31] = v.x; Kt[ks][c + 1][t & 31] = v.y; Kt[ks][c + 2][t & 31] = v.z; Kt[ks][c + 3][t & 31] = v.w;
             }
-            int vkey = k0 + (t >> 3);
+            int vkey = k0 + ks * KT + (t >> 3);
             if (vkey > wg_last) vkey = wg_last;
             const float *vr = vbase + (int64_t)vkey * a.tok_stride + (t & 7) * PART;
 #pragma unroll
             for (int j = 0; j < PART; j += 4)
-                *reinterpret_cast<float4 *>(&Vs[t >> 3][(t & 7) * PART + j]) = *reinterpret_cast<const float4 *>(vr + j);
+                *reinterpret_cast<float4 *>(&Vs[ks][t >> 3][(t & 7) * PART + j]) = *reinterpret_cast<const float4 *>(vr + j);
         }
         __syncthreads();
-        if (k0 <= wave_last) {                              // wave-uniform
+        const int kb0 = k0 + kset * KT;                     // this wavefront's tile of the round
+        if (kb0 <= wave_last) {                             // wave-uniform
             floatx16 st;
 #pragma unroll
             for (int e = 0; e < 16; e++) st[e] = 0.0f;
 #pragma unroll
             for (int kk = 0; kk < HD / 2; kk++)
-                st = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[2 * kk + half][l32], qreg[kk], st, 0, 0, 0);
-            // st[e] = q . k for key k0 + 8*(e/4) + 4*half + e%4 and this lane's query
+                st = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[kset][2 * kk + half][l32], qreg[kk], st, 0, 0, 0);
+            // st[e] = q . k for key kb0 + 8*(e/4) + 4*half + e%4 and this lane's query
             float tmax = -INFINITY;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                int key = k0 + 8 * (e >> 2) + 4 * half + (e & 3);
+                int key = kb0 + 8 * (e >> 2) + 4 * half + (e & 3);
                 float sv = (q_ok && key <= qpos) ? st[e] * a.scale : -INFINITY;      // scale after the product
                 st[e] = sv;
                 tmax = fmaxf(tmax, sv);
@@ -264,10 +277,31 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
                 const int key = 8 * (kk >> 2) + 4 * half + (kk & 3);
 #pragma unroll
                 for (int i = 0; i < NT; i++)
-                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[key][32 * i + l32], st[kk], acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[kset][key][32 * i + l32], st[kk], acc[i], 0, 0, 0);
             }
         }
         __syncthreads();
+    }
+    if constexpr (KSETS > 1) {
+        // merge the two key sets' states of the same queries: set 1 parks (m, l, acc) lane by lane, set 0 adds them
+        float *mg = lds + (int64_t)(qw * 64 + lane) * (NT * 16 + 2);
+        if (kset == 1) {
+            mg[0] = m; mg[1] = l;
+#pragma unroll
+            for (int i = 0; i < NT; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) mg[2 + i * 16 + e] = acc[i][e];
+        }
+        __syncthreads();
+        if (kset == 1) return;
+        const float m1 = mg[0], l1 = mg[1];
+        const float mn = fmaxf(m, m1);
+        const float w0 = (m == -INFINITY) ? 0.0f : expf(m - mn), w1 = (m1 == -INFINITY) ? 0.0f : expf(m1 - mn);
+        l = l * w0 + l1 * w1;
+#pragma unroll
+        for (int i = 0; i < NT; i++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][e] = acc[i][e] * w0 + mg[2 + i * 16 + e] * w1;
     }
     l += __shfl_xor(l, 32, 64);
     if (q_ok) {
@@ -664,10 +698,20 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
     a.scale = (float)(1.0 / sqrt((double)p.hd));
     if (p.s >= 16) {                     // enough rows to share key tiles: matrix-core kernel
         dim3 tg(p.h, (p.s + 127) / 128);
+        if ((int64_t)tg.x * tg.y < kAttnFullGrid) {      // too few workgroups for the chip: 64 rows each, keys in two sets
+            dim3 tg2(p.h, (p.s + 63) / 64);
+            switch (p.hd) {
+                case 32: hipLaunchKernelGGL((k_attention_tiled<32, 2>), tg2, dim3(256), 0, s, a); break;
+                case 64: hipLaunchKernelGGL((k_attention_tiled<64, 2>), tg2, dim3(256), 0, s, a); break;
+                case 128: hipLaunchKernelGGL((k_attention_tiled<128, 2>), tg2, dim3(256), 0, s, a); break;
+                default: fail("attention: head dim must be 32, 64 or 128");
+            }
+            return;
+        }
         switch (p.hd) {
-            case 32: hipLaunchKernelGGL(k_attention_tiled<32>, tg, dim3(256), 0, s, a); break;
-            case 64: hipLaunchKernelGGL(k_attention_tiled<64>, tg, dim3(256), 0, s, a); break;
-            case 128: hipLaunchKernelGGL(k_attention_tiled<128>, tg, dim3(256), 0, s, a); break;
+            case 32: hipLaunchKernelGGL((k_attention_tiled<32, 1>), tg, dim3(256), 0, s, a); break;
+            case 64: hipLaunchKernelGGL((k_attention_tiled<64, 1>), tg, dim3(256), 0, s, a); break;
+            case 128: hipLaunchKernelGGL((k_attention_tiled<128, 1>), tg, dim3(256), 0, s, a); break;
             default: fail("attention: head dim must be 32, 64 or 128");
         }
         return;
