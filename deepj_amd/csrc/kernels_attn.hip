@@ -26,7 +26,7 @@ using namespace dev;
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kAttnFullGrid = 256;        // workgroups that give every CU one
+constexpr int kAttnFullGrid = 512;        // workgroups that give every CU one
 
 // ── RoPE on the fused projection + cache append ─────────────────────────────
 // qkv [S x 3d]: Q | K | V.  Row i sits at position state[0] + i.
@@ -167,16 +167,16 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 // beyond every query of a wavefront is skipped by it.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-// KSETS = 2 (for grids that would leave CUs idle): a workgroup takes 64 query rows; its wavefronts 0, 1 walk the
-// even key tiles and 2, 3 the odd ones for the SAME queries, two tiles are staged per round, and the two partial
-// soft-max states are merged through LDS at the end - twice the workgroups and half the rounds.
+// KSETS = 2 or 4 (for grids that would leave CUs idle): a workgroup takes 64 or 32 query rows; its wavefronts are
+// 2 or 4 sets that walk every KSETS-th key tile for the SAME queries, KSETS tiles are staged per round, and the
+// sets' partial soft-max states are merged through LDS at the end - more workgroups and fewer rounds.
 template <int HD, int KSETS>
 __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     constexpr int KT = 32, NT = HD / 32;
     constexpr int QW = 4 / KSETS;                           // wavefronts that hold distinct query rows
     constexpr int QWG = 32 * QW;                            // query rows per workgroup
     constexpr int kKtFloats = KSETS * HD * (KT + 1), kVsFloats = KSETS * KT * HD;
-    constexpr int kMergeFloats = KSETS > 1 ? QW * 64 * (NT * 16 + 2) : 0;
+    constexpr int kMergeFloats = (KSETS - 1) * QW * 64 * (NT * 16 + 2);
     __shared__ __align__(16) float lds[kKtFloats + kVsFloats > kMergeFloats ? kKtFloats + kVsFloats : kMergeFloats];
     float(*Kt)[HD][KT + 1] = reinterpret_cast<float(*)[HD][KT + 1]>(lds);              // [set][j][key]: transposed
     float(*Vs)[KT][HD] = reinterpret_cast<float(*)[KT][HD]>(lds + kKtFloats);          // [set][key][j]
@@ -283,9 +283,11 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
         __syncthreads();
     }
     if constexpr (KSETS > 1) {
-        // merge the two key sets' states of the same queries: set 1 parks (m, l, acc) lane by lane, set 0 adds them
-        float *mg = lds + (int64_t)(qw * 64 + lane) * (NT * 16 + 2);
-        if (kset == 1) {
+        // merge the key sets' states of the same queries: every set but the first parks (m, l, acc) lane by lane,
+        // set 0 adds them
+        constexpr int REC = NT * 16 + 2;
+        if (kset > 0) {
+            float *mg = lds + (int64_t)(((kset - 1) * QW + qw) * 64 + lane) * REC;
             mg[0] = m; mg[1] = l;
 #pragma unroll
             for (int i = 0; i < NT; i++)
@@ -293,15 +295,20 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
                 for (int e = 0; e < 16; e++) mg[2 + i * 16 + e] = acc[i][e];
         }
         __syncthreads();
-        if (kset == 1) return;
-        const float m1 = mg[0], l1 = mg[1];
-        const float mn = fmaxf(m, m1);
-        const float w0 = (m == -INFINITY) ? 0.0f : expf(m - mn), w1 = (m1 == -INFINITY) ? 0.0f : expf(m1 - mn);
-        l = l * w0 + l1 * w1;
+        if (kset > 0) return;
 #pragma unroll
-        for (int i = 0; i < NT; i++)
+        for (int ks = 1; ks < KSETS; ks++) {
+            const float *mg = lds + (int64_t)(((ks - 1) * QW + qw) * 64 + lane) * REC;
+            const float m1 = mg[0], l1 = mg[1];
+            const float mn = fmaxf(m, m1);
+            const float w0 = (m == -INFINITY) ? 0.0f : expf(m - mn), w1 = (m1 == -INFINITY) ? 0.0f : expf(m1 - mn);
+            l = l * w0 + l1 * w1;
+            m = mn;
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][e] = acc[i][e] * w0 + mg[2 + i * 16 + e] * w1;
+            for (int i = 0; i < NT; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][e] = acc[i][e] * w0 + mg[2 + i * 16 + e] * w1;
+        }
     }
     l += __shfl_xor(l, 32, 64);
     if (q_ok) {
@@ -698,7 +705,17 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
     a.scale = (float)(1.0 / sqrt((double)p.hd));
     if (p.s >= 16) {                     // enough rows to share key tiles: matrix-core kernel
         dim3 tg(p.h, (p.s + 127) / 128);
-        if ((int64_t)tg.x * tg.y < kAttnFullGrid) {      // too few workgroups for the chip: 64 rows each, keys in two sets
+        if ((int64_t)tg.x * tg.y * 2 < kAttnFullGrid) {  // far too few workgroups for the chip: 32 rows each, keys in four sets
+            dim3 tg4(p.h, (p.s + 31) / 32);
+            switch (p.hd) {
+                case 32: hipLaunchKernelGGL((k_attention_tiled<32, 4>), tg4, dim3(256), 0, s, a); break;
+                case 64: hipLaunchKernelGGL((k_attention_tiled<64, 4>), tg4, dim3(256), 0, s, a); break;
+                case 128: hipLaunchKernelGGL((k_attention_tiled<128, 4>), tg4, dim3(256), 0, s, a); break;
+                default: fail("attention: head dim must be 32, 64 or 128");
+            }
+            return;
+        }
+        if ((int64_t)tg.x * tg.y < kAttnFullGrid) {      // too few: 64 rows each, keys in two sets
             dim3 tg2(p.h, (p.s + 63) / 64);
             switch (p.hd) {
                 case 32: hipLaunchKernelGGL((k_attention_tiled<32, 2>), tg2, dim3(256), 0, s, a); break;

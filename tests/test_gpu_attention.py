@@ -26,7 +26,10 @@ def oracle_attention(q, k, v, H, cos, sin):
 
 
 @pytest.mark.parametrize("H,hd,max_seq,chunks", [(8, 32, 256, [32, 1, 1, 1]), (4, 64, 200, [70, 1, 1, 60, 1]),
-                                                 (2, 128, 130, [5, 1, 124]), (32, 64, 2048, [3, 1])])
+                                                 (2, 128, 130, [5, 1, 124]), (32, 64, 2048, [3, 1]),
+                                                 # grids of 288 and 576 workgroups at 128 rows each: the prefill kernel's
+                                                 # two-key-set and one-key-set variants (the small shapes above use four)
+                                                 (32, 64, 1200, [1100, 1, 20]), (64, 32, 1150, [1100, 1])])
 def test_rope_store_attention_prefill_and_decode(H, hd, max_seq, chunks):
     d = H * hd
     total = sum(chunks)
