@@ -32,6 +32,7 @@ struct GemmEpilogue {
     const int32_t *m_dev;   // when set, only rows < min(M, m_dev[0] + m_extra) exist (row count kept on the device)
     int m_extra;
     int gelu;               // GELU (tanh form, tensor/cpu/CpuBackend.java:338, used by activations/GELU.java:15-18) on acc + bias, before the residual
+    int swiglu;             // Q8 GEMM only: columns are interleaved gate/up pairs; C is [M x N/2], C[r][j] = SiLU(gate_j) * up_j
 };
 
 __device__ __forceinline__ float gemm_gelu(float x) {
@@ -398,7 +399,8 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
         __syncthreads();
         if (k0 + QBK < K) fetch(k0 + QBK);     // next step's global loads fly while this step multiplies
 
-#pragma unroll
+        // (a run-time loop on purpose: unrolled, the products of consecutive groups get interleaved and the kernel
+        // measured 4-10 % slower)
         for (int grp = kset; grp < G; grp += KS) {
         floatx16 g[WT][WT];                    // this group's unscaled partial sums
 #pragma unroll
@@ -473,6 +475,18 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int row = m0 + wm * 32 * WT + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                if (ep.swiglu) {
+                    // gate and up of one output sit in neighbouring lanes (columns 2j, 2j + 1); N is even, so a
+                    // pair is inside or outside the matrix together (SiLU.java:20-24, SwiGLULayer.java:69)
+                    float v = acc[i][jn][e];
+                    if (ep.bias) v = v + badd;
+                    const float other = __shfl_xor(v, 1, 64);
+                    if (row < M && (col & 1) == 0) {
+                        const float sg = v * (1.0f / (1.0f + expf(-v)));
+                        C[(int64_t)row * (N >> 1) + (col >> 1)] = sg * other;
+                    }
+                    continue;
+                }
                 if (row < M) {
                     float v = acc[i][jn][e];
                     if (ep.bias) v = v + badd;
@@ -499,7 +513,7 @@ inline bool use_big_tile(int m, int n) {
 void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out, int m, int n, int k) {
     if (m <= 0 || n <= 0) return;
     if (k <= 0) { launch_fill(s, reinterpret_cast<uint32_t *>(out), 0u, (int64_t)m * n); return; }
-    GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0, 0};
+    GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0};
     if (use_big_tile(m, n)) {
         dim3 grid2((n + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
         hipLaunchKernelGGL(k_gemm128, grid2, dim3(256), 0, s, a, b, out, m, n, k, ep);
@@ -513,9 +527,10 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
 // (= output columns of this launch; 2N for an interleaved gate/up weight).
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu) {
+                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu, int swiglu) {
     if (m <= 0 || n_rows <= 0) return;
-    GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu};
+    if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
+    GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu, swiglu};
     if (!m_dev && use_big_tile(m, n_rows)) {       // a device-side row count is usually far below m: keep small tiles
         dim3 grid2((n_rows + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
         hipLaunchKernelGGL((k_gemm_q8<2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
