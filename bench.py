@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE.json configs[2], the configuration the headline metric is quoted on):
+Workload (the configuration the headline metric is quoted on):
 Llama decode, dModel 2048, 16 layers, 32 heads (head dim 64), SwiGLU hidden 5632, vocab
 32000, maxSeq 2048; weights = new LlamaModel(cfg, 42) (java.util.Random Gaussians x 0.1),
 all matmul weights Q8; prompt = 512 ids from Random(3).nextInt(32000); batch-1 greedy decode

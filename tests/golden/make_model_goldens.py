@@ -22,10 +22,10 @@ sys.path.insert(0, ROOT)
 from oracle import cpu_ref as ref  # noqa: E402
 
 CONFIGS = {
-    # BASELINE.json configs[2]: Llama decode workload
+    # the Llama decode workload of the benchmark
     "c3": dict(model=dict(vocab=32000, max_seq=2048, d=2048, heads=32, layers=16, dff=5632), seed=42,
                prompt_seed=3, prompt_len=512, new_tokens=64),
-    # BASELINE.json configs[4]: DeepSeek-style MLA (qRank = d/2, kvRank = d/4 as the reference's README suggests).
+    # DeepSeek-style MLA at the same width (qRank = d/2, kvRank = d/4 as the reference's README suggests).
     # With the reference's initialiser (N(0,1)*0.1, Tensor.java random) at this width the attention scores
     # q.k/sqrt(hd) have a standard deviation near 150: every softmax row is a hard arg-max, and any change of
     # fp32 summation order flips near-ties, so two correct fp32 implementations differ by O(1) in the logits
@@ -35,7 +35,7 @@ CONFIGS = {
     # seeded reference initialisation.
     "c5": dict(model=dict(vocab=32000, max_seq=512, d=2048, heads=16, layers=16, dff=5632, q_rank=1024, kv_rank=512),
                seed=42, prompt_seed=5, prompt_len=256, new_tokens=64, mla_weight_scale=0.25),
-    # GPT path at the size of GPT-2 small (GPTModel.java; not a BASELINE config): LayerNorm, GELU feed-forward,
+    # GPT path at the size of GPT-2 small (GPTModel.java): LayerNorm, GELU feed-forward,
     # learned positions, an odd vocabulary, dModel = 768 (a Q8 row shorter than one 1 KiB chunk).  initScale 1:
     # with GPTConfig's default 0.2 every LayerNorm gain is 0.2 too and the logits of a random model shrink to a
     # few 1e-4, where the top-1/top-2 gap is no longer far above fp32 noise.  Prompt seed 8: the smallest

@@ -2,7 +2,7 @@
 LlamaModel forward + TextGenerator, restated) on identical seeded weights: the oracle runs on
 the dequantised Q8 weights, so the only differences are fp32 summation order.
 
-Gates (BASELINE.json): per-row logits max-abs 1e-3; greedy token ids identical over 64 tokens.
+Gates: per-row logits max-abs 1e-3; greedy token ids identical over 64 tokens.
 Config 1 of the baseline is the tiny Llama: vocab 256, dModel 256, 4 layers, 8 heads,
 dFF 688, maxSeq 256, seed 42, prompt = 32 ids from Random(7), 64 greedy tokens."""
 import numpy as np

@@ -1,6 +1,6 @@
 """Q8 weight path through the C ABI: quantiser bit-exact against the host quantiser, decode
 matvec and prefill GEMM (with their fused prologue/epilogues) against the CPU oracle run on
-the dequantised weights.  Shapes of BASELINE.json's isolated linear-op sweep at reduced N
+the dequantised weights.  Shapes of the isolated linear-op sweep at reduced N
 where the oracle would be slow, plus ragged K (688 = 21*32 + 16)."""
 import numpy as np
 import pytest
