@@ -193,6 +193,20 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
     }
 }
 
+// LDS layout of the staged activation row.  A lane multiplies the 16 consecutive activations of "its" 16-byte
+// weight chunk (chunk = 64 * c + lane) and reads them as four 128-bit words; stored in order, consecutive lanes
+// would be 64 bytes apart and four of every sixteen lanes would hit the same banks on every read.  So the row is
+// kept as planes: plane 4 * c + q holds the q-th word of every lane's slice of chunk row c, lane after lane
+// (conflict free to read), and a plane is padded by 16 floats so that the staging writes - consecutive threads
+// write the four words of one slice, i.e. to four planes - spread over the banks as well.
+constexpr int kXsPlane = 64 * 4 + 16;                              // floats per plane
+__host__ __device__ inline int xs_floats(int kp) { return ((kp + 1023) / 1024) * 4 * kXsPlane; }
+// offset of activation e (any e < Kp rounded up to 1024)
+__device__ __forceinline__ int xs_at(int e) {
+    const int chunk = e >> 4, q = (e >> 2) & 3;
+    return ((chunk >> 6) * 4 + q) * kXsPlane + (chunk & 63) * 4 + (e & 3);
+}
+
 // NC: 1 KiB chunks of one row a lane visits (ceil(Kp/1024)); B: outputs per batch.
 //
 // Batches of outputs are dealt round-robin to the wavefronts.  The weight loads of a
@@ -209,7 +223,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     constexpr bool GELU = MODE == 1;
     constexpr bool MERGE = MODE == 2;
     constexpr int NS = kAttnRecordSplits;
-    extern __shared__ __align__(16) float xs[];   // Kp floats
+    extern __shared__ __align__(16) float xs[];   // the activation row, laid out by xs_at() below
     __shared__ float red[kWaves], red2[kWaves];
     constexpr int RPO = SWIGLU ? 2 : 1;           // Q8 rows per output
     constexpr int R = B * RPO;                    // rows per batch
@@ -339,7 +353,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             float4 y;
             y.x = (xv[j].x / sd) * gv[j].x + bv[j].x; y.y = (xv[j].y / sd) * gv[j].y + bv[j].y;
             y.z = (xv[j].z / sd) * gv[j].z + bv[j].z; y.w = (xv[j].w / sd) * gv[j].w + bv[j].w;
-            if (e < p.kp) *reinterpret_cast<float4 *>(xs + e) = y;      // e >= k: x, gamma and beta are all zero
+            if (e < p.kp) *reinterpret_cast<float4 *>(xs + xs_at(e)) = y;      // e >= k: x, gamma and beta are all zero
         }
     } else if (vec) {
         if (p.gamma) {
@@ -361,13 +375,13 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
 #pragma unroll
         for (int j = 0; j < NC; j++) {
             int e = (tid + kThreads * j) * 4;
-            if (e < p.kp) *reinterpret_cast<float4 *>(xs + e) = xv[j];
+            if (e < p.kp) *reinterpret_cast<float4 *>(xs + xs_at(e)) = xv[j];
         }
     } else {
         float ss = 0.0f;
         for (int i = tid; i < p.kp; i += kThreads) {
             float v = i < p.k ? p.x[i] : 0.0f;
-            xs[i] = v;
+            xs[xs_at(i)] = v;
             ss += v * v;
         }
         if (p.beta) {
@@ -378,19 +392,19 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             lds_barrier();
             float mean = (red[0] + red[1] + red[2] + red[3]) * (1.0f / (float)p.k);
             float sv = 0.0f;
-            for (int i = tid; i < p.k; i += kThreads) { float c = xs[i] - mean; sv += c * c; }
+            for (int i = tid; i < p.k; i += kThreads) { float c = xs[xs_at(i)] - mean; sv += c * c; }
             sv = wave_sum_dpp(sv);
             if (lane == 0) red2[wave] = sv;
             lds_barrier();
             float sd = sqrtf((red2[0] + red2[1] + red2[2] + red2[3]) * (1.0f / (float)p.k) + kLayerNormEps);
-            for (int i = tid; i < p.k; i += kThreads) xs[i] = ((xs[i] - mean) / sd) * p.gamma[i] + p.beta[i];
+            for (int i = tid; i < p.k; i += kThreads) xs[xs_at(i)] = ((xs[xs_at(i)] - mean) / sd) * p.gamma[i] + p.beta[i];
         } else if (p.gamma) {
             ss = wave_sum_dpp(ss);
             if (lane == 0) red[wave] = ss;
             lds_barrier();
             float tot = red[0] + red[1] + red[2] + red[3];
             float rms = sqrtf(tot * (1.0f / (float)p.k) + kRmsEps);
-            for (int i = tid; i < p.k; i += kThreads) xs[i] = (xs[i] / rms) * p.gamma[i];
+            for (int i = tid; i < p.k; i += kThreads) xs[xs_at(i)] = (xs[xs_at(i)] / rms) * p.gamma[i];
         }
     }
     lds_barrier();
@@ -409,7 +423,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
         bool active = kb < p.kp;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            float4 v = active ? *reinterpret_cast<const float4 *>(xs + kb + 4 * j) : make_float4(0, 0, 0, 0);
+            float4 v = active ? *reinterpret_cast<const float4 *>(xs + (c * 4 + j) * kXsPlane + lane * 4) : make_float4(0, 0, 0, 0);
             xr[c][4 * j] = v.x; xr[c][4 * j + 1] = v.y; xr[c][4 * j + 2] = v.z; xr[c][4 * j + 3] = v.w;
         }
     }
@@ -434,7 +448,7 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     int grid = (batches + kWaves - 1) / kWaves;
     if (grid > mv_grid_cap()) grid = mv_grid_cap();
     if (grid < 1) grid = 1;
-    size_t lds = (size_t)a.kp * sizeof(float);
+    size_t lds = (size_t)xs_floats(a.kp) * sizeof(float);
     hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE>), dim3(grid), dim3(kThreads), lds, s, a);
 }
 
