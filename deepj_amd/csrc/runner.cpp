@@ -285,9 +285,10 @@ void init_seeded(Runner &r, int64_t seed, int threads, float init_scale) {
 
 // ── buffers ────────────────────────────────────────────────────────────────
 
+// Buffers for `rows` rows (they only ever grow: every op takes its row count explicitly).
 void alloc_acts(Runner &r, Acts &a, int rows) {
     const Config &c = r.cfg;
-    if (a.rows == rows) return;
+    if (a.rows >= rows) return;
     for (int32_t *id : {&a.x, &a.x2, &a.qkv, &a.q, &a.att, &a.ff, &a.ids, &a.cq}) r.release(*id);
     int64_t S = rows, d = c.d;
     a.x = r.alloc(S * d); a.x2 = r.alloc(S * d); a.q = r.alloc(S * d); a.att = r.alloc(S * d);
@@ -344,6 +345,8 @@ void finalize(Runner &r) {
     }
     r.run(s);
     alloc_acts(r, r.dec, 1);
+    // the prompt-sized buffers for the longest prompt the cache can take, so that no request pays for allocation
+    alloc_acts(r, r.pre, c.max_seq);
     r.finalized = true;
 }
 
