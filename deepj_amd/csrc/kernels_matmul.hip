@@ -282,7 +282,7 @@ __device__ __forceinline__ float top_bits(float x) {      // the leading 8 signi
     return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & 0xffff0000u);
 }
 
-// WT = 1: workgroup tile 64 x 64, one 32 x 32 accumulator per wavefront; WT = 2: 128 x 128, four.
+// Workgroup tile 64 WTM x 64 WTN, WTM x WTN accumulators of 32 x 32 per wavefront (1 x 1: 64 x 64 tile; 2 x 2: 128 x 128).
 // G: scale groups (of 32 k) per step.  A step costs two barriers and an LDS round trip whatever its size, and a
 // 64 x 64 tile has only six products per wavefront and group to set against that, so it takes several groups a step.
 // Operand element j of lane l is k = 16*step + 8*(l / 32) + j for A and B alike, so the pairing of the MFMA's
@@ -290,21 +290,24 @@ __device__ __forceinline__ float top_bits(float x) {      // the leading 8 signi
 // KS: wavefront sets per workgroup (256 threads each).  Set s multiplies the groups s, s + KS, ... of every step
 // into accumulators of its own and the sets are added through LDS at the end: with a grid of one small tile per
 // CU this is what puts a second wavefront on every SIMD, so one set's conversions overlap the other's products.
-template <int WT, int G, int KS>
+template <int WTM, int WTN, int G, int KS>
 __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ A, const int8_t *__restrict__ Bq,
                                                  const float *__restrict__ Bs, float *__restrict__ C, int M,
                                                  const int N, const int K, const int kp, GemmEpilogue ep) {
-    constexpr int TM = 64 * WT, TN = 64 * WT;
+    constexpr int TM = 64 * WTM, TN = 64 * WTN;
     constexpr int QBK = kQ8Group * G;        // k per step
     constexpr int LDK = QBK + 8;             // LDS row: the step's bf16 payload + 8 of padding (16-byte aligned, spreads banks)
     constexpr int NT = 256 * KS;
-    constexpr int EL = TM * QBK / NT;        // activation floats (and weight bytes) a thread stages per step
-    constexpr int TPR = QBK / EL;            // threads per tile row
-    static_assert(EL >= 8 && EL <= kQ8Group && kQ8Group % EL == 0, "a thread's share of a row lies inside one scale group");
+    constexpr int EL = TM * QBK / NT;        // activation floats a thread stages per step ...
+    constexpr int TPR = QBK / EL;            // ... as one of TPR threads per tile row
+    constexpr int ELB = TN * QBK / NT;       // weight bytes a thread stages per step ...
+    constexpr int TPRB = QBK / ELB;          // ... as one of TPRB threads per tile column
+    static_assert(EL >= 8 && EL <= kQ8Group && kQ8Group % EL == 0 && ELB >= 8 && ELB <= kQ8Group && kQ8Group % ELB == 0,
+                  "a thread's share of a row lies inside one scale group");
     static_assert(G % KS == 0, "the step's groups divide over the sets");
     // One LDS block: the step's operands, and after the last step the sums the sets exchange.
     constexpr int kXsBytes = 3 * TM * LDK * 2, kWlBytes = TN * LDK * 2, kSsBytes = G * TN * 4;
-    constexpr int kRedBytes = (KS - 1) * 4 * WT * WT * 16 * 64 * 4;
+    constexpr int kRedBytes = (KS - 1) * 4 * WTM * WTN * 16 * 64 * 4;
     constexpr int kOperandBytes = kXsBytes + kWlBytes + kSsBytes;
     __shared__ __align__(16) unsigned char lds[kOperandBytes > kRedBytes ? kOperandBytes : kRedBytes];
     uint16_t(*Xs)[TM][LDK] = reinterpret_cast<uint16_t(*)[TM][LDK]>(lds);             // hi / mid / lo pieces, k contiguous
@@ -323,20 +326,22 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
     }
     const int groups = kp / kQ8Group;
 
-    floatx16 acc[WT][WT];
+    floatx16 acc[WTM][WTN];
 #pragma unroll
-    for (int i = 0; i < WT; i++)
+    for (int i = 0; i < WTM; i++)
 #pragma unroll
-        for (int j = 0; j < WT; j++)
+        for (int j = 0; j < WTN; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    const int s_row = t / TPR;               // tile row (A) and tile column (B) this thread stages
+    const int s_row = t / TPR;               // tile row of A this thread stages, from k offset s_k
     const int s_k = (t % TPR) * EL;
+    const int s_col = t / TPRB;              // tile column (row of B) this thread stages, from k offset s_kb
+    const int s_kb = (t % TPRB) * ELB;
     const bool a_vec = (K & 3) == 0;
 
     float va[EL];
-    int qraw[EL / 4];
+    int qraw[ELB / 4];
     float qsc = 0.0f;
     auto fetch = [&](int k0) {
         const int gr = m0 + s_row;
@@ -354,20 +359,20 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
                 va[j] = (gr < M && gk < K) ? A[(int64_t)gr * K + gk] : 0.0f;
             }
         }
-        const int gn = n0 + s_row;
-        if (gn < N && k0 + s_k < kp) {
-            const int *p = reinterpret_cast<const int *>(Bq + (int64_t)gn * kp + k0 + s_k);   // kp is a multiple of 32: in bounds
+        const int gn = n0 + s_col;
+        if (gn < N && k0 + s_kb < kp) {
+            const int *p = reinterpret_cast<const int *>(Bq + (int64_t)gn * kp + k0 + s_kb);  // kp is a multiple of 32: in bounds
 #pragma unroll
-            for (int q = 0; q < EL / 4; q++) qraw[q] = p[q];
-            qsc = Bs[(int64_t)gn * groups + (k0 + s_k) / kQ8Group];
+            for (int q = 0; q < ELB / 4; q++) qraw[q] = p[q];
+            qsc = Bs[(int64_t)gn * groups + (k0 + s_kb) / kQ8Group];
         } else {
 #pragma unroll
-            for (int q = 0; q < EL / 4; q++) qraw[q] = 0;
+            for (int q = 0; q < ELB / 4; q++) qraw[q] = 0;
             qsc = 0.0f;
         }
     };
     auto stage = [&]() {
-        uint32_t ph[EL / 2], pm[EL / 2], pl[EL / 2], pw[EL / 2];
+        uint32_t ph[EL / 2], pm[EL / 2], pl[EL / 2], pw[ELB / 2];
 #pragma unroll
         for (int j = 0; j < EL / 2; j++) {
             const float x0 = va[2 * j], x1 = va[2 * j + 1];
@@ -378,7 +383,7 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
             ph[j] = pack_bf16_hi(h0, h1); pm[j] = pack_bf16_hi(c0, c1); pl[j] = pack_bf16_hi(l0, l1);
         }
 #pragma unroll
-        for (int q = 0; q < EL / 4; q++) {
+        for (int q = 0; q < ELB / 4; q++) {
             const int r = qraw[q];
             pw[2 * q] = pack_bf16_hi((float)(int8_t)(r & 0xff), (float)(int8_t)((r >> 8) & 0xff));
             pw[2 * q + 1] = pack_bf16_hi((float)(int8_t)((r >> 16) & 0xff), (float)(int8_t)((r >> 24) & 0xff));
@@ -388,9 +393,11 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
             reinterpret_cast<uint4 *>(&Xs[0][s_row][s_k])[q] = make_uint4(ph[4 * q], ph[4 * q + 1], ph[4 * q + 2], ph[4 * q + 3]);
             reinterpret_cast<uint4 *>(&Xs[1][s_row][s_k])[q] = make_uint4(pm[4 * q], pm[4 * q + 1], pm[4 * q + 2], pm[4 * q + 3]);
             reinterpret_cast<uint4 *>(&Xs[2][s_row][s_k])[q] = make_uint4(pl[4 * q], pl[4 * q + 1], pl[4 * q + 2], pl[4 * q + 3]);
-            reinterpret_cast<uint4 *>(&Wl[s_row][s_k])[q] = make_uint4(pw[4 * q], pw[4 * q + 1], pw[4 * q + 2], pw[4 * q + 3]);
         }
-        if (s_k % kQ8Group == 0) Ss[s_k / kQ8Group][s_row] = qsc;
+#pragma unroll
+        for (int q = 0; q < ELB / 8; q++)
+            reinterpret_cast<uint4 *>(&Wl[s_col][s_kb])[q] = make_uint4(pw[4 * q], pw[4 * q + 1], pw[4 * q + 2], pw[4 * q + 3]);
+        if (s_kb % kQ8Group == 0) Ss[s_kb / kQ8Group][s_col] = qsc;
     };
 
     if (K > 0) fetch(0);
@@ -402,35 +409,35 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
         // (a run-time loop on purpose: unrolled, the products of consecutive groups get interleaved and the kernel
         // measured 4-10 % slower)
         for (int grp = kset; grp < G; grp += KS) {
-        floatx16 g[WT][WT];                    // this group's unscaled partial sums
+        floatx16 g[WTM][WTN];                  // this group's unscaled partial sums
 #pragma unroll
-        for (int i = 0; i < WT; i++)
+        for (int i = 0; i < WTM; i++)
 #pragma unroll
-            for (int j = 0; j < WT; j++)
+            for (int j = 0; j < WTN; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) g[i][j][e] = 0.0f;
 #pragma unroll
         for (int step = 0; step < kQ8Group / 16; step++) {
             const int kofs = grp * kQ8Group + step * 16 + half * 8;
-            bf16x8 b[WT];
+            bf16x8 b[WTN];
 #pragma unroll
-            for (int tn = 0; tn < WT; tn++) b[tn] = *reinterpret_cast<const bf16x8 *>(&Wl[wn * 32 * WT + 32 * tn + l32][kofs]);
+            for (int tn = 0; tn < WTN; tn++) b[tn] = *reinterpret_cast<const bf16x8 *>(&Wl[wn * 32 * WTN + 32 * tn + l32][kofs]);
 #pragma unroll
             for (int piece = 0; piece < 3; piece++) {
 #pragma unroll
-                for (int tm = 0; tm < WT; tm++) {
-                    const bf16x8 a = *reinterpret_cast<const bf16x8 *>(&Xs[piece][wm * 32 * WT + 32 * tm + l32][kofs]);
+                for (int tm = 0; tm < WTM; tm++) {
+                    const bf16x8 a = *reinterpret_cast<const bf16x8 *>(&Xs[piece][wm * 32 * WTM + 32 * tm + l32][kofs]);
 #pragma unroll
-                    for (int tn = 0; tn < WT; tn++) g[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[tn], g[tm][tn], 0, 0, 0);
+                    for (int tn = 0; tn < WTN; tn++) g[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[tn], g[tm][tn], 0, 0, 0);
                 }
             }
         }
         // every accumulator entry of a lane belongs to one output column: one scale per lane and tile column
 #pragma unroll
-        for (int tn = 0; tn < WT; tn++) {
-            const float sc = Ss[grp][wn * 32 * WT + 32 * tn + l32];
+        for (int tn = 0; tn < WTN; tn++) {
+            const float sc = Ss[grp][wn * 32 * WTN + 32 * tn + l32];
 #pragma unroll
-            for (int tm = 0; tm < WT; tm++)
+            for (int tm = 0; tm < WTM; tm++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[tm][tn][e] = fmaf(g[tm][tn][e], sc, acc[tm][tn][e]);
         }
@@ -440,41 +447,41 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
 
     if constexpr (KS > 1) {
         // add the sets' sums: every set but the first parks its accumulators in the (no longer read) piece buffers
-        float *red = reinterpret_cast<float *>(lds);                // [KS - 1][4 wavefronts][WT*WT*16][64 lanes]
+        float *red = reinterpret_cast<float *>(lds);                // [KS - 1][4 wavefronts][WTM*WTN*16][64 lanes]
         if (kset > 0) {
 #pragma unroll
-            for (int i = 0; i < WT; i++)
+            for (int i = 0; i < WTM; i++)
 #pragma unroll
-                for (int j = 0; j < WT; j++)
+                for (int j = 0; j < WTN; j++)
 #pragma unroll
                     for (int e = 0; e < 16; e++)
-                        red[((((kset - 1) * 4 + wave) * WT * WT + i * WT + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+                        red[((((kset - 1) * 4 + wave) * WTM * WTN + i * WTN + j) * 16 + e) * 64 + lane] = acc[i][j][e];
         }
         __syncthreads();
         if (kset > 0) return;
 #pragma unroll
         for (int ks = 1; ks < KS; ks++)
 #pragma unroll
-            for (int i = 0; i < WT; i++)
+            for (int i = 0; i < WTM; i++)
 #pragma unroll
-                for (int j = 0; j < WT; j++)
+                for (int j = 0; j < WTN; j++)
 #pragma unroll
                     for (int e = 0; e < 16; e++)
-                        acc[i][j][e] += red[((((ks - 1) * 4 + wave) * WT * WT + i * WT + j) * 16 + e) * 64 + lane];
+                        acc[i][j][e] += red[((((ks - 1) * 4 + wave) * WTM * WTN + i * WTN + j) * 16 + e) * 64 + lane];
     }
 
     // epilogue: acc[i][jn][e] is C[32*i + 8*(e/4) + 4*(lane/32) + e%4][32*jn + lane%32] of the wavefront's block
 #pragma unroll
-    for (int jn = 0; jn < WT; jn++) {
-        const int col = n0 + wn * 32 * WT + 32 * jn + l32;
+    for (int jn = 0; jn < WTN; jn++) {
+        const int col = n0 + wn * 32 * WTN + 32 * jn + l32;
         if (col >= N) continue;
         float badd = 0.0f;
         if (ep.bias) badd = ep.interleaved_bias ? ((col & 1) ? ep.bias2[col >> 1] : ep.bias[col >> 1]) : ep.bias[col];
 #pragma unroll
-        for (int i = 0; i < WT; i++) {
+        for (int i = 0; i < WTM; i++) {
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                const int row = m0 + wm * 32 * WT + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                const int row = m0 + wm * 32 * WTM + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
                 if (ep.swiglu) {
                     // gate and up of one output sit in neighbouring lanes (columns 2j, 2j + 1); N is even, so a
                     // pair is inside or outside the matrix together (SiLU.java:20-24, SwiGLULayer.java:69)
@@ -533,15 +540,24 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
     GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu, swiglu};
     if (!m_dev && use_big_tile(m, n_rows)) {       // a device-side row count is usually far below m: keep small tiles
         dim3 grid2((n_rows + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
-        hipLaunchKernelGGL((k_gemm_q8<2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        // Two 128 x 128 workgroups fit a CU, so the tiles run in rounds of 512; when the last round would be mostly
+        // empty (352 or 704 tiles), 64 x 128 tiles - twice as many, three to four per CU - finish sooner
+        // (512 x 11264 x 2048: 101 against 113 us; 1024 rows: 194 against 229 us).
+        const int64_t tiles = (int64_t)grid2.x * grid2.y, rounds = (tiles + 511) / 512;
+        if (tiles * 100 < rounds * 512 * 85) {
+            dim3 gridw(grid2.x, (m + 63) / 64);
+            hipLaunchKernelGGL((k_gemm_q8<1, 2, 2, 1>), gridw, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+            return;
+        }
+        hipLaunchKernelGGL((k_gemm_q8<2, 2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
         return;
     }
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
     // few tiles (about one per CU): a workgroup brings its own second wavefront per SIMD
     if ((int64_t)grid.x * grid.y <= kFewTiles)
-        hipLaunchKernelGGL((k_gemm_q8<1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        hipLaunchKernelGGL((k_gemm_q8<1, 1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
     else
-        hipLaunchKernelGGL((k_gemm_q8<1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        hipLaunchKernelGGL((k_gemm_q8<1, 1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
 }
 
 }  // namespace dj
