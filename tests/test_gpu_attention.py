@@ -29,7 +29,9 @@ def oracle_attention(q, k, v, H, cos, sin):
                                                  (2, 128, 130, [5, 1, 124]), (32, 64, 2048, [3, 1]),
                                                  # grids of 288 and 576 workgroups at 128 rows each: the prefill kernel's
                                                  # two-key-set and one-key-set variants (the small shapes above use four)
-                                                 (32, 64, 1200, [1100, 1, 20]), (64, 32, 1150, [1100, 1])])
+                                                 (32, 64, 1200, [1100, 1, 20]), (64, 32, 1150, [1100, 1]),
+                                                 # ragged chunks around the 16-row threshold and the 32-row query tile
+                                                 (4, 64, 200, [17, 1, 33, 15, 16, 65]), (3, 128, 150, [31, 97])])
 def test_rope_store_attention_prefill_and_decode(H, hd, max_seq, chunks):
     d = H * hd
     total = sum(chunks)
