@@ -109,9 +109,9 @@ def test_q8_matvec_fused_prologue_epilogue(dev, flags):
         assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"{flags} {k}x{n}")
 
 
-@pytest.mark.parametrize("m", [1, 64])
-def test_q8_swiglu_gate_up(dev, m):
-    k, n = 256, 688
+@pytest.mark.parametrize("m,k,n", [(1, 256, 688), (64, 256, 688),
+                                   (520, 96, 4500), (1000, 160, 3500), (600, 64, 2000)])   # 64x128, 128x128, many 64x64 tiles
+def test_q8_swiglu_gate_up(dev, m, k, n):
     wg, wu = gaussian(k, n, 21, 0.05), gaussian(k, n, 22, 0.05)
     bg, bu = gaussian(1, n, 23, 0.1), gaussian(1, n, 24, 0.1)
     x, gamma = gaussian(m, k, 25, 1.0), 1.0 + gaussian(1, k, 26, 0.02)
@@ -125,12 +125,15 @@ def test_q8_swiglu_gate_up(dev, m):
     gate = ref.linear(h, ref.q8_roundtrip(wg), bg)
     up = ref.linear(h, ref.q8_roundtrip(wu), bu)
     exp = ref.multiply(ref.silu(gate), up)
-    assert_close(exp, dev.download(ob, (m, n)), atol=2e-6, rtol=1e-4, what=f"swiglu m={m}")
+    assert_close(exp, dev.download(ob, (m, n)), atol=2e-6, rtol=1e-4, what=f"swiglu {m}x{k}x{n}")
 
 
 @pytest.mark.parametrize("m,k,n", [(64, 2048, 512), (512, 2048, 256), (64, 688, 256), (7, 96, 33), (130, 5632, 128),
                                    (64, 4096, 344), (96, 11008, 128),
-                                   (1300, 688, 1400), (1024, 2048, 2100)])     # 128 x 128 tile, ragged edges
+                                   (1300, 688, 1400), (1024, 2048, 2100),      # many 64 x 64 tiles, ragged edges
+                                   # 440 tiles of 128 x 128 (one well-filled round of 512), ragged in M, N and K; 355 such
+                                   # tiles (a mostly empty second round) -> 64 x 128 tiles; exactly 512
+                                   (1000, 160, 7000), (520, 96, 9000), (1024, 64, 8192)])
 def test_q8_gemm_matches_oracle(dev, m, k, n):
     exp, got = linear_case(dev, m, k, n, norm=True, bias=True, residual=True, seed=30)
     scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
