@@ -208,6 +208,34 @@ __global__ void __launch_bounds__(kThreads) k_cross_entropy(const float *__restr
 __global__ void __launch_bounds__(kThreads) k_rmsnorm(const float *__restrict__ x, const float *__restrict__ gamma,
                                                       float *__restrict__ out, int rows, int cols) {
     __shared__ float lds[kWaves];
+    constexpr int NV = 4;                                        // 128-bit words a thread keeps of one row
+    if ((cols & 3) == 0 && cols <= kThreads * 4 * NV) {
+        // the row stays in registers between the sum of squares and the scaling: one pass over memory
+        const int n4 = cols >> 2;
+        for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+            const float4 *row4 = reinterpret_cast<const float4 *>(x + (int64_t)r * cols);
+            float4 *out4 = reinterpret_cast<float4 *>(out + (int64_t)r * cols);
+            float4 v[NV], g[NV];
+            float s = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int i = threadIdx.x + j * kThreads;
+                v[j] = i < n4 ? row4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                g[j] = i < n4 ? reinterpret_cast<const float4 *>(gamma)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                s += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+            }
+            s = block_sum(s, lds);
+            const float rms = sqrtf(s * (1.0f / (float)cols) + kRmsEps);
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int i = threadIdx.x + j * kThreads;
+                if (i < n4)
+                    out4[i] = make_float4((v[j].x / rms) * g[j].x, (v[j].y / rms) * g[j].y, (v[j].z / rms) * g[j].z,
+                                          (v[j].w / rms) * g[j].w);
+            }
+        }
+        return;
+    }
     for (int r = blockIdx.x; r < rows; r += gridDim.x) {
         const float *row = x + (int64_t)r * cols;
         float *orow = out + (int64_t)r * cols;

@@ -155,6 +155,12 @@ def test_fused_rmsnorm_silu_mul_embed_argmax(dev):
     xb, gb, ob = dev.upload(x), dev.upload(gamma), dev.alloc(x.size)
     Stream().rmsnorm(xb, gb, ob, 9, 2048).run()
     assert_close(ref.rmsnorm(x, gamma), dev.download(ob, x.shape), 1e-6, 1e-5)
+    # rows kept in registers (cols a multiple of 4 up to 4096) and the strided fallback (wider or ragged rows)
+    for rows, cols in ((3, 36), (600, 4096), (5, 4100), (7, 70), (2, 8192)):
+        xr, gr = gaussian(rows, cols, 44, 1.5), 1.0 + gaussian(1, cols, 45, 0.1)
+        o = dev.alloc(xr.size)
+        Stream().rmsnorm(dev.upload(xr), dev.upload(gr), o, rows, cols).run()
+        assert_close(ref.rmsnorm(xr, gr), dev.download(o, xr.shape), 1e-6, 1e-5, what=f"rmsnorm {rows}x{cols}")
     g, u = gaussian(5, 5632, 42, 2.0), gaussian(5, 5632, 43, 1.0)
     o2 = dev.alloc(g.size)
     Stream().silu_mul(dev.upload(g), dev.upload(u), o2, g.size).run()
