@@ -12,7 +12,9 @@
 // and an fp32 activation is the exact sum of three bf16 numbers (its top, middle and bottom 8 significant bits,
 // taken by truncation), so x . q = hi . q + mid . q + lo . q with every product exact and fp32 accumulation: three
 // bf16 MFMAs of K = 16 replace eight fp32 MFMAs of K = 2 at four times the rate.  The group scale multiplies the
-// finished 32-k partial sums (one scale per accumulator column per step).
+// finished 32-k partial sums (one scale per accumulator column per step).  Tile shapes (64 x 64, 64 x 128,
+// 128 x 128), scale groups per step and wavefront sets per workgroup are template arguments chosen per problem
+// shape by launch_q8_gemm; the epilogue adds bias / GELU / residual or pairs interleaved gate/up columns (SwiGLU).
 #include "dj_common.h"
 
 namespace dj {

@@ -8,11 +8,11 @@
 // [-127, 127]; dequantised weight = float(q) * scale (one fp32 rounding, so host
 // and device agree bit for bit).  1.125 bytes per weight.
 //
-// Decode (M = 1) is HBM bound: every weight byte is read exactly once.  One
+// Decode (M = 1): every weight byte is read from HBM exactly once.  One
 // wavefront owns an output row at a time; its 64 lanes read the row with 128-bit
 // loads (1 KiB per wave-load, fully coalesced), convert int8 -> fp32 in registers,
 // multiply with the activation slice the lane keeps in VGPRs for the whole kernel,
-// and reduce across the wavefront with shuffles.  The activation vector is staged
+// and reduce across the wavefront with DPP row operations.  The activation vector is staged
 // once per workgroup through LDS, where the optional prologue is applied (RMSNorm,
 // LayerNorm, or the merge of the decode attention's per-split records), so norm +
 // projection (+ bias, + GELU, + residual, or the SwiGLU gate) is one launch.
