@@ -115,7 +115,10 @@ def test_fused_decode_attention_and_decode_next(H, hd, max_seq, prefill, steps):
 
 
 @pytest.mark.parametrize("H,hd,max_seq,start,steps", [(8, 32, 256, 0, 6), (32, 64, 2048, 515, 3), (4, 128, 96, 55, 41),
-                                                      (2, 64, 1, 0, 1), (5, 32, 700, 509, 5)])
+                                                      (2, 64, 1, 0, 1), (5, 32, 700, 509, 5),
+                                                      # splits longer than one key/value round (two rounds in flight),
+                                                      # and longer than two (the loop comes round again)
+                                                      (32, 64, 2048, 1500, 2), (4, 128, 700, 600, 3), (2, 128, 1100, 1090, 3)])
 def test_decode_attention_records_merged_by_the_q8_linear_prologue(H, hd, max_seq, start, steps):
     """ATTN_DECODE_RECORDS leaves one record per (head, key split); the ATTN_MERGE prologue of the following
     Q8_LINEAR merges them.  With an identity-like projection out of reach (Q8), the check is against the oracle's
