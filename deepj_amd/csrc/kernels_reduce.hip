@@ -292,6 +292,11 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
     if (!vn && v != bv) return v > bv;
     return i < bi;
 }
+// The same order for a candidate that is known to come AFTER the incumbent (i > bi), or for an empty incumbent
+// (bi = INT_MAX): it wins only with a strictly larger value, or as the first NaN.
+__device__ __forceinline__ bool better_later(float v, float bv, int bi) {
+    return (v > bv) || ((v != v) && (bv == bv)) || bi == 0x7fffffff;
+}
 __global__ void __launch_bounds__(kThreads) k_argmax_rows(const float *__restrict__ a, int32_t *__restrict__ out,
                                                           int rows, int cols) {
     __shared__ float sv[kWaves];
@@ -334,6 +339,9 @@ __global__ void __launch_bounds__(1024) k_decode_next(const float *__restrict__ 
     __shared__ int s_tok;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
+    // the counters the last phase updates: requested now, used after the reduction
+    int st_pos = 0, st_gen = 0;
+    if (threadIdx.x == 0) { st_pos = state[0]; st_gen = state[2]; }
     // eight independent 128-bit loads per thread per round: one memory round trip per 32768 logits
     const int v4 = vocab >> 2;
     const float4 *l4 = reinterpret_cast<const float4 *>(logits);
@@ -347,11 +355,11 @@ __global__ void __launch_bounds__(1024) k_decode_next(const float *__restrict__ 
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             int c = (base + u * 1024 + threadIdx.x) * 4;
-            if (c < (v4 << 2)) {
-                if (better(t[u].x, c, bv, bi)) { bv = t[u].x; bi = c; }
-                if (better(t[u].y, c + 1, bv, bi)) { bv = t[u].y; bi = c + 1; }
-                if (better(t[u].z, c + 2, bv, bi)) { bv = t[u].z; bi = c + 2; }
-                if (better(t[u].w, c + 3, bv, bi)) { bv = t[u].w; bi = c + 3; }
+            if (c < (v4 << 2)) {                    // a thread meets its candidates in rising index order
+                if (better_later(t[u].x, bv, bi)) { bv = t[u].x; bi = c; }
+                if (better_later(t[u].y, bv, bi)) { bv = t[u].y; bi = c + 1; }
+                if (better_later(t[u].z, bv, bi)) { bv = t[u].z; bi = c + 2; }
+                if (better_later(t[u].w, bv, bi)) { bv = t[u].w; bi = c + 3; }
             }
         }
     }
@@ -371,10 +379,10 @@ __global__ void __launch_bounds__(1024) k_decode_next(const float *__restrict__ 
     if (threadIdx.x == 0) {
         for (int w = 1; w < 16; w++)
             if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
-        int g = state[2];
+        const int g = st_gen;
         if (g < capacity) tokens[g] = bi;
         state[1] = bi;
-        state[0] = state[0] + n_positions;
+        state[0] = st_pos + n_positions;
         state[2] = g + 1;
         s_tok = bi;
     }

@@ -114,6 +114,42 @@ def test_fused_decode_attention_and_decode_next(H, hd, max_seq, prefill, steps):
         dev.release_all()
 
 
+@pytest.mark.parametrize("vocab", [50, 4099, 32000, 40001])
+def test_decode_next_orders_logits_like_float_compare(vocab):
+    """DECODE_NEXT picks what TextGenerator's stable descending sort puts first (TextGenerator.java:163-170 with
+    Float.compare): the largest value, the lowest index among equals, NaN above everything (the first NaN wins),
+    index 0 when every logit is -inf; vocabularies below, at and beyond one round of the kernel's loads and not a
+    multiple of four."""
+    d = 8
+    rng = np.random.default_rng(vocab)
+    table = gaussian(vocab, d, 7)
+    cases = []
+    base = (rng.standard_normal(vocab) * 3).astype(np.float32)
+    cases.append((base.copy(), int(np.argmax(base))))
+    t = base.copy(); hi = float(t.max()) + 1.0
+    for i in (vocab - 1, vocab // 2, 3): t[i] = hi
+    cases.append((t, 3))                                            # ties: lowest index
+    t = base.copy(); t[vocab - 2] = np.nan; t[vocab // 3] = np.nan; t[1] = np.inf
+    cases.append((t, vocab // 3))                                   # NaN outranks +inf; the first NaN wins
+    cases.append((np.full(vocab, -np.inf, np.float32), 0))          # nothing is larger than anything: index 0
+    t = np.full(vocab, -np.inf, np.float32); t[vocab - 1] = -1e30
+    cases.append((t, vocab - 1))
+    dev = DeviceBuffers()
+    try:
+        state, tokens = dev.upload(np.zeros(4, np.int32)), dev.alloc(64)
+        logits_b, x_b, table_b = dev.alloc(vocab), dev.alloc(d), dev.upload(table)
+        for n, (logits, want) in enumerate(cases):
+            dev.write(logits_b, logits)
+            Stream().decode_next(logits_b, state, tokens, 64, table_b, x_b, vocab, d).run()
+            st = dev.download(state, (4,), np.int32)
+            assert (st[0], st[1], st[2]) == (n + 1, want, n + 1), f"case {n}: {st}"
+            assert np.array_equal(dev.download(x_b, (d,)), table[want])
+        got = dev.download(tokens, (64,), np.int32)[:len(cases)]
+        assert list(got) == [w for _, w in cases]
+    finally:
+        dev.release_all()
+
+
 @pytest.mark.parametrize("H,hd,max_seq,start,steps", [(8, 32, 256, 0, 6), (32, 64, 2048, 515, 3), (4, 128, 96, 55, 41),
                                                       (2, 64, 1, 0, 1), (5, 32, 700, 509, 5),
                                                       # splits longer than one key/value round (two rounds in flight),
