@@ -218,7 +218,9 @@ __device__ __forceinline__ int xs_at(int e) {
 // (its double-precision tanh costs some forty registers); 2 = ATTN_MERGE prologue: x is not the activation row
 // but the per-split records [head][kAttnRecordSplits][hd + 4] = {max, sum, -, -, o[hd]} the decode attention
 // kernel left, and the row is their merge  x[h*hd + j] = sum_s w_s o_s[j] / sum_s w_s l_s,  w_s = exp(max_s - max).
-template <int NC, int B, bool SWIGLU, int MODE>
+// PRO (compile time too: an operand that is not there must not be loaded - a workgroup's activation-sized loads
+// are as many bytes as its weight rows): 0 = no prologue, 1 = RMSNorm (gamma), 2 = LayerNorm (gamma and beta).
+template <int NC, int B, bool SWIGLU, int MODE, int PRO>
 __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     constexpr bool GELU = MODE == 1;
     constexpr bool MERGE = MODE == 2;
@@ -264,16 +266,17 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     } else if (vec) {
         // The activation, gain and beta loads go out first: they hit in L2 and come back while the weight loads
         // issued right behind them are still on their way from HBM.  All of them are unconditional (clamped
-        // address, dummy pointer for an absent operand), so the wait for them is a counted one that leaves the
-        // weight loads in flight.
-        const float *gp = p.gamma ? p.gamma : p.x, *bp = p.beta ? p.beta : p.x;
+        // address; which operands exist is known at compile time), so the wait for them is a counted one that
+        // leaves the weight loads in flight.
 #pragma unroll
         for (int j = 0; j < NC; j++) {
             const int e = (tid + kThreads * j) * 4;
             const int ec = e < p.k ? e : 0;
             xv[j] = *reinterpret_cast<const float4 *>(p.x + ec);
-            gv[j] = *reinterpret_cast<const float4 *>(gp + ec);
-            bv[j] = *reinterpret_cast<const float4 *>(bp + ec);
+            if constexpr (PRO >= 1) gv[j] = *reinterpret_cast<const float4 *>(p.gamma + ec);
+            else gv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if constexpr (PRO == 2) bv[j] = *reinterpret_cast<const float4 *>(p.beta + ec);
+            else bv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
     asm volatile("" ::: "memory");      // the loads above are issued before the ones below ...
@@ -314,7 +317,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             float x0 = xv[j].x, x1 = xv[j].y, x2 = xv[j].z, x3 = xv[j].w;
             asm volatile("" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
             const bool ok = (tid + kThreads * j) * 4 < p.k;
-            const bool okg = ok && p.gamma;
+            const bool okg = ok && PRO >= 1;
             xv[j] = make_float4(ok ? x0 : 0.f, ok ? x1 : 0.f, ok ? x2 : 0.f, ok ? x3 : 0.f);
             gv[j] = make_float4(okg ? gv[j].x : 0.f, okg ? gv[j].y : 0.f, okg ? gv[j].z : 0.f, okg ? gv[j].w : 0.f);
             bv[j] = make_float4(ok ? bv[j].x : 0.f, ok ? bv[j].y : 0.f, ok ? bv[j].z : 0.f, ok ? bv[j].w : 0.f);
@@ -324,7 +327,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
     // Stage the activation row through LDS (zero beyond K so padded weights meet zeros).
     // All global loads of the prologue - x and, for the RMSNorm prologue, gamma - were
     // issued together, so it costs one memory round trip, not one per element.
-    if (vec && p.beta) {
+    if (vec && PRO == 2) {
         // LayerNorm prologue (LayerNorm1D.java:34-66): mean, then the population variance about it, then
         // ((x - mean) / sqrt(var + 1e-5)) * gamma + beta goes to LDS.
         const float inv_k = 1.0f / (float)p.k;
@@ -356,7 +359,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
             if (e < p.kp) *reinterpret_cast<float4 *>(xs + xs_at(e)) = y;      // e >= k: x, gamma and beta are all zero
         }
     } else if (vec) {
-        if (p.gamma) {
+        if (PRO == 1) {
             // RMSNorm prologue (RMSNorm1D.java:46-57).  W.(g * x / rms) = (W.(g * x)) / rms: the staged row is
             // g * x, which needs no reduction, and the division by rms is applied to the finished sums, so the
             // sum of squares is reduced while the weight rows are still streaming in.
@@ -449,7 +452,19 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     if (grid > mv_grid_cap()) grid = mv_grid_cap();
     if (grid < 1) grid = 1;
     size_t lds = (size_t)xs_floats(a.kp) * sizeof(float);
-    hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE>), dim3(grid), dim3(kThreads), lds, s, a);
+    // the prologue the operands ask for: gamma and beta = LayerNorm, gamma alone = RMSNorm
+    const int pro = a.gamma ? (a.beta ? 2 : 1) : 0;
+    if constexpr (MODE == 2) {
+        hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 0>), dim3(grid), dim3(kThreads), lds, s, a);
+    } else if constexpr (SW) {
+        if (pro == 2) fail("q8_linear: SWIGLU cannot be combined with LAYERNORM");
+        if (pro == 1) hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 1>), dim3(grid), dim3(kThreads), lds, s, a);
+        else hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 0>), dim3(grid), dim3(kThreads), lds, s, a);
+    } else {
+        if (pro == 2) hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 2>), dim3(grid), dim3(kThreads), lds, s, a);
+        else if (pro == 1) hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 1>), dim3(grid), dim3(kThreads), lds, s, a);
+        else hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 0>), dim3(grid), dim3(kThreads), lds, s, a);
+    }
 }
 
 // Batch depth B (outputs a wavefront multiplies per step).  Small matrices want B = 1: every
