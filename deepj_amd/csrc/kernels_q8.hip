@@ -115,7 +115,8 @@ struct MatvecArgs {
 template <int NC, int R> struct RowBatch {
     int4 w[R][NC];
     float sc[R][NC];
-    float eb[R], eb2[R], er[R];       // bias, second bias and residual of the batch's outputs (index = output)
+    float ev;                         // epilogue operands of the batch: lane u holds the bias of output u, lane B + u its
+                                      // second bias, lane 2B + u its residual (one load instruction for all of them)
 };
 
 // The epilogue operands of outputs o0 .. o0+B-1 are requested together with the weight rows, so the
@@ -127,14 +128,12 @@ __device__ __forceinline__ void load_epilogue(RowBatch<NC, R> &b, const MatvecAr
     // later wait for an EARLIER load would have to be a wait for all of them.
     const float *bias = p.bias ? p.bias : p.scales, *bias2 = (SWIGLU && p.bias2) ? p.bias2 : p.scales;
     const float *residual = p.residual ? p.residual : p.scales;
-#pragma unroll
-    for (int u = 0; u < B; u++) {
-        int o = o0 + u < p.n_out ? o0 + u : p.n_out - 1;
-        o = o < 0 ? 0 : o;
-        b.eb[u] = bias[o];
-        if constexpr (SWIGLU) b.eb2[u] = bias2[o]; else b.eb2[u] = 0.0f;
-        b.er[u] = residual[o];
-    }
+    const int lane = threadIdx.x & 63;
+    const int kind = lane / B, u = lane - kind * B;         // lanes past 3B repeat a valid address
+    int o = o0 + u < p.n_out ? o0 + u : p.n_out - 1;
+    o = o < 0 ? 0 : o;
+    const float *src = kind == 1 ? bias2 : (kind == 2 ? residual : bias);
+    b.ev = src[o];
 }
 
 // Loads are unconditional: rows past the wave's range are clamped to its last row and
@@ -169,6 +168,13 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
         for (int c = 0; c < NC; c++) a = fmaf(dot16(b.w[u][c], xr[c]), b.sc[u][c], a);
         acc[u] = wave_sum_dpp(a) / rms;        // rms = 1 unless the RMSNorm scale was deferred to here
     }
+    float eb[B], eb2[B], er[B];
+#pragma unroll
+    for (int u = 0; u < B; u++) {
+        eb[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.ev), u));
+        eb2[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.ev), B + u));
+        er[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.ev), 2 * B + u));
+    }
     if (lane == 0) {
 #pragma unroll
         for (int u = 0; u < B; u++) {
@@ -177,16 +183,16 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
                 float v;
                 if constexpr (SWIGLU) {
                     float gate = acc[2 * u], up = acc[2 * u + 1];
-                    if (p.bias) gate = gate + b.eb[u];
-                    if (p.bias2) up = up + b.eb2[u];
+                    if (p.bias) gate = gate + eb[u];
+                    if (p.bias2) up = up + eb2[u];
                     float sg = gate * d_sigmoid(gate);     // SiLU.java:20-24
                     v = sg * up;                            // SwiGLULayer.java:69
                 } else {
                     v = acc[u];
-                    if (p.bias) v = v + b.eb[u];
+                    if (p.bias) v = v + eb[u];
                     if constexpr (GELU) v = d_gelu(v);
                 }
-                if (p.residual) v = b.er[u] + v;
+                if (p.residual) v = er[u] + v;
                 p.out[o] = v;
             }
         }
