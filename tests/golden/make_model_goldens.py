@@ -8,7 +8,7 @@ weights; nothing from the reference tree is imported or executed.  The reference
 no logits or token values for any model, so these fixtures pin the GPU path to the oracle, not to
 a JVM run.
 
-    python tests/golden/make_model_goldens.py c3 [c5] [g2]      # minutes per config on 8 cores
+    python tests/golden/make_model_goldens.py c3 [c4] [c5] [g2]      # minutes per config on 8 cores
 """
 import json
 import os
@@ -25,6 +25,9 @@ CONFIGS = {
     # the Llama decode workload of the benchmark
     "c3": dict(model=dict(vocab=32000, max_seq=2048, d=2048, heads=32, layers=16, dff=5632), seed=42,
                prompt_seed=3, prompt_len=512, new_tokens=64),
+    # the prefill workload: 7B-class widths (head dim 128), eight layers, a 2048-token prompt
+    "c4": dict(model=dict(vocab=32000, max_seq=2080, d=4096, heads=32, layers=8, dff=11008), seed=42,
+               prompt_seed=4, prompt_len=2048, new_tokens=32),
     # DeepSeek-style MLA at the same width (qRank = d/2, kvRank = d/4 as the reference's README suggests).
     # With the reference's initialiser (N(0,1)*0.1, Tensor.java random) at this width the attention scores
     # q.k/sqrt(hd) have a standard deviation near 150: every softmax row is a hard arg-max, and any change of
