@@ -133,7 +133,9 @@ def test_q8_swiglu_gate_up(dev, m, k, n):
                                    (1300, 688, 1400), (1024, 2048, 2100),      # many 64 x 64 tiles, ragged edges
                                    # 440 tiles of 128 x 128 (one well-filled round of 512), ragged in M, N and K; 355 such
                                    # tiles (a mostly empty second round) -> 64 x 128 tiles; exactly 512
-                                   (1000, 160, 7000), (520, 96, 9000), (1024, 64, 8192)])
+                                   (1000, 160, 7000), (520, 96, 9000), (1024, 64, 8192),
+                                   # the linear-op sweep's own shapes at M = 512, full width
+                                   (512, 2048, 5632), (512, 5632, 2048), (512, 4096, 11008)])
 def test_q8_gemm_matches_oracle(dev, m, k, n):
     exp, got = linear_case(dev, m, k, n, norm=True, bias=True, residual=True, seed=30)
     scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
