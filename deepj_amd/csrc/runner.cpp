@@ -298,6 +298,8 @@ void alloc_acts(Runner &r, Acts &a, int rows) {
     a.rows = rows;
 }
 
+void warm_up(Runner &r);
+
 void finalize(Runner &r) {
     const Config &c = r.cfg;
     if (r.finalized) return;
@@ -348,6 +350,7 @@ void finalize(Runner &r) {
     // the prompt-sized buffers for the longest prompt the cache can take, so that no request pays for allocation
     alloc_acts(r, r.pre, c.max_seq);
     r.finalized = true;
+    warm_up(r);
 }
 
 // ── command streams ────────────────────────────────────────────────────────
@@ -475,6 +478,29 @@ void reset(Runner &r) {
     hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
     r.pos = 0;
     r.generated = 0;
+}
+
+// The runtime builds a kernel's function object on its first launch (a few hundred microseconds each), and the
+// decode graphs are captured on first use.  One pass over prompts of the lengths that select the different GEMM and
+// attention variants, and a few graph-replayed tokens, move those costs from the first request to finalize();
+// the sequence state is cleared afterwards (the cache rows written here are never read: every row is rewritten
+// before the position counter reaches it).
+void decode_greedy(Runner &r, int steps, int mode);
+void warm_up(Runner &r) {
+    const Config &c = r.cfg;
+    std::vector<int32_t> ids((size_t)std::min(c.max_seq, 2048), 0);
+    for (int n : {2048, 1024, 512, 256, 128, 64, 32, 16, 4}) {
+        if (n > (int)ids.size()) continue;
+        reset(r);
+        prefill(r, ids.data(), n, nullptr, true);
+    }
+    reset(r);
+    const int steps = kGraphUnroll + 1;
+    if (c.max_seq >= steps + 2) {
+        prefill(r, ids.data(), 1, nullptr, true);
+        decode_greedy(r, steps, 1);
+    }
+    reset(r);
 }
 
 // All `steps` tokens in one launch of the persistent decode kernel.
