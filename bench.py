@@ -157,7 +157,7 @@ def main() -> int:
     t0 = time.perf_counter()
     model.prefill(prompt)
     HipNative.synchronize()
-    t_first_prefill = time.perf_counter() - t0      # includes the one-time allocation of the prompt-sized buffers
+    t_first_prefill = time.perf_counter() - t0      # the first request after the model was built
     model.reset()
     t0 = time.perf_counter()
     model.prefill(prompt)
