@@ -23,6 +23,7 @@
 // Matrices are given in the reference's orientation, fp32 [dIn x dOut] row-major.
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <string>
@@ -488,6 +489,8 @@ void reset(Runner &r) {
 void decode_greedy(Runner &r, int steps, int mode);
 void warm_up(Runner &r) {
     const Config &c = r.cfg;
+    const char *env = getenv("DEEPJ_HIP_WARMUP");           // "0": skip (profiling runs that want only the request's launches)
+    if (env && env[0] == '0') return;
     std::vector<int32_t> ids((size_t)std::min(c.max_seq, 2048), 0);
     for (int n : {2048, 1024, 512, 256, 128, 64, 32, 16, 4}) {
         if (n > (int)ids.size()) continue;
