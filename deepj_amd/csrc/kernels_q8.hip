@@ -447,6 +447,7 @@ __global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
 }
 
 constexpr int kMvGridCap = 768;          // three workgroups per CU
+constexpr int kMvGridCapWide = 1024;     // four for the widest matrices (the LM head: two batches per wavefront instead of three, 14.7 -> 14.0 us)
 inline int mv_grid_cap() { return kMvGridCap; }
 
 template <int NC, int B, bool SW, int MODE = 0>
@@ -455,7 +456,13 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     // more wavefronts than outputs.
     int batches = (a.n_out + B - 1) / B;
     int grid = (batches + kWaves - 1) / kWaves;
-    if (grid > mv_grid_cap()) grid = mv_grid_cap();
+    const int cap = a.n_out >= 16384 ? kMvGridCapWide : mv_grid_cap();
+    if (grid > cap) {
+        // every wavefront the same number of batches: fewer workgroups than the cap rather than a last, partly
+        // filled round (gate/up: 704 workgroups of exactly two batches per wavefront instead of 768 with one or two)
+        const int rounds = (batches + cap * kWaves - 1) / (cap * kWaves);
+        grid = (batches + kWaves * rounds - 1) / (kWaves * rounds);
+    }
     if (grid < 1) grid = 1;
     size_t lds = (size_t)xs_floats(a.kp) * sizeof(float);
     // the prologue the operands ask for: gamma and beta = LayerNorm, gamma alone = RMSNorm
