@@ -18,8 +18,12 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not used by this library's kernels.
+# kernarg preload: a kernel's leading scalar arguments (pointers, sizes; as many as fit in 14 registers) reach a
+# wavefront in registers at launch instead of through a load from the argument buffer that every other load of the
+# kernel would have to wait for.  The latency-bound decode kernels take their operands as separate arguments,
+# the first-needed ones in front, for this reason.
 COMMON = ["-x", "hip", f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 # Kernels whose results are compared element by element with the CPU backend keep
 # a*b+c unfused (the CPU never fuses); the contraction kernels use fma on purpose.

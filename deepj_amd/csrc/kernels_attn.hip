@@ -488,9 +488,19 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
 constexpr int kRecThreads = 1024;
 constexpr int kRecWaves = kRecThreads / 64;
 
+// Separate scalar arguments, the ones the first loads need in front (they can reach a wavefront in registers at
+// launch; a by-value struct is always fetched from the argument buffer first).
 template <int LPK>
-__global__ void __launch_bounds__(kRecThreads) k_attn_decode_records(DecodeArgs a) {
+__global__ void __launch_bounds__(kRecThreads)
+k_attn_decode_records(const int32_t *a_state, float *a_k_cache, float *a_v_cache, const float *a_qkv,
+                      const float *a_cos_t, const float *a_sin_t, int a_max_seq, int a_H, float *a_records,
+                      float a_scale) {
     constexpr int HD = LPK * 4;
+    DecodeArgs a;
+    a.qkv = a_qkv; a.k_cache = a_k_cache; a.v_cache = a_v_cache; a.tok_stride = HD;
+    a.head_stride = (int64_t)a_max_seq * HD; a.out = nullptr; a.state = a_state; a.scratch = a_records;
+    a.cos_t = a_cos_t; a.sin_t = a_sin_t; a.H = a_H; a.hd = HD; a.max_seq = a_max_seq; a.nsplit = kAttnRecordSplits;
+    a.scale = a_scale; a.counters = nullptr;
     constexpr int KPW = 64 / LPK;                  // keys a wavefront handles at a time
     constexpr int STRIDE = kRecWaves * KPW;        // keys per workgroup round
     constexpr int U = 4;
@@ -669,18 +679,16 @@ void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *
 void launch_attn_decode_records(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *records,
                                 const int32_t *state, const float *cos_t, const float *sin_t, int H, int hd,
                                 int max_seq) {
-    DecodeArgs a;
-    a.counters = nullptr;
-    a.qkv = qkv; a.k_cache = k_cache; a.v_cache = v_cache; a.out = nullptr; a.state = state; a.scratch = records;
-    a.tok_stride = hd; a.head_stride = (int64_t)max_seq * hd;
-    a.cos_t = cos_t; a.sin_t = sin_t; a.H = H; a.hd = hd; a.max_seq = max_seq;
-    a.nsplit = kAttnRecordSplits;
-    a.scale = (float)(1.0 / sqrt((double)hd));
+    const float scale = (float)(1.0 / sqrt((double)hd));
     dim3 grid(H, kAttnRecordSplits);
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(kRecThreads), 0, s, state, k_cache, v_cache, qkv, cos_t, sin_t, max_seq, H,
+                           records, scale);
+    };
     switch (hd) {
-        case 32: hipLaunchKernelGGL((k_attn_decode_records<8>), grid, dim3(kRecThreads), 0, s, a); break;
-        case 64: hipLaunchKernelGGL((k_attn_decode_records<16>), grid, dim3(kRecThreads), 0, s, a); break;
-        case 128: hipLaunchKernelGGL((k_attn_decode_records<32>), grid, dim3(kRecThreads), 0, s, a); break;
+        case 32: go(k_attn_decode_records<8>); break;
+        case 64: go(k_attn_decode_records<16>); break;
+        case 128: go(k_attn_decode_records<32>); break;
         default: fail("attention: head dim must be 32, 64 or 128");
     }
 }

@@ -226,8 +226,16 @@ __device__ __forceinline__ int xs_at(int e) {
 // kernel left, and the row is their merge  x[h*hd + j] = sum_s w_s o_s[j] / sum_s w_s l_s,  w_s = exp(max_s - max).
 // PRO (compile time too: an operand that is not there must not be loaded - a workgroup's activation-sized loads
 // are as many bytes as its weight rows): 0 = no prologue, 1 = RMSNorm (gamma), 2 = LayerNorm (gamma and beta).
+// The operands arrive as separate kernel arguments, the ones every lane needs first in front: leading scalar
+// arguments can be handed to a wavefront in registers at launch (a by-value struct is always fetched from the
+// argument buffer, a dependent load ahead of every other load of the kernel).
 template <int NC, int B, bool SWIGLU, int MODE, int PRO>
-__global__ void __launch_bounds__(kThreads) k_q8_matvec(MatvecArgs p) {
+__global__ void __launch_bounds__(kThreads)
+k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *a_out, int a_k, int a_kp, int a_n_out,
+            const float *a_gamma, int a_rec_hd, const float *a_bias, const float *a_bias2, const float *a_residual,
+            const float *a_beta) {
+    const MatvecArgs p{a_x, a_wq, a_scales, a_out, a_k, a_kp, a_n_out, a_gamma, a_bias, a_bias2, a_residual, a_beta,
+                       a_rec_hd};
     constexpr bool GELU = MODE == 1;
     constexpr bool MERGE = MODE == 2;
     constexpr int NS = kAttnRecordSplits;
@@ -467,16 +475,20 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     size_t lds = (size_t)xs_floats(a.kp) * sizeof(float);
     // the prologue the operands ask for: gamma and beta = LayerNorm, gamma alone = RMSNorm
     const int pro = a.gamma ? (a.beta ? 2 : 1) : 0;
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, s, a.x, a.wq, a.scales, a.out, a.k, a.kp, a.n_out,
+                           a.gamma, a.rec_hd, a.bias, a.bias2, a.residual, a.beta);
+    };
     if constexpr (MODE == 2) {
-        hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 0>), dim3(grid), dim3(kThreads), lds, s, a);
+        go(k_q8_matvec<NC, B, SW, MODE, 0>);
     } else if constexpr (SW) {
         if (pro == 2) fail("q8_linear: SWIGLU cannot be combined with LAYERNORM");
-        if (pro == 1) hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 1>), dim3(grid), dim3(kThreads), lds, s, a);
-        else hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 0>), dim3(grid), dim3(kThreads), lds, s, a);
+        if (pro == 1) go(k_q8_matvec<NC, B, SW, MODE, 1>);
+        else go(k_q8_matvec<NC, B, SW, MODE, 0>);
     } else {
-        if (pro == 2) hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 2>), dim3(grid), dim3(kThreads), lds, s, a);
-        else if (pro == 1) hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 1>), dim3(grid), dim3(kThreads), lds, s, a);
-        else hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, 0>), dim3(grid), dim3(kThreads), lds, s, a);
+        if (pro == 2) go(k_q8_matvec<NC, B, SW, MODE, 2>);
+        else if (pro == 1) go(k_q8_matvec<NC, B, SW, MODE, 1>);
+        else go(k_q8_matvec<NC, B, SW, MODE, 0>);
     }
 }
 
