@@ -18,6 +18,7 @@
 // projection (+ bias, + GELU, + residual, or the SwiGLU gate) is one launch.
 // M > 1 goes to the MFMA GEMM in kernels_matmul.hip.
 #include <cstdlib>
+#include <type_traits>
 
 #include "dj_common.h"
 #include "dj_device.h"
@@ -229,7 +230,10 @@ __device__ __forceinline__ int xs_at(int e) {
 // The operands arrive as separate kernel arguments, the ones every lane needs first in front: leading scalar
 // arguments can be handed to a wavefront in registers at launch (a by-value struct is always fetched from the
 // argument buffer, a dependent load ahead of every other load of the kernel).
-template <int NC, int B, bool SWIGLU, int MODE, int PRO>
+// VEC (compile time): K is a multiple of 4 and the row is loaded as float4s.  A run-time choice between the two
+// staging paths made the compiler merge their registers with copies placed right behind the first activation
+// load - a wait for it ahead of every weight load.
+template <int NC, int B, bool SWIGLU, int MODE, int PRO, bool VEC>
 __global__ void __launch_bounds__(kThreads)
 k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *a_out, int a_k, int a_kp, int a_n_out,
             const float *a_gamma, int a_rec_hd, const float *a_bias, const float *a_bias2, const float *a_residual,
@@ -258,7 +262,7 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
 
     RowBatch<NC, R> ba, bb;
     bool deferred_norm = false;
-    const bool vec = (p.k & 3) == 0;              // kernel-uniform
+    constexpr bool vec = VEC;
     float4 xv[NC], gv[NC], bv[NC];
     float2 rml[MERGE ? NC : 1][NS];
     float4 rov[MERGE ? NC : 1][NS];
@@ -460,6 +464,9 @@ inline int mv_grid_cap() { return kMvGridCap; }
 
 template <int NC, int B, bool SW, int MODE = 0>
 void launch_mv(hipStream_t s, const MatvecArgs &a) {
+    if constexpr (B != 1 && MODE != 2) {
+        if ((a.k & 3) != 0) { launch_mv<NC, 1, SW, MODE>(s, a); return; }
+    }
     // Three workgroups (12 wavefronts) per CU when there are outputs for them; never
     // more wavefronts than outputs.
     int batches = (a.n_out + B - 1) / B;
@@ -475,20 +482,33 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     size_t lds = (size_t)xs_floats(a.kp) * sizeof(float);
     // the prologue the operands ask for: gamma and beta = LayerNorm, gamma alone = RMSNorm
     const int pro = a.gamma ? (a.beta ? 2 : 1) : 0;
-    auto go = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, s, a.x, a.wq, a.scales, a.out, a.k, a.kp, a.n_out,
-                           a.gamma, a.rec_hd, a.bias, a.bias2, a.residual, a.beta);
+    // ragged K (not a multiple of 4): the scalar staging path, built for one output per wavefront only
+    const bool vec = (a.k & 3) == 0;
+    auto go = [&](auto pro_tag) {
+        constexpr int PRO = decltype(pro_tag)::value;
+        if (vec) {
+            hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, PRO, true>), dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
+                               a.scales, a.out, a.k, a.kp, a.n_out, a.gamma, a.rec_hd, a.bias, a.bias2, a.residual, a.beta);
+        } else if constexpr (B == 1 && MODE != 2) {
+            hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, PRO, false>), dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
+                               a.scales, a.out, a.k, a.kp, a.n_out, a.gamma, a.rec_hd, a.bias, a.bias2, a.residual, a.beta);
+        } else {
+            fail("q8_linear: no matvec kernel for this shape");     // launch_mv sends ragged K to B = 1
+        }
     };
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    using P2 = std::integral_constant<int, 2>;
     if constexpr (MODE == 2) {
-        go(k_q8_matvec<NC, B, SW, MODE, 0>);
+        go(P0{});
     } else if constexpr (SW) {
         if (pro == 2) fail("q8_linear: SWIGLU cannot be combined with LAYERNORM");
-        if (pro == 1) go(k_q8_matvec<NC, B, SW, MODE, 1>);
-        else go(k_q8_matvec<NC, B, SW, MODE, 0>);
+        if (pro == 1) go(P1{});
+        else go(P0{});
     } else {
-        if (pro == 2) go(k_q8_matvec<NC, B, SW, MODE, 2>);
-        else if (pro == 1) go(k_q8_matvec<NC, B, SW, MODE, 1>);
-        else go(k_q8_matvec<NC, B, SW, MODE, 0>);
+        if (pro == 2) go(P2{});
+        else if (pro == 1) go(P1{});
+        else go(P0{});
     }
 }
 
