@@ -235,11 +235,12 @@ __device__ __forceinline__ int xs_at(int e) {
 // load - a wait for it ahead of every weight load.
 template <int NC, int B, bool SWIGLU, int MODE, int PRO, bool VEC>
 __global__ void __launch_bounds__(kThreads)
-k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *a_out, int a_k, int a_kp, int a_n_out,
-            const float *a_gamma, int a_rec_hd, const float *a_bias, const float *a_bias2, const float *a_residual,
+k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *a_out, int a_k, int a_grid, int a_n_out,
+            int a_rec_hd, const float *a_gamma, const float *a_bias, const float *a_bias2, const float *a_residual,
             const float *a_beta) {
-    const MatvecArgs p{a_x, a_wq, a_scales, a_out, a_k, a_kp, a_n_out, a_gamma, a_bias, a_bias2, a_residual, a_beta,
-                       a_rec_hd};
+    // (the grid size comes as an argument: gridDim.x is one more value fetched from the argument buffer)
+    const MatvecArgs p{a_x, a_wq, a_scales, a_out, a_k, (a_k + kQ8Group - 1) / kQ8Group * kQ8Group, a_n_out, a_gamma,
+                       a_bias, a_bias2, a_residual, a_beta, a_rec_hd};
     constexpr bool GELU = MODE == 1;
     constexpr bool MERGE = MODE == 2;
     constexpr int NS = kAttnRecordSplits;
@@ -250,7 +251,7 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int groups = p.kp / kQ8Group;
     const int wave_global = blockIdx.x * kWaves + wave;
-    const int wave_count = gridDim.x * kWaves;
+    const int wave_count = a_grid * kWaves;
     // Batches are dealt round-robin: batch j of wave w is batch w + j*wave_count of the
     // matrix, so at any moment the rows in flight across the chip are neighbours in memory.
     const int n_batches = (p.n_out + B - 1) / B;
@@ -488,10 +489,10 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
         constexpr int PRO = decltype(pro_tag)::value;
         if (vec) {
             hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, PRO, true>), dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
-                               a.scales, a.out, a.k, a.kp, a.n_out, a.gamma, a.rec_hd, a.bias, a.bias2, a.residual, a.beta);
+                               a.scales, a.out, a.k, grid, a.n_out, a.rec_hd, a.gamma, a.bias, a.bias2, a.residual, a.beta);
         } else if constexpr (B == 1 && MODE != 2) {
             hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, PRO, false>), dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
-                               a.scales, a.out, a.k, a.kp, a.n_out, a.gamma, a.rec_hd, a.bias, a.bias2, a.residual, a.beta);
+                               a.scales, a.out, a.k, grid, a.n_out, a.rec_hd, a.gamma, a.bias, a.bias2, a.residual, a.beta);
         } else {
             fail("q8_linear: no matvec kernel for this shape");     // launch_mv sends ragged K to B = 1
         }
