@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # HBM bytes read + written per matvec launch (mean over the 65 launches of one token), from rocprofv3
 # FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
 # (profiles/q8_matvec_llama_d2048_decode_hbm_traffic.txt); algorithmic bytes are 15.40 MB.
-MATVEC_TRAFFIC_BYTES_PER_LAUNCH = 15_820_000
+MATVEC_TRAFFIC_BYTES_PER_LAUNCH = 15_800_000
 
 
 def q8_linear_bytes(k: int, n_rows: int) -> int:
