@@ -97,7 +97,8 @@ def test_q8_linear_layernorm_prologue(dev, m, k, n):
 @pytest.mark.parametrize("m", [1, 9, 200])
 def test_q8_linear_gelu_epilogue(dev, m):
     for k, n, flags in [(512, 1024, dict(gelu=True)), (256, 130, dict(gelu=True, layernorm=True)),
-                        (64, 40, dict(gelu=True, residual=True, bias=False))]:
+                        (64, 40, dict(gelu=True, residual=True, bias=False)),
+                        (250, 5000, dict(gelu=True))]:                 # K not a multiple of 4, many outputs
         exp, got = gpt_linear_case(dev, m, k, n, seed=30, **flags)
         scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
         assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"gelu m={m} {k}x{n} {flags}")

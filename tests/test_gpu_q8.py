@@ -92,7 +92,9 @@ def linear_case(dev, m, k, n, *, norm=False, bias=False, residual=False, seed=0)
 
 
 @pytest.mark.parametrize("k,n", [(2048, 2048), (2048, 5632), (5632, 2048), (4096, 1100), (11008, 512), (4096, 11008),
-                                 (688, 256), (256, 688), (32, 1), (1024, 5)])
+                                 (688, 256), (256, 688), (32, 1), (1024, 5),
+                                 # K not a multiple of 4: the scalar staging path, one output per wavefront whatever N
+                                 (70, 9), (1023, 300), (2050, 7000)])
 def test_q8_matvec_matches_oracle(dev, k, n):
     exp, got = linear_case(dev, 1, k, n)
     # fp32 sums of K terms in a different order: |err| <~ 1e-6 * sqrt(K) * |x||w|; outputs can sit near 0
@@ -103,13 +105,13 @@ def test_q8_matvec_matches_oracle(dev, k, n):
 @pytest.mark.parametrize("flags", [dict(norm=True), dict(bias=True), dict(residual=True),
                                    dict(norm=True, bias=True, residual=True)])
 def test_q8_matvec_fused_prologue_epilogue(dev, flags):
-    for k, n in [(2048, 768), (688, 256)]:
+    for k, n in [(2048, 768), (688, 256), (1023, 300)]:
         exp, got = linear_case(dev, 1, k, n, seed=10, **flags)
         scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
         assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"{flags} {k}x{n}")
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 256, 688), (64, 256, 688),
+@pytest.mark.parametrize("m,k,n", [(1, 256, 688), (1, 254, 688), (1, 2050, 6000), (64, 256, 688),
                                    (520, 96, 4500), (1000, 160, 3500), (600, 64, 2000)])   # 64x128, 128x128, many 64x64 tiles
 def test_q8_swiglu_gate_up(dev, m, k, n):
     wg, wu = gaussian(k, n, 21, 0.05), gaussian(k, n, 22, 0.05)
