@@ -40,3 +40,14 @@ def test_no_silent_cpu_fallback_without_a_device():
     with pytest.raises(RuntimeError):
         HipNative.nativeFlushOps(np.array([1, 0, 0, 0, 4], dtype=np.int32), 5)
     assert HipNative.q8Floats(64, 2) == (256 + 2 * 2 * 4) // 4      # pure size arithmetic needs no device
+
+
+def test_device_code_is_built_for_gfx950_with_the_required_flags():
+    """Every HIP source is compiled for gfx950 with packed-FP32 instructions switched off and with the leading
+    kernel arguments preloaded into registers (the decode kernels' argument order relies on it)."""
+    from deepj_amd import build
+    assert build.ARCH == "gfx950"
+    flags = " ".join(build.COMMON)
+    assert "-Xclang -target-feature -Xclang -packed-fp32-ops" in flags
+    assert "-mllvm -amdgpu-kernarg-preload-count=16" in flags
+    assert all(os.path.exists(os.path.join(build.CSRC, src)) for src in build.SOURCES)
