@@ -32,9 +32,13 @@ struct Buffer {
     int64_t floats = 0;       // size the caller asked for
 };
 
+// A captured graph holds raw device addresses.  The buffers its stream named (id, address at capture time) and
+// the workspace it used are remembered, and a replay is refused once any of them is gone or has moved.
 struct Graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    std::vector<std::pair<int32_t, void *>> refs;
+    float *workspace = nullptr;       // set when the stream needs workspace
 };
 
 struct Runtime {
@@ -53,6 +57,7 @@ struct Runtime {
     std::unordered_map<int32_t, Graph> graphs;
     int32_t next_graph = 1;
     unsigned *attn_counters = nullptr;             // kAttnCounterHeads zeroed words: decode attention's split arrivals
+    std::vector<std::pair<int32_t, void *>> *track = nullptr;   // graph capture: buffers the dry pass resolves
     void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
     std::vector<int64_t> decode_table_key;
 };
@@ -208,6 +213,7 @@ float *buf(int32_t id, int64_t floats, int op, const char *role) {
     if (floats < 0 || floats > it->second.floats)
         fail(std::string(op_name(op)) + ": buffer id=" + std::to_string(id) + " (" + role + ") holds " +
              std::to_string(it->second.floats) + " floats, op needs " + std::to_string(floats));
+    if (g.track) g.track->emplace_back(id, it->second.ptr);
     return static_cast<float *>(it->second.ptr);
 }
 float *buf_opt(int32_t id, int64_t floats, int op, const char *role) {
@@ -625,6 +631,7 @@ void exec_one(Cursor &c) {
         }
         case DJ_OP_LLAMA_DECODE: {
             const int len = w[1];
+            if (len < 29) fail("OP_LLAMA_DECODE: length word below the 29 header words");    // before any of them is read
             const int64_t steps = w[2], d = w[3], H = w[4], dff = w[5], vocab = w[6], max_seq = w[7], L = w[8], cap = w[9];
             if (steps < 0 || d <= 0 || H <= 0 || dff <= 0 || vocab <= 0 || max_seq <= 0 || L <= 0 || cap < 0 || d % H)
                 fail("OP_LLAMA_DECODE: bad shape");
@@ -991,10 +998,20 @@ int deepj_hip_graph_capture(const int32_t *cmd, int32_t len, int32_t *handle) {
         ensure_init();
         if (!handle) fail("graph_capture: null handle");
         int64_t ws = 0;
-        walk(cmd, len, true, &ws);
-        ensure_workspace(ws);
-        DJ_HIP(hipStreamSynchronize(g.stream));
         Graph gr;
+        g.track = &gr.refs;
+        try {
+            walk(cmd, len, true, &ws);
+        } catch (...) {
+            g.track = nullptr;
+            throw;
+        }
+        g.track = nullptr;
+        std::sort(gr.refs.begin(), gr.refs.end());
+        gr.refs.erase(std::unique(gr.refs.begin(), gr.refs.end()), gr.refs.end());
+        ensure_workspace(ws);
+        if (ws > 0) gr.workspace = g.workspace;
+        DJ_HIP(hipStreamSynchronize(g.stream));
         DJ_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal));
         g.capturing = true;
         try {
@@ -1023,6 +1040,17 @@ int deepj_hip_graph_launch(int32_t handle, int32_t times) {
     return guarded([&] {
         auto it = g.graphs.find(handle);
         if (it == g.graphs.end()) fail("graph_launch: unknown graph handle " + std::to_string(handle));
+        // the graph replays raw addresses: refuse when a buffer it names was released or now lives elsewhere,
+        // or when the workspace it used has been replaced by a larger one
+        for (const auto &ref : it->second.refs) {
+            auto b = g.live.find(ref.first);
+            if (b == g.live.end() || b->second.ptr != ref.second)
+                fail("graph_launch: buffer id=" + std::to_string(ref.first) + " was released or reallocated after graph " +
+                     std::to_string(handle) + " was captured; capture the stream again");
+        }
+        if (it->second.workspace && it->second.workspace != g.workspace)
+            fail("graph_launch: the workspace was reallocated after graph " + std::to_string(handle) +
+                 " was captured; capture the stream again");
         // Bounded run-ahead: at most kRing windows of kWindow replays are queued behind the one the
         // device is executing, so a long run never piles tens of thousands of dispatches (and their
         // kernel-argument blocks) into the queue; the device is never left idle by this.

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from deepj_amd import HipNative, Tensor
+from deepj_amd import opcodes as op
 from oracle import cpu_ref as ref
 from gpu_util import assert_close, backend, rnd, tensor
 
@@ -253,6 +254,45 @@ def test_native_errors_surface_as_exceptions_and_runtime_survives():
         HipNative.nativeReleaseBuffers([900001, 900002, 424242], 3)             # unknown id ignored (:1545-1547)
     with backend() as be:                                                       # still works afterwards
         assert_close([[3.0]], be.add(tensor([[1.0]]), tensor([[2.0]])), 0, 0)
+
+
+def test_graph_replay_is_refused_once_a_captured_buffer_or_the_workspace_is_gone():
+    """A captured graph replays raw device addresses: after a buffer it names is released (or re-created elsewhere),
+    or after the workspace it used was replaced by a larger one, a launch must fail and run nothing."""
+    from deepj_amd.fused import DeviceBuffers, Stream
+    HipNative.init(0)
+    dev = DeviceBuffers()
+    try:
+        a, out = dev.upload(np.arange(8, dtype=np.float32)), dev.alloc(8)
+        add = Stream().emit(op.OP_ADD_SCALAR, a, out, np.float32(1.0).view(np.int32), 8).array()
+        g1 = HipNative.graphCapture(add)
+        HipNative.graphLaunch(g1, 2)
+        assert list(dev.download(out, (8,))) == [1, 2, 3, 4, 5, 6, 7, 8]
+        dev.write(out, np.zeros(8, np.float32))
+        dev.release(a)
+        with pytest.raises(RuntimeError, match="released or reallocated"):
+            HipNative.graphLaunch(g1, 1)
+        assert not dev.download(out, (8,)).any(), "a refused replay must launch nothing"
+        HipNative.graphDestroy(g1)
+        # a graph that uses the workspace (normalised rows of an M > 1 Q8_LINEAR), then a stream that needs a larger one
+        m, k, n = 8, 64, 4
+        x, gm, w, o = dev.alloc(m * k), dev.alloc(k), dev.alloc(HipNative.q8Floats(k, n)), dev.alloc(m * n)
+        Stream().fill(x, 0, m * k).fill(gm, 0, k).fill(w, 0, HipNative.q8Floats(k, n)).run()
+        g2 = HipNative.graphCapture(Stream().q8_linear(x, w, o, m, k, n, gamma=gm).array())
+        HipNative.graphLaunch(g2, 1)
+        big_m, big_k = 16384, 2048                   # 32 Mi floats of normalised rows: more than any other test's stream needs
+        bx, bg, bw, bo = (dev.alloc(big_m * big_k), dev.alloc(big_k), dev.alloc(HipNative.q8Floats(big_k, n)),
+                          dev.alloc(big_m * n))
+        Stream().fill(bx, 0, big_m * big_k).fill(bg, 0, big_k).fill(bw, 0, HipNative.q8Floats(big_k, n)).run()
+        Stream().q8_linear(bx, bw, bo, big_m, big_k, n, gamma=bg).run()
+        with pytest.raises(RuntimeError, match="workspace was reallocated"):
+            HipNative.graphLaunch(g2, 1)
+        HipNative.graphDestroy(g2)
+        # a stream whose variable-length op claims fewer words than its fixed header is refused before its words are read
+        with pytest.raises(RuntimeError, match="length word below"):
+            HipNative.nativeFlushOps(np.array([op.OP_LLAMA_DECODE, 2], np.int32), 2)
+    finally:
+        dev.release_all()
 
 
 def test_released_buffers_are_recycled_without_new_driver_allocations():
