@@ -29,6 +29,7 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_download.argtypes = [C.c_int32, C.c_void_p, C.c_int64]
     lib.deepj_hip_release.argtypes = [_i32p, C.c_int32]
     lib.deepj_hip_flush_ops.argtypes = [_i32p, C.c_int32]
+    lib.deepj_hip_flush_ops_noalloc.argtypes = [_i32p, C.c_int32]
     lib.deepj_hip_last_error.restype = C.c_char_p
     lib.deepj_hip_pool_stats.argtypes = [C.POINTER(C.c_int64)]
     lib.deepj_hip_stream.restype = C.c_void_p
@@ -39,7 +40,7 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_graph_launch.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_graph_destroy.argtypes = [C.c_int32]
     for name in ("deepj_hip_init", "deepj_hip_alloc_buffers", "deepj_hip_upload", "deepj_hip_download",
-                 "deepj_hip_release", "deepj_hip_flush_ops", "deepj_hip_synchronize", "deepj_hip_shutdown",
+                 "deepj_hip_release", "deepj_hip_flush_ops", "deepj_hip_flush_ops_noalloc", "deepj_hip_synchronize", "deepj_hip_shutdown",
                  "deepj_hip_trim", "deepj_hip_pool_stats", "deepj_hip_time_ops", "deepj_hip_graph_capture",
                  "deepj_hip_graph_launch", "deepj_hip_graph_destroy"):
         getattr(lib, name).restype = C.c_int
@@ -108,6 +109,12 @@ class HipNative:
     def nativeFlushOps(cmd_stream, length: int) -> None:
         cmd = _ids(cmd_stream)
         _check(library().deepj_hip_flush_ops(cmd.ctypes.data_as(_i32p), length))
+
+    @staticmethod
+    def flushOpsNoAlloc(cmd_stream, length: int) -> None:
+        """flushOps over the library's static scratch array: no device allocation on this path."""
+        cmd = _ids(cmd_stream)
+        _check(library().deepj_hip_flush_ops_noalloc(cmd.ctypes.data_as(_i32p), length))
 
     # ── runtime control ─────────────────────────────────────────────────────
     @staticmethod

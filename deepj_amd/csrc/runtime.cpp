@@ -57,6 +57,8 @@ struct Runtime {
     std::unordered_map<int32_t, Graph> graphs;
     int32_t next_graph = 1;
     unsigned *attn_counters = nullptr;             // kAttnCounterHeads zeroed words: decode attention's split arrivals
+    unsigned char *static_scratch = nullptr;       // device address of `scratch` below on g.device
+    bool no_alloc = false;                         // inside deepj_hip_flush_ops_noalloc: nothing may allocate
     std::vector<std::pair<int32_t, void *>> *track = nullptr;   // graph capture: buffers the dry pass resolves
     void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
     std::vector<int64_t> decode_table_key;
@@ -64,6 +66,14 @@ struct Runtime {
 
 Runtime g;
 thread_local std::string g_error;
+
+// Scratch memory of deepj_hip_flush_ops_noalloc, part of the loaded code object (each GPU the library runs on
+// holds its own copy until the process ends): the arrival counters of the split decode attention, then the
+// workspace that Q8_LINEAR's GEMM path writes its normalised activation rows to.  Host code never uses the
+// symbol itself as an address: ensure_init() asks the runtime where the array lives on the current device.
+constexpr size_t kStaticCounterBytes = (size_t)kAttnCounterHeads * sizeof(unsigned);
+constexpr int64_t kStaticWorkspaceFloats = DEEPJ_HIP_NOALLOC_WORKSPACE_FLOATS;   // 8 MiB: e.g. 512 rows of 4096 floats
+static __device__ __align__(256) unsigned char scratch[kStaticCounterBytes + (size_t)kStaticWorkspaceFloats * 4];
 
 void ensure_init(int device = 0) {
     if (g.ready) return;
@@ -77,6 +87,10 @@ void ensure_init(int device = 0) {
     DJ_HIP(hipHostMalloc(&g.staging, g.staging_bytes, hipHostMallocDefault));
     DJ_HIP(hipMalloc((void **)&g.attn_counters, kAttnCounterHeads * sizeof(unsigned)));
     DJ_HIP(hipMemset(g.attn_counters, 0, kAttnCounterHeads * sizeof(unsigned)));
+    g.static_scratch = nullptr;
+    DJ_HIP(hipGetSymbolAddress((void **)&g.static_scratch, HIP_SYMBOL(scratch)));
+    if (!g.static_scratch) fail("deepj_hip: the static scratch array has no device address");
+    DJ_HIP(hipMemset(g.static_scratch, 0, kStaticCounterBytes));
     g.device = device;
     g.ready = true;
 }
@@ -100,6 +114,7 @@ void *pool_alloc(size_t cls) {
         return p;
     }
     if (g.capturing) fail("deepj_hip: device allocation requested while a graph is being captured");
+    if (g.no_alloc) fail("deepj_hip: device allocation requested inside the allocation-free entry point");
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, cls);
     if (e != hipSuccess) {
@@ -134,6 +149,12 @@ void pool_free(void *p, size_t cls) {
 }
 
 void ensure_workspace(int64_t floats) {
+    if (g.no_alloc) {
+        if (floats > kStaticWorkspaceFloats)
+            fail("flush_ops_noalloc: the stream needs " + std::to_string(floats) + " floats of workspace, the static "
+                 "scratch holds " + std::to_string(kStaticWorkspaceFloats) + " (use deepj_hip_flush_ops)");
+        return;
+    }
     if (floats <= g.workspace_floats) return;
     if (g.capturing) fail("deepj_hip: workspace would have to grow during graph capture; run the stream once first");
     DJ_HIP(hipStreamSynchronize(g.stream));
@@ -632,6 +653,7 @@ void exec_one(Cursor &c) {
         case DJ_OP_LLAMA_DECODE: {
             const int len = w[1];
             if (len < 29) fail("OP_LLAMA_DECODE: length word below the 29 header words");    // before any of them is read
+            if (g.no_alloc) fail("OP_LLAMA_DECODE keeps a device copy of its layer table and cannot run allocation-free");
             const int64_t steps = w[2], d = w[3], H = w[4], dff = w[5], vocab = w[6], max_seq = w[7], L = w[8], cap = w[9];
             if (steps < 0 || d <= 0 || H <= 0 || dff <= 0 || vocab <= 0 || max_seq <= 0 || L <= 0 || cap < 0 || d % H)
                 fail("OP_LLAMA_DECODE: bad shape");
@@ -888,6 +910,35 @@ int deepj_hip_flush_ops(const int32_t *cmd, int32_t len) {
     return guarded([&] {
         ensure_init();
         run_stream(cmd, len);
+    });
+}
+
+// The same interpreter over the static scratch array instead of the runtime's own (growable) workspace and
+// counters: no hipMalloc / hipFree on this path.  The counters are cleared by a fill kernel first (the array keeps
+// whatever the last call left); calls that overlap on one GPU would share the array and race.
+int deepj_hip_flush_ops_noalloc(const int32_t *cmd, int32_t len) {
+    return guarded([&] {
+        if (!g.ready)
+            fail("flush_ops_noalloc: the runtime is not initialised (initialisation allocates: call deepj_hip_init first)");
+        struct Scope {
+            float *ws = g.workspace; int64_t wsf = g.workspace_floats; unsigned *ctr = g.attn_counters;
+            Scope() {
+                g.no_alloc = true;
+                g.attn_counters = reinterpret_cast<unsigned *>(g.static_scratch);
+                g.workspace = reinterpret_cast<float *>(g.static_scratch + kStaticCounterBytes);
+                g.workspace_floats = kStaticWorkspaceFloats;
+            }
+            ~Scope() { g.no_alloc = false; g.workspace = ws; g.workspace_floats = wsf; g.attn_counters = ctr; }
+        } scope;
+        if (len < 0) fail("flushOps: negative stream length");
+        if (len > 0 && !cmd) fail("flushOps: null command stream");
+        int64_t ws = 0;
+        walk(cmd, len, true, &ws);
+        ensure_workspace(ws);           // only checks the need against the static size here
+        launch_fill(g.stream, reinterpret_cast<uint32_t *>(g.attn_counters), 0u, kAttnCounterHeads);
+        walk(cmd, len, false, nullptr);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) fail(std::string("kernel launch failed: ") + hipGetErrorString(e));
     });
 }
 

@@ -52,6 +52,20 @@ int deepj_hip_release(const int32_t *ids, int32_t count);
  * only enqueues work: results are observable through deepj_hip_download. */
 int deepj_hip_flush_ops(const int32_t *cmd, int32_t len);
 
+/* deepj_hip_flush_ops for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same streams, same
+ * kernels, same results; the device scratch those kernels need - the workspace that Q8_LINEAR with a norm
+ * prologue and M > 1 writes its normalised rows to, and the arrival counters of the split decode attention
+ * (ATTENTION / ATTENTION_KV with S = 1, ATTN_DECODE) - is a fixed array inside the library's code object instead
+ * of memory the runtime allocates and grows.  The call never calls hipMalloc or hipFree: it fails when the
+ * runtime is not initialised yet (deepj_hip_init allocates), when the stream needs more than
+ * DEEPJ_HIP_NOALLOC_WORKSPACE_FLOATS floats of workspace (M * K of the largest such Q8_LINEAR), and on
+ * LLAMA_DECODE.  Every buffer the stream names must already exist.  All calls on a GPU share the one array,
+ * which keeps the previous call's contents (the counters are cleared by a kernel at the start of each call);
+ * calls that overlap on one GPU would race - the single-caller rule above already excludes that. */
+#define DEEPJ_HIP_NOALLOC_WORKSPACE_FLOATS (2 << 20)
+int deepj_hip_flush_ops_noalloc(const int32_t *cmd, int32_t len);
+
 /* Message of the last failure on this thread ("" if none). */
 const char *deepj_hip_last_error(void);
 
