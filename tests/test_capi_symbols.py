@@ -51,3 +51,6 @@ def test_device_code_is_built_for_gfx950_with_the_required_flags():
     assert "-Xclang -target-feature -Xclang -packed-fp32-ops" in flags
     assert "-mllvm -amdgpu-kernarg-preload-count=16" in flags
     assert all(os.path.exists(os.path.join(build.CSRC, src)) for src in build.SOURCES)
+    # the device pass honours the flag (the host pass only notes that it does not know the feature): a float2 probe
+    # kernel compiled with it holds no v_pk_*_f32 instruction, and holds one without it
+    build.verify_packed_fp32_off()
