@@ -12,10 +12,13 @@ per-token HIP graph).  Prints ONE JSON line.
 
 Besides tok/s the line carries
   roofline     - the Q8 matvec kernel (the dominant kernel): algorithmic bytes per launch /
-                 average launch duration, measured with HIP events on the library's stream
-                 over back-to-back launches on the model's own weights (1 GB of distinct
-                 weights per token, so nothing is served from the 256 MB Infinity Cache; the
-                 cache-warm figure - the first four layers cycled - is reported beside it)
+                 mean kernel duration, measured live with a start and a stop HIP event on every
+                 dispatch of the per-token stream run in order on the model's own weights (1 GB of
+                 distinct weights per token, so nothing is served from the 256 MB Infinity Cache) -
+                 the quantity rocprofv3 --kernel-trace reports; `per_kernel` holds the same for
+                 every kernel of the token, `floor` an empty kernel and a pure streaming read of the
+                 very same weight buffers by the same method; the back-to-back launch period
+                 (no events, launch cost hidden behind the previous kernel) is reported beside it
   cpu_baseline - the CPU oracle (a C restatement of the reference's CpuBackend + layers,
                  not the JVM) on this box's host cores, on a bounded sample of the workload
 """
@@ -44,41 +47,114 @@ def q8_linear_bytes(k: int, n_rows: int) -> int:
     return k * n_rows + 4 * k * n_rows // 32 + 4 * k + 4 * n_rows
 
 
-def matvec_roofline(model, iters: int = 20):
-    """Times only the Q8_LINEAR ops of the per-token stream, in order, on the real weights."""
-    from deepj_amd import HipNative, opcodes as op
-    stream = model.decodeStream()
-    strides = op.FUSED_STRIDES
-    pos, lin, total_bytes, launches = 0, [], 0, 0
+VARIANTS = {  # (K, Q8 rows) of the workload's five matvec shapes
+    (2048, 6144): "qkv", (2048, 2048): "wo", (2048, 11264): "gate_up", (5632, 2048): "down", (2048, 32000): "lm_head"}
+
+
+def decode_ops(stream):
+    """(opcode, words) of every op of a fused command stream."""
+    from deepj_amd import opcodes as op
+    pos, ops = 0, []
     while pos < len(stream):
         code = int(stream[pos])
-        n = strides[code]
-        if code == op.OP_Q8_LINEAR:
-            w = stream[pos:pos + n]
-            m, k, nn, flags = int(w[4]), int(w[5]), int(w[6]), int(w[7])
-            if m == 1:
-                rows = 2 * nn if flags & op.LIN_SWIGLU else nn
-                total_bytes += q8_linear_bytes(k, rows)
-                launches += 1
-                lin.extend(int(x) for x in w)
+        n = op.FUSED_STRIDES[code]
+        ops.append((code, [int(x) for x in stream[pos:pos + n]]))
         pos += n
-    words = len(lin) // launches                                # every Q8_LINEAR op has the same length
+    return ops
+
+
+def matvec_roofline(model, position: int, iters: int = 12):
+    """Per-kernel durations of one decoded token, measured live: the per-token stream runs in order (1 GB of distinct
+    weights per pass, so nothing is served from the 256 MB Infinity Cache) with a start and a stop event on every
+    dispatch; a kernel's duration is the time between the two on the device - what a kernel trace reports for it.
+    `achieved` = algorithmic bytes of the 65 Q8 matvec launches / the sum of their durations."""
+    from deepj_amd import HipNative, opcodes as op
+    from deepj_amd.fused import DeviceBuffers, Stream
+    cfg = model.cfg
+    stream = model.decodeStream()
+    ops = decode_ops(stream)
+    HipNative.profileOps(stream, 2)                               # warm-up
+    us = HipNative.profileOps(stream, iters)
+    table, lin, lin_bytes, lin_us, weights = {}, [], 0, 0.0, []
+
+    def add(name, nbytes, t):
+        e = table.setdefault(name, {"launches_per_token": 0, "bytes": int(nbytes), "us": 0.0})
+        e["launches_per_token"] += 1
+        e["us"] += float(t)
+
+    for (code, w), t in zip(ops, us):
+        if code == op.OP_Q8_LINEAR and w[4] == 1:
+            k, nn, flags = w[5], w[6], w[7]
+            rows = 2 * nn if flags & op.LIN_SWIGLU else nn
+            nbytes = q8_linear_bytes(k, rows)
+            add(VARIANTS.get((k, rows), f"{k}x{rows}"), nbytes, t)
+            lin_bytes += nbytes
+            lin_us += float(t)
+            lin.extend(w)
+            weights.append((w[2], HipNative.q8Floats(k, rows), VARIANTS.get((k, rows), f"{k}x{rows}")))
+        elif code == op.OP_ATTN_DECODE_RECORDS:
+            add("attention", 2 * position * cfg.dModel * 4, t)    # K and V rows of the live context, fp32
+        elif code == op.OP_DECODE_NEXT:
+            add("decode_next", 4 * cfg.vocabSize, t)
+    for e in table.values():
+        e["us"] = round(e["us"] / e["launches_per_token"], 3)
+        e["GBs"] = round(e["bytes"] / e["us"] / 1e3, 1)
+        e["frac"] = round(e["bytes"] / e["us"] / 1e3 / HBM_PEAK_GBS, 4)
+    launches = len(weights)
+    achieved = lin_bytes / lin_us / 1e3
+
+    # the same 65 launches back to back without events (launch cost hidden behind the previous kernel, gaps included)
     lin = np.asarray(lin, dtype=np.int32)
-    HipNative.timeOps(lin, 2)                                   # warm-up
-    ms = HipNative.timeOps(lin, iters)
-    avg_launch_s = ms * 1e-3 / (iters * launches)
-    achieved = (total_bytes / launches) / avg_launch_s / 1e9
-    # the cache-warm figure, reported apart: the launches of the first four layers only (232 MB), which stay
-    # resident in the 256 MB Infinity Cache from one pass to the next
-    warm_n = min(16, launches)
+    HipNative.timeOps(lin, 2)
+    b2b_us = HipNative.timeOps(lin, iters) * 1e3 / (iters * launches)
+    words = len(lin) // launches
+    warm_n = min(16, launches)                                    # first four layers: 232 MB, Infinity-Cache resident
     warm = lin[:warm_n * words]
     HipNative.timeOps(warm, 4)
     warm_us = HipNative.timeOps(warm, 4 * iters) * 1e3 / (4 * iters * warm_n)
+
+    # floors, by the same method: an empty kernel of the matvec's grid size (what a dependent launch costs with no
+    # work in it), and a pure streaming read of the very same weight buffers in the same order
+    dev = DeviceBuffers()
+    sink = dev.alloc(4)
+    nops = Stream()
+    for _ in range(64):
+        nops.nop(768)
+    nops.profile(2)
+    empty_us = float(np.mean(nops.profile(iters)))
+    empty_period_us = nops.time(iters) * 1e3 / (iters * 64)
+    reads = Stream()
+    for wid, floats, _ in weights:
+        reads.stream_read(wid, sink, floats)
+    reads.profile(2)
+    rus = reads.profile(iters)
+    read_tab = {}
+    for (wid, floats, name), t in zip(weights, rus):
+        e = read_tab.setdefault(name, {"bytes": floats * 4, "us": 0.0, "n": 0})
+        e["us"] += float(t)
+        e["n"] += 1
+    for e in read_tab.values():
+        e["us"] = round(e["us"] / e.pop("n"), 3)
+        e["GBs"] = round(e["bytes"] / e["us"] / 1e3, 1)
+    read_avg_us = float(np.sum(rus)) / launches
+    read_b2b_us = reads.time(iters) * 1e3 / (iters * launches)
+    dev.release_all()
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MATVEC_TRAFFIC_BYTES_PER_LAUNCH,
-            "kernel": "k_q8_matvec", "launches_per_token": launches,
-            "bytes_per_launch": total_bytes // launches, "avg_launch_us": round(avg_launch_s * 1e6, 3),
-            "cache_warm_avg_launch_us": round(warm_us, 3)}
+            "traffic_source": "profiles/q8_matvec_llama_d2048_decode_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
+                              "WRITE_SIZE, scaled by k_copy)",
+            "kernel": "k_q8_matvec", "launches_per_token": launches, "bytes_per_launch": lin_bytes // launches,
+            "avg_launch_us": round(lin_us / launches, 3),
+            "timing": "mean kernel duration (start/stop events on each dispatch, whole token in order, HBM-cold); "
+                      "rocprofv3 --kernel-trace reports the same quantity",
+            "back_to_back_avg_launch_us": round(b2b_us, 3), "cache_warm_avg_launch_us": round(warm_us, 3),
+            "per_kernel": table,
+            "floor": {"empty_kernel_us": round(empty_us, 3), "empty_launch_period_us": round(empty_period_us, 3),
+                      "stream_read": read_tab, "stream_read_avg_us": round(read_avg_us, 3),
+                      "stream_read_back_to_back_avg_us": round(read_b2b_us, 3),
+                      # what a kernel that only READS the same weight buffers reaches by the same measure
+                      "stream_read_frac_of_peak": round(lin_bytes / launches / read_avg_us / 1e3 / HBM_PEAK_GBS, 4),
+                      "matvec_time_over_stream_read_time": round(lin_us / launches / read_avg_us, 3)}}
 
 
 def calibration_copy(mib: int = 256, repeats: int = 3) -> None:
@@ -173,7 +249,8 @@ def main() -> int:
     toks = model.tokens()
     assert len(toks) == 1 + args.warmup + args.steps
 
-    roof = matvec_roofline(model)
+    roof = matvec_roofline(model, args.prompt + args.warmup + args.steps)
+    model.reset()
     calibration_copy()
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg, args.prompt)
 

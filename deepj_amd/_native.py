@@ -36,12 +36,13 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_floats.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_q8_floats.restype = C.c_int64
     lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
+    lib.deepj_hip_profile_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p, C.c_int32, _i32p]
     lib.deepj_hip_graph_capture.argtypes = [_i32p, C.c_int32, _i32p]
     lib.deepj_hip_graph_launch.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_graph_destroy.argtypes = [C.c_int32]
     for name in ("deepj_hip_init", "deepj_hip_alloc_buffers", "deepj_hip_upload", "deepj_hip_download",
                  "deepj_hip_release", "deepj_hip_flush_ops", "deepj_hip_flush_ops_noalloc", "deepj_hip_synchronize", "deepj_hip_shutdown",
-                 "deepj_hip_trim", "deepj_hip_pool_stats", "deepj_hip_time_ops", "deepj_hip_graph_capture",
+                 "deepj_hip_trim", "deepj_hip_pool_stats", "deepj_hip_time_ops", "deepj_hip_profile_ops", "deepj_hip_graph_capture",
                  "deepj_hip_graph_launch", "deepj_hip_graph_destroy"):
         getattr(lib, name).restype = C.c_int
 
@@ -149,6 +150,16 @@ class HipNative:
         ms = C.c_float()
         _check(library().deepj_hip_time_ops(cmd.ctypes.data_as(_i32p), cmd.size, iters, C.byref(ms)))
         return float(ms.value)
+
+    @staticmethod
+    def profileOps(cmd_stream, iters: int, max_ops: int = 4096) -> np.ndarray:
+        """Mean kernel duration (microseconds, start/stop events on each op's dispatch) of every op of the stream."""
+        cmd = _ids(cmd_stream)
+        out = np.empty(max_ops, dtype=np.float32)
+        n = C.c_int32()
+        _check(library().deepj_hip_profile_ops(cmd.ctypes.data_as(_i32p), cmd.size, iters,
+                                               out.ctypes.data_as(_f32p), max_ops, C.byref(n)))
+        return out[: n.value].copy()
 
     @staticmethod
     def graphCapture(cmd_stream) -> int:

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdint>
 #include <stdexcept>
@@ -35,6 +36,26 @@ inline int64_t q8_bytes(int k, int rows) {
     return q8_scale_offset_bytes(k, rows) + (int64_t)rows * (q8_padded_k(k) / kQ8Group) * 4;
 }
 
+// Per-kernel timing for deepj_hip_profile_ops: while `armed`, the next kernel that goes through launch_kernel()
+// is launched with a start and a stop event attached to that one dispatch (its begin and end time stamps on the
+// device, the quantity a kernel trace reports); every other launch is an ordinary one.
+struct LaunchTiming {
+    hipEvent_t start = nullptr, stop = nullptr;
+    bool armed = false;
+};
+extern LaunchTiming g_launch_timing;
+
+template <typename... Params, typename... Args>
+inline void launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, hipStream_t s, Args... args) {
+    if (g_launch_timing.armed) {
+        g_launch_timing.armed = false;
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, g_launch_timing.start, g_launch_timing.stop, 0,
+                              static_cast<Params>(args)...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<Params>(args)...);
+    }
+}
+
 // ── launchers (each validates nothing: the interpreter has already checked
 //    ids, sizes and shapes on the host before any of these is called) ──────
 
@@ -50,6 +71,9 @@ void launch_scatter_add(hipStream_t s, float *target, const float *idx, const fl
                         int cols, int n_idx);
 void launch_fill(hipStream_t s, uint32_t *dst, uint32_t bits, int64_t n);
 void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n);
+// measurement floors: a pure streaming read of n floats (nothing kept), and an empty kernel of `grid` workgroups
+void launch_stream_read(hipStream_t s, const float *src, float *sink, int64_t n);
+void launch_nop(hipStream_t s, int grid);
 void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n);
 void launch_append_rows(hipStream_t s, const float *src, float *dst, const int32_t *state, int rows, int row_floats,
                         int max_rows);

@@ -682,8 +682,8 @@ void launch_attn_decode_records(hipStream_t s, const float *qkv, float *k_cache,
     const float scale = (float)(1.0 / sqrt((double)hd));
     dim3 grid(H, kAttnRecordSplits);
     auto go = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, grid, dim3(kRecThreads), 0, s, state, k_cache, v_cache, qkv, cos_t, sin_t, max_seq, H,
-                           records, scale);
+        launch_kernel(kernel, grid, dim3(kRecThreads), 0, s, state, k_cache, v_cache, qkv, cos_t, sin_t, max_seq, H,
+                      records, scale);
     };
     switch (hd) {
         case 32: go(k_attn_decode_records<8>); break;

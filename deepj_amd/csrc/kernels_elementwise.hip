@@ -203,6 +203,29 @@ __global__ void __launch_bounds__(kThreads) k_fill(uint32_t *__restrict__ dst, u
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = bits;
 }
 
+// Measurement floor of the HBM-bound decode kernels: the same bytes read with 128-bit loads, eight in flight per
+// lane, nothing computed but an AND over the words (so that no load can be dropped) and nothing stored unless
+// every bit of the buffer is set.
+__global__ void __launch_bounds__(kThreads) k_stream_read(const uint4 *__restrict__ src, uint32_t *__restrict__ sink,
+                                                          int64_t n16, int64_t tail_from, const uint32_t *src_words,
+                                                          int64_t n_words) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint32_t acc = 0xffffffffu;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = src[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc &= v[u].x & v[u].y & v[u].z & v[u].w;
+    }
+    for (; i < n16; i += stride) { uint4 v = src[i]; acc &= v.x & v.y & v.z & v.w; }
+    for (int64_t j = tail_from + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n_words; j += stride) acc &= src_words[j];
+    if (acc == 0xffffffffu && n_words > 0 && src_words[0] == 0xffffffffu) sink[0] = acc;     // practically never
+}
+
+__global__ void k_nop() {}
+
 __global__ void __launch_bounds__(kThreads) k_copy(const float *__restrict__ src, float *__restrict__ dst, int64_t n) {
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
@@ -353,6 +376,20 @@ void launch_scatter_add(hipStream_t s, float *target, const float *idx, const fl
 void launch_fill(hipStream_t s, uint32_t *dst, uint32_t bits, int64_t n) {
     if (n <= 0) return;
     DJ_LAUNCH(k_fill, grid_for(n), kThreads, s, dst, bits, n);
+}
+
+void launch_stream_read(hipStream_t s, const float *src, float *sink, int64_t n) {
+    if (n <= 0) return;
+    const int64_t n16 = n / 4;
+    int64_t grid = (n16 + (int64_t)kThreads * 8 - 1) / ((int64_t)kThreads * 8);
+    if (grid > 768) grid = 768;            // three workgroups per CU, as the matvec
+    if (grid < 1) grid = 1;
+    launch_kernel(k_stream_read, dim3((int)grid), dim3(kThreads), 0, s, reinterpret_cast<const uint4 *>(src),
+                  reinterpret_cast<uint32_t *>(sink), n16, n16 * 4, reinterpret_cast<const uint32_t *>(src), n);
+}
+
+void launch_nop(hipStream_t s, int grid) {
+    launch_kernel(k_nop, dim3(grid < 1 ? 1 : grid), dim3(kThreads), 0, s);
 }
 
 void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n) {

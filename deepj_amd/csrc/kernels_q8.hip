@@ -488,11 +488,11 @@ void launch_mv(hipStream_t s, const MatvecArgs &a) {
     auto go = [&](auto pro_tag) {
         constexpr int PRO = decltype(pro_tag)::value;
         if (vec) {
-            hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, PRO, true>), dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
-                               a.scales, a.out, a.k, grid, a.n_out, a.rec_hd, a.gamma, a.bias, a.bias2, a.residual, a.beta);
+            launch_kernel(k_q8_matvec<NC, B, SW, MODE, PRO, true>, dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
+                          a.scales, a.out, a.k, grid, a.n_out, a.rec_hd, a.gamma, a.bias, a.bias2, a.residual, a.beta);
         } else if constexpr (B == 1 && MODE != 2) {
-            hipLaunchKernelGGL((k_q8_matvec<NC, B, SW, MODE, PRO, false>), dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
-                               a.scales, a.out, a.k, grid, a.n_out, a.rec_hd, a.gamma, a.bias, a.bias2, a.residual, a.beta);
+            launch_kernel(k_q8_matvec<NC, B, SW, MODE, PRO, false>, dim3(grid), dim3(kThreads), lds, s, a.x, a.wq,
+                          a.scales, a.out, a.k, grid, a.n_out, a.rec_hd, a.gamma, a.bias, a.bias2, a.residual, a.beta);
         } else {
             fail("q8_linear: no matvec kernel for this shape");     // launch_mv sends ragged K to B = 1
         }

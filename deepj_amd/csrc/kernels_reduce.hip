@@ -469,7 +469,7 @@ void launch_add_positions(hipStream_t s, float *x, const float *table, const int
 
 void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
                         const float *table, float *x, int vocab, int d, int n_positions) {
-    hipLaunchKernelGGL(k_decode_next, dim3(1), dim3(1024), 0, s, logits, state, tokens, capacity, table, x, vocab, d,
+    launch_kernel(k_decode_next, dim3(1), dim3(1024), 0, s, logits, state, tokens, capacity, table, x, vocab, d,
                        n_positions);
 }
 

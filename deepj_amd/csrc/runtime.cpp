@@ -24,6 +24,9 @@
 #include "dj_common.h"
 
 namespace dj {
+
+LaunchTiming g_launch_timing;
+
 namespace {
 
 struct Buffer {
@@ -220,6 +223,8 @@ int stride_of(int op) {
         case DJ_OP_LAYERNORM: return 7;
         case DJ_OP_ATTN_DECODE_RECORDS: return 12;
         case DJ_OP_ADD_POSITIONS: return 7;
+        case DJ_OP_STREAM_READ: return 4;
+        case DJ_OP_NOP: return 2;
         default: return -1;
     }
 }
@@ -732,6 +737,20 @@ void exec_one(Cursor &c) {
             if (run) launch_copy(s, a + so, o + dof, n);
             break;
         }
+        case DJ_OP_STREAM_READ: {
+            // [op, src, sink, n]: reads n floats of src and keeps nothing (sink holds >= 1 float)
+            int64_t n = w[3]; need_positive(op, "n", n);
+            const float *a = buf(w[1], n, op, "src");
+            float *o = buf(w[2], 1, op, "sink");
+            if (run) launch_stream_read(s, a, o, n);
+            break;
+        }
+        case DJ_OP_NOP: {
+            // [op, grid]: an empty kernel of `grid` workgroups of 256 threads
+            if (w[1] < 1 || w[1] > 65535) fail("OP_NOP: grid must be 1..65535");
+            if (run) launch_nop(s, w[1]);
+            break;
+        }
         case DJ_OP_FILL: {
             int64_t n = w[3]; need_positive(op, "n", n);
             float *o = buf(w[1], n, op, "dst");
@@ -806,6 +825,8 @@ const char *op_name(int op) {
         case DJ_OP_APPEND_ROWS: return "OP_APPEND_ROWS";
         case DJ_OP_Q8_LINEAR_DYN: return "OP_Q8_LINEAR_DYN";
         case DJ_OP_LLAMA_DECODE: return "OP_LLAMA_DECODE";
+        case DJ_OP_STREAM_READ: return "OP_STREAM_READ";
+        case DJ_OP_NOP: return "OP_NOP";
         default: return "OP_?";
     }
 }
@@ -1039,6 +1060,66 @@ int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms
         DJ_HIP(hipEventElapsedTime(ms_total, e0, e1));
         (void)hipEventDestroy(e0);
         (void)hipEventDestroy(e1);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) fail(std::string("kernel launch failed: ") + hipGetErrorString(e));
+    });
+}
+
+// Per-op kernel durations: every op of the stream is launched with a start and a stop event on its (first) kernel
+// dispatch, the stream runs `iters` times in order, and us_per_op[i] receives the mean begin-to-end time of op i's
+// kernel on the device in microseconds (-1 for an op none of whose launches can carry events).
+int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float *us_per_op, int32_t capacity,
+                          int32_t *n_ops) {
+    return guarded([&] {
+        ensure_init();
+        if (iters <= 0 || !us_per_op || capacity < 0) fail("profile_ops: bad arguments");
+        int64_t ws = 0;
+        walk(cmd, len, true, &ws);
+        ensure_workspace(ws);
+        std::vector<int32_t> starts;                 // word offset of every op
+        for (int32_t pos = 0; pos < len;) {
+            starts.push_back(pos);
+            int stride = stride_of(cmd[pos]);
+            pos += stride == 0 ? cmd[pos + 1] : stride;
+        }
+        const int n = (int)starts.size();
+        if (n_ops) *n_ops = n;
+        if (n > capacity) fail("profile_ops: the stream holds " + std::to_string(n) + " ops, the output only " + std::to_string(capacity));
+        std::vector<hipEvent_t> ev((size_t)2 * n, nullptr);
+        std::vector<double> sum((size_t)n, 0.0);
+        std::vector<int> count((size_t)n, 0);
+        auto cleanup = [&] {
+            g_launch_timing = LaunchTiming{};
+            for (hipEvent_t e : ev) if (e) (void)hipEventDestroy(e);
+        };
+        try {
+            for (auto &e : ev) DJ_HIP(hipEventCreate(&e));
+            for (int it = 0; it < iters; it++) {
+                std::vector<char> timed((size_t)n, 0);
+                for (int i = 0; i < n; i++) {
+                    Cursor c{cmd, len, starts[(size_t)i], false, 0};
+                    g_launch_timing.start = ev[(size_t)2 * i];
+                    g_launch_timing.stop = ev[(size_t)2 * i + 1];
+                    g_launch_timing.armed = true;
+                    exec_one(c);
+                    timed[(size_t)i] = !g_launch_timing.armed;
+                    g_launch_timing.armed = false;
+                }
+                DJ_HIP(hipStreamSynchronize(g.stream));
+                for (int i = 0; i < n; i++) {
+                    if (!timed[(size_t)i]) continue;
+                    float ms = 0.0f;
+                    DJ_HIP(hipEventElapsedTime(&ms, ev[(size_t)2 * i], ev[(size_t)2 * i + 1]));
+                    sum[(size_t)i] += (double)ms * 1e3;
+                    count[(size_t)i]++;
+                }
+            }
+        } catch (...) {
+            cleanup();
+            throw;
+        }
+        cleanup();
+        for (int i = 0; i < n; i++) us_per_op[i] = count[(size_t)i] ? (float)(sum[(size_t)i] / count[(size_t)i]) : -1.0f;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) fail(std::string("kernel launch failed: ") + hipGetErrorString(e));
     });

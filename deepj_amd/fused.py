@@ -140,6 +140,8 @@ class Stream:
 
     def copy(self, src, dst, n, src_off=0, dst_off=0): return self.emit(op.OP_COPY, src, dst, n, src_off, dst_off)
     def fill(self, dst, bits, n): return self.emit(op.OP_FILL, dst, bits, n)
+    def stream_read(self, src, sink, n): return self.emit(op.OP_STREAM_READ, src, sink, n)
+    def nop(self, grid=1): return self.emit(op.OP_NOP, grid)
     def matmul(self, a, b, out, m, n, k): return self.emit(op.OP_MATMUL, a, b, out, m, n, k)
 
     # execution -----------------------------------------------------------------
@@ -149,6 +151,10 @@ class Stream:
     def run(self) -> None:
         a = self.array()
         HipNative.nativeFlushOps(a, a.size)
+
+    def profile(self, iters: int) -> np.ndarray:
+        """Mean kernel duration of every op in microseconds (events on each op's own dispatch)."""
+        return HipNative.profileOps(self.array(), iters)
 
     def time(self, iters: int) -> float:
         """Milliseconds for `iters` back-to-back executions (HIP events on the library's stream)."""

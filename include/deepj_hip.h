@@ -84,6 +84,14 @@ void *deepj_hip_stream(void);
  * recorded on the library's stream; *ms_total receives the elapsed time. */
 int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total);
 
+/* Runs a validated stream `iters` times in order with a start and a stop event attached to each op's (first)
+ * kernel dispatch: us_per_op[i] receives the mean begin-to-end time of op i's kernel on the device, in
+ * microseconds - the duration a kernel trace reports for it (-1 for ops whose launches carry no events: every
+ * decode-path op does - Q8_LINEAR with M = 1, ATTN_DECODE_RECORDS, DECODE_NEXT, STREAM_READ, NOP).  *n_ops = ops in
+ * the stream; fails when capacity is smaller. */
+int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float *us_per_op, int32_t capacity,
+                          int32_t *n_ops);
+
 /* Captures a command stream into a HIP graph (no allocation may be pending:
  * every buffer it names must exist) and replays it.  Used for the per-token
  * decode stream, whose position and token live in device memory. */
@@ -179,13 +187,15 @@ enum {
      * ADD_POSITIONS [op, x, table, state, rows, d, maxSeq]
      *     x[i, :] += table[state[0] + i, :]: the learned positional rows of J/models/gpt/GPTModel.java:52-54 for
      *     rows that sit at positions state[0].. of the sequence
+     * STREAM_READ   [op, src, sink, n]    measurement floor: reads n floats of src with 128-bit loads and keeps nothing
+     * NOP           [op, grid]            measurement floor: an empty kernel of `grid` workgroups of 256 threads
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
     DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82, DJ_OP_LAYERNORM = 83,
-    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85
+    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85, DJ_OP_STREAM_READ = 86, DJ_OP_NOP = 87
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8, DJ_LIN_LAYERNORM = 16,

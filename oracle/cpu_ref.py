@@ -492,6 +492,8 @@ lib.ref_model_weight.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(_I), C.POINTE
 lib.ref_model_weight.restype = f32p
 lib.ref_model_forward.argtypes = [C.c_void_p, i32p, _I, f32p]
 lib.ref_model_forward.restype = _I
+lib.ref_model_hidden.argtypes = [C.c_void_p, i32p, _I, _I, f32p]
+lib.ref_model_hidden.restype = _I
 lib.ref_model_reset_cache.argtypes = [C.c_void_p]
 lib.ref_model_forward_cached.argtypes = [C.c_void_p, i32p, _I, f32p, _I]
 lib.ref_model_forward_cached.restype = _I
@@ -568,6 +570,15 @@ class Model:
             raise ValueError(f"seqLen {len(ids)} exceeds maxSeq {self.max_seq}")
         if rc != 0:
             raise ValueError("Token id out of range")
+        return out
+
+    def hidden(self, ids, n_layers: int) -> np.ndarray:
+        """The block stack's state after its first n_layers blocks, [len(ids) x d]: the input of block n_layers."""
+        ids = i32(ids)
+        out = np.empty((len(ids), self.d), dtype=np.float32)
+        rc = lib.ref_model_hidden(self._h, _ip(ids), len(ids), n_layers, _fp(out))
+        if rc != 0:
+            raise ValueError(f"hidden failed rc={rc}")
         return out
 
     def reset_cache(self):

@@ -487,6 +487,25 @@ static void gpt_forward(ref_model *m, float *x, float *h, float *a, float *x2, i
     ref_linear(h, m->wlm, m->blm, logits, n, d, c->vocab);
 }
 
+/* LlamaTransformerBlock.java:50-53 / DeepSeekTransformerBlock.java:54-57, the first n_layers blocks in order */
+static void run_blocks(ref_model *m, float *x, float *h, float *a, float *x2, int n, int n_layers) {
+    const ref_config *c = &m->cfg;
+    int d = c->d;
+    for (int l = 0; l < n_layers; l++) {
+        const ref_layer *L = &m->layer[l];
+        ref_rmsnorm(x, L->g1, h, n, d);
+        if (c->kind == 0)
+            ref_mhsa_forward(h, L->wq, L->wk, L->wv, L->wo, a, n, d, c->heads, m->cos_t, m->sin_t, 1);
+        else
+            ref_mla_forward(h, L->wdq, L->wuq, L->wdkv, L->wuk, L->wuv, L->wo, a, n, d, c->heads,
+                            c->q_rank, c->kv_rank, m->cos_t, m->sin_t);
+        ref_add(x, a, x2, n, d);
+        ref_rmsnorm(x2, L->g2, h, n, d);
+        ref_swiglu(h, L->wg, L->bg, L->wu, L->bu, L->wd, L->bd, a, n, d, c->dff);
+        ref_add(x2, a, x, n, d);
+    }
+}
+
 /* DecoderOnlyModel.java:58-64 with Llama/DeepSeek blocks */
 int ref_model_forward(ref_model *m, const int32_t *ids, int n, float *logits) {
     const ref_config *c = &m->cfg;
@@ -500,21 +519,25 @@ int ref_model_forward(ref_model *m, const int32_t *ids, int n, float *logits) {
         free(x); free(h); free(a); free(x2);
         return 0;
     }
-    for (int l = 0; l < c->layers; l++) {
-        const ref_layer *L = &m->layer[l];
-        ref_rmsnorm(x, L->g1, h, n, d);
-        if (c->kind == 0)
-            ref_mhsa_forward(h, L->wq, L->wk, L->wv, L->wo, a, n, d, c->heads, m->cos_t, m->sin_t, 1);
-        else
-            ref_mla_forward(h, L->wdq, L->wuq, L->wdkv, L->wuk, L->wuv, L->wo, a, n, d, c->heads,
-                            c->q_rank, c->kv_rank, m->cos_t, m->sin_t);
-        ref_add(x, a, x2, n, d);
-        ref_rmsnorm(x2, L->g2, h, n, d);
-        ref_swiglu(h, L->wg, L->bg, L->wu, L->bu, L->wd, L->bd, a, n, d, c->dff);
-        ref_add(x2, a, x, n, d);
-    }
+    run_blocks(m, x, h, a, x2, n, c->layers);
     ref_rmsnorm(x, m->gf, h, n, d);
     ref_linear(h, m->wlm, m->blm, logits, n, d, c->vocab);
+    free(x); free(h); free(a); free(x2);
+    return 0;
+}
+
+/* The block stack's state after its first n_layers blocks (TransformerStack.java:28-35 stopped early), [n x d]:
+ * the input the next block sees.  Llama / DeepSeek only.  Test infrastructure: lets a test feed one block of a deep
+ * model the exact input the CPU path gives it. */
+int ref_model_hidden(ref_model *m, const int32_t *ids, int n, int n_layers, float *x_out) {
+    const ref_config *c = &m->cfg;
+    int d = c->d;
+    int64_t nd = (int64_t)n * d;
+    if (c->kind == 2 || n_layers < 0 || n_layers > c->layers) return -3;
+    float *x = falloc(nd), *h = falloc(nd), *a = falloc(nd), *x2 = falloc(nd);
+    if (embed(m, ids, n, x) != 0) { free(x); free(h); free(a); free(x2); return -1; }
+    run_blocks(m, x, h, a, x2, n, n_layers);
+    memcpy(x_out, x, (size_t)nd * sizeof(float));
     free(x); free(h); free(a); free(x2);
     return 0;
 }

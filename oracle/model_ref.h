@@ -119,6 +119,8 @@ float     *ref_model_weight(ref_model *m, const char *name, int *rows, int *cols
 
 /* DecoderOnlyModel.forward: logits [n x vocab] for the whole context. Returns 0, or -1 on a bad id. */
 int ref_model_forward(ref_model *m, const int32_t *ids, int n, float *logits);
+/* x after the first n_layers blocks, [n x d] (Llama / DeepSeek); -1 bad token id, -3 bad layer count or GPT */
+int ref_model_hidden(ref_model *m, const int32_t *ids, int n, int n_layers, float *x_out);
 /* Incremental: appends n rows after the m->cached rows already seen; logits [n x vocab]
  * (or only the last row when last_only != 0: logits [1 x vocab]). */
 void ref_model_reset_cache(ref_model *m);

@@ -73,11 +73,23 @@ def build(name):
     return LlamaModel(cfg, c["seed"]), c
 
 
+def logit_gate(name):
+    """Max-abs gate for GPU-vs-oracle logits of a full-size fixture: the baseline's 1e-3 wherever the oracle itself is
+    well inside it relative to float64 (fixture "fp64_step0": 2e-4 for "c5" and "g2"), FULL_SIZE_LOGIT_ATOL where the
+    oracle's own fp32 arithmetic is already further than 1e-3 from exact ("c3": 3.4e-3, "c4")."""
+    f = GOLD[name].get("fp64_step0")
+    if f and f["oracle_max_abs_err_all_cols"] <= 2.5e-4:
+        return 1e-3
+    return FULL_SIZE_LOGIT_ATOL
+
+
 @pytest.mark.parametrize("name", ["c3", "c4", "c5", "g2"])
 def test_full_size_greedy_tokens_and_logits_match_oracle_fixture(name):
     if name not in GOLD:
         pytest.skip(f"no fixture for {name} (run tests/golden/make_model_goldens.py {name})")
     g = GOLD[name]
+    assert "fp64_step0" in g, "every full-size fixture carries the float64 probe that justifies its logit gate"
+    FULL_SIZE_LOGIT_ATOL = logit_gate(name)      # noqa: N806 - shadows the module default for this configuration
     model, c = build(name)
     try:
         prompt = JavaRandom(c["prompt_seed"]).ints(c["prompt_len"], c["model"]["vocab"])
@@ -95,7 +107,8 @@ def test_full_size_greedy_tokens_and_logits_match_oracle_fixture(name):
             exact, cpu = np.array(f["fp64"]), np.array(f["oracle_fp32"])
             gpu_err = float(np.max(np.abs(l0[f["cols"]] - exact)))
             cpu_err = float(np.max(np.abs(cpu - exact)))
-            print(f"\n[{name}] max-abs error vs float64 on {len(exact)} logits: GPU {gpu_err:.2e}, CPU oracle {cpu_err:.2e}")
+            print(f"\n[{name}] max-abs error vs float64 on {len(exact)} logits: GPU {gpu_err:.2e}, CPU oracle {cpu_err:.2e}; "
+                  f"GPU vs oracle {float(np.max(np.abs(l0[f['cols']] - cpu))):.2e} (gate {FULL_SIZE_LOGIT_ATOL:g})")
             assert gpu_err <= 1.25 * cpu_err + 1e-4
             assert float(np.max(np.abs(l0[f["cols"]] - cpu))) <= FULL_SIZE_LOGIT_ATOL
         # greedy generation through the captured graph
@@ -118,3 +131,161 @@ def test_full_size_greedy_tokens_and_logits_match_oracle_fixture(name):
             assert float(np.max(np.abs(model.lastLogits() - full[t]))) <= FULL_SIZE_LOGIT_ATOL
     finally:
         model.close()
+
+
+# ── the DeepSeek configuration exactly as stated: reference initialisation, nothing scaled ─────────────────────
+#
+# At this width the reference's initialiser (N(0,1) * 0.1) gives attention scores with a standard deviation near 150:
+# every softmax row is a hard arg-max, a near-tie between the two best keys flips with the summation order, and one
+# flip replaces a whole value row.  The fixture's float64 probe measures the consequence on the CPU side alone: the
+# oracle's fp32 logits of the last prompt row are 4.8 (max-abs; 1.2 rms, logits of +-20) away from the float64 value,
+# and a second fp32 evaluation in numpy's summation order is 4.3 away from the oracle.  "Token-identical to the CPU
+# path" is therefore not a property any other summation order can have at this initialisation - two CPU orders do not
+# have it either - and the model is checked in the ways that stay meaningful:
+#   * end to end: GPU-vs-float64 distance no larger than the CPU path's own (x1.25); greedy ids identical to the
+#     oracle's under teacher forcing up to the first step whose oracle top-1/top-2 gap is below the measured
+#     GPU-vs-oracle distance (that step is reported); graph replay == eager (bit-identical kernels);
+#   * block by block: every tested block of the 16, fed the oracle's own input to that block, agrees with the oracle
+#     (prefill rows and cached decode rows) - the check that does not compound.
+
+def seeded_deepseek_weights(cfg, seed):
+    """The parameters of new DeepSeekModel(cfg, seed) by name (DeepSeekModel.java:31-47, draw order of
+    DeepSeekTransformerBuilder.java:56-68), from the java.util.Random twin."""
+    emb_r, stack_r, head_r = JavaRandom(seed), JavaRandom(seed), JavaRandom(seed + 1)
+    d = cfg.dModel
+    w = {"emb": emb_r.tensor(cfg.vocabSize, d)}
+    shapes = dict(wdq=(d, cfg.qRank), wuq=(cfg.qRank, d), wdkv=(d, cfg.kvRank), wuk=(cfg.kvRank, d),
+                  wuv=(cfg.kvRank, d), wo=(d, d), wg=(d, cfg.dFF), wu=(d, cfg.dFF), wd=(cfg.dFF, d))
+    for l in range(cfg.nLayers):
+        w[f"L{l}.g1"] = np.ones((1, d), np.float32)
+        w[f"L{l}.g2"] = np.ones((1, d), np.float32)
+        for name, (r, c) in shapes.items():
+            w[f"L{l}.{name}"] = stack_r.tensor(r, c)
+        for b, n in (("bg", cfg.dFF), ("bu", cfg.dFF), ("bd", d)):
+            w[f"L{l}.{b}"] = np.zeros((1, n), np.float32)
+    w["gf"] = np.ones((1, d), np.float32)
+    w["wlm"] = head_r.tensor(d, cfg.vocabSize)
+    w["blm"] = np.zeros((1, cfg.vocabSize), np.float32)
+    return w
+
+
+def test_deepseek_at_the_stated_init_end_to_end():
+    name = "c5_ref_init"
+    if name not in GOLD or "fp64_step0" not in GOLD[name]:
+        pytest.skip("no fixture (run tests/golden/make_model_goldens.py c5_ref_init and make_fp64_probe.py c5_ref_init)")
+    g, f = GOLD[name], GOLD[name]["fp64_step0"]
+    model, c = build(name)
+    try:
+        prompt = JavaRandom(c["prompt_seed"]).ints(c["prompt_len"], c["model"]["vocab"])
+        assert [int(x) for x in prompt[:8]] == g["prompt_head"]
+        exp = np.array(g["tokens"], dtype=np.int32)
+        # step 0 against float64 and against the oracle
+        model.reset()
+        model.prefill(prompt, choose_next=False)
+        l0 = model.lastLogits()
+        exact, cpu = np.array(f["fp64"]), np.array(f["oracle_fp32"])
+        gpu_err = float(np.max(np.abs(l0[f["cols"]] - exact)))
+        cpu_err = float(np.max(np.abs(cpu - exact)))
+        dist = float(np.max(np.abs(l0[f["cols"]] - cpu)))
+        print(f"\n[{name}] step 0, max-abs over {len(exact)} logits: GPU vs float64 {gpu_err:.3f}, oracle vs float64 "
+              f"{cpu_err:.3f} (all columns {f['oracle_max_abs_err_all_cols']:.3f}; a second CPU fp32 order "
+              f"{f['alt_fp32_max_abs_err_all_cols']:.3f}), GPU vs oracle {dist:.3f}")
+        assert np.all(np.isfinite(l0))
+        assert gpu_err <= 1.25 * max(cpu_err, f["oracle_max_abs_err_all_cols"])
+        # teacher forcing: the GPU sees the oracle's tokens; its arg-max may leave the oracle's only at a step whose
+        # oracle gap is below the measured distance
+        first_part, agree = None, 0
+        for t, (i1, l1, i2, l2) in enumerate(g["steps"]):
+            if t > 0:
+                model.step(int(exp[t - 1]))
+            same = int(np.argmax(model.lastLogits())) == i1
+            agree += same
+            if not same and first_part is None:
+                first_part = t
+                assert l1 - l2 < dist, (f"step {t}: the GPU leaves the oracle's token although the oracle's top-1/top-2 "
+                                        f"gap {l1 - l2:.3f} exceeds the GPU-vs-oracle logit distance {dist:.3f}")
+        print(f"[{name}] teacher-forced arg-max equals the oracle's at {agree} of {len(exp)} steps; first parting at step "
+              f"{first_part} (oracle gap there {g['steps'][first_part][1] - g['steps'][first_part][3]:.3f})"
+              if first_part is not None else f"[{name}] all {len(exp)} teacher-forced steps agree")
+        # the GPU's own greedy sequence: graph replay and eager launches run the same kernels on the same data
+        a = TextGenerator.generate(model, prompt, 24, top_k=1, use_graph=True)
+        b = TextGenerator.generate(model, prompt, 24, top_k=1, use_graph=False)
+        assert np.array_equal(a, b)
+        # decode row against prefill row: two GPU summation orders (matvec and GEMM kernels) of a model whose CPU
+        # orders are O(1) apart; reported, and bounded by the CPU path's own distance from float64
+        ids = np.concatenate([prompt[:40], exp[:3]])
+        full = model.forward(ids)
+        model.reset()
+        model.prefill(ids[:40], choose_next=False)
+        worst = 0.0
+        for t in range(40, 43):
+            model.step(int(ids[t]))
+            worst = max(worst, float(np.max(np.abs(model.lastLogits() - full[t]))))
+        print(f"[{name}] decode row vs prefill row at full depth: max-abs {worst:.3f}")
+        assert worst <= 1.25 * f["oracle_max_abs_err_all_cols"]
+    finally:
+        model.close()
+
+
+@pytest.mark.parametrize("layer", range(16))
+def test_deepseek_at_the_stated_init_block_by_block(layer, stated_init):
+    """Block `layer` of the 16-block model at the stated initialisation, fed the oracle's own input to that block:
+    a one-block GPU model whose embedding table holds those input rows against a one-block oracle with the same
+    weights.  Prefill rows (GEMM kernels) and cached decode rows (matvec kernels, KV cache)."""
+    from oracle import cpu_ref as ref
+    cfg, w, cpu16, ids = stated_init
+    S, d = len(ids), cfg.dModel
+    x_in = cpu16.hidden(ids, layer)                                  # [S x d], what block `layer` sees on the CPU
+    one = DeepSeekConfig(S, S, d, cfg.nHeads, 1, cfg.dFF, cfg.qRank, cfg.kvRank)     # vocabulary = the S input rows
+    names = ("g1", "g2", "wdq", "wuq", "wdkv", "wuk", "wuv", "wo", "wg", "bg", "wu", "bu", "wd", "bd")
+    head = np.ascontiguousarray(w["wlm"][:, :S])
+    gpu = DeepSeekModel(one, None)
+    cpu = ref.Model(vocab=S, max_seq=S, d=d, heads=cfg.nHeads, layers=1, dff=cfg.dFF, seed=1, q_rank=cfg.qRank,
+                    kv_rank=cfg.kvRank, timing_only_fill=True)
+    try:
+        for n in names:
+            gpu.setWeight(f"L0.{n}", w[f"L{layer}.{n}"])
+            cpu.weight(f"L0.{n}")[...] = w[f"L{layer}.{n}"]
+        for n, v in (("emb", x_in), ("gf", w["gf"]), ("wlm", head), ("blm", np.zeros((1, S), np.float32))):
+            gpu.setWeight(n, v)
+            cpu.weight(n)[...] = v
+        gpu.finalize()
+        cpu.q8_roundtrip()
+        rows = np.arange(S, dtype=np.int32)
+        exp = cpu.forward(rows)
+        got = gpu.forward(rows)
+        err = float(np.max(np.abs(got - exp)))
+        scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+        gpu.reset()
+        gpu.prefill(rows[:S - 4], choose_next=False)
+        derr = 0.0
+        for t in range(S - 4, S):
+            gpu.step(int(rows[t]))
+            derr = max(derr, float(np.max(np.abs(gpu.lastLogits() - exp[t]))))
+        print(f"\n[c5 stated init, block {layer}] input rms {float(np.sqrt(np.mean(x_in.astype(np.float64) ** 2))):.2f}, "
+              f"logit rms {scale:.2f}: prefill rows max-abs {err:.2e}, decode rows {derr:.2e}")
+        assert err <= 1e-3 and derr <= 1e-3              # the baseline's logit tolerance
+    finally:
+        gpu.close()
+        cpu.close()
+
+
+@pytest.fixture(scope="module")
+def stated_init():
+    """The 16-block DeepSeek model of the baseline at its stated initialisation on the CPU oracle (weights from the
+    java.util.Random twin, which tests/test_host_random.py pins bit for bit to the oracle's), and a 48-token prompt."""
+    from oracle import cpu_ref as ref
+    m = GOLD["c5_ref_init"]["config"]["model"] if "c5_ref_init" in GOLD else dict(
+        vocab=32000, max_seq=512, d=2048, heads=16, layers=16, dff=5632, q_rank=1024, kv_rank=512)
+    cfg = DeepSeekConfig(m["vocab"], m["max_seq"], m["d"], m["heads"], m["layers"], m["dff"], m["q_rank"], m["kv_rank"])
+    w = seeded_deepseek_weights(cfg, 42)
+    ref.set_threads(ref.default_threads())
+    cpu16 = ref.Model(vocab=cfg.vocabSize, max_seq=cfg.maxSeqLen, d=cfg.dModel, heads=cfg.nHeads, layers=cfg.nLayers,
+                      dff=cfg.dFF, seed=42, q_rank=cfg.qRank, kv_rank=cfg.kvRank, timing_only_fill=True)
+    for n in cpu16.weight_names():
+        cpu16.weight(n)[...] = w[n]
+    cpu16.q8_roundtrip()
+    ids = JavaRandom(5).ints(48, cfg.vocabSize)
+    yield cfg, w, cpu16, ids
+    cpu16.close()
+    ref.set_threads(1)
