@@ -41,8 +41,10 @@ float deepj_host_random_next_float(void *h);
 namespace {
 
 struct Config {
-    int32_t kind;       // 0 Llama, 1 DeepSeek (MLA), 2 GPT
+    int32_t kind;       // 0 Llama, 1 DeepSeek (MLA), 2 GPT; DeepSeek with the latent KV cache arrives as kind 3 and
+                        // is kept here as kind 1 with `latent` set
     int32_t vocab, max_seq, d, heads, layers, dff, q_rank, kv_rank;
+    bool latent = false;
 };
 
 struct Error : std::runtime_error { using std::runtime_error::runtime_error; };
@@ -57,13 +59,15 @@ struct Layer {
     int32_t g1 = -1, g2 = -1, be1 = -1, be2 = -1;     // be*: LayerNorm betas (GPT)
     int32_t wqkv = -1, wo = -1;                       // Llama: fused [3d x d]
     int32_t wdown = -1, wup = -1;                     // MLA: stacked down-projections, block up-projection
+    int32_t wdq = -1, wuq = -1, wdkv = -1, wukv = -1; // MLA with the latent cache: Wdq, Wuq, Wdkv, and [Wuk | Wuv] by output row
     int32_t wgu = -1, bg = -1, bu = -1, wd = -1, bd = -1;
 };
 
 struct Acts {          // activation buffers for S rows
     int32_t rows = 0;
     int32_t x = -1, x2 = -1, qkv = -1, q = -1, att = -1, ff = -1, ids = -1;
-    int32_t cq = -1;                                                 // MLA: [cQ | pad | cKV] rows
+    int32_t cq = -1;                                                 // MLA: [cQ | pad | cKV] rows (latent cache: cQ rows)
+    int32_t ckv = -1;                                                // MLA with the latent cache: cKV rows
 };
 
 struct Runner {
@@ -76,6 +80,7 @@ struct Runner {
     int32_t cos_t = -1, sin_t = -1, kc = -1, vc = -1;
     int32_t state = -1, tokens = -1, scratch = -1, logits = -1, last_x = -1;
     int32_t records = -1;                                  // decode attention records (merged by the Wo matvec)
+    int32_t latent = -1, kv_all = -1;                      // latent cache [L][maxSeq][kvRank]; re-expanded [maxSeq][K | V] of one layer
     int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
     int64_t p_sync_floats = 0;
     bool p_pending = false;                                // a persistent launch has not been checked yet
@@ -169,6 +174,14 @@ void set_weight(Runner &r, const std::string &name, const float *data, int rows,
             expect_shape(name, rows, cols, d, d);
             int part = w == "wq" ? 0 : (w == "wk" ? 1 : 2);
             quantize_into(r, L.wqkv, data, d, d, part * d, 1, 3 * d);
+        }
+        else if (c.latent && w == "wdq") { expect_shape(name, rows, cols, d, c.q_rank); quantize_into(r, L.wdq, data, d, c.q_rank, 0, 1, c.q_rank); }
+        else if (c.latent && w == "wuq") { expect_shape(name, rows, cols, c.q_rank, d); quantize_into(r, L.wuq, data, c.q_rank, d, 0, 1, d); }
+        else if (c.latent && w == "wdkv") { expect_shape(name, rows, cols, d, c.kv_rank); quantize_into(r, L.wdkv, data, d, c.kv_rank, 0, 1, c.kv_rank); }
+        else if (c.latent && (w == "wuk" || w == "wuv")) {
+            // Q8 rows [0, d) = the columns of Wuk, [d, 2d) = those of Wuv: one product re-expands a latent row to [K | V]
+            expect_shape(name, rows, cols, c.kv_rank, d);
+            quantize_into(r, L.wukv, data, c.kv_rank, d, w == "wuk" ? 0 : d, 1, 2 * d);
         }
         else if (c.kind == 1 && (w == "wdq" || w == "wdkv")) {
             // output rows [0, qRank) = Wdq, [qRankPadded, +kvRank) = Wdkv; the pad rows stay zero (the buffer is
@@ -290,12 +303,13 @@ void init_seeded(Runner &r, int64_t seed, int threads, float init_scale) {
 void alloc_acts(Runner &r, Acts &a, int rows) {
     const Config &c = r.cfg;
     if (a.rows >= rows) return;
-    for (int32_t *id : {&a.x, &a.x2, &a.qkv, &a.q, &a.att, &a.ff, &a.ids, &a.cq}) r.release(*id);
+    for (int32_t *id : {&a.x, &a.x2, &a.qkv, &a.q, &a.att, &a.ff, &a.ids, &a.cq, &a.ckv}) r.release(*id);
     int64_t S = rows, d = c.d;
     a.x = r.alloc(S * d); a.x2 = r.alloc(S * d); a.q = r.alloc(S * d); a.att = r.alloc(S * d);
     a.ff = r.alloc(S * c.dff); a.ids = r.alloc(std::max<int64_t>(S, 4));
     a.qkv = r.alloc(S * 3 * d);
-    if (c.kind == 1) a.cq = r.alloc(S * r.latent_width());
+    if (c.latent) { a.cq = r.alloc(S * c.q_rank); a.ckv = r.alloc(S * c.kv_rank); }
+    else if (c.kind == 1) a.cq = r.alloc(S * r.latent_width());
     a.rows = rows;
 }
 
@@ -325,8 +339,16 @@ void finalize(Runner &r) {
     // be cached instead (kvRank floats per token rather than 2*dModel), but the reference rotates K after the
     // up-projection (MultiHeadLatentAttention.java:108-112), so the up-projection cannot be folded into the query
     // and every step would have to re-expand and re-rotate all cached positions.
-    r.kc = r.alloc(per_layer * c.layers);
-    r.vc = r.alloc(per_layer * c.layers);
+    if (c.latent) {
+        // The latent cache (MultiHeadLatentAttention.java:98-106 computes K and V from cKV = x.Wdkv): kvRank floats per
+        // token and layer instead of 2 * dModel.  Every step re-expands the layer's cached rows to [K | V] and rotates
+        // K (the reference rotates K after the up-projection, :108-112), into ONE buffer all layers take turns with.
+        r.latent = r.alloc((int64_t)c.layers * c.max_seq * c.kv_rank);
+        r.kv_all = r.alloc((int64_t)c.max_seq * 2 * c.d);
+    } else {
+        r.kc = r.alloc(per_layer * c.layers);
+        r.vc = r.alloc(per_layer * c.layers);
+    }
     r.state = r.alloc(4);
     r.tokens = r.alloc(c.max_seq);
     r.logits = r.alloc(c.vocab);
@@ -365,7 +387,23 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
     // GPT: LayerNorm instead of RMSNorm and no rotation                  GPTTransformerBlock.java:66-68
     // DeepSeek: [Q|K|V] = ([cQ|cKV] = norm1(x).[Wdq|Wdkv]) . blockdiag(Wuq, [Wuk|Wuv])   MultiHeadLatentAttention.java:92-123
-    if (c.kind == 1) {
+    if (c.latent) {
+        // cQ = norm1(x).Wdq, Q = cQ.Wuq, cKV = norm1(x).Wdkv appended to the layer's latent rows; then, for ALL
+        // cached positions, [K | V] = cKV.[Wuk | Wuv] (the row count lives on the device), RoPE on the K halves and
+        // on Q, attention over the token-major rows (MultiHeadLatentAttention.java:92-123).
+        const int qr = c.q_rank, kvr = c.kv_rank;
+        const int64_t lat_off = (int64_t)l * c.max_seq * kvr;
+        q8_linear(s, a.x, L.wdq, a.cq, S, d, qr, DJ_LIN_RMSNORM, L.g1);
+        q8_linear(s, a.cq, L.wuq, a.qkv, S, qr, d, 0);
+        q8_linear(s, a.x, L.wdkv, a.ckv, S, d, kvr, DJ_LIN_RMSNORM, L.g1);
+        emit(s, DJ_OP_APPEND_ROWS, a.ckv, r.latent, r.state, S, kvr, c.max_seq, lat_off);
+        emit(s, DJ_OP_Q8_LINEAR_DYN, r.latent, L.wukv, r.kv_all, c.max_seq, kvr, 2 * d, r.state, S, lat_off);
+        emit(s, DJ_OP_ROPE_ROWS, r.kv_all, r.kv_all, r.state, r.cos_t, r.sin_t, c.max_seq, H, hd, c.max_seq, 1, 2 * d, S);
+        emit(s, DJ_OP_ROPE_ROWS, a.qkv, a.q, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, 0, 0, -1);
+        emit(s, DJ_OP_ATTENTION_KV, a.q, r.kv_all, r.kv_all, a.att, r.state, r.scratch, S, H, hd, c.max_seq, 0, 2 * d, d);
+        q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);
+        wo_done = true;
+    } else if (c.kind == 1) {
         const int k2 = r.latent_width();
         q8_linear(s, a.x, L.wdown, a.cq, S, d, k2, DJ_LIN_RMSNORM, L.g1);
         q8_linear(s, a.cq, L.wup, a.qkv, S, k2, 3 * d, 0);
@@ -374,7 +412,9 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     } else {
         q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
     }
-    if (S == 1 && &a == &r.dec) {
+    if (c.latent) {
+        // attention and Wo were emitted above
+    } else if (S == 1 && &a == &r.dec) {
         // the key splits' records go straight to the Wo matvec, whose prologue merges them
         emit(s, DJ_OP_ATTN_DECODE_RECORDS, a.qkv, r.kc, r.vc, r.records, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
         emit(s, DJ_OP_Q8_LINEAR, r.records, L.wo, a.x2, 1, d, d, DJ_LIN_RESIDUAL | DJ_LIN_ATTN_MERGE, hd, -1, -1, a.x);
@@ -707,6 +747,7 @@ extern "C" {
 // runner may use (pick a range the ComputeGraph never reaches, e.g. 1 << 29).
 void *deepj_runner_create(const int32_t cfg[9], int32_t id_base) {
     Config c{cfg[0], cfg[1], cfg[2], cfg[3], cfg[4], cfg[5], cfg[6], cfg[7], cfg[8]};
+    if (c.kind == 3) { c.kind = 1; c.latent = true; }      // DeepSeek with the latent KV cache
     // TransformerConfig.validateCommon (models/TransformerConfig.java:19-31) + DeepSeekConfig.java:31-35
     if (c.vocab <= 0 || c.max_seq <= 0 || c.d <= 0 || c.heads <= 0 || c.layers <= 0 || c.dff <= 0) return nullptr;
     if (c.d % c.heads != 0) return nullptr;
@@ -731,13 +772,15 @@ void deepj_runner_destroy(void *h) {
     std::vector<int32_t> ids;
     auto add = [&](int32_t id) { if (id >= 0) ids.push_back(id); };
     for (auto &L : r->layers)
-        for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdown, L.wup, L.wgu, L.bg, L.bu, L.wd, L.bd}) add(id);
+        for (int32_t id : {L.g1, L.g2, L.be1, L.be2, L.wqkv, L.wo, L.wdown, L.wup, L.wdq, L.wuq, L.wdkv, L.wukv, L.wgu, L.bg,
+                           L.bu, L.wd, L.bd})
+            add(id);
     for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->state,
                        r->tokens, r->scratch, r->records, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
-                       r->pos_table, r->bf})
+                       r->pos_table, r->bf, r->latent, r->kv_all})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
-        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq}) add(id);
+        for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv}) add(id);
     if (!ids.empty()) deepj_hip_release(ids.data(), (int32_t)ids.size());
     delete r;
 }

@@ -155,11 +155,13 @@ _next_id_base = [1 << 29]
 
 
 class _DecoderOnlyModel:
-    def __init__(self, cfg, seed: int | None, threads: int = 0):
+    def __init__(self, cfg, seed: int | None, threads: int = 0, latent_cache: bool = False):
         _validate(cfg)
         self.cfg = cfg
         kind = 1 if isinstance(cfg, DeepSeekConfig) else (2 if isinstance(cfg, GPTConfig) else 0)
-        arr = (C.c_int32 * 9)(kind, cfg.vocabSize, cfg.maxSeqLen, cfg.dModel, cfg.nHeads, cfg.nLayers, cfg.dFF,
+        if latent_cache and kind != 1:
+            raise ValueError("the latent KV cache belongs to the DeepSeek (MLA) model")
+        arr = (C.c_int32 * 9)(3 if latent_cache else kind, cfg.vocabSize, cfg.maxSeqLen, cfg.dModel, cfg.nHeads, cfg.nLayers, cfg.dFF,
                               getattr(cfg, "qRank", 0), getattr(cfg, "kvRank", 0))
         base = _next_id_base[0]
         _next_id_base[0] += 1 << 20
@@ -259,10 +261,12 @@ class LlamaModel(_DecoderOnlyModel):
 
 
 class DeepSeekModel(_DecoderOnlyModel):
-    """new DeepSeekModel(cfg, seed) (DeepSeekModel.java:29-46)."""
+    """new DeepSeekModel(cfg, seed) (DeepSeekModel.java:29-46).  latent_cache: keep cKV (kvRank floats per token and
+    layer) instead of the rotated K and V (2 * dModel) and re-expand it every step - eight times less cache at the
+    README's ranks, at the price of a [context x kvRank] x [kvRank x 2 dModel] product per layer and token."""
 
-    def __init__(self, cfg: DeepSeekConfig, seed: int | None = 42, threads: int = 0):
-        super().__init__(cfg, seed, threads)
+    def __init__(self, cfg: DeepSeekConfig, seed: int | None = 42, threads: int = 0, latent_cache: bool = False):
+        super().__init__(cfg, seed, threads, latent_cache)
 
 
 class GPTModel(_DecoderOnlyModel):

@@ -226,8 +226,11 @@ float   deepj_host_random_next_float(void *rng);
  * TextGenerator of the reference (J/models/DecoderOnlyModel.java:58-64,
  * J/models/TextGenerator.java:66-181) with a device-resident KV cache, Q8 weights and one
  * fused command stream per token replayed as a HIP graph.  It uses only the functions
- * above.  cfg = {kind (0 Llama, 1 DeepSeek, 2 GPT), vocab, maxSeq, dModel, nHeads, nLayers, dFF,
- * qRank, kvRank}; id_base = first buffer id the runner may use.  Weight names: "emb",
+ * above.  cfg = {kind (0 Llama, 1 DeepSeek, 2 GPT, 3 DeepSeek with the latent KV cache), vocab, maxSeq, dModel,
+ * nHeads, nLayers, dFF, qRank, kvRank}; id_base = first buffer id the runner may use.  Kind 1 caches the rotated
+ * K and V of every position (2 * dModel floats per token and layer) like the Llama path; kind 3 caches the MLA
+ * latent rows cKV = norm(x).Wdkv (kvRank floats per token and layer, J/layers/transformer/attention/
+ * MultiHeadLatentAttention.java:98-106) and re-expands and re-rotates them every step - less memory, more work.  Weight names: "emb",
  * "gf", "wlm", "blm", "L<i>.g1|g2|wq|wk|wv|wo|wdq|wuq|wdkv|wuk|wuv|wg|bg|wu|bu|wd|bd";
  * GPT (J/models/gpt/GPTModel.java:27-45, J/layers/transformer/blocks/GPTTransformerBlock.java:52-73) adds
  * "pos" [maxSeq x dModel], "bf" and "L<i>.be1|be2" (LayerNorm betas; g1, g2, gf are the gammas), names its

@@ -33,11 +33,11 @@ FULL_SIZE_LOGIT_ATOL = 5e-3
 MLA_PROJECTIONS = ("wdq", "wuq", "wdkv", "wuk", "wuv")
 
 
-def seeded_deepseek_with_scaled_mla(cfg, seed, scale):
+def seeded_deepseek_with_scaled_mla(cfg, seed, scale, latent_cache=False):
     """new DeepSeekModel(cfg, seed) (DeepSeekModel.java:31-47: embedding from Random(seed), the block
     stack from its own Random(seed), the LM head from Random(seed+1); Tensor.random = N(0,1)*0.1) with the
     five MLA projection matrices multiplied by `scale`, loaded through setWeight."""
-    model = DeepSeekModel(cfg, None)
+    model = DeepSeekModel(cfg, None, latent_cache=latent_cache)
     emb_r, stack_r, head_r = JavaRandom(seed), JavaRandom(seed), JavaRandom(seed + 1)
     d = cfg.dModel
     model.setWeight("emb", emb_r.tensor(cfg.vocabSize, d))
@@ -129,6 +129,28 @@ def test_full_size_greedy_tokens_and_logits_match_oracle_fixture(name):
         for t in range(40, 43):
             model.step(int(ids[t]))
             assert float(np.max(np.abs(model.lastLogits() - full[t]))) <= FULL_SIZE_LOGIT_ATOL
+    finally:
+        model.close()
+
+
+def test_full_size_deepseek_with_the_latent_cache_matches_the_fixture():
+    """The "c5" fixture again with cKV cached instead of K and V (runner kind 3): step-0 logits inside the same
+    gate, the 64 greedy tokens identical."""
+    g = GOLD.get("c5")
+    if not g:
+        pytest.skip("no c5 fixture")
+    c, m = g["config"], g["config"]["model"]
+    cfg = DeepSeekConfig(m["vocab"], m["max_seq"], m["d"], m["heads"], m["layers"], m["dff"], m["q_rank"], m["kv_rank"])
+    model = seeded_deepseek_with_scaled_mla(cfg, c["seed"], c["mla_weight_scale"], latent_cache=True)
+    try:
+        prompt = JavaRandom(c["prompt_seed"]).ints(c["prompt_len"], m["vocab"])
+        model.reset()
+        model.prefill(prompt, choose_next=False)
+        l0 = model.lastLogits()
+        f = g["fp64_step0"]
+        assert float(np.max(np.abs(l0[f["cols"]] - np.array(f["oracle_fp32"])))) <= logit_gate("c5")
+        got = TextGenerator.generate(model, prompt, c["new_tokens"], top_k=1, use_graph=True)
+        assert np.array_equal(got[c["prompt_len"]:], np.array(g["tokens"], dtype=np.int32))
     finally:
         model.close()
 

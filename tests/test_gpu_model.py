@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from deepj_amd import DeepSeekConfig, DeepSeekModel, HipNative, LlamaConfig, LlamaModel, TextGenerator
+from deepj_amd.models import _DecoderOnlyModel
 from oracle import cpu_ref as ref
 
 pytestmark = pytest.mark.gpu
@@ -191,6 +192,59 @@ def test_deepseek_decode_row_equals_prefill_row(ds):
     for t in range(20, 30):
         gpu.step(int(ids[t]))
         assert float(np.max(np.abs(gpu.lastLogits() - full[t]))) <= 2e-4, t
+
+
+# ── DeepSeek with the latent KV cache (runner kind 3) ────────────────────────
+
+@pytest.fixture(scope="module")
+def ds_latent():
+    ref.set_threads(ref.default_threads())
+    gpu = DeepSeekModel(DS, 42, latent_cache=True)
+    cpu = oracle_model(DS, 42, q_rank=64, kv_rank=32)
+    yield gpu, cpu
+    gpu.close()
+    ref.set_threads(1)
+
+
+def test_deepseek_latent_cache_logits_and_tokens_match_oracle(ds_latent, ds):
+    """The same tiny DeepSeek model with cKV cached instead of the rotated K and V: prompt logits within 1e-3 of the
+    oracle, 64 greedy tokens identical to the oracle and to the full-cache mode, graph replay == eager."""
+    gpu, cpu = ds_latent
+    prompt = ref.JavaRandom(5).ints(24, 256)
+    got, exp = gpu.forward(prompt), cpu.forward(prompt)
+    err = float(np.max(np.abs(got - exp)))
+    assert err <= 1e-3, f"logits max-abs error {err}"
+    want = cpu.generate(prompt, 64, top_k=1, use_cache=True)
+    a = TextGenerator.generate(gpu, prompt, 64, top_k=1, use_graph=True)
+    assert np.array_equal(a, want), f"first mismatch at {int(np.argmax(a != want))}"
+    b = TextGenerator.generate(gpu, prompt, 64, top_k=1, use_graph=False)
+    assert np.array_equal(b, want)
+    full_cache = TextGenerator.generate(ds[0], prompt, 64, top_k=1, use_graph=True)
+    assert np.array_equal(full_cache, want)
+    sampled = TextGenerator.generate(gpu, prompt, 20, temperature=0.8, top_k=5, seed=9)
+    assert np.array_equal(sampled, cpu.generate(prompt, 20, temperature=0.8, top_k=5, seed=9, use_cache=True))
+
+
+def test_deepseek_latent_cache_decode_row_equals_prefill_row(ds_latent):
+    gpu, _ = ds_latent
+    ids = ref.JavaRandom(12).ints(30, 256)
+    full = gpu.forward(ids)
+    gpu.reset()
+    gpu.prefill(ids[:20], choose_next=False)
+    for t in range(20, 30):
+        gpu.step(int(ids[t]))
+        assert float(np.max(np.abs(gpu.lastLogits() - full[t]))) <= 2e-4, t
+    # a second prefill chunk on top of a filled cache re-expands the earlier rows as well
+    gpu.reset()
+    gpu.prefill(ids[:13], choose_next=False)
+    gpu.prefill(ids[13:29], choose_next=False)
+    gpu.step(int(ids[29]))
+    assert float(np.max(np.abs(gpu.lastLogits() - full[29]))) <= 2e-4
+
+
+def test_latent_cache_is_a_deepseek_option_only():
+    with pytest.raises(ValueError, match="latent KV cache belongs to the DeepSeek"):
+        _DecoderOnlyModel(C1, None, 0, True)
 
 
 def test_deepseek_one_full_width_layer_at_reference_init():

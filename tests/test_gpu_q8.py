@@ -180,3 +180,58 @@ def test_fused_rmsnorm_silu_mul_embed_argmax(dev):
     Stream().argmax_rows(dev.upload(logits), o4, 3, 32000).run()
     got = dev.download(o4, (3,), np.int32)
     assert list(got) == [int(np.argmax(logits[0])), 777, int(np.argmax(logits[2]))]
+
+
+# ── the two ops the latent KV cache is built from: rows appended at a device-side fill level, and a Q8 product
+#    over the rows that exist so far ──────────────────────────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("level,rows", [(0, 3), (5, 1), (9, 4), (12, 2), (-2, 3), (40, 2)])
+def test_append_rows_at_the_device_side_fill_level(dev, level, rows):
+    """dst[dstOff + (state[0] + i) * rowFloats ...] = src row i; rows that would land outside [0, maxRows) are
+    dropped (a fill level that is negative or beyond the cache never makes the kernel write out of bounds)."""
+    rf, max_rows, off = 24, 12, 7
+    before = gaussian(1, off + max_rows * rf + 5, 61, 1.0).reshape(-1)
+    src = gaussian(rows, rf, 62, 1.0)
+    dst, sb = dev.upload(before), dev.upload(src)
+    state = dev.upload(np.array([level, 0, 0, 0], np.int32))
+    Stream().append_rows(sb, dst, state, rows, rf, max_rows, off).run()
+    exp = before.copy()
+    for i in range(rows):
+        r = level + i
+        if 0 <= r < max_rows:
+            exp[off + r * rf: off + (r + 1) * rf] = src[i]
+    assert np.array_equal(dev.download(dst, exp.shape), exp)
+
+
+@pytest.mark.parametrize("level,extra", [(0, 1), (6, 1), (37, 16), (150, 1), (199, 1), (-3, 1), (500, 4)])
+def test_q8_linear_over_the_rows_a_growing_cache_holds(dev, level, extra):
+    """Q8_LINEAR_DYN: rows [0, min(Mmax, state[0] + extraRows)) of x + xOff times W; the rows beyond stay untouched."""
+    m_max, k, n, x_off = 200, 96, 136, 64
+    w = gaussian(k, n, 71, 0.05)
+    x = gaussian(m_max, k, 72, 1.0)
+    wq = quantize_on_device(dev, w)
+    xb = dev.upload(np.concatenate([np.zeros(x_off, np.float32), x.reshape(-1)]))
+    marker = np.full((m_max, n), 123.0, np.float32)
+    ob = dev.upload(marker)
+    state = dev.upload(np.array([level, 0, 0, 0], np.int32))
+    Stream().q8_linear_dyn(xb, wq, ob, m_max, k, n, state, extra, x_off).run()
+    got = dev.download(ob, (m_max, n))
+    live = max(0, min(m_max, level + extra))
+    if live:
+        exp = ref.matmul(x[:live], ref.q8_roundtrip(w))
+        scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+        assert_close(exp, got[:live], atol=1e-4 * scale, rtol=1e-4, what=f"live rows at level {level}")
+    assert np.array_equal(got[live:], marker[live:]), "rows beyond the fill level were written"
+
+
+def test_latent_ops_reject_bad_streams(dev):
+    a, st = dev.alloc(64), dev.upload(np.zeros(4, np.int32))
+    with pytest.raises(RuntimeError, match="op needs"):
+        Stream().append_rows(a, a, st, 2, 16, 8, 0).run()                 # dst must hold 8 rows of 16 floats
+    with pytest.raises(RuntimeError, match="bad shape"):
+        Stream().append_rows(a, a, st, 0, 16, 4, 0).run()
+    w = dev.alloc(HipNative.q8Floats(32, 4))
+    with pytest.raises(RuntimeError, match="op needs"):
+        Stream().q8_linear_dyn(a, w, a, 4, 32, 4, st, 1, 0).run()         # x holds 64 floats, 4 rows of 32 need 128
+    with pytest.raises(RuntimeError, match="bad shape"):
+        Stream().q8_linear_dyn(a, w, a, 1, 32, 4, st, -1, 0).run()
