@@ -359,15 +359,6 @@ void finalize(Runner &r) {
     r.records = r.alloc((int64_t)c.heads * 4 * (hd + 4));
     Stream s;
     emit(s, DJ_OP_FILL, r.state, 0, 4);
-    if (c.kind == 0) {
-        int64_t psf = 0, paf = 0;
-        hip(deepj_hip_llama_decode_plan(c.heads, hd, nullptr, nullptr, &psf, &paf));
-        r.p_scratch = r.alloc(psf);
-        r.p_argbuf = r.alloc(paf);
-        r.p_sync_floats = deepj_hip_llama_decode_sync_floats();
-        r.p_sync = r.alloc(r.p_sync_floats);
-        emit(s, DJ_OP_FILL, r.p_sync, 0, r.p_sync_floats);
-    }
     r.run(s);
     alloc_acts(r, r.dec, 1);
     // the prompt-sized buffers for the longest prompt the cache can take, so that no request pays for allocation
@@ -546,9 +537,25 @@ void warm_up(Runner &r) {
     reset(r);
 }
 
+// The persistent decode kernel (experimental: about half the speed of the replayed graph) gets its buffers on first use.
+void ensure_persistent(Runner &r) {
+    if (r.p_sync >= 0) return;
+    const Config &c = r.cfg;
+    int64_t psf = 0, paf = 0;
+    hip(deepj_hip_llama_decode_plan(c.heads, r.hd(), nullptr, nullptr, &psf, &paf));
+    r.p_scratch = r.alloc(psf);
+    r.p_argbuf = r.alloc(paf);
+    r.p_sync_floats = deepj_hip_llama_decode_sync_floats();
+    r.p_sync = r.alloc(r.p_sync_floats);
+    Stream s;
+    emit(s, DJ_OP_FILL, r.p_sync, 0, r.p_sync_floats);
+    r.run(s);
+}
+
 // All `steps` tokens in one launch of the persistent decode kernel.
 Stream persistent_stream(Runner &r, int steps) {
     const Config &c = r.cfg;
+    ensure_persistent(r);
     Stream s;
     emit(s, DJ_OP_LLAMA_DECODE, 29 + 9 * c.layers, steps, c.d, c.heads, c.dff, c.vocab, c.max_seq, c.layers, c.max_seq,
          r.emb, r.cos_t, r.sin_t, r.kc, r.vc, r.state, r.tokens, r.dec.x, r.dec.x2, r.dec.qkv, r.dec.att, r.dec.ff,
