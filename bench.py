@@ -75,7 +75,7 @@ def matvec_roofline(model, position: int, iters: int = 12):
     ops = decode_ops(stream)
     HipNative.profileOps(stream, 2)                               # warm-up
     us = HipNative.profileOps(stream, iters)
-    table, lin, lin_bytes, lin_us, weights = {}, [], 0, 0.0, []
+    table, lin, lin_bytes, lin_us, weights, kv_cache_id = {}, [], 0, 0.0, [], None
 
     def add(name, nbytes, t):
         e = table.setdefault(name, {"launches_per_token": 0, "bytes": int(nbytes), "us": 0.0})
@@ -94,6 +94,7 @@ def matvec_roofline(model, position: int, iters: int = 12):
             weights.append((w[2], HipNative.q8Floats(k, rows), VARIANTS.get((k, rows), f"{k}x{rows}")))
         elif code == op.OP_ATTN_DECODE_RECORDS:
             add("attention", 2 * position * cfg.dModel * 4, t)    # K and V rows of the live context, fp32
+            kv_cache_id = w[2]
         elif code == op.OP_DECODE_NEXT:
             add("decode_next", 4 * cfg.vocabSize, t)
     for e in table.values():
@@ -138,6 +139,14 @@ def matvec_roofline(model, position: int, iters: int = 12):
         e["GBs"] = round(e["bytes"] / e["us"] / 1e3, 1)
     read_avg_us = float(np.sum(rus)) / launches
     read_b2b_us = reads.time(iters) * 1e3 / (iters * launches)
+    # the decode attention's floor: as many bytes of the K cache as one layer's K and V rows of the live context
+    kv = Stream()
+    for _ in range(cfg.nLayers):
+        kv.stream_read(kv_cache_id, sink, 2 * position * cfg.dModel)
+    kv.profile(2)
+    kv_us = float(np.mean(kv.profile(iters)))
+    read_tab["attention_kv"] = {"bytes": 2 * position * cfg.dModel * 4, "us": round(kv_us, 3),
+                                "GBs": round(2 * position * cfg.dModel * 4 / kv_us / 1e3, 1)}
     dev.release_all()
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MATVEC_TRAFFIC_BYTES_PER_LAUNCH,
@@ -195,6 +204,11 @@ def cpu_baseline(cfg, ctx: int, tokens: int = 12):
     for i in range(1, tokens):
         m.forward_cached(ids[ctx + i:ctx + i + 1], last_only=True)
     per_token = (time.perf_counter() - t0) / (tokens - 1)
+    # the reference itself has no KV cache: every new token is a forward of the whole context, logits for every row
+    # (TextGenerator.java:91-100, DecoderOnlyModel.java:58-64) - one such forward, timed
+    t0 = time.perf_counter()
+    m.forward(ids[:ctx + 1])
+    t_full = time.perf_counter() - t0
     m.close()
     ref.set_threads(1)
     return {"value": round(1.0 / per_token, 4), "unit": "tok/s", "cores": 1, "kind": "port",
@@ -202,8 +216,7 @@ def cpu_baseline(cfg, ctx: int, tokens: int = 12):
                       f"weights, KV cache at context {ctx}, {tokens - 1} timed tokens; S=1 matmul is single-threaded "
                       f"by construction (CpuBackend.java:175)",
             "prefill_tok_s": round(ctx / t_prefill, 2), "prefill_threads": threads,
-            # the reference itself has no KV cache: every new token re-runs the whole context (TextGenerator.java:91-100)
-            "no_kv_cache_s_per_token": round(t_prefill * (ctx + 1) / ctx, 2)}
+            "no_kv_cache_s_per_token": round(t_full, 2), "no_kv_cache_threads": threads}
 
 
 def main() -> int:
@@ -251,6 +264,16 @@ def main() -> int:
 
     roof = matvec_roofline(model, args.prompt + args.warmup + args.steps)
     model.reset()
+    # the same decode at three times the context (the cache read grows with the position, the weights do not)
+    long_prompt = JavaRandom(3).ints(1536, cfg.vocabSize)
+    model.prefill(long_prompt)
+    model.decode(8)
+    HipNative.synchronize()
+    t0 = time.perf_counter()
+    model.decode(128)
+    HipNative.synchronize()
+    t_long = (time.perf_counter() - t0) / 128
+    model.reset()
     calibration_copy()
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg, args.prompt)
 
@@ -273,7 +296,8 @@ def main() -> int:
         "end_to_end": {"bytes_per_token": int(weights + kv), "achieved_GBs": round((weights + kv) * tok_s / 1e9, 1),
                        "frac_of_hbm_peak": round((weights + kv) * tok_s / 1e9 / HBM_PEAK_GBS, 4),
                        "prefill_tok_s": round(args.prompt / t_prefill, 1),
-                       "first_prefill_ms": round(t_first_prefill * 1e3, 2), "model_build_s": round(t_build, 1)},
+                       "first_prefill_ms": round(t_first_prefill * 1e3, 2), "model_build_s": round(t_build, 1),
+                       "decode_tok_s_at_context_1536": round(1.0 / t_long, 1)},
     }
     print(json.dumps(line))
     model.close()
