@@ -203,21 +203,22 @@ __global__ void __launch_bounds__(kThreads) k_fill(uint32_t *__restrict__ dst, u
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = bits;
 }
 
-// Measurement floor of the HBM-bound decode kernels: the same bytes read with 128-bit loads, eight in flight per
-// lane, nothing computed but an AND over the words (so that no load can be dropped) and nothing stored unless
-// every bit of the buffer is set.
+// Measurement floor of the HBM-bound decode kernels: the same bytes read with 128-bit loads, D in flight per lane,
+// nothing computed but an AND over the words (so that no load can be dropped) and nothing stored unless every bit of
+// the buffer is set.
+template <int D>
 __global__ void __launch_bounds__(kThreads) k_stream_read(const uint4 *__restrict__ src, uint32_t *__restrict__ sink,
                                                           int64_t n16, int64_t tail_from, const uint32_t *src_words,
                                                           int64_t n_words) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint32_t acc = 0xffffffffu;
-    for (; i + 7 * stride < n16; i += 8 * stride) {
-        uint4 v[8];
+    for (; i + (D - 1) * stride < n16; i += D * stride) {
+        uint4 v[D];
 #pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = src[i + u * stride];
+        for (int u = 0; u < D; u++) v[u] = src[i + u * stride];
 #pragma unroll
-        for (int u = 0; u < 8; u++) acc &= v[u].x & v[u].y & v[u].z & v[u].w;
+        for (int u = 0; u < D; u++) acc &= v[u].x & v[u].y & v[u].z & v[u].w;
     }
     for (; i < n16; i += stride) { uint4 v = src[i]; acc &= v.x & v.y & v.z & v.w; }
     for (int64_t j = tail_from + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n_words; j += stride) acc &= src_words[j];
@@ -380,12 +381,22 @@ void launch_fill(hipStream_t s, uint32_t *dst, uint32_t bits, int64_t n) {
 
 void launch_stream_read(hipStream_t s, const float *src, float *sink, int64_t n) {
     if (n <= 0) return;
-    const int64_t n16 = n / 4;
-    int64_t grid = (n16 + (int64_t)kThreads * 8 - 1) / ((int64_t)kThreads * 8);
-    if (grid > 768) grid = 768;            // three workgroups per CU, as the matvec
+    const int64_t n16 = n / 4, per_lane = (n16 + kThreads - 1) / kThreads;    // 128-bit loads a lane would issue in a grid of one
+    // as many loads in flight per lane as leave at least two workgroups per CU, at most three (the matvec's grid)
+    int depth = 8;
+    while (depth > 1 && per_lane / depth < 512) depth >>= 1;
+    int64_t grid = (per_lane + depth - 1) / depth;
+    if (grid > 768) grid = 768;
     if (grid < 1) grid = 1;
-    launch_kernel(k_stream_read, dim3((int)grid), dim3(kThreads), 0, s, reinterpret_cast<const uint4 *>(src),
-                  reinterpret_cast<uint32_t *>(sink), n16, n16 * 4, reinterpret_cast<const uint32_t *>(src), n);
+    const uint4 *p = reinterpret_cast<const uint4 *>(src);
+    uint32_t *o = reinterpret_cast<uint32_t *>(sink);
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(src);
+    switch (depth) {
+        case 8: launch_kernel(k_stream_read<8>, dim3((int)grid), dim3(kThreads), 0, s, p, o, n16, n16 * 4, w, n); break;
+        case 4: launch_kernel(k_stream_read<4>, dim3((int)grid), dim3(kThreads), 0, s, p, o, n16, n16 * 4, w, n); break;
+        case 2: launch_kernel(k_stream_read<2>, dim3((int)grid), dim3(kThreads), 0, s, p, o, n16, n16 * 4, w, n); break;
+        default: launch_kernel(k_stream_read<1>, dim3((int)grid), dim3(kThreads), 0, s, p, o, n16, n16 * 4, w, n); break;
+    }
 }
 
 void launch_nop(hipStream_t s, int grid) {
