@@ -35,6 +35,10 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_stream.restype = C.c_void_p
     lib.deepj_hip_q8_floats.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_q8_floats.restype = C.c_int64
+    lib.deepj_hip_q8_prepared_floats.argtypes = [C.c_int32, C.c_int32]
+    lib.deepj_hip_q8_prepared_floats.restype = C.c_int64
+    lib.deepj_hip_q8_gemm_path.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+    lib.deepj_hip_q8_gemm_path.restype = C.c_int32
     lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
     lib.deepj_hip_profile_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p, C.c_int32, _i32p]
     lib.deepj_hip_graph_capture.argtypes = [_i32p, C.c_int32, _i32p]
@@ -143,6 +147,16 @@ class HipNative:
     @staticmethod
     def q8Floats(k: int, rows: int) -> int:
         return int(library().deepj_hip_q8_floats(k, rows))
+
+    @staticmethod
+    def q8PreparedFloats(k: int, rows: int) -> int:
+        """Floats of the buffer OP_Q8_PREPARE fills for a Q8 weight of `rows` rows over k inputs."""
+        return int(library().deepj_hip_q8_prepared_floats(k, rows))
+
+    @staticmethod
+    def q8GemmPath(m: int, k: int, rows: int) -> int:
+        """1 when a Q8_LINEAR of m rows over such a weight runs on the fp16 direct-load GEMM, 0 on the bf16 kernels."""
+        return int(library().deepj_hip_q8_gemm_path(m, k, rows))
 
     @staticmethod
     def timeOps(cmd_stream, iters: int) -> float:

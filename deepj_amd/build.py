@@ -34,6 +34,7 @@ SOURCES = {
     # matrix-core accumulators in ordinary vector registers: the kernels rescale or mask them with vector
     # instructions after every few products, and each trip through the accumulator file costs a move per value
     "kernels_matmul.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "kernels_gemm_f16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "kernels_q8.hip": [],
     "kernels_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "kernels_decode.hip": [],

@@ -111,6 +111,7 @@ struct Q8Linear {
     int rec_hd = 0;                   // ATTN_MERGE prologue only: head width of the records in x
     const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
     int m_extra = 0;
+    const float *prepared = nullptr;  // the weights in the fp16 GEMM's layout (launch_q8_prepare), or null: converted per call
 };
 void launch_q8_quantize(hipStream_t s, const float *w, int8_t *q, float *scales, int k, int n, int row_off,
                         int row_step);
@@ -118,6 +119,20 @@ void launch_q8_dequantize(hipStream_t s, const int8_t *q, const float *scales, f
                           int row_off, int row_step);
 void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_t workspace_floats);
 int64_t q8_linear_workspace_floats(int m, int k, int n, int flags);
+// The size at which launch_q8_linear takes its fastest path (>= the one above); callers that may grow their workspace
+// offer this much, callers that may not offer what they have.
+int64_t q8_linear_preferred_workspace_floats(int m, int k, int n, int flags, bool prepared);
+
+// kernels_gemm_f16.hip: the many-row Q8 GEMM on fp16 matrix cores (two-piece activations, direct loads to LDS)
+bool q8_gemm_f16_shape_ok(int m, int n_rows, int k);
+int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared);
+// floats of the weights in that kernel's layout: fp16 [rows up to a multiple of 256][Kp + 64], then the scales as
+// [Kp / 32][rows up to a multiple of 256]
+int64_t q8_prepared_floats(int k, int n_rows);
+void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, float *prepared, int k, int n_rows);
+void launch_q8_gemm_f16(hipStream_t s, const float *x, const int8_t *wq, const float *scales, const float *prepared, float *out, int m,
+                        int k, int n_rows, const float *bias, const float *bias2, const float *residual, int interleaved_bias, int gelu,
+                        int swiglu, float *workspace, int64_t workspace_floats);
 
 // kernels_attn.hip
 struct AttnArgs {

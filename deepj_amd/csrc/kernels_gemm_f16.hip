@@ -1,0 +1,366 @@
+// Q8 GEMM for many rows (prefill): C[M x N] = X[M x K] . dequant(W)^T, W int8 [N x Kp] with one fp32 scale per 32 k.
+//
+// Arithmetic.  An int8 weight is exact in fp16.  A row of activations is multiplied by a power of two that brings its
+// largest magnitude into [2^14, 2^15) (exact, undone at the end) and every element is then written as hi + lo, two
+// fp16 numbers: hi = fp16(v) by round-to-nearest, lo = fp16(v - hi).  hi carries 11 significant bits and lo the next 11
+// (down to 2^-24 of the row's scale, where fp16 subnormals end), so hi + lo holds v to about 2^-23 relative - the fp32
+// value itself for all practical rows - and x . q = hi . q + lo . q with exact products and fp32 accumulation: two
+// v_mfma_f32_32x32x16_f16 per 16 k instead of three bf16 ones.  The group scale multiplies the finished 32-k partial
+// sum, as in the reference's dequantise-then-multiply (Q8 layout: q8_format notes in dj_common.h).
+//
+// Data path.  Both operands are prepared in global memory in the exact byte layout the matrix cores want: two fp16
+// planes of X (k_split_f16) and an fp16 copy of W with its scales transposed to [group][row] (k_q8_to_f16).  The GEMM
+// kernel then moves them with direct global -> LDS loads (global_load_lds_dwordx4: no vector registers, no LDS
+// store instructions), three stages deep, and spends its vector instructions on the per-group scaling only.
+//
+// Shape.  Workgroup tile 128 x 256, 256 threads = 4 wavefronts (2 x 2), one wavefront per SIMD; a wavefront owns
+// 64 x 128 of C = 8 MFMA tiles of 32 x 32 = 128 fp32 accumulators per lane, kept in ordinary vector registers because
+// the scaling reads and writes them with vector instructions.  All MFMA operands are in ordinary vector registers as
+// well: products whose A/B operands sit in the accumulation registers run at about two thirds of the rate here.
+// That budget (128 accumulators + 32 partial sums + 64 operand registers of 256) fixes the schedule: a K step of
+// 32 is 8 passes of one 32 x 32 tile (4 dependent MFMAs: 2 K halves x hi/lo), two partial-sum tiles alternate, and in
+// the shadow of a pass's MFMAs the wavefront issues the previous tile's 16 multiply-adds, the LDS reads of the
+// operands it needs next, and its share of the loads for the step after next.  __builtin_amdgcn_sched_barrier pins
+// that interleaving; the compiler still allocates registers and inserts the MFMA hazard waits.
+//
+// Stages and barriers.  Stage s % 3 holds K step s.  During step s a wavefront reads stage s (the second tile row,
+// column 3) and, after a mid-step barrier, stage s + 1 (the next step's first tile row, columns 0-2, scales); the
+// loads of step s + 2 are issued in the first half of step s into the stage that step s - 1 used, which every
+// wavefront has left by the barrier at the top of step s.  Loads past the last step are clamped to it and land in a
+// stage nobody reads again, so every step issues the same number of loads and the wait counts are constants.
+// The direct loads are inline assembly (the compiler would otherwise wait for ALL of them before any LDS read), and
+// the matching s_waitcnt vmcnt are written by hand; the kernel contains no other vector memory loads before its
+// epilogue, so the compiler's own counting is not disturbed.
+//
+// Epilogue.  A wavefront passes its accumulators through its own quarter of LDS to turn the MFMA layout (a lane owns a
+// column) into rows, then applies the row's power of two, bias / GELU / residual or the SwiGLU pairing on float4s and
+// stores 16 bytes per lane.
+#include "dj_common.h"
+#include "gemm_epilogue.h"
+#include <cstdlib>
+
+namespace dj {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+
+namespace {
+
+constexpr int TM = 128, TN = 256;
+constexpr int kXs = 2 * TM * 64;            // bytes of the two activation planes of one stage: [plane][row][32 k] fp16
+constexpr int kWl = TN * 64;                // bytes of the weights of one stage: [row][32 k] fp16
+constexpr int kStage = kXs + kWl + TN * 4;  // + one scale per weight row
+constexpr int kStages = 3;
+constexpr int kLoads = 9;                   // direct loads per wavefront per stage: 4 of X, 4 of W, 1 of scales
+
+struct GemmF16Args {
+    const uint16_t *planes;     // [2][m_pad][pitch] fp16: hi plane, lo plane
+    const uint16_t *w16;        // [n_pad][pitch] fp16
+    const float *scales_t;      // [kp / 32][n_pad]
+    const float *unscale;       // [m_pad]: 2^-s of the row
+    float *out;
+    int m, n, m_pad, n_pad, kp, pitch;
+    GemmEpilogue ep;
+};
+
+// 64 lanes x 16 bytes from base + off[lane] into LDS bytes [dst, dst + 1024), lane order
+__device__ __forceinline__ void load_to_lds16(const void *base, uint32_t off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void load_to_lds4(const void *base, uint32_t off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
+}
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16(const GemmF16Args a) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+    float acc[2][4][16];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    // A stage is made of 1 KB blocks of 16 rows x 4 chunks of 16 bytes (8 fp16); row r keeps chunk c at slot
+    // c ^ ((r >> 2) & 3), which spreads the 32 rows an MFMA operand read touches over all LDS banks.  A direct load
+    // writes lane order, so lane p fetches the chunk that belongs at slot p & 3 of row p >> 2.  The lane's byte
+    // offset is the same in every block; a block's origin is wave-uniform.
+    const int prow = lane >> 2, pchunk = (lane & 3) ^ ((prow >> 2) & 3);
+    const uint32_t op_lane = (uint32_t)((prow * a.pitch + pchunk * 8) * 2), s_lane = lane * 4;
+    const unsigned char *x_base[4], *w_base[4];
+    uint32_t x_dst[4], w_dst[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int blk = wave * 4 + i, pl = blk >> 3, rb = blk & 7;      // X: 2 planes x 8 row blocks; W: 16 row blocks
+        x_base[i] = reinterpret_cast<const unsigned char *>(a.planes) + (pl * plane_elems + (int64_t)(m0 + rb * 16) * a.pitch) * 2;
+        x_dst[i] = pl * TM * 64 + rb * 1024;
+        w_base[i] = reinterpret_cast<const unsigned char *>(a.w16) + (int64_t)(n0 + blk * 16) * a.pitch * 2;
+        w_dst[i] = kXs + blk * 1024;
+    }
+    const unsigned char *s_base = reinterpret_cast<const unsigned char *>(a.scales_t) + (int64_t)(n0 + wave * 64) * 4;
+    const uint32_t s_dst = kXs + kWl + wave * 256;
+    const int steps = a.kp / 32, last = steps - 1;
+    auto load_one = [&](int i, int step, int stage) {
+        const uint32_t sb = lds0 + stage * kStage;
+        step = min(step, last);
+        if (i < 4) load_to_lds16(x_base[i] + (int64_t)step * 64, op_lane, sb + x_dst[i]);
+        else if (i < 8) load_to_lds16(w_base[i - 4] + (int64_t)step * 64, op_lane, sb + w_dst[i - 4]);
+        else load_to_lds4(s_base + (int64_t)step * a.n_pad * 4, s_lane, sb + s_dst);
+    };
+
+    // MFMA operand addresses: lane l32 + 32 * half reads row l32, K chunk 2 * sub + half of its tile
+    const int sw = (l32 >> 2) & 3;
+    const int lane_sub0 = (l32 << 6) + (((0 + half) ^ sw) << 4), lane_sub1 = (l32 << 6) + (((2 + half) ^ sw) << 4);
+    const int x_wave = wm * 64 * 64, w_wave = kXs + wn * 128 * 64, s_wave = kXs + kWl + wn * 128 * 4 + l32 * 4;
+    const floatx16 z16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    halfx8 fx[2][2][2];                 // [tile row][K half][hi, lo]
+    halfx8 fw[2][4];                    // [K half][tile column]
+    float sc[4];                        // [tile column]
+    floatx16 g[2] = {z16, z16};         // partial sums of the tile in flight and of the one being scaled
+#pragma unroll
+    for (int j = 0; j < 4; j++) sc[j] = 0.f;
+    struct Addr { const unsigned char *x0, *x1, *w0, *w1, *s; };
+    auto addr_of = [&](int stage) {
+        const unsigned char *sb = lds + stage * kStage;
+        return Addr{sb + x_wave + lane_sub0, sb + x_wave + lane_sub1, sb + w_wave + lane_sub0, sb + w_wave + lane_sub1, sb + s_wave};
+    };
+    auto read_x = [&](int tm, int q, const Addr &ad) {      // q = K half * 2 + piece
+        const int sub = q >> 1, piece = q & 1;
+        fx[tm][sub][piece] = *reinterpret_cast<const halfx8 *>((sub ? ad.x1 : ad.x0) + piece * TM * 64 + tm * 2048);
+    };
+    auto read_w = [&](int sub, int tn, const Addr &ad) { fw[sub][tn] = *reinterpret_cast<const halfx8 *>((sub ? ad.w1 : ad.w0) + tn * 2048); };
+
+    auto k_step = [&](int step, int stage) {
+        const int sy = stage == 2 ? 0 : stage + 1, sz = sy == 2 ? 0 : sy + 1;
+        const Addr ax = addr_of(stage);
+        const int dy = (sy - stage) * kStage;
+        __builtin_amdgcn_s_barrier();                                  // every wavefront has left stage sz
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int tm = k >> 2, tn = k & 3, par = k & 1;
+            const int pk = (k + 7) & 7, ptm = pk >> 2, ptn = pk & 3;   // the tile finished by the previous pass
+            if (k == 4) {
+                asm volatile("s_waitcnt vmcnt(9)" ::: "memory");      // this wavefront's loads of step + 1 have landed ...
+                __builtin_amdgcn_s_barrier();                          // ... and so have everyone's
+                asm volatile("" ::: "memory");
+            }
+            const Addr ay = Addr{ax.x0 + dy, ax.x1 + dy, ax.w0 + dy, ax.w1 + dy, ax.s + dy};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int sub = i >> 1, piece = i & 1;
+                g[par] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx[tm][sub][piece], fw[sub][tn], i == 0 ? z16 : g[par], 0, 0, 0);
+                // the previous tile's scaling, one slot away from the MFMA that completed it
+                const int f0 = i <= 1 ? 0 : i == 2 ? 6 : 11, f1 = i == 0 ? 0 : i == 1 ? 6 : i == 2 ? 11 : 16;
+#pragma unroll
+                for (int f = f0; f < f1; f++) acc[ptm][ptn][f] = fmaf(g[1 - par][f], sc[ptn], acc[ptm][ptn][f]);
+                // column 3 of this step (operands, scale) in pass 0; columns 0-2 of the next step as this step leaves them
+                if (k == 0 && i < 2) read_w(i, 3, ax);
+                if (k >= 5 && i < 2) read_w(i, k - 5, ay);
+                if (k == 0 && i == 3) sc[3] = *reinterpret_cast<const float *>(ax.s + 3 * 128);
+                if (k >= 5 && i == 3) sc[k - 5] = *reinterpret_cast<const float *>(ay.s + (k - 5) * 128);
+                // the second tile row of this step in passes 0-3, the first tile row of the next step in passes 4-7
+                if (k < 4 && i == 2) read_x(1, k, ax);
+                if (k >= 4 && i == 2) read_x(0, k - 4, ay);
+                // the loads of step + 2
+                if (k < 4 && (i == 1 || i == 3)) load_one(k * 2 + (i >> 1), step + 2, sz);
+                if (k == 3 && i == 0) load_one(8, step + 2, sz);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    for (int s = 0; s < 2; s++)
+        for (int i = 0; i < kLoads; i++) load_one(i, s, s);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    {
+        const Addr a0 = addr_of(0);
+        for (int q = 0; q < 4; q++) read_x(0, q, a0);
+        for (int tn = 0; tn < 3; tn++) { read_w(0, tn, a0); read_w(1, tn, a0); }
+        for (int tn = 0; tn < 3; tn++) sc[tn] = *reinterpret_cast<const float *>(a0.s + tn * 128);
+    }
+    int stage = 0;
+    for (int step = 0; step < steps; step++) {
+        k_step(step, stage);
+        stage = stage == 2 ? 0 : stage + 1;
+    }
+    // the last tile's scaling; its scale (column 3 of the last step) is still in place
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[1][3][e] = fmaf(g[1][e], sc[3], acc[1][3][e]);
+    // no direct load may still be writing LDS when the epilogue reuses it or the workgroup ends
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // Epilogue.  acc[tm][tn][e] is C[32 tm + 8 (e / 4) + 4 half + e % 4][32 tn + l32] of the wavefront's 64 x 128 block.
+    // Per tile row: 32 x 128 floats go through this wavefront's 16 KB of LDS and come back as rows of float4.
+    float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
+    const GemmEpilogue &ep = a.ep;
+    const int out_n = ep.swiglu ? a.n >> 1 : a.n;
+#pragma unroll
+    for (int tm = 0; tm < 2; tm++) {
+#pragma unroll
+        for (int tn = 0; tn < 4; tn++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * 128 + 32 * tn + l32] = acc[tm][tn][e];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int col = n0 + wn * 128 + l32 * 4;                       // first of this lane's four columns
+        float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (ep.bias && col < a.n) {
+            if (ep.interleaved_bias) {                                 // even column n: bias[n / 2], odd: bias2[n / 2]
+                const float2 be = *reinterpret_cast<const float2 *>(ep.bias + (col >> 1)), bo = *reinterpret_cast<const float2 *>(ep.bias2 + (col >> 1));
+                b4 = make_float4(be.x, bo.x, be.y, bo.y);
+            } else {
+                b4 = *reinterpret_cast<const float4 *>(ep.bias + col);
+            }
+        }
+#pragma unroll 4
+        for (int i = 0; i < 16; i++) {
+            const int rl = i * 2 + half, row = m0 + wm * 64 + 32 * tm + rl;
+            float4 v = *reinterpret_cast<const float4 *>(stage_f + rl * 128 + l32 * 4);
+            if (row >= a.m || col >= a.n) continue;
+            const float us = a.unscale[row];
+            v.x = v.x * us; v.y = v.y * us; v.z = v.z * us; v.w = v.w * us;
+            if (ep.bias) { v.x = v.x + b4.x; v.y = v.y + b4.y; v.z = v.z + b4.z; v.w = v.w + b4.w; }
+            if (ep.swiglu) {
+                // (gate, up) pairs in neighbouring columns (SiLU.java:20-24, SwiGLULayer.java:69)
+                float2 o;
+                o.x = v.x * (1.0f / (1.0f + expf(-v.x))) * v.y;
+                o.y = v.z * (1.0f / (1.0f + expf(-v.z))) * v.w;
+                *reinterpret_cast<float2 *>(a.out + (int64_t)row * out_n + (col >> 1)) = o;
+                continue;
+            }
+            if (ep.gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
+            if (ep.residual) {
+                const float4 r = *reinterpret_cast<const float4 *>(ep.residual + (int64_t)row * a.n + col);
+                v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
+            }
+            *reinterpret_cast<float4 *>(a.out + (int64_t)row * a.n + col) = v;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");              // the rows are in registers before the next tile row overwrites them
+    }
+}
+
+// One workgroup per row of X: the row's largest magnitude, then the two fp16 planes of x * 2^s.  Columns [k, kp) are
+// written as zeros (the weights' padding is zero as well, but 0 x garbage could be a NaN); rows [m, m_pad) are left
+// alone: they only feed output rows that are never stored.
+__global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, uint16_t *__restrict__ planes, float *__restrict__ unscale,
+                                                   int m, int k, int kp, int pitch, int64_t plane_elems) {
+    __shared__ float red[4];
+    const int row = blockIdx.x, t = threadIdx.x;
+    const float *xr = x + (int64_t)row * k;
+    float mx = 0.f;
+    for (int c = t; c < k; c += 256) mx = fmaxf(mx, fabsf(xr[c]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if ((t & 63) == 0) red[t >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    // mx = f * 2^e with f in [0.5, 1): s = 15 - e puts it in [2^14, 2^15).  Zero, infinite or NaN rows stay unscaled;
+    // s is kept where 2^s and 2^-s are both normal numbers.
+    int s = 0;
+    if (mx > 0.f && mx < __builtin_inff()) {
+        int e;
+        (void)frexpf(mx, &e);
+        s = max(-126, min(126, 15 - e));
+    }
+    const float up = ldexpf(1.0f, s);
+    if (t == 0) unscale[row] = ldexpf(1.0f, -s);
+    uint16_t *hi = planes + (int64_t)row * pitch, *lo = hi + plane_elems;
+    for (int c = t; c < kp; c += 256) {
+        const float v = c < k ? xr[c] * up : 0.f;
+        const _Float16 h = (_Float16)v;
+        const _Float16 l = (_Float16)(v - (float)h);
+        hi[c] = __builtin_bit_cast(uint16_t, h);
+        lo[c] = __builtin_bit_cast(uint16_t, l);
+    }
+}
+
+// int8 weights [rows x kp] -> fp16 [rows x pitch] (8 per thread), scales [rows x groups] -> [groups x n_pad]
+__global__ void __launch_bounds__(256) k_q8_to_f16(const int8_t *__restrict__ wq, const float *__restrict__ scales, uint16_t *__restrict__ w16,
+                                                   float *__restrict__ scales_t, int rows, int kp, int pitch, int n_pad) {
+    const int chunks = kp >> 3;
+    const int64_t total = (int64_t)rows * chunks;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int row = (int)(idx / chunks), c = (int)(idx % chunks);
+        const int2 q = *reinterpret_cast<const int2 *>(wq + (int64_t)row * kp + c * 8);
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int w = j < 2 ? q.x : q.y, sh = (j & 1) * 16;
+            const _Float16 a = (_Float16)(float)(int8_t)((w >> sh) & 0xff), b = (_Float16)(float)(int8_t)((w >> (sh + 8)) & 0xff);
+            o[j] = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+        }
+        *reinterpret_cast<uint4 *>(w16 + (int64_t)row * pitch + c * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+        if ((c & 3) == 0) scales_t[(int64_t)(c >> 2) * n_pad + row] = scales[(int64_t)row * (kp >> 5) + (c >> 2)];
+    }
+}
+
+}  // namespace
+
+bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) {
+    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels (for comparisons)
+    static const bool enabled = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return !(e && e[0] == '0'); }();
+    if (!enabled) return false;
+    // few tiles leave most of the chip idle (one 128 x 256 tile per CU at a time); the bf16 kernels with their smaller
+    // tiles take those.  Four columns per lane in the epilogue need n_rows % 4 == 0.
+    const int64_t tiles = (int64_t)((m + TM - 1) / TM) * ((n_rows + TN - 1) / TN);
+    return m >= 256 && (n_rows & 3) == 0 && tiles >= 160 && k >= 64;
+}
+
+// the weights in this kernel's layout: fp16 rows, then the transposed scales (each part 256-byte aligned)
+int64_t q8_prepared_floats(int k, int n_rows) {
+    const int64_t kp = q8_padded_k(k), pitch = kp + 64, n_pad = round_up(n_rows, TN);
+    return round_up(n_pad * pitch / 2, 64) + round_up((kp / 32) * n_pad, 64);
+}
+
+// floats of workspace: planes, row factors and, unless the caller holds prepared weights, those
+int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared) {
+    const int64_t kp = q8_padded_k(k), pitch = kp + 64, m_pad = round_up(m, TM);
+    return round_up(m_pad * pitch, 64) + round_up(m_pad, 64) + (prepared ? 0 : q8_prepared_floats(k, n_rows));
+}
+
+void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, float *prepared, int k, int n_rows) {
+    if (k <= 0 || n_rows <= 0) return;
+    const int kp = q8_padded_k(k), pitch = kp + 64, n_pad = (int)round_up(n_rows, TN);
+    uint16_t *w16 = reinterpret_cast<uint16_t *>(prepared);
+    float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
+    const int64_t items = (int64_t)n_rows * (kp / 8);
+    launch_kernel(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
+}
+
+void launch_q8_gemm_f16(hipStream_t s, const float *x, const int8_t *wq, const float *scales, const float *prepared, float *out, int m,
+                        int k, int n_rows, const float *bias, const float *bias2, const float *residual, int interleaved_bias, int gelu,
+                        int swiglu, float *workspace, int64_t workspace_floats) {
+    if (!q8_gemm_f16_shape_ok(m, n_rows, k)) fail("q8_gemm_f16: shape outside this kernel's range");
+    if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
+    if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
+    const int kp = q8_padded_k(k), pitch = kp + 64, m_pad = (int)round_up(m, TM), n_pad = (int)round_up(n_rows, TN);
+    float *w = workspace;
+    uint16_t *planes = reinterpret_cast<uint16_t *>(w); w += round_up((int64_t)m_pad * pitch, 64);
+    float *unscale = w;                                  w += round_up(m_pad, 64);
+    launch_kernel(k_split_f16, dim3(m), dim3(256), 0, s, x, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
+    if (!prepared) {
+        launch_q8_prepare(s, wq, scales, w, k, n_rows);
+        prepared = w;
+    }
+    const uint16_t *w16 = reinterpret_cast<const uint16_t *>(prepared);
+    const float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
+    GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch,
+                  GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}};
+    static bool configured = false;
+    if (!configured) {
+        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
+        configured = true;
+    }
+    launch_kernel(k_gemm_q8_f16, dim3(n_pad / TN, m_pad / TM), dim3(256), (size_t)kStages * kStage, s, a);
+}
+
+}  // namespace dj

@@ -16,6 +16,7 @@
 // 128 x 128), scale groups per step and wavefront sets per workgroup are template arguments chosen per problem
 // shape by launch_q8_gemm; the epilogue adds bias / GELU / residual or pairs interleaved gate/up columns (SwiGLU).
 #include "dj_common.h"
+#include "gemm_epilogue.h"
 
 namespace dj {
 
@@ -25,24 +26,6 @@ namespace {
 
 constexpr int BM = 64, BN = 64, BK = 32;
 constexpr int PAD = 4;
-
-struct GemmEpilogue {
-    const float *bias;      // [N] or null; with interleave: even col n -> bias[n/2], odd col -> bias2[n/2]
-    const float *bias2;
-    const float *residual;  // [M x N] or null
-    int interleaved_bias;
-    const int32_t *m_dev;   // when set, only rows < min(M, m_dev[0] + m_extra) exist (row count kept on the device)
-    int m_extra;
-    int gelu;               // GELU (tanh form, tensor/cpu/CpuBackend.java:338, used by activations/GELU.java:15-18) on acc + bias, before the residual
-    int swiglu;             // Q8 GEMM only: columns are interleaved gate/up pairs; C is [M x N/2], C[r][j] = SiLU(gate_j) * up_j
-};
-
-__device__ __forceinline__ float gemm_gelu(float x) {
-    float c = sqrtf(2.0f / 3.14159265358979323846f);
-    float x3 = x * x * x;
-    float t = c * (x + 0.044715f * x3);
-    return 0.5f * x * (1.0f + (float)tanh((double)t));
-}
 
 __global__ void __launch_bounds__(256) k_gemm(const float *__restrict__ A, const float *__restrict__ Bf,
                                               float *__restrict__ C, int M, const int N, const int K,

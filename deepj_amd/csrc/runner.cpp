@@ -84,6 +84,8 @@ struct Runner {
     int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
     int64_t p_sync_floats = 0;
     bool p_pending = false;                                // a persistent launch has not been checked yet
+    std::vector<int32_t> prepared;                         // the weights in the many-row GEMM's layout (first long prompt)
+    bool prepared_done = false;
     Acts dec, pre;
     int32_t graph = 0, graph_unrolled = 0;                 // one token per replay / kGraphUnroll tokens per replay
     bool finalized = false;
@@ -459,6 +461,31 @@ Stream decode_stream(Runner &r, bool sample_on_device) {
     return s;
 }
 
+// A long prompt runs its projections on the GEMM that loads fp16 weights straight into LDS.  The first such prompt
+// writes the weights once in that layout (about 2 bytes per weight more, kept until the runner goes) instead of every
+// call converting them into the workspace.  (finalize()'s warm-up pass runs long prompts when maxSeqLen allows them, so
+// with the warm-up on the copies exist from the start.)
+void ensure_prepared(Runner &r, int n) {
+    if (r.prepared_done || n < 256) return;
+    r.prepared_done = true;
+    const Config &c = r.cfg;
+    const int d = c.d;
+    Stream s;
+    auto prepare = [&](int32_t w, int k, int rows) {
+        if (w < 0 || !deepj_hip_q8_gemm_path(c.max_seq, k, rows)) return;
+        int32_t p = r.alloc(deepj_hip_q8_prepared_floats(k, rows));
+        r.prepared.push_back(p);
+        emit(s, DJ_OP_Q8_PREPARE, w, p, k, rows);
+    };
+    for (const Layer &L : r.layers) {
+        prepare(L.wqkv, d, 3 * d);
+        prepare(L.wo, d, d);
+        prepare(L.wgu, d, c.kind == 2 ? c.dff : 2 * c.dff);
+        prepare(L.wd, c.dff, d);
+    }
+    if (!s.empty()) r.run(s);
+}
+
 void check_ids(const Config &c, const int32_t *ids, int n) {
     for (int i = 0; i < n; i++)
         if (ids[i] < 0 || ids[i] >= c.vocab) throw Error("Token id out of range: " + std::to_string(ids[i]));   // Embedding.java:30-32
@@ -474,6 +501,7 @@ void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choos
     if (r.pos + n > c.max_seq)
         throw Error("context of " + std::to_string(r.pos + n) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
     alloc_acts(r, r.pre, n);
+    ensure_prepared(r, n);
     hip(deepj_hip_upload(r.pre.ids, reinterpret_cast<const float *>(ids), n));
     Stream s;
     emit(s, DJ_OP_EMBED_GATHER, r.emb, r.pre.ids, r.pre.x, n, c.d, c.vocab, 0);
@@ -788,6 +816,7 @@ void deepj_runner_destroy(void *h) {
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
         for (int32_t id : {a->x, a->x2, a->qkv, a->q, a->att, a->ff, a->ids, a->cq, a->ckv}) add(id);
+    for (int32_t id : r->prepared) add(id);
     if (!ids.empty()) deepj_hip_release(ids.data(), (int32_t)ids.size());
     delete r;
 }

@@ -63,6 +63,8 @@ struct Runtime {
     unsigned char *static_scratch = nullptr;       // device address of `scratch` below on g.device
     bool no_alloc = false;                         // inside deepj_hip_flush_ops_noalloc: nothing may allocate
     std::vector<std::pair<int32_t, void *>> *track = nullptr;   // graph capture: buffers the dry pass resolves
+    struct Prepared { int32_t id; int k, rows; };
+    std::unordered_map<int32_t, Prepared> prepared;   // Q8 weight buffer -> its copy in the fp16 GEMM's layout (OP_Q8_PREPARE)
     void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
     std::vector<int64_t> decode_table_key;
 };
@@ -96,6 +98,13 @@ void ensure_init(int device = 0) {
     DJ_HIP(hipMemset(g.static_scratch, 0, kStaticCounterBytes));
     g.device = device;
     g.ready = true;
+}
+
+// A prepared copy stops standing for its Q8 buffer as soon as either is released or written.
+void forget_prepared(int32_t id) {
+    if (g.prepared.empty()) return;
+    g.prepared.erase(id);
+    for (auto it = g.prepared.begin(); it != g.prepared.end();) it = it->second.id == id ? g.prepared.erase(it) : std::next(it);
 }
 
 // 256 B granularity up to 64 KiB, then four classes per power of two (<= 25 % slack).
@@ -225,6 +234,7 @@ int stride_of(int op) {
         case DJ_OP_ADD_POSITIONS: return 7;
         case DJ_OP_STREAM_READ: return 4;
         case DJ_OP_NOP: return 2;
+        case DJ_OP_Q8_PREPARE: return 5;
         default: return -1;
     }
 }
@@ -395,6 +405,7 @@ void exec_one(Cursor &c) {
             float *src = buf(w[1], quant ? k * n : qfloats, op, "src");
             float *dst = buf(w[2], quant ? qfloats : k * n, op, "dst");
             if (run) {
+                forget_prepared(w[2]);
                 if (quant) {
                     int8_t *q = reinterpret_cast<int8_t *>(dst);
                     float *sc = reinterpret_cast<float *>(q + q8_scale_offset_bytes((int)k, (int)total));
@@ -442,7 +453,14 @@ void exec_one(Cursor &c) {
             p.bias = (flags & DJ_LIN_BIAS) ? buf(w[9], n, op, "bias") : nullptr;
             p.bias2 = ((flags & DJ_LIN_BIAS) && sw) ? buf(w[10], n, op, "bias2") : nullptr;
             p.residual = (flags & DJ_LIN_RESIDUAL) ? buf(w[11], m * n, op, "residual") : nullptr;
-            int64_t ws = q8_linear_workspace_floats((int)m, (int)k, (int)n, flags);
+            // a workspace that may grow is sized for the kernel's fastest path; the fixed one for the smallest
+            if (m > 1) {
+                auto pit = g.prepared.find(w[2]);
+                if (pit != g.prepared.end() && pit->second.k == k && pit->second.rows == rows)
+                    p.prepared = buf(pit->second.id, q8_prepared_floats((int)k, (int)rows), op, "prepared weights");
+            }
+            int64_t ws = g.no_alloc ? q8_linear_workspace_floats((int)m, (int)k, (int)n, flags)
+                                    : q8_linear_preferred_workspace_floats((int)m, (int)k, (int)n, flags, p.prepared != nullptr);
             if (c.dry) c.ws_need = std::max(c.ws_need, ws);
             if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
             break;
@@ -734,7 +752,22 @@ void exec_one(Cursor &c) {
             if (n < 0 || so < 0 || dof < 0) fail("OP_COPY: bad range");
             const float *a = buf(w[1], so + n, op, "src");
             float *o = buf(w[2], dof + n, op, "dst");
-            if (run) launch_copy(s, a + so, o + dof, n);
+            if (run) { forget_prepared(w[2]); launch_copy(s, a + so, o + dof, n); }
+            break;
+        }
+        case DJ_OP_Q8_PREPARE: {
+            // [op, weight, prepared, K, rows]: writes the weights in the many-row GEMM's layout and lets that buffer
+            // stand for them in later Q8_LINEARs with more than one row, until either buffer is released or written
+            int64_t k = w[3], rows = w[4]; need_positive(op, "K", k); need_positive(op, "rows", rows);
+            if (w[1] == w[2]) fail("OP_Q8_PREPARE: the prepared copy needs a buffer of its own");
+            const float *wq = buf(w[1], (q8_bytes((int)k, (int)rows) + 3) / 4, op, "weight");
+            float *prep = buf(w[2], q8_prepared_floats((int)k, (int)rows), op, "prepared");
+            if (run) {
+                const int8_t *q = reinterpret_cast<const int8_t *>(wq);
+                launch_q8_prepare(s, q, reinterpret_cast<const float *>(q + q8_scale_offset_bytes((int)k, (int)rows)), prep, (int)k, (int)rows);
+                forget_prepared(w[2]);
+                g.prepared[w[1]] = Runtime::Prepared{w[2], (int)k, (int)rows};
+            }
             break;
         }
         case DJ_OP_STREAM_READ: {
@@ -754,7 +787,7 @@ void exec_one(Cursor &c) {
         case DJ_OP_FILL: {
             int64_t n = w[3]; need_positive(op, "n", n);
             float *o = buf(w[1], n, op, "dst");
-            if (run) launch_fill(s, reinterpret_cast<uint32_t *>(o), (uint32_t)w[2], n);
+            if (run) { forget_prepared(w[1]); launch_fill(s, reinterpret_cast<uint32_t *>(o), (uint32_t)w[2], n); }
             break;
         }
         default:
@@ -827,6 +860,7 @@ const char *op_name(int op) {
         case DJ_OP_LLAMA_DECODE: return "OP_LLAMA_DECODE";
         case DJ_OP_STREAM_READ: return "OP_STREAM_READ";
         case DJ_OP_NOP: return "OP_NOP";
+        case DJ_OP_Q8_PREPARE: return "OP_Q8_PREPARE";
         default: return "OP_?";
     }
 }
@@ -886,6 +920,7 @@ int deepj_hip_upload(int32_t id, const float *src, int64_t n) {
                  std::to_string(it->second.floats));
         if (n == 0) return;
         if (!src) fail("uploadBuffer: null source");
+        forget_prepared(id);
         size_t bytes = (size_t)n * 4;
         // The caller's array is only borrowed: the copy out of it has finished on return.
         if (bytes <= g.staging_bytes) {
@@ -923,6 +958,7 @@ int deepj_hip_release(const int32_t *ids, int32_t count) {
             g.live_bytes -= (int64_t)it->second.capacity;
             pool_free(it->second.ptr, it->second.capacity);
             g.live.erase(it);
+            forget_prepared(ids[i]);
         }
     });
 }
@@ -1041,6 +1077,16 @@ int64_t deepj_hip_llama_decode_sync_floats(void) { return llama_decode_sync_word
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows) {
     if (k <= 0 || rows <= 0) return 0;
     return (q8_bytes(k, rows) + 3) / 4;
+}
+
+int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows) {
+    if (k <= 0 || rows <= 0) return 0;
+    return q8_prepared_floats(k, rows);
+}
+
+int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows) {
+    if (m <= 1 || k <= 0 || rows <= 0) return 0;
+    return q8_gemm_f16_shape_ok(m, rows, k) ? 1 : 0;
 }
 
 int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total) {

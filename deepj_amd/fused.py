@@ -142,6 +142,7 @@ class Stream:
     def fill(self, dst, bits, n): return self.emit(op.OP_FILL, dst, bits, n)
     def stream_read(self, src, sink, n): return self.emit(op.OP_STREAM_READ, src, sink, n)
     def nop(self, grid=1): return self.emit(op.OP_NOP, grid)
+    def q8_prepare(self, w, prepared, k, rows): return self.emit(op.OP_Q8_PREPARE, w, prepared, k, rows)
     def matmul(self, a, b, out, m, n, k): return self.emit(op.OP_MATMUL, a, b, out, m, n, k)
 
     # execution -----------------------------------------------------------------

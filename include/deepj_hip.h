@@ -189,13 +189,20 @@ enum {
      *     rows that sit at positions state[0].. of the sequence
      * STREAM_READ   [op, src, sink, n]    measurement floor: reads n floats of src with 128-bit loads and keeps nothing
      * NOP           [op, grid]            measurement floor: an empty kernel of `grid` workgroups of 256 threads
+     * Q8_PREPARE    [op, weight, prepared, K, rows]
+     *     Writes the Q8 weight [rows x K] into `prepared` (deepj_hip_q8_prepared_floats(K, rows) floats, a buffer of
+     *     its own) as fp16 rows plus scales transposed to [group][row], the layout the many-row GEMM loads straight
+     *     into LDS, and lets `prepared` stand for `weight` in later Q8_LINEARs with M > 1 (they otherwise convert the
+     *     weights into the workspace on every call).  The association ends when either buffer is released, uploaded
+     *     to, or the destination of Q8_QUANTIZE / COPY / FILL; a graph captured before that keeps the copy it was
+     *     captured with.  Results are the same with and without it.
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
     DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82, DJ_OP_LAYERNORM = 83,
-    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85, DJ_OP_STREAM_READ = 86, DJ_OP_NOP = 87
+    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85, DJ_OP_STREAM_READ = 86, DJ_OP_NOP = 87, DJ_OP_Q8_PREPARE = 88
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8, DJ_LIN_LAYERNORM = 16,
@@ -209,6 +216,12 @@ int64_t deepj_hip_llama_decode_sync_floats(void);
 
 /* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
+
+/* Floats of the buffer Q8_PREPARE fills for such a weight (about 2 bytes per weight), and whether a Q8_LINEAR of m
+ * rows over it runs on the fp16 direct-load GEMM (1) or on the bf16 kernels (0) when its workspace may grow.
+ * No counterpart in the reference, whose weights are fp32 (J/layers/Linear.java:9-24). */
+int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows);
+int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);
 
 /* ── host side: java.util.Random twin ─────────────────────────────────────
  * Tensor.random(rows, cols, Random) of the reference (J/tensor/cpu/CpuBackend.java:148-152)

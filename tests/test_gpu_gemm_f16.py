@@ -1,0 +1,190 @@
+"""The many-row Q8 GEMM on fp16 matrix cores (two-piece activations, direct loads into LDS) through the C ABI against
+the CPU oracle: fp32 CpuBackend.matmul (tensor/cpu/CpuBackend.java:168-188, ikj order) on the dequantised weights.
+
+Shapes are chosen so that the library takes this kernel (HipNative.q8GemmPath says so for each); what the tests vary:
+ragged M and N (not multiples of the 128 x 256 tile), K that is not a multiple of the 32-group, every epilogue
+(bias, GELU, residual, interleaved SwiGLU with both biases), the RMSNorm / LayerNorm prologue, rows whose magnitudes span
+twelve decades with outliers and tiny values inside a row, all-zero rows, prepared weights (OP_Q8_PREPARE) against
+per-call conversion, and the loss of that association when the weights are rewritten.
+Gate: |expected - actual| <= atol + 1e-4 |expected| with atol = 1e-4 of the output's rms (the per-op gate of
+src/test/java/io/github/kirstenali/deepj/tensor/metal/MetalBackendTest.java:452-466)."""
+import numpy as np
+import pytest
+
+from deepj_amd import HipNative, JavaRandom
+from deepj_amd.fused import DeviceBuffers, Stream
+from oracle import cpu_ref as ref
+from gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    ref.set_threads(ref.default_threads())
+    d = DeviceBuffers()
+    yield d
+    d.release_all()
+    ref.set_threads(1)
+
+
+def quantised(dev, w):
+    """Uploads w [K x N], quantises it with the library and returns (buffer, the oracle's dequantised copy)."""
+    k, n = w.shape
+    src = dev.upload(w)
+    wq = dev.alloc(HipNative.q8Floats(k, n))
+    Stream().q8_quantize(src, wq, k, n).run()
+    dev.release(src)
+    return wq, ref.q8_roundtrip(w)
+
+
+def gate(exp):
+    return 1e-4 * float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+
+
+def test_path_query_matches_the_documented_rule():
+    assert HipNative.q8GemmPath(512, 2048, 11264) == 1        # 4 x 44 tiles
+    assert HipNative.q8GemmPath(2048, 4096, 4096) == 1        # 16 x 16
+    assert HipNative.q8GemmPath(512, 2048, 6144) == 0         # 96 tiles: most of the chip would idle
+    assert HipNative.q8GemmPath(1, 2048, 32000) == 0          # the matvec's case
+    assert HipNative.q8GemmPath(512, 2048, 11266) == 0        # four columns per lane in the epilogue
+    assert HipNative.q8PreparedFloats(2048, 11264) == (11264 * (2048 + 64)) // 2 + 64 * 11264
+
+
+@pytest.mark.parametrize("m,k,n", [(300, 1000, 13828), (257, 96, 40964), (640, 2048, 8192)])
+def test_plain_product_ragged_shapes(dev, m, k, n):
+    assert HipNative.q8GemmPath(m, k, n) == 1
+    w = JavaRandom(11).tensor(k, n, 0.02)
+    x = JavaRandom(12).tensor(m, k, 1.0)
+    wq, deq = quantised(dev, w)
+    exp = ref.matmul(x, deq)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    Stream().q8_linear(xb, wq, ob, m, k, n).run()
+    got = dev.download(ob, (m, n))
+    dev.release(xb, ob, wq)
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear M={m} K={k} N={n}")
+
+
+def test_rows_spanning_twelve_decades_with_outliers(dev):
+    """Each row gets its own power of two before the fp16 split: a row of 1e-6 magnitudes must come out as exact as a
+    row of 1e6; inside a row, values 300 times the typical size and values 1e-4 of it share the row's scale."""
+    m, k, n = 260, 512, 40960
+    assert HipNative.q8GemmPath(m, k, n) == 1
+    x = JavaRandom(21).tensor(m, k, 1.0)
+    x *= (10.0 ** ((np.arange(m) % 13) - 6)).astype(np.float32)[:, None]
+    x[:, 5::97] *= 300.0
+    x[:, 7::89] *= 1e-4
+    x[17, :] = 0.0                                                # an all-zero row
+    x[18, 3] = 0.0
+    w = JavaRandom(22).tensor(k, n, 0.02)
+    wq, deq = quantised(dev, w)
+    exp = ref.matmul(x, deq)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    Stream().q8_linear(xb, wq, ob, m, k, n).run()
+    got = dev.download(ob, (m, n))
+    dev.release(xb, ob, wq)
+    assert not got[17].any()
+    # per row: the row's own rms sets the tolerance (the rows differ by twelve decades)
+    rms = np.sqrt(np.mean(exp.astype(np.float64) ** 2, axis=1, keepdims=True))
+    err = np.abs(got.astype(np.float64) - exp) - 1e-4 * np.abs(exp)
+    worst = float(np.max(err / np.maximum(rms, 1e-300)))
+    print(f"\n[rows 1e-6 .. 1e6] worst (|err| - 1e-4 |exp|) / row rms = {worst:.2e}")
+    assert worst <= 1e-4
+
+
+@pytest.mark.parametrize("epilogue", ["bias", "bias_gelu", "bias_residual", "residual"])
+def test_epilogues(dev, epilogue):
+    m, k, n = 384, 256, 14336
+    assert HipNative.q8GemmPath(m, k, n) == 1
+    x = JavaRandom(31).tensor(m, k, 1.0)
+    w = JavaRandom(32).tensor(k, n, 0.05)
+    b = JavaRandom(33).tensor(1, n, 0.3)
+    r = JavaRandom(34).tensor(m, n, 1.0)
+    wq, deq = quantised(dev, w)
+    exp = ref.matmul(x, deq)
+    kw = {}
+    if "bias" in epilogue:
+        exp = ref.add_row_vector(exp, b)
+        kw["bias"] = dev.upload(b)
+    if "gelu" in epilogue:
+        exp = ref.gelu(exp)
+        kw["gelu"] = True
+    if "residual" in epilogue:
+        exp = ref.add(r, exp)
+        kw["residual"] = dev.upload(r)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    Stream().q8_linear(xb, wq, ob, m, k, n, **kw).run()
+    got = dev.download(ob, (m, n))
+    dev.release(xb, ob, wq, *[v for v in kw.values() if not isinstance(v, bool)])
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear + {epilogue}")
+
+
+@pytest.mark.parametrize("norm", ["rms", "layer"])
+def test_swiglu_and_norm_prologues(dev, norm):
+    """gate/up rows interleaved in one Q8 buffer, SiLU(gate) * up in the epilogue (SwiGLULayer.java:63-70), behind an
+    RMSNorm prologue; LayerNorm prologue with a plain bias epilogue (GPT's first MLP projection)."""
+    m, d, dff = 300, 320, 10368
+    x = JavaRandom(41).tensor(m, d, 1.5)
+    gamma = (1.0 + JavaRandom(42).tensor(1, d, 0.1)).astype(np.float32)
+    xb, gb = dev.upload(x), dev.upload(gamma)
+    if norm == "rms":
+        assert HipNative.q8GemmPath(m, d, 2 * dff) == 1
+        wg, wu = JavaRandom(43).tensor(d, dff, 0.05), JavaRandom(44).tensor(d, dff, 0.05)
+        bg, bu = JavaRandom(45).tensor(1, dff, 0.2), JavaRandom(46).tensor(1, dff, 0.2)
+        h = ref.rmsnorm(x, gamma)
+        exp = ref.multiply(ref.silu(ref.add_row_vector(ref.matmul(h, ref.q8_roundtrip(wg)), bg)),
+                           ref.add_row_vector(ref.matmul(h, ref.q8_roundtrip(wu)), bu))
+        wgu = dev.alloc(HipNative.q8Floats(d, 2 * dff))
+        for w, off in ((wg, 0), (wu, 1)):
+            src = dev.upload(w)
+            Stream().q8_quantize(src, wgu, d, dff, off, 2, 2 * dff).run()
+            dev.release(src)
+        ob = dev.alloc(m * dff)
+        Stream().q8_linear(xb, wgu, ob, m, d, dff, gamma=gb, bias=dev.upload(bg), bias2=dev.upload(bu), swiglu=True).run()
+        got = dev.download(ob, (m, dff))
+        dev.release(wgu, ob)
+    else:
+        n = 2 * dff
+        assert HipNative.q8GemmPath(m, d, n) == 1
+        beta = JavaRandom(47).tensor(1, d, 0.1)
+        w, b = JavaRandom(48).tensor(d, n, 0.05), JavaRandom(49).tensor(1, n, 0.2)
+        wq, deq = quantised(dev, w)
+        exp = ref.add_row_vector(ref.matmul(ref.layernorm(x, gamma, beta), deq), b)
+        ob = dev.alloc(m * n)
+        Stream().q8_linear(xb, wq, ob, m, d, n, gamma=gb, beta=dev.upload(beta), bias=dev.upload(b)).run()
+        got = dev.download(ob, (m, n))
+        dev.release(wq, ob)
+    dev.release(xb, gb)
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"{norm}-norm prologue")
+
+
+def test_prepared_weights_give_the_same_bits_and_follow_the_weights(dev):
+    m, k, n = 512, 512, 10240
+    assert HipNative.q8GemmPath(m, k, n) == 1
+    x = JavaRandom(51).tensor(m, k, 1.0)
+    w1, w2 = JavaRandom(52).tensor(k, n, 0.02), JavaRandom(53).tensor(k, n, 0.02)
+    wq, deq1 = quantised(dev, w1)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    lin = Stream().q8_linear(xb, wq, ob, m, k, n)
+    lin.run()
+    plain = dev.download(ob, (m, n))
+    prep = dev.alloc(HipNative.q8PreparedFloats(k, n))
+    Stream().q8_prepare(wq, prep, k, n).run()
+    lin.run()
+    with_prepared = dev.download(ob, (m, n))
+    assert np.array_equal(plain.view(np.int32), with_prepared.view(np.int32))
+    # new weights in the same buffer: the copy no longer stands for them
+    src = dev.upload(w2)
+    Stream().q8_quantize(src, wq, k, n).run()
+    lin.run()
+    got = dev.download(ob, (m, n))
+    exp = ref.matmul(x, ref.q8_roundtrip(w2))
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what="after re-quantising a prepared weight")
+    # prepared again, then the copy is released: back to per-call conversion, same result
+    Stream().q8_prepare(wq, prep, k, n).run()
+    dev.release(prep)
+    lin.run()
+    assert np.array_equal(dev.download(ob, (m, n)).view(np.int32), got.view(np.int32))
+    with pytest.raises(RuntimeError, match="a buffer of its own"):
+        Stream().q8_prepare(wq, wq, k, n).run()
+    dev.release(src, wq, xb, ob)

@@ -280,7 +280,7 @@ def test_graph_replay_is_refused_once_a_captured_buffer_or_the_workspace_is_gone
         Stream().fill(x, 0, m * k).fill(gm, 0, k).fill(w, 0, HipNative.q8Floats(k, n)).run()
         g2 = HipNative.graphCapture(Stream().q8_linear(x, w, o, m, k, n, gamma=gm).array())
         HipNative.graphLaunch(g2, 1)
-        big_m, big_k = 16384, 2048                   # 32 Mi floats of normalised rows: more than any other test's stream needs
+        big_m, big_k = 16384, 8192                   # 128 Mi floats of normalised rows: more than any other test's stream needs
         bx, bg, bw, bo = (dev.alloc(big_m * big_k), dev.alloc(big_k), dev.alloc(HipNative.q8Floats(big_k, n)),
                           dev.alloc(big_m * n))
         Stream().fill(bx, 0, big_m * big_k).fill(bg, 0, big_k).fill(bw, 0, HipNative.q8Floats(big_k, n)).run()
