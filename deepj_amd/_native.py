@@ -155,7 +155,8 @@ class HipNative:
 
     @staticmethod
     def q8GemmPath(m: int, k: int, rows: int) -> int:
-        """1 when a Q8_LINEAR of m rows over such a weight runs on the fp16 direct-load GEMM, 0 on the bf16 kernels."""
+        """128 or 64 (rows per workgroup tile) when a Q8_LINEAR of m rows over such a weight runs on the fp16 direct-load
+        GEMM, 0 when it runs on the bf16 kernels or the matvec."""
         return int(library().deepj_hip_q8_gemm_path(m, k, rows))
 
     @staticmethod

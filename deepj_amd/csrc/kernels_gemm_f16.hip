@@ -38,6 +38,7 @@
 #include "dj_common.h"
 #include "gemm_epilogue.h"
 #include <cstdlib>
+#include <type_traits>
 
 namespace dj {
 
@@ -69,6 +70,53 @@ __device__ __forceinline__ void load_to_lds16(const void *base, uint32_t off, ui
 }
 __device__ __forceinline__ void load_to_lds4(const void *base, uint32_t off, uint32_t dst) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
+}
+
+// One tile row of a wavefront's block: acc[tn][e] is C[row0 + 8 (e / 4) + 4 half + e % 4][col0 + 32 tn + l32].  The 32 x 128
+// floats go through 16 KB of LDS that belong to this wavefront alone and come back as rows of float4 (lane l32 + 32 half:
+// rows 2 i + half, columns 4 l32 ..), which get the row's power of two, bias / GELU / residual or the SwiGLU pairing.
+__device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stage_f, const float (&acc)[4][16], int row0, int col0, int half, int l32) {
+    const GemmEpilogue &ep = a.ep;
+    const int out_n = ep.swiglu ? a.n >> 1 : a.n;
+#pragma unroll
+    for (int tn = 0; tn < 4; tn++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * 128 + 32 * tn + l32] = acc[tn][e];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int col = col0 + l32 * 4;                                    // first of this lane's four columns
+    float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (ep.bias && col < a.n) {
+        if (ep.interleaved_bias) {                                     // even column n: bias[n / 2], odd: bias2[n / 2]
+            const float2 be = *reinterpret_cast<const float2 *>(ep.bias + (col >> 1)), bo = *reinterpret_cast<const float2 *>(ep.bias2 + (col >> 1));
+            b4 = make_float4(be.x, bo.x, be.y, bo.y);
+        } else {
+            b4 = *reinterpret_cast<const float4 *>(ep.bias + col);
+        }
+    }
+#pragma unroll 4
+    for (int i = 0; i < 16; i++) {
+        const int rl = i * 2 + half, row = row0 + rl;
+        float4 v = *reinterpret_cast<const float4 *>(stage_f + rl * 128 + l32 * 4);
+        if (row >= a.m || col >= a.n) continue;
+        const float us = a.unscale[row];
+        v.x = v.x * us; v.y = v.y * us; v.z = v.z * us; v.w = v.w * us;
+        if (ep.bias) { v.x = v.x + b4.x; v.y = v.y + b4.y; v.z = v.z + b4.z; v.w = v.w + b4.w; }
+        if (ep.swiglu) {
+            // (gate, up) pairs in neighbouring columns (SiLU.java:20-24, SwiGLULayer.java:69)
+            float2 o;
+            o.x = v.x * (1.0f / (1.0f + expf(-v.x))) * v.y;
+            o.y = v.z * (1.0f / (1.0f + expf(-v.z))) * v.w;
+            *reinterpret_cast<float2 *>(a.out + (int64_t)row * out_n + (col >> 1)) = o;
+            continue;
+        }
+        if (ep.gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
+        if (ep.residual) {
+            const float4 r = *reinterpret_cast<const float4 *>(ep.residual + (int64_t)row * a.n + col);
+            v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
+        }
+        *reinterpret_cast<float4 *>(a.out + (int64_t)row * a.n + col) = v;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                  // the rows are in registers before anything overwrites them
 }
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16(const GemmF16Args a) {
@@ -199,53 +247,135 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
-    // Epilogue.  acc[tm][tn][e] is C[32 tm + 8 (e / 4) + 4 half + e % 4][32 tn + l32] of the wavefront's 64 x 128 block.
-    // Per tile row: 32 x 128 floats go through this wavefront's 16 KB of LDS and come back as rows of float4.
     float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
-    const GemmEpilogue &ep = a.ep;
-    const int out_n = ep.swiglu ? a.n >> 1 : a.n;
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) {
+    for (int tm = 0; tm < 2; tm++) store_tile_row(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * 128, half, l32);
+}
+
+// The same product on a 64 x 256 workgroup tile, for problems whose 128-row tiles would leave most of the chip idle
+// (a 512-row prompt against 6144 output rows is 96 such tiles on 256 compute units, 192 of these).  A wavefront owns
+// one tile row (32 x 128, 64 accumulators), which leaves registers for two complete operand sets: everything step
+// s + 1 needs is read from its stage during step s, a stage is only ever read during the step before its own, and
+// the loads of step s + 3 go into the stage of step s at the top of step s, behind one barrier per step - two
+// steps of distance for the direct loads instead of one.  Stage: 8 KB of X (2 planes x 64 rows), 16 KB of W, scales.
+constexpr int TM64 = 64;
+constexpr int kXs64 = 2 * TM64 * 64;
+constexpr int kStage64 = kXs64 + kWl + TN * 4;
+constexpr int kLoads64 = 7;                 // per wavefront per stage: 2 of X, 4 of W, 1 of scales
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16_m64(const GemmF16Args a) {
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
+    const int m0 = blockIdx.y * TM64, n0 = blockIdx.x * TN;
+    const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+    float acc[4][16];
 #pragma unroll
-        for (int tn = 0; tn < 4; tn++)
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * 128 + 32 * tn + l32] = acc[tm][tn][e];
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const int col = n0 + wn * 128 + l32 * 4;                       // first of this lane's four columns
-        float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ep.bias && col < a.n) {
-            if (ep.interleaved_bias) {                                 // even column n: bias[n / 2], odd: bias2[n / 2]
-                const float2 be = *reinterpret_cast<const float2 *>(ep.bias + (col >> 1)), bo = *reinterpret_cast<const float2 *>(ep.bias2 + (col >> 1));
-                b4 = make_float4(be.x, bo.x, be.y, bo.y);
-            } else {
-                b4 = *reinterpret_cast<const float4 *>(ep.bias + col);
-            }
-        }
-#pragma unroll 4
-        for (int i = 0; i < 16; i++) {
-            const int rl = i * 2 + half, row = m0 + wm * 64 + 32 * tm + rl;
-            float4 v = *reinterpret_cast<const float4 *>(stage_f + rl * 128 + l32 * 4);
-            if (row >= a.m || col >= a.n) continue;
-            const float us = a.unscale[row];
-            v.x = v.x * us; v.y = v.y * us; v.z = v.z * us; v.w = v.w * us;
-            if (ep.bias) { v.x = v.x + b4.x; v.y = v.y + b4.y; v.z = v.z + b4.z; v.w = v.w + b4.w; }
-            if (ep.swiglu) {
-                // (gate, up) pairs in neighbouring columns (SiLU.java:20-24, SwiGLULayer.java:69)
-                float2 o;
-                o.x = v.x * (1.0f / (1.0f + expf(-v.x))) * v.y;
-                o.y = v.z * (1.0f / (1.0f + expf(-v.z))) * v.w;
-                *reinterpret_cast<float2 *>(a.out + (int64_t)row * out_n + (col >> 1)) = o;
-                continue;
-            }
-            if (ep.gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
-            if (ep.residual) {
-                const float4 r = *reinterpret_cast<const float4 *>(ep.residual + (int64_t)row * a.n + col);
-                v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
-            }
-            *reinterpret_cast<float4 *>(a.out + (int64_t)row * a.n + col) = v;
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");              // the rows are in registers before the next tile row overwrites them
+        for (int e = 0; e < 16; e++) acc[j][e] = 0.f;
+
+    const int prow = lane >> 2, pchunk = (lane & 3) ^ ((prow >> 2) & 3);
+    const uint32_t op_lane = (uint32_t)((prow * a.pitch + pchunk * 8) * 2), s_lane = lane * 4;
+    const unsigned char *x_base[2], *w_base[4];
+    uint32_t x_dst[2], w_dst[4];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int blk = wave * 2 + i, pl = blk >> 2, rb = blk & 3;      // X: 2 planes x 4 row blocks
+        x_base[i] = reinterpret_cast<const unsigned char *>(a.planes) + (pl * plane_elems + (int64_t)(m0 + rb * 16) * a.pitch) * 2;
+        x_dst[i] = pl * TM64 * 64 + rb * 1024;
     }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int blk = wave * 4 + i;                                   // W: 16 row blocks
+        w_base[i] = reinterpret_cast<const unsigned char *>(a.w16) + (int64_t)(n0 + blk * 16) * a.pitch * 2;
+        w_dst[i] = kXs64 + blk * 1024;
+    }
+    const unsigned char *s_base = reinterpret_cast<const unsigned char *>(a.scales_t) + (int64_t)(n0 + wave * 64) * 4;
+    const uint32_t s_dst = kXs64 + kWl + wave * 256;
+    const int steps = a.kp / 32, last = steps - 1;
+    auto load_one = [&](int i, int step, int stage) {
+        const uint32_t sb = lds0 + stage * kStage64;
+        step = min(step, last);
+        if (i < 2) load_to_lds16(x_base[i] + (int64_t)step * 64, op_lane, sb + x_dst[i]);
+        else if (i < 6) load_to_lds16(w_base[i - 2] + (int64_t)step * 64, op_lane, sb + w_dst[i - 2]);
+        else load_to_lds4(s_base + (int64_t)step * a.n_pad * 4, s_lane, sb + s_dst);
+    };
+
+    const int sw = (l32 >> 2) & 3;
+    const int lane_sub0 = (l32 << 6) + (((0 + half) ^ sw) << 4), lane_sub1 = (l32 << 6) + (((2 + half) ^ sw) << 4);
+    const int x_wave = wm * 32 * 64, w_wave = kXs64 + wn * 128 * 64, s_wave = kXs64 + kWl + wn * 128 * 4 + l32 * 4;
+    const floatx16 z16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    halfx8 fx[2][2][2];                 // [set][K half][hi, lo]
+    halfx8 fw[2][2][4];                 // [set][K half][tile column]
+    float sc[2][4];                     // [set][tile column]
+    floatx16 g[2] = {z16, z16};
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) sc[i][j] = 0.f;
+    // read n of the 16 LDS reads that fetch a step's operands, in the order of their first use
+    auto read_one = [&](auto set_c, int n, const unsigned char *x0, const unsigned char *x1, const unsigned char *w0, const unsigned char *w1, const unsigned char *sp) {
+        constexpr int set = decltype(set_c)::value;
+        if (n < 4) fx[set][n >> 1][n & 1] = *reinterpret_cast<const halfx8 *>(((n >> 1) ? x1 : x0) + (n & 1) * TM64 * 64);
+        else if (n < 12) { const int tn = (n - 4) >> 1, sub = (n - 4) & 1; fw[set][sub][tn] = *reinterpret_cast<const halfx8 *>((sub ? w1 : w0) + tn * 2048); }
+        else sc[set][n - 12] = *reinterpret_cast<const float *>(sp + (n - 12) * 128);
+    };
+    auto k_step = [&](auto set_c, int step, int stage) {
+        constexpr int set = decltype(set_c)::value;
+        asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory");   // step + 1 has landed (step + 2 may be in flight); this step's operands are in registers
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const int next = stage == 2 ? 0 : stage + 1;
+        const unsigned char *nb = lds + next * kStage64;
+        const unsigned char *x0 = nb + x_wave + lane_sub0, *x1 = nb + x_wave + lane_sub1, *w0 = nb + w_wave + lane_sub0, *w1 = nb + w_wave + lane_sub1, *sp = nb + s_wave;
+#pragma unroll
+        for (int tn = 0; tn < 4; tn++) {
+            const int par = tn & 1, ptn = (tn + 3) & 3, pset = tn == 0 ? 1 - set : set;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int sub = i >> 1, piece = i & 1, slot = tn * 4 + i;
+                g[par] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fx[set][sub][piece], fw[set][sub][tn], i == 0 ? z16 : g[par], 0, 0, 0);
+                const int f0 = i <= 1 ? 0 : i == 2 ? 6 : 11, f1 = i == 0 ? 0 : i == 1 ? 6 : i == 2 ? 11 : 16;
+#pragma unroll
+                for (int f = f0; f < f1; f++) acc[ptn][f] = fmaf(g[1 - par][f], sc[pset][ptn], acc[ptn][f]);
+                read_one(std::integral_constant<int, 1 - set>{}, slot, x0, x1, w0, w1, sp);
+                if ((slot & 1) && (slot >> 1) < kLoads64) load_one(slot >> 1, step + 3, stage);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    for (int s = 0; s < 3; s++)
+        for (int i = 0; i < kLoads64; i++) load_one(i, s, s);
+    asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    {
+        const unsigned char *x0 = lds + x_wave + lane_sub0, *x1 = lds + x_wave + lane_sub1, *w0 = lds + w_wave + lane_sub0, *w1 = lds + w_wave + lane_sub1, *sp = lds + s_wave;
+        for (int n = 0; n < 16; n++) read_one(std::integral_constant<int, 0>{}, n, x0, x1, w0, w1, sp);
+    }
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    int stage = 0, step = 0;
+    for (; step + 1 < steps; step += 2) {
+        const int st1 = stage == 2 ? 0 : stage + 1;
+        k_step(S0{}, step, stage);
+        k_step(S1{}, step + 1, st1);
+        stage = st1 == 2 ? 0 : st1 + 1;
+    }
+    if (step < steps) k_step(S0{}, step, stage);
+    // the last tile's scaling: column 3 of the last step, whose set is the parity of that step
+    {
+        const bool odd = (steps - 1) & 1;
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[3][e] = fmaf(g[1][e], odd ? sc[1][3] : sc[0][3], acc[3][e]);
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    store_tile_row(a, reinterpret_cast<float *>(lds + wave * (32 * 128 * 4)), acc, m0 + wm * 32, n0 + wn * 128, half, l32);
 }
 
 // One workgroup per row of X: the row's largest magnitude, then the two fp16 planes of x * 2^s.  Columns [k, kp) are
@@ -305,15 +435,25 @@ __global__ void __launch_bounds__(256) k_q8_to_f16(const int8_t *__restrict__ wq
 
 }  // namespace
 
-bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) {
-    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels (for comparisons)
-    static const bool enabled = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return !(e && e[0] == '0'); }();
-    if (!enabled) return false;
-    // few tiles leave most of the chip idle (one 128 x 256 tile per CU at a time); the bf16 kernels with their smaller
-    // tiles take those.  Four columns per lane in the epilogue need n_rows % 4 == 0.
-    const int64_t tiles = (int64_t)((m + TM - 1) / TM) * ((n_rows + TN - 1) / TN);
-    return m >= 256 && (n_rows & 3) == 0 && tiles >= 160 && k >= 64;
+// 128 or 64: the workgroup tile's rows for this problem; 0: the problem is not for these kernels.  A compute unit runs one
+// workgroup at a time, so what counts is how many of the 256 a launch keeps busy and for how many rounds.
+int q8_gemm_f16_tile_rows(int m, int n_rows, int k) {
+    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels, =64 / =128 forces a tile (for comparisons)
+    static const int forced = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return e ? atoi(e) : -1; }();
+    if (forced == 0) return 0;
+    // four columns per lane in the epilogue need n_rows % 4 == 0
+    if (m < 256 || (n_rows & 3) != 0 || k < 64) return 0;
+    const int64_t cols = (n_rows + TN - 1) / TN, t128 = (int64_t)((m + TM - 1) / TM) * cols, t64 = (int64_t)((m + TM64 - 1) / TM64) * cols;
+    if (forced == 128 || forced == 64) return t64 >= 128 ? forced : 0;
+    // measured on 512 rows x K 2048: 11264 output rows (176 / 352 tiles) 84 us with 128-row tiles, 91 us with 64-row
+    // ones; 6144 output rows (96 / 192 tiles) 76 us on the bf16 kernel, 53 us with 64-row tiles; below 128 of the
+    // small tiles (2048 output rows) the bf16 kernels with their 64 x 64 tiles stay ahead
+    if (t128 >= 160) return 128;
+    if (t64 >= 128) return 64;
+    return 0;
 }
+
+bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) { return q8_gemm_f16_tile_rows(m, n_rows, k) != 0; }
 
 // the weights in this kernel's layout: fp16 rows, then the transposed scales (each part 256-byte aligned)
 int64_t q8_prepared_floats(int k, int n_rows) {
@@ -358,9 +498,13 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const int8_t *wq, const f
     static bool configured = false;
     if (!configured) {
         hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
+        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage64), "hipFuncSetAttribute(k_gemm_q8_f16_m64)");
         configured = true;
     }
-    launch_kernel(k_gemm_q8_f16, dim3(n_pad / TN, m_pad / TM), dim3(256), (size_t)kStages * kStage, s, a);
+    if (q8_gemm_f16_tile_rows(m, n_rows, k) == 64)
+        launch_kernel(k_gemm_q8_f16_m64, dim3(n_pad / TN, (m + TM64 - 1) / TM64), dim3(256), (size_t)kStages * kStage64, s, a);
+    else
+        launch_kernel(k_gemm_q8_f16, dim3(n_pad / TN, m_pad / TM), dim3(256), (size_t)kStages * kStage, s, a);
 }
 
 }  // namespace dj

@@ -1086,7 +1086,7 @@ int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows) {
 
 int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows) {
     if (m <= 1 || k <= 0 || rows <= 0) return 0;
-    return q8_gemm_f16_shape_ok(m, rows, k) ? 1 : 0;
+    return q8_gemm_f16_tile_rows(m, rows, k);
 }
 
 int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total) {

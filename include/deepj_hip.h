@@ -217,8 +217,9 @@ int64_t deepj_hip_llama_decode_sync_floats(void);
 /* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
 
-/* Floats of the buffer Q8_PREPARE fills for such a weight (about 2 bytes per weight), and whether a Q8_LINEAR of m
- * rows over it runs on the fp16 direct-load GEMM (1) or on the bf16 kernels (0) when its workspace may grow.
+/* Floats of the buffer Q8_PREPARE fills for such a weight (about 2 bytes per weight), and which kernel a Q8_LINEAR of m
+ * rows over it runs on when its workspace may grow: the fp16 direct-load GEMM with 128 or 64 rows per workgroup tile
+ * (returns 128 or 64), or the bf16 kernels / the matvec (returns 0).
  * No counterpart in the reference, whose weights are fp32 (J/layers/Linear.java:9-24). */
 int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows);
 int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);

@@ -1,7 +1,8 @@
 """The many-row Q8 GEMM on fp16 matrix cores (two-piece activations, direct loads into LDS) through the C ABI against
 the CPU oracle: fp32 CpuBackend.matmul (tensor/cpu/CpuBackend.java:168-188, ikj order) on the dequantised weights.
 
-Shapes are chosen so that the library takes this kernel (HipNative.q8GemmPath says so for each); what the tests vary:
+Shapes are chosen so that the library takes this kernel (HipNative.q8GemmPath says so for each), with its 128-row
+and its 64-row workgroup tile (the shapes with about 160 tiles or more of 128 x 256 take the former); what the tests vary:
 ragged M and N (not multiples of the 128 x 256 tile), K that is not a multiple of the 32-group, every epilogue
 (bias, GELU, residual, interleaved SwiGLU with both biases), the RMSNorm / LayerNorm prologue, rows whose magnitudes span
 twelve decades with outliers and tiny values inside a row, all-zero rows, prepared weights (OP_Q8_PREPARE) against
@@ -43,17 +44,19 @@ def gate(exp):
 
 
 def test_path_query_matches_the_documented_rule():
-    assert HipNative.q8GemmPath(512, 2048, 11264) == 1        # 4 x 44 tiles
-    assert HipNative.q8GemmPath(2048, 4096, 4096) == 1        # 16 x 16
-    assert HipNative.q8GemmPath(512, 2048, 6144) == 0         # 96 tiles: most of the chip would idle
+    assert HipNative.q8GemmPath(512, 2048, 11264) == 128      # 4 x 44 tiles of 128 x 256
+    assert HipNative.q8GemmPath(2048, 4096, 4096) == 128      # 16 x 16
+    assert HipNative.q8GemmPath(512, 2048, 6144) == 64        # 96 such tiles would idle most of the chip: 192 of 64 x 256
+    assert HipNative.q8GemmPath(512, 2048, 2048) == 0         # 64 even of those: the bf16 kernels' 64 x 64 tiles
     assert HipNative.q8GemmPath(1, 2048, 32000) == 0          # the matvec's case
     assert HipNative.q8GemmPath(512, 2048, 11266) == 0        # four columns per lane in the epilogue
     assert HipNative.q8PreparedFloats(2048, 11264) == (11264 * (2048 + 64)) // 2 + 64 * 11264
 
 
-@pytest.mark.parametrize("m,k,n", [(300, 1000, 13828), (257, 96, 40964), (640, 2048, 8192)])
-def test_plain_product_ragged_shapes(dev, m, k, n):
-    assert HipNative.q8GemmPath(m, k, n) == 1
+@pytest.mark.parametrize("m,k,n,tile", [(300, 1000, 13828, 128), (257, 96, 40964, 128), (640, 2048, 8192, 128),
+                                         (300, 1000, 8196, 64), (512, 2048, 6144, 64), (257, 96, 13000, 64)])
+def test_plain_product_ragged_shapes(dev, m, k, n, tile):
+    assert HipNative.q8GemmPath(m, k, n) == tile
     w = JavaRandom(11).tensor(k, n, 0.02)
     x = JavaRandom(12).tensor(m, k, 1.0)
     wq, deq = quantised(dev, w)
@@ -69,7 +72,7 @@ def test_rows_spanning_twelve_decades_with_outliers(dev):
     """Each row gets its own power of two before the fp16 split: a row of 1e-6 magnitudes must come out as exact as a
     row of 1e6; inside a row, values 300 times the typical size and values 1e-4 of it share the row's scale."""
     m, k, n = 260, 512, 40960
-    assert HipNative.q8GemmPath(m, k, n) == 1
+    assert HipNative.q8GemmPath(m, k, n) == 128
     x = JavaRandom(21).tensor(m, k, 1.0)
     x *= (10.0 ** ((np.arange(m) % 13) - 6)).astype(np.float32)[:, None]
     x[:, 5::97] *= 300.0
@@ -92,10 +95,11 @@ def test_rows_spanning_twelve_decades_with_outliers(dev):
     assert worst <= 1e-4
 
 
+@pytest.mark.parametrize("n,tile", [(14336, 128), (9216, 64)])
 @pytest.mark.parametrize("epilogue", ["bias", "bias_gelu", "bias_residual", "residual"])
-def test_epilogues(dev, epilogue):
-    m, k, n = 384, 256, 14336
-    assert HipNative.q8GemmPath(m, k, n) == 1
+def test_epilogues(dev, epilogue, n, tile):
+    m, k = 384, 256
+    assert HipNative.q8GemmPath(m, k, n) == tile
     x = JavaRandom(31).tensor(m, k, 1.0)
     w = JavaRandom(32).tensor(k, n, 0.05)
     b = JavaRandom(33).tensor(1, n, 0.3)
@@ -119,16 +123,17 @@ def test_epilogues(dev, epilogue):
     assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear + {epilogue}")
 
 
+@pytest.mark.parametrize("dff,tile", [(10368, 128), (4352, 64)])
 @pytest.mark.parametrize("norm", ["rms", "layer"])
-def test_swiglu_and_norm_prologues(dev, norm):
+def test_swiglu_and_norm_prologues(dev, norm, dff, tile):
     """gate/up rows interleaved in one Q8 buffer, SiLU(gate) * up in the epilogue (SwiGLULayer.java:63-70), behind an
     RMSNorm prologue; LayerNorm prologue with a plain bias epilogue (GPT's first MLP projection)."""
-    m, d, dff = 300, 320, 10368
+    m, d = 300, 320
     x = JavaRandom(41).tensor(m, d, 1.5)
     gamma = (1.0 + JavaRandom(42).tensor(1, d, 0.1)).astype(np.float32)
     xb, gb = dev.upload(x), dev.upload(gamma)
     if norm == "rms":
-        assert HipNative.q8GemmPath(m, d, 2 * dff) == 1
+        assert HipNative.q8GemmPath(m, d, 2 * dff) == tile
         wg, wu = JavaRandom(43).tensor(d, dff, 0.05), JavaRandom(44).tensor(d, dff, 0.05)
         bg, bu = JavaRandom(45).tensor(1, dff, 0.2), JavaRandom(46).tensor(1, dff, 0.2)
         h = ref.rmsnorm(x, gamma)
@@ -145,7 +150,7 @@ def test_swiglu_and_norm_prologues(dev, norm):
         dev.release(wgu, ob)
     else:
         n = 2 * dff
-        assert HipNative.q8GemmPath(m, d, n) == 1
+        assert HipNative.q8GemmPath(m, d, n) == tile
         beta = JavaRandom(47).tensor(1, d, 0.1)
         w, b = JavaRandom(48).tensor(d, n, 0.05), JavaRandom(49).tensor(1, n, 0.2)
         wq, deq = quantised(dev, w)
@@ -160,7 +165,7 @@ def test_swiglu_and_norm_prologues(dev, norm):
 
 def test_prepared_weights_give_the_same_bits_and_follow_the_weights(dev):
     m, k, n = 512, 512, 10240
-    assert HipNative.q8GemmPath(m, k, n) == 1
+    assert HipNative.q8GemmPath(m, k, n) == 128
     x = JavaRandom(51).tensor(m, k, 1.0)
     w1, w2 = JavaRandom(52).tensor(k, n, 0.02), JavaRandom(53).tensor(k, n, 0.02)
     wq, deq1 = quantised(dev, w1)
