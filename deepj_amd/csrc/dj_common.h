@@ -131,9 +131,10 @@ int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared);
 // [Kp / 32][rows up to a multiple of 256]
 int64_t q8_prepared_floats(int k, int n_rows);
 void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, float *prepared, int k, int n_rows);
-void launch_q8_gemm_f16(hipStream_t s, const float *x, const int8_t *wq, const float *scales, const float *prepared, float *out, int m,
-                        int k, int n_rows, const float *bias, const float *bias2, const float *residual, int interleaved_bias, int gelu,
-                        int swiglu, float *workspace, int64_t workspace_floats);
+// gamma (and beta): the rows are RMS- (Layer-) normalised on their way into the kernel's layout
+void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
+                        const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
+                        const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats);
 
 // kernels_attn.hip
 struct AttnArgs {

@@ -62,6 +62,8 @@ struct GemmF16Args {
     float *out;
     int m, n, m_pad, n_pad, kp, pitch;
     GemmEpilogue ep;
+    int split_steps;            // 64-row kernel only: K steps per workgroup along blockIdx.z (0: all of K, no partial sums)
+    float *partial;             // [gridDim.z][m][n] partial products when split_steps > 0
 };
 
 // 64 lanes x 16 bytes from base + off[lane] into LDS bytes [dst, dst + 1024), lane order
@@ -262,6 +264,7 @@ constexpr int TM64 = 64;
 constexpr int kXs64 = 2 * TM64 * 64;
 constexpr int kStage64 = kXs64 + kWl + TN * 4;
 constexpr int kLoads64 = 7;                 // per wavefront per stage: 2 of X, 4 of W, 1 of scales
+constexpr int kMinSplitSteps = 32;          // K steps a workgroup must at least have when several share a tile's K
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16_m64(const GemmF16Args a) {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -294,10 +297,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
     const unsigned char *s_base = reinterpret_cast<const unsigned char *>(a.scales_t) + (int64_t)(n0 + wave * 64) * 4;
     const uint32_t s_dst = kXs64 + kWl + wave * 256;
-    const int steps = a.kp / 32, last = steps - 1;
+    // this workgroup's share of K: all of it, or split_steps steps from blockIdx.z * split_steps (a partial product)
+    const int all_steps = a.kp / 32, first = a.split_steps ? (int)blockIdx.z * a.split_steps : 0;
+    const int steps = a.split_steps ? min(a.split_steps, all_steps - first) : all_steps, last = first + steps - 1;
     auto load_one = [&](int i, int step, int stage) {
         const uint32_t sb = lds0 + stage * kStage64;
-        step = min(step, last);
+        step = min(first + step, last);
         if (i < 2) load_to_lds16(x_base[i] + (int64_t)step * 64, op_lane, sb + x_dst[i]);
         else if (i < 6) load_to_lds16(w_base[i - 2] + (int64_t)step * 64, op_lane, sb + w_dst[i - 2]);
         else load_to_lds4(s_base + (int64_t)step * a.n_pad * 4, s_lane, sb + s_dst);
@@ -375,41 +380,168 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    store_tile_row(a, reinterpret_cast<float *>(lds + wave * (32 * 128 * 4)), acc, m0 + wm * 32, n0 + wn * 128, half, l32);
+    float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
+    if (a.split_steps) {
+        // a partial product: the bare sums (times the row's power of two) into this split's slab; k_sum_partials finishes them
+        GemmF16Args b = a;
+        b.out = a.partial + (int64_t)blockIdx.z * a.m * a.n;
+        b.ep = GemmEpilogue{nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0};
+        store_tile_row(b, stage_f, acc, m0 + wm * 32, n0 + wn * 128, half, l32);
+        return;
+    }
+    store_tile_row(a, stage_f, acc, m0 + wm * 32, n0 + wn * 128, half, l32);
 }
 
-// One workgroup per row of X: the row's largest magnitude, then the two fp16 planes of x * 2^s.  Columns [k, kp) are
-// written as zeros (the weights' padding is zero as well, but 0 x garbage could be a NaN); rows [m, m_pad) are left
-// alone: they only feed output rows that are never stored.
-__global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, uint16_t *__restrict__ planes, float *__restrict__ unscale,
-                                                   int m, int k, int kp, int pitch, int64_t plane_elems) {
+// out = epilogue(sum over the splits of partial[z]) on float4s: bias, GELU, residual as in store_tile_row (a fixed order
+// of additions, so a run repeats bit for bit - which adding into C with atomics would not)
+__global__ void __launch_bounds__(256) k_sum_partials(const float *__restrict__ partial, float *__restrict__ out, int splits, int64_t mn4, int n4,
+                                                     const float *__restrict__ bias, const float *__restrict__ residual, int gelu) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < mn4; i += (int64_t)gridDim.x * 256) {
+        float4 v = reinterpret_cast<const float4 *>(partial)[i];
+        for (int z = 1; z < splits; z++) {
+            const float4 p = reinterpret_cast<const float4 *>(partial)[(int64_t)z * mn4 + i];
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        if (bias) {
+            const float4 b = reinterpret_cast<const float4 *>(bias)[i % n4];
+            v.x = v.x + b.x; v.y = v.y + b.y; v.z = v.z + b.z; v.w = v.w + b.w;
+        }
+        if (gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
+        if (residual) {
+            const float4 r = reinterpret_cast<const float4 *>(residual)[i];
+            v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
+        }
+        reinterpret_cast<float4 *>(out)[i] = v;
+    }
+}
+
+// One workgroup per row of X: the row's normalisation if asked for (NORM 1: gamma * x / sqrt(mean(x^2) + 1e-6),
+// RMSNorm1D.java:46-57; NORM 2: gamma * (x - mean) / sqrt(var + 1e-5) + beta, LayerNorm1D.java:34-66; the same formulas
+// and unfused multiply-adds as the stand-alone kernels), the largest magnitude of the result, then the two fp16 planes
+// of it times 2^s.  Rows of up to 8192 floats stay in registers in between; longer or ragged ones are read three or four
+// times, from L2 after the first.  Columns [k, kp) are written as zeros
+// (the weights' padding is zero as well, but 0 x garbage could be a NaN); rows [m, m_pad) are left alone: they only
+// feed output rows that are never stored.
+template <int NORM>
+__global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                   uint16_t *__restrict__ planes, float *__restrict__ unscale, int m, int k, int kp, int pitch,
+                                                   int64_t plane_elems) {
+#pragma clang fp contract(off)
     __shared__ float red[4];
     const int row = blockIdx.x, t = threadIdx.x;
     const float *xr = x + (int64_t)row * k;
-    float mx = 0.f;
-    for (int c = t; c < k; c += 256) mx = fmaxf(mx, fabsf(xr[c]));
+    auto block_reduce = [&](float v, bool is_max) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-    if ((t & 63) == 0) red[t >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    // mx = f * 2^e with f in [0.5, 1): s = 15 - e puts it in [2^14, 2^15).  Zero, infinite or NaN rows stay unscaled;
-    // s is kept where 2^s and 2^-s are both normal numbers.
-    int s = 0;
-    if (mx > 0.f && mx < __builtin_inff()) {
-        int e;
-        (void)frexpf(mx, &e);
-        s = max(-126, min(126, 15 - e));
-    }
-    const float up = ldexpf(1.0f, s);
-    if (t == 0) unscale[row] = ldexpf(1.0f, -s);
+        for (int o = 32; o > 0; o >>= 1) { const float u = __shfl_xor(v, o, 64); v = is_max ? fmaxf(v, u) : v + u; }
+        __syncthreads();
+        if ((t & 63) == 0) red[t >> 6] = v;
+        __syncthreads();
+        return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : ((red[0] + red[1]) + red[2]) + red[3];
+    };
+    auto scale_of = [&](float mx) {
+        // mx = f * 2^e with f in [0.5, 1): s = 15 - e puts it in [2^14, 2^15).  Zero, infinite or NaN rows stay
+        // unscaled; s is kept where 2^s and 2^-s are both normal numbers.
+        int s = 0;
+        if (mx > 0.f && mx < __builtin_inff()) {
+            int e;
+            (void)frexpf(mx, &e);
+            s = max(-126, min(126, 15 - e));
+        }
+        if (t == 0) unscale[row] = ldexpf(1.0f, -s);
+        return ldexpf(1.0f, s);
+    };
+    auto halves = [](float v, uint16_t &h, uint16_t &l) {
+        const _Float16 hh = (_Float16)v;
+        const _Float16 ll = (_Float16)(v - (float)hh);
+        h = __builtin_bit_cast(uint16_t, hh);
+        l = __builtin_bit_cast(uint16_t, ll);
+    };
     uint16_t *hi = planes + (int64_t)row * pitch, *lo = hi + plane_elems;
+    constexpr int NV = 8;                                            // 128-bit words a thread keeps of one row
+    if ((k & 3) == 0 && k == kp && k <= 256 * 4 * NV) {
+        // the row stays in registers: one pass over memory
+        const int n4 = k >> 2;
+        const float4 *row4 = reinterpret_cast<const float4 *>(xr);
+        float4 v[NV];
+        float s1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = t + j * 256;
+            v[j] = i < n4 ? row4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (NORM == 1) s1 += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+            if (NORM == 2) s1 += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+        }
+        if (NORM == 1) {
+            const float rms = sqrtf(block_reduce(s1, false) * (1.0f / (float)k) + kRmsEps);
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int i = t + j * 256;
+                if (i >= n4) continue;
+                const float4 g = reinterpret_cast<const float4 *>(gamma)[i];
+                v[j] = make_float4((v[j].x / rms) * g.x, (v[j].y / rms) * g.y, (v[j].z / rms) * g.z, (v[j].w / rms) * g.w);
+            }
+        } else if (NORM == 2) {
+            const float inv = 1.0f / (float)k, mean = block_reduce(s1, false) * inv;
+            float var = 0.f;
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                if (t + j * 256 >= n4) continue;
+                const float a = v[j].x - mean, b = v[j].y - mean, c = v[j].z - mean, d = v[j].w - mean;
+                var += (a * a + b * b) + (c * c + d * d);
+            }
+            const float sd = sqrtf(block_reduce(var, false) * inv + kLayerNormEps);
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int i = t + j * 256;
+                if (i >= n4) continue;
+                const float4 g = reinterpret_cast<const float4 *>(gamma)[i], bt = reinterpret_cast<const float4 *>(beta)[i];
+                v[j] = make_float4(((v[j].x - mean) / sd) * g.x + bt.x, ((v[j].y - mean) / sd) * g.y + bt.y,
+                                   ((v[j].z - mean) / sd) * g.z + bt.z, ((v[j].w - mean) / sd) * g.w + bt.w);
+            }
+        }
+        float mx = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[j].x), fabsf(v[j].y)), fmaxf(fabsf(v[j].z), fabsf(v[j].w))));
+        const float up = scale_of(block_reduce(mx, true));
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = t + j * 256;
+            if (i >= n4) continue;
+            uint16_t h[4], l[4];
+            halves(v[j].x * up, h[0], l[0]); halves(v[j].y * up, h[1], l[1]); halves(v[j].z * up, h[2], l[2]); halves(v[j].w * up, h[3], l[3]);
+            reinterpret_cast<uint2 *>(hi)[i] = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+            reinterpret_cast<uint2 *>(lo)[i] = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
+        }
+        return;
+    }
+    float mean = 0.f, denom = 1.f;
+    if (NORM == 1) {
+        float ss = 0.f;
+        for (int c = t; c < k; c += 256) { const float v = xr[c]; ss += v * v; }
+        denom = sqrtf(block_reduce(ss, false) * (1.0f / (float)k) + kRmsEps);
+    } else if (NORM == 2) {
+        const float inv = 1.0f / (float)k;
+        float sm = 0.f;
+        for (int c = t; c < k; c += 256) sm += xr[c];
+        mean = block_reduce(sm, false) * inv;
+        float var = 0.f;
+        for (int c = t; c < k; c += 256) { const float d = xr[c] - mean; var += d * d; }
+        denom = sqrtf(block_reduce(var, false) * inv + kLayerNormEps);
+    }
+    auto value = [&](int c) {
+        const float v = xr[c];
+        if (NORM == 1) return (v / denom) * gamma[c];
+        if (NORM == 2) return ((v - mean) / denom) * gamma[c] + beta[c];
+        return v;
+    };
+    float mx = 0.f;
+    for (int c = t; c < k; c += 256) mx = fmaxf(mx, fabsf(value(c)));
+    const float up = scale_of(block_reduce(mx, true));
     for (int c = t; c < kp; c += 256) {
-        const float v = c < k ? xr[c] * up : 0.f;
-        const _Float16 h = (_Float16)v;
-        const _Float16 l = (_Float16)(v - (float)h);
-        hi[c] = __builtin_bit_cast(uint16_t, h);
-        lo[c] = __builtin_bit_cast(uint16_t, l);
+        uint16_t h, l;
+        halves(c < k ? value(c) * up : 0.f, h, l);
+        hi[c] = h;
+        lo[c] = l;
     }
 }
 
@@ -435,24 +567,33 @@ __global__ void __launch_bounds__(256) k_q8_to_f16(const int8_t *__restrict__ wq
 
 }  // namespace
 
-// 128 or 64: the workgroup tile's rows for this problem; 0: the problem is not for these kernels.  A compute unit runs one
-// workgroup at a time, so what counts is how many of the 256 a launch keeps busy and for how many rounds.
-int q8_gemm_f16_tile_rows(int m, int n_rows, int k) {
+// How these kernels take a problem: tile_rows 128 or 64 (0: not at all), and for the 64-row kernel the number of
+// workgroups that share K (1: none).  A compute unit runs one workgroup at a time, so what counts is how many of the
+// 256 a launch keeps busy and for how many rounds.
+struct GemmF16Plan { int tile_rows, splits; };
+
+GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
     // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels, =64 / =128 forces a tile (for comparisons)
     static const int forced = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return e ? atoi(e) : -1; }();
-    if (forced == 0) return 0;
+    if (forced == 0) return {0, 1};
     // four columns per lane in the epilogue need n_rows % 4 == 0
-    if (m < 256 || (n_rows & 3) != 0 || k < 64) return 0;
+    if (m < 256 || (n_rows & 3) != 0 || k < 64) return {0, 1};
     const int64_t cols = (n_rows + TN - 1) / TN, t128 = (int64_t)((m + TM - 1) / TM) * cols, t64 = (int64_t)((m + TM64 - 1) / TM64) * cols;
-    if (forced == 128 || forced == 64) return t64 >= 128 ? forced : 0;
+    if (forced == 128 || forced == 64) return {t64 >= 128 ? forced : 0, 1};
     // measured on 512 rows x K 2048: 11264 output rows (176 / 352 tiles) 84 us with 128-row tiles, 91 us with 64-row
-    // ones; 6144 output rows (96 / 192 tiles) 76 us on the bf16 kernel, 53 us with 64-row tiles; below 128 of the
-    // small tiles (2048 output rows) the bf16 kernels with their 64 x 64 tiles stay ahead
-    if (t128 >= 160) return 128;
-    if (t64 >= 128) return 64;
-    return 0;
+    // ones; 6144 output rows (96 / 192 tiles) 76 us on the bf16 kernel, 53 us with 64-row tiles
+    if (t128 >= 160) return {128, 1};
+    if (t64 >= 128) return {64, 1};
+    // few tiles but a long K (512 x 2048 output over K 5632: 64 tiles, 71 us on the bf16 kernel, 47 us as 4 x 64
+    // workgroups): several workgroups per tile, each with a share of K of at least kMinSplitSteps steps, their partial
+    // products summed by a second kernel.  With K 2048 (two shares) it is a tie with the bf16 kernel, which keeps it.
+    const int steps = q8_padded_k(k) / 32;
+    const int splits = (int)std::min<int64_t>(std::min<int64_t>(8, 256 / t64), steps / kMinSplitSteps);
+    if (t64 >= 32 && splits >= 3) return {64, splits};
+    return {0, 1};
 }
 
+int q8_gemm_f16_tile_rows(int m, int n_rows, int k) { return q8_gemm_f16_plan(m, n_rows, k).tile_rows; }
 bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) { return q8_gemm_f16_tile_rows(m, n_rows, k) != 0; }
 
 // the weights in this kernel's layout: fp16 rows, then the transposed scales (each part 256-byte aligned)
@@ -464,7 +605,9 @@ int64_t q8_prepared_floats(int k, int n_rows) {
 // floats of workspace: planes, row factors and, unless the caller holds prepared weights, those
 int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared) {
     const int64_t kp = q8_padded_k(k), pitch = kp + 64, m_pad = round_up(m, TM);
-    return round_up(m_pad * pitch, 64) + round_up(m_pad, 64) + (prepared ? 0 : q8_prepared_floats(k, n_rows));
+    const int splits = q8_gemm_f16_plan(m, n_rows, k).splits;
+    return round_up(m_pad * pitch, 64) + round_up(m_pad, 64) + (prepared ? 0 : q8_prepared_floats(k, n_rows)) +
+           (splits > 1 ? round_up((int64_t)splits * m * n_rows, 64) : 0);
 }
 
 void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, float *prepared, int k, int n_rows) {
@@ -476,9 +619,9 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
     launch_kernel(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
 }
 
-void launch_q8_gemm_f16(hipStream_t s, const float *x, const int8_t *wq, const float *scales, const float *prepared, float *out, int m,
-                        int k, int n_rows, const float *bias, const float *bias2, const float *residual, int interleaved_bias, int gelu,
-                        int swiglu, float *workspace, int64_t workspace_floats) {
+void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
+                        const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
+                        const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats) {
     if (!q8_gemm_f16_shape_ok(m, n_rows, k)) fail("q8_gemm_f16: shape outside this kernel's range");
     if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
@@ -486,24 +629,35 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const int8_t *wq, const f
     float *w = workspace;
     uint16_t *planes = reinterpret_cast<uint16_t *>(w); w += round_up((int64_t)m_pad * pitch, 64);
     float *unscale = w;                                  w += round_up(m_pad, 64);
-    launch_kernel(k_split_f16, dim3(m), dim3(256), 0, s, x, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
+    // gamma alone: RMSNorm of the rows first; gamma and beta: LayerNorm
+    auto split = !gamma ? k_split_f16<0> : beta ? k_split_f16<2> : k_split_f16<1>;
+    launch_kernel(split, dim3(m), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
     if (!prepared) {
         launch_q8_prepare(s, wq, scales, w, k, n_rows);
         prepared = w;
+        w += q8_prepared_floats(k, n_rows);
     }
+    const GemmF16Plan plan = q8_gemm_f16_plan(m, n_rows, k);
+    if (plan.splits > 1 && swiglu) fail("q8_gemm_f16: no SwiGLU epilogue on partial products");
     const uint16_t *w16 = reinterpret_cast<const uint16_t *>(prepared);
     const float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
+    const int split_steps = plan.splits > 1 ? (kp / 32 + plan.splits - 1) / plan.splits : 0;
     GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch,
-                  GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}};
+                  GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}, split_steps, w};
     static bool configured = false;
     if (!configured) {
         hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
         hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage64), "hipFuncSetAttribute(k_gemm_q8_f16_m64)");
         configured = true;
     }
-    if (q8_gemm_f16_tile_rows(m, n_rows, k) == 64)
-        launch_kernel(k_gemm_q8_f16_m64, dim3(n_pad / TN, (m + TM64 - 1) / TM64), dim3(256), (size_t)kStages * kStage64, s, a);
-    else
+    if (plan.tile_rows == 64) {
+        launch_kernel(k_gemm_q8_f16_m64, dim3(n_pad / TN, (m + TM64 - 1) / TM64, plan.splits), dim3(256), (size_t)kStages * kStage64, s, a);
+        if (plan.splits > 1) {
+            const int64_t mn4 = (int64_t)m * n_rows / 4;
+            launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
+                          mn4, n_rows / 4, bias, residual, gelu);
+        }
+    } else
         launch_kernel(k_gemm_q8_f16, dim3(n_pad / TN, m_pad / TM), dim3(256), (size_t)kStages * kStage, s, a);
 }
 

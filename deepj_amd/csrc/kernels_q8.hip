@@ -581,10 +581,10 @@ int64_t q8_linear_workspace_floats(int m, int k, int n, int flags) {
 }
 
 int64_t q8_linear_preferred_workspace_floats(int m, int k, int n, int flags, bool prepared) {
-    int64_t ws = q8_linear_workspace_floats(m, k, n, flags);
+    const int64_t ws = q8_linear_workspace_floats(m, k, n, flags);
     const int n_rows = (flags & DJ_LIN_SWIGLU) ? 2 * n : n;
     const bool mv = (m == 1) && matvec_supported(k);
-    if (!mv && q8_gemm_f16_shape_ok(m, n_rows, k)) ws += q8_gemm_f16_workspace_floats(m, n_rows, k, prepared);
+    if (!mv && q8_gemm_f16_shape_ok(m, n_rows, k)) return std::max(ws, q8_gemm_f16_workspace_floats(m, n_rows, k, prepared));
     return ws;
 }
 
@@ -623,6 +623,15 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     // GEMM path
     if (p.flags & DJ_LIN_ATTN_MERGE) fail("q8_linear: the ATTN_MERGE prologue exists for M = 1 only");
     if (workspace_floats < q8_linear_workspace_floats(p.m, p.k, p.n, p.flags)) fail("q8_linear: workspace too small");
+    if (swiglu && residual) fail("q8_linear: SWIGLU with RESIDUAL is not supported");   // no caller combines them
+    // many rows and enough tiles: the fp16 kernel, when the caller's workspace also holds its prepared operands; the
+    // normalisation happens on the rows' way into that layout
+    const int n_rows = swiglu ? 2 * p.n : p.n;
+    if (!p.m_dev && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
+        launch_q8_gemm_f16(s, p.x, gamma, beta, p.wq, p.scales, p.prepared, p.out, p.m, p.k, n_rows, bias, swiglu ? bias2 : nullptr,
+                           swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, workspace, workspace_floats);
+        return;
+    }
     const float *x = p.x;
     float *ws = workspace;
     if (gamma) {
@@ -630,15 +639,6 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
         else launch_rmsnorm(s, p.x, gamma, ws, p.m, p.k);
         x = ws;
         ws += (int64_t)p.m * p.k;
-    }
-    if (swiglu && residual) fail("q8_linear: SWIGLU with RESIDUAL is not supported");   // no caller combines them
-    // many rows and enough tiles: the fp16 kernel, when the caller's workspace also holds its prepared operands
-    const int n_rows = swiglu ? 2 * p.n : p.n;
-    const int64_t ws_left = workspace_floats - (ws - workspace);
-    if (!p.m_dev && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && ws_left >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
-        launch_q8_gemm_f16(s, x, p.wq, p.scales, p.prepared, p.out, p.m, p.k, n_rows, bias, swiglu ? bias2 : nullptr,
-                           swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, ws, ws_left);
-        return;
     }
     if (swiglu) {
         // the GEMM's epilogue pairs the interleaved gate/up columns, so the 2N-wide product never reaches memory

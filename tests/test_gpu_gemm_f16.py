@@ -5,7 +5,8 @@ Shapes are chosen so that the library takes this kernel (HipNative.q8GemmPath sa
 and its 64-row workgroup tile (the shapes with about 160 tiles or more of 128 x 256 take the former); what the tests vary:
 ragged M and N (not multiples of the 128 x 256 tile), K that is not a multiple of the 32-group, every epilogue
 (bias, GELU, residual, interleaved SwiGLU with both biases), the RMSNorm / LayerNorm prologue, rows whose magnitudes span
-twelve decades with outliers and tiny values inside a row, all-zero rows, prepared weights (OP_Q8_PREPARE) against
+twelve decades with outliers and tiny values inside a row, all-zero rows, K shared by several workgroups whose partial
+products a second kernel sums (few tiles, long K), prepared weights (OP_Q8_PREPARE) against
 per-call conversion, and the loss of that association when the weights are rewritten.
 Gate: |expected - actual| <= atol + 1e-4 |expected| with atol = 1e-4 of the output's rms (the per-op gate of
 src/test/java/io/github/kirstenali/deepj/tensor/metal/MetalBackendTest.java:452-466)."""
@@ -48,6 +49,7 @@ def test_path_query_matches_the_documented_rule():
     assert HipNative.q8GemmPath(2048, 4096, 4096) == 128      # 16 x 16
     assert HipNative.q8GemmPath(512, 2048, 6144) == 64        # 96 such tiles would idle most of the chip: 192 of 64 x 256
     assert HipNative.q8GemmPath(512, 2048, 2048) == 0         # 64 even of those: the bf16 kernels' 64 x 64 tiles
+    assert HipNative.q8GemmPath(512, 5632, 2048) == 64        # the same 64 tiles over a long K: four workgroups share each
     assert HipNative.q8GemmPath(1, 2048, 32000) == 0          # the matvec's case
     assert HipNative.q8GemmPath(512, 2048, 11266) == 0        # four columns per lane in the epilogue
     assert HipNative.q8PreparedFloats(2048, 11264) == (11264 * (2048 + 64)) // 2 + 64 * 11264
@@ -95,10 +97,10 @@ def test_rows_spanning_twelve_decades_with_outliers(dev):
     assert worst <= 1e-4
 
 
-@pytest.mark.parametrize("n,tile", [(14336, 128), (9216, 64)])
+@pytest.mark.parametrize("k,n,tile", [(256, 14336, 128), (256, 9216, 64), (4000, 2052, 64)])   # the last: K shared by four workgroups
 @pytest.mark.parametrize("epilogue", ["bias", "bias_gelu", "bias_residual", "residual"])
-def test_epilogues(dev, epilogue, n, tile):
-    m, k = 384, 256
+def test_epilogues(dev, epilogue, k, n, tile):
+    m = 384
     assert HipNative.q8GemmPath(m, k, n) == tile
     x = JavaRandom(31).tensor(m, k, 1.0)
     w = JavaRandom(32).tensor(k, n, 0.05)
