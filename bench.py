@@ -166,6 +166,52 @@ def matvec_roofline(model, position: int, iters: int = 12):
                       "matvec_time_over_stream_read_time": round(lin_us / launches / read_avg_us, 3)}}
 
 
+MFMA_PEAK_TFLOPS = 2500.0       # MI355X dense fp16 / bf16 matrix-core peak
+
+
+def prefill_roofline(model, n: int, iters: int = 6):
+    """Per-kernel durations of the n-token prompt's command stream, measured live like the decode table (a start and a
+    stop event on each op's main dispatch; the small helpers of a Q8_LINEAR - the activation split, the sum of partial
+    products - are inside the whole-prompt time but not in the per-kernel figure).  A projection's algorithmic work is
+    one multiply-add per weight per row, 2 M K N flops; the fp16 kernels issue two matrix-core products for it (hi and
+    lo halves of the activation), the bf16 kernels three - `issued` counts those against the same peak."""
+    from deepj_amd import HipNative, opcodes as op
+    stream = model.prefillStream(n)
+    ops = decode_ops(stream)
+    HipNative.profileOps(stream, 2)
+    us = HipNative.profileOps(stream, iters)
+    names = {(2048, 6144): "qkv", (2048, 2048): "wo", (2048, 11264): "gate_up", (5632, 2048): "down"}
+    table, flops, gemm_us, issued = {}, 0.0, 0.0, 0.0
+    for (code, w), t in zip(ops, us):
+        if code == op.OP_Q8_LINEAR and w[4] > 1 and t > 0:
+            m, k, nn, flags = w[4], w[5], w[6], w[7]
+            rows = 2 * nn if flags & op.LIN_SWIGLU else nn
+            tile = HipNative.q8GemmPath(m, k, rows)
+            f = 2.0 * m * k * rows
+            e = table.setdefault(names.get((k, rows), f"{k}x{rows}"), {
+                "launches": 0, "us": 0.0, "flops": f,
+                "kernel": f"k_gemm_q8_f16 ({tile} x 256 tiles, fp16 x 2)" if tile else "k_gemm_q8 (bf16 x 3)"})
+            e["launches"] += 1
+            e["us"] += float(t)
+            flops += f
+            gemm_us += float(t)
+            issued += f * (2 if tile else 3)
+        elif code == op.OP_ATTENTION and t > 0:
+            e = table.setdefault("attention", {"launches": 0, "us": 0.0, "kernel": "k_attention_tiled (fp32 matrix cores)"})
+            e["launches"] += 1
+            e["us"] += float(t)
+    for e in table.values():
+        e["us"] = round(e["us"] / e["launches"], 2)
+        if "flops" in e:
+            e["TFLOPs"] = round(e.pop("flops") / e["us"] / 1e6, 1)
+            e["frac"] = round(e["TFLOPs"] / MFMA_PEAK_TFLOPS, 4)
+    achieved = flops / gemm_us / 1e6
+    return {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "issued_frac": round(issued / gemm_us / 1e6 / MFMA_PEAK_TFLOPS, 4),
+            "kernel": "Q8 GEMM of the prompt's projections", "rows": n, "per_kernel": table,
+            "timing": "mean kernel duration (start/stop events on each dispatch, whole prompt in order)"}
+
+
 def calibration_copy(mib: int = 256, repeats: int = 3) -> None:
     """A plain device copy of known size (reads `mib` MiB, writes `mib` MiB per launch), so that a
     hardware-counter run of this script has a kernel (k_copy) whose FETCH_SIZE / WRITE_SIZE readings
@@ -226,6 +272,12 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--eager", action="store_true",
+                    help="decode without the HIP graph (same kernels, launched one by one): for runs under a tracer")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="stop after the prompt: prints the prefill object alone (short runs under a counter-collecting profiler)")
+    ap.add_argument("--table-iters", type=int, default=12,
+                    help="passes behind the per-kernel tables; counter-collecting profilers serialise every dispatch, 1 keeps such runs short")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (one MI355X per box); --gpus > 1 is not supported", file=sys.stderr)
@@ -252,25 +304,36 @@ def main() -> int:
     model.prefill(prompt)
     HipNative.synchronize()
     t_prefill = time.perf_counter() - t0
+    model.reset()
+    prefill_roof = prefill_roofline(model, args.prompt, max(1, args.table_iters // 2))
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s, Q8 Llama d=2048 L=16, 1 GPU", "value": round(args.prompt / t_prefill, 1),
+                          "unit": "tok/s", "n_gpus": 1, "prompt_tokens": args.prompt, "prefill": prefill_roof}))
+        model.close()
+        return 0
+    model.reset()
+    model.prefill(prompt)
+    HipNative.synchronize()
 
-    model.decode(args.warmup)                       # captures the graph on first use
+    graph = False if args.eager else None
+    model.decode(args.warmup, use_graph=graph)      # captures the graph on first use
     HipNative.synchronize()
     t0 = time.perf_counter()
-    model.decode(args.steps)
+    model.decode(args.steps, use_graph=graph)
     HipNative.synchronize()
     elapsed = time.perf_counter() - t0
     toks = model.tokens()
     assert len(toks) == 1 + args.warmup + args.steps
 
-    roof = matvec_roofline(model, args.prompt + args.warmup + args.steps)
+    roof = matvec_roofline(model, args.prompt + args.warmup + args.steps, args.table_iters)
     model.reset()
     # the same decode at three times the context (the cache read grows with the position, the weights do not)
     long_prompt = JavaRandom(3).ints(1536, cfg.vocabSize)
     model.prefill(long_prompt)
-    model.decode(8)
+    model.decode(8, use_graph=graph)
     HipNative.synchronize()
     t0 = time.perf_counter()
-    model.decode(128)
+    model.decode(128, use_graph=graph)
     HipNative.synchronize()
     t_long = (time.perf_counter() - t0) / 128
     model.reset()
@@ -298,6 +361,7 @@ def main() -> int:
                        "prefill_tok_s": round(args.prompt / t_prefill, 1),
                        "first_prefill_ms": round(t_first_prefill * 1e3, 2), "model_build_s": round(t_build, 1),
                        "decode_tok_s_at_context_1536": round(1.0 / t_long, 1)},
+        "prefill": prefill_roof,
     }
     print(json.dumps(line))
     model.close()

@@ -628,7 +628,7 @@ void launch_rope_kv_store(hipStream_t s, const float *qkv, float *q_out, float *
     if (total <= 0) return;
     int64_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(k_rope_kv_store, dim3((int)blocks), dim3(kThreads), 0, s, qkv, q_out, k_cache, v_cache, state,
+    launch_kernel(k_rope_kv_store, dim3((int)blocks), dim3(kThreads), 0, s, qkv, q_out, k_cache, v_cache, state,
                        cos_t, sin_t, S, H, hd, max_seq);
 }
 
@@ -716,9 +716,9 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
         if ((int64_t)tg.x * tg.y * 2 < kAttnFullGrid) {  // far too few workgroups for the chip: 32 rows each, keys in four sets
             dim3 tg4(p.h, (p.s + 31) / 32);
             switch (p.hd) {
-                case 32: hipLaunchKernelGGL((k_attention_tiled<32, 4>), tg4, dim3(256), 0, s, a); break;
-                case 64: hipLaunchKernelGGL((k_attention_tiled<64, 4>), tg4, dim3(256), 0, s, a); break;
-                case 128: hipLaunchKernelGGL((k_attention_tiled<128, 4>), tg4, dim3(256), 0, s, a); break;
+                case 32: launch_kernel((k_attention_tiled<32, 4>), tg4, dim3(256), 0, s, a); break;
+                case 64: launch_kernel((k_attention_tiled<64, 4>), tg4, dim3(256), 0, s, a); break;
+                case 128: launch_kernel((k_attention_tiled<128, 4>), tg4, dim3(256), 0, s, a); break;
                 default: fail("attention: head dim must be 32, 64 or 128");
             }
             return;
@@ -726,17 +726,17 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
         if ((int64_t)tg.x * tg.y < kAttnFullGrid) {      // too few: 64 rows each, keys in two sets
             dim3 tg2(p.h, (p.s + 63) / 64);
             switch (p.hd) {
-                case 32: hipLaunchKernelGGL((k_attention_tiled<32, 2>), tg2, dim3(256), 0, s, a); break;
-                case 64: hipLaunchKernelGGL((k_attention_tiled<64, 2>), tg2, dim3(256), 0, s, a); break;
-                case 128: hipLaunchKernelGGL((k_attention_tiled<128, 2>), tg2, dim3(256), 0, s, a); break;
+                case 32: launch_kernel((k_attention_tiled<32, 2>), tg2, dim3(256), 0, s, a); break;
+                case 64: launch_kernel((k_attention_tiled<64, 2>), tg2, dim3(256), 0, s, a); break;
+                case 128: launch_kernel((k_attention_tiled<128, 2>), tg2, dim3(256), 0, s, a); break;
                 default: fail("attention: head dim must be 32, 64 or 128");
             }
             return;
         }
         switch (p.hd) {
-            case 32: hipLaunchKernelGGL((k_attention_tiled<32, 1>), tg, dim3(256), 0, s, a); break;
-            case 64: hipLaunchKernelGGL((k_attention_tiled<64, 1>), tg, dim3(256), 0, s, a); break;
-            case 128: hipLaunchKernelGGL((k_attention_tiled<128, 1>), tg, dim3(256), 0, s, a); break;
+            case 32: launch_kernel((k_attention_tiled<32, 1>), tg, dim3(256), 0, s, a); break;
+            case 64: launch_kernel((k_attention_tiled<64, 1>), tg, dim3(256), 0, s, a); break;
+            case 128: launch_kernel((k_attention_tiled<128, 1>), tg, dim3(256), 0, s, a); break;
             default: fail("attention: head dim must be 32, 64 or 128");
         }
         return;

@@ -61,6 +61,7 @@ struct GemmF16Args {
     const float *unscale;       // [m_pad]: 2^-s of the row
     float *out;
     int m, n, m_pad, n_pad, kp, pitch;
+    int m_tiles, n_tiles;       // tiles of the launched kernel's size along M and N
     GemmEpilogue ep;
     int split_steps;            // 64-row kernel only: K steps per workgroup along blockIdx.z (0: all of K, no partial sums)
     float *partial;             // [gridDim.z][m][n] partial products when split_steps > 0
@@ -72,6 +73,17 @@ __device__ __forceinline__ void load_to_lds16(const void *base, uint32_t off, ui
 }
 __device__ __forceinline__ void load_to_lds4(const void *base, uint32_t off, uint32_t dst) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
+}
+
+// Workgroup -> tile.  Workgroups go to the eight XCDs (each with its own L2) round-robin by their linear index, so index L
+// runs on XCD L % 8.  All row tiles of one column tile get indices that agree mod 8: the column tile's weights - the
+// bulk of the traffic - are then fetched into one L2 instead of up to eight.  Groups of eight column tiles; the grid is
+// padded to whole groups and the surplus workgroups leave at once.
+__device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int &m_tile, int &n_tile) {
+    const int per_group = 8 * m_tiles, g = blockIdx.x / per_group, r = blockIdx.x % per_group;
+    n_tile = g * 8 + (r & 7);
+    m_tile = r >> 3;
+    return n_tile < n_tiles;
 }
 
 // One tile row of a wavefront's block: acc[tn][e] is C[row0 + 8 (e / 4) + 4 half + e % 4][col0 + 32 tn + l32].  The 32 x 128
@@ -125,7 +137,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     extern __shared__ __align__(16) unsigned char lds[];
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
-    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    int m_tile, n_tile;
+    if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
+    const int m0 = m_tile * TM, n0 = n_tile * TN;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
     float acc[2][4][16];
@@ -270,7 +284,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     extern __shared__ __align__(16) unsigned char lds[];
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
-    const int m0 = blockIdx.y * TM64, n0 = blockIdx.x * TN;
+    int m_tile, n_tile;
+    if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
+    const int m0 = m_tile * TM64, n0 = n_tile * TN;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
     float acc[4][16];
@@ -616,7 +632,7 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
     uint16_t *w16 = reinterpret_cast<uint16_t *>(prepared);
     float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
     const int64_t items = (int64_t)n_rows * (kp / 8);
-    launch_kernel(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
+    hipLaunchKernelGGL(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
 }
 
 void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
@@ -631,7 +647,8 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     float *unscale = w;                                  w += round_up(m_pad, 64);
     // gamma alone: RMSNorm of the rows first; gamma and beta: LayerNorm
     auto split = !gamma ? k_split_f16<0> : beta ? k_split_f16<2> : k_split_f16<1>;
-    launch_kernel(split, dim3(m), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
+    // (the helpers are ordinary launches: per-kernel timing of this op, launch_kernel's business, is the GEMM's)
+    hipLaunchKernelGGL(split, dim3(m), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
     if (!prepared) {
         launch_q8_prepare(s, wq, scales, w, k, n_rows);
         prepared = w;
@@ -642,7 +659,9 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     const uint16_t *w16 = reinterpret_cast<const uint16_t *>(prepared);
     const float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
     const int split_steps = plan.splits > 1 ? (kp / 32 + plan.splits - 1) / plan.splits : 0;
-    GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch,
+    const int n_tiles = n_pad / TN, m_tiles = plan.tile_rows == 64 ? (m + TM64 - 1) / TM64 : m_pad / TM;
+    const unsigned grid_x = (unsigned)((n_tiles + 7) / 8 * 8 * m_tiles);
+    GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch, m_tiles, n_tiles,
                   GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}, split_steps, w};
     static bool configured = false;
     if (!configured) {
@@ -651,14 +670,14 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
         configured = true;
     }
     if (plan.tile_rows == 64) {
-        launch_kernel(k_gemm_q8_f16_m64, dim3(n_pad / TN, (m + TM64 - 1) / TM64, plan.splits), dim3(256), (size_t)kStages * kStage64, s, a);
+        launch_kernel(k_gemm_q8_f16_m64, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * kStage64, s, a);
         if (plan.splits > 1) {
             const int64_t mn4 = (int64_t)m * n_rows / 4;
-            launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
-                          mn4, n_rows / 4, bias, residual, gelu);
+            hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
+                               mn4, n_rows / 4, bias, residual, gelu);
         }
     } else
-        launch_kernel(k_gemm_q8_f16, dim3(n_pad / TN, m_pad / TM), dim3(256), (size_t)kStages * kStage, s, a);
+        launch_kernel(k_gemm_q8_f16, dim3(grid_x), dim3(256), (size_t)kStages * kStage, s, a);
 }
 
 }  // namespace dj

@@ -531,18 +531,18 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
         const int64_t tiles = (int64_t)grid2.x * grid2.y, rounds = (tiles + 511) / 512;
         if (tiles * 100 < rounds * 512 * 85) {
             dim3 gridw(grid2.x, (m + 63) / 64);
-            hipLaunchKernelGGL((k_gemm_q8<1, 2, 2, 1>), gridw, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+            launch_kernel((k_gemm_q8<1, 2, 2, 1>), gridw, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
             return;
         }
-        hipLaunchKernelGGL((k_gemm_q8<2, 2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        launch_kernel((k_gemm_q8<2, 2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
         return;
     }
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
     // few tiles (about one per CU): a workgroup brings its own second wavefront per SIMD
     if ((int64_t)grid.x * grid.y <= kFewTiles)
-        hipLaunchKernelGGL((k_gemm_q8<1, 1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        launch_kernel((k_gemm_q8<1, 1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
     else
-        hipLaunchKernelGGL((k_gemm_q8<1, 1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        launch_kernel((k_gemm_q8<1, 1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
 }
 
 }  // namespace dj

@@ -491,18 +491,11 @@ void check_ids(const Config &c, const int32_t *ids, int n) {
         if (ids[i] < 0 || ids[i] >= c.vocab) throw Error("Token id out of range: " + std::to_string(ids[i]));   // Embedding.java:30-32
 }
 
-// Runs the prompt rows through the model, filling the cache.  Leaves the last row's
-// logits in r.logits; with choose != 0 also picks the next token greedily on the device.
-void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choose) {
+// The command stream that takes the n token ids in r.pre.ids through the model at the current position.
+Stream prompt_stream(Runner &r, int n, bool choose) {
     const Config &c = r.cfg;
-    if (!r.finalized) finalize(r);
-    if (n <= 0) throw Error("prefill: empty prompt");
-    check_ids(c, ids, n);
-    if (r.pos + n > c.max_seq)
-        throw Error("context of " + std::to_string(r.pos + n) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
     alloc_acts(r, r.pre, n);
     ensure_prepared(r, n);
-    hip(deepj_hip_upload(r.pre.ids, reinterpret_cast<const float *>(ids), n));
     Stream s;
     emit(s, DJ_OP_EMBED_GATHER, r.emb, r.pre.ids, r.pre.x, n, c.d, c.vocab, 0);
     positions(r, s, r.pre.x, n);
@@ -513,6 +506,20 @@ void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choos
         emit(s, DJ_OP_DECODE_NEXT, r.logits, r.state, r.tokens, c.max_seq, r.emb, r.dec.x, c.vocab, c.d, n);
         if (r.pos + n < c.max_seq) positions(r, s, r.dec.x, 1);     // a full cache takes no further token
     }
+    return s;
+}
+
+// Runs the prompt rows through the model, filling the cache.  Leaves the last row's
+// logits in r.logits; with choose != 0 also picks the next token greedily on the device.
+void prefill(Runner &r, const int32_t *ids, int n, float *all_logits, bool choose) {
+    const Config &c = r.cfg;
+    if (!r.finalized) finalize(r);
+    if (n <= 0) throw Error("prefill: empty prompt");
+    check_ids(c, ids, n);
+    if (r.pos + n > c.max_seq)
+        throw Error("context of " + std::to_string(r.pos + n) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
+    Stream s = prompt_stream(r, n, choose);
+    hip(deepj_hip_upload(r.pre.ids, reinterpret_cast<const float *>(ids), n));   // (prompt_stream sized r.pre for n rows)
     r.run(s);
     if (all_logits) {
         // DecoderOnlyModel.forward returns logits for every row; only parity tests ask for them.
@@ -900,6 +907,19 @@ int deepj_runner_generate(void *h, const int32_t *prompt, int32_t n_prompt, int3
     return guarded(r, [&] {
         if (mode < 0 || mode > 2) throw Error("generate: mode must be 0 (eager), 1 (graph) or 2 (persistent kernel)");
         generate(*r, prompt, n_prompt, max_new, temperature, top_k, seed, out, mode);
+    });
+}
+
+// The command stream of an n-token prompt at the current position, over the ids of the last prefill of that length
+// (for inspection and timing by the caller; running it advances nothing on the host side).
+int deepj_runner_prefill_stream(void *h, int32_t n, int32_t *out, int32_t capacity, int32_t *len) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] {
+        if (!r->finalized) finalize(*r);
+        if (n <= 0 || r->pos + n > r->cfg.max_seq) throw Error("prefill_stream: row count outside the context window");
+        Stream s = prompt_stream(*r, n, false);
+        if (len) *len = (int32_t)s.size();
+        if (out && capacity >= (int32_t)s.size()) std::memcpy(out, s.data(), s.size() * sizeof(int32_t));
     });
 }
 

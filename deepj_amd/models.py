@@ -44,6 +44,7 @@ def _lib():
         lib.deepj_runner_generate.argtypes = [C.c_void_p, _i32p, C.c_int32, C.c_int32, C.c_float, C.c_int32,
                                               C.c_int64, C.c_int32, _i32p]
         lib.deepj_runner_decode_stream.argtypes = [C.c_void_p, _i32p, C.c_int32, _i32p]
+        lib.deepj_runner_prefill_stream.argtypes = [C.c_void_p, C.c_int32, _i32p, C.c_int32, _i32p]
         lib.deepj_host_random_create.argtypes = [C.c_int64]
         lib.deepj_host_random_create.restype = C.c_void_p
         lib.deepj_host_random_destroy.argtypes = [C.c_void_p]
@@ -244,6 +245,14 @@ class _DecoderOnlyModel:
         n = C.c_int32()
         self._check(_lib().deepj_runner_tokens(self._h, out.ctypes.data_as(_i32p), out.size, C.byref(n)))
         return out[: n.value].copy()
+
+    def prefillStream(self, n: int) -> np.ndarray:
+        """The command stream of an n-token prompt at the current position (ids: those of the last prefill)."""
+        ln = C.c_int32()
+        self._check(_lib().deepj_runner_prefill_stream(self._h, n, None, 0, C.byref(ln)))
+        out = np.empty(ln.value, dtype=np.int32)
+        self._check(_lib().deepj_runner_prefill_stream(self._h, n, out.ctypes.data_as(_i32p), out.size, C.byref(ln)))
+        return out
 
     def decodeStream(self) -> np.ndarray:
         n = C.c_int32()

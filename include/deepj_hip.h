@@ -269,6 +269,8 @@ int deepj_runner_tokens(void *runner, int32_t *out, int32_t capacity, int32_t *n
 int deepj_runner_generate(void *runner, const int32_t *prompt, int32_t n_prompt, int32_t max_new,
                           float temperature, int32_t top_k, int64_t seed, int32_t mode, int32_t *out);
 int deepj_runner_decode_stream(void *runner, int32_t *out, int32_t capacity, int32_t *len);
+/* the command stream of an n-token prompt at the current position (over the ids the last prefill uploaded) */
+int deepj_runner_prefill_stream(void *runner, int32_t n, int32_t *out, int32_t capacity, int32_t *len);
 
 #ifdef __cplusplus
 }
