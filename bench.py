@@ -304,16 +304,13 @@ def main() -> int:
     model.prefill(prompt)
     HipNative.synchronize()
     t_prefill = time.perf_counter() - t0
-    model.reset()
-    prefill_roof = prefill_roofline(model, args.prompt, max(1, args.table_iters // 2))
     if args.prefill_only:
+        model.reset()
+        prefill_roof = prefill_roofline(model, args.prompt, max(1, args.table_iters // 2))
         print(json.dumps({"metric": "prefill tok/s, Q8 Llama d=2048 L=16, 1 GPU", "value": round(args.prompt / t_prefill, 1),
                           "unit": "tok/s", "n_gpus": 1, "prompt_tokens": args.prompt, "prefill": prefill_roof}))
         model.close()
         return 0
-    model.reset()
-    model.prefill(prompt)
-    HipNative.synchronize()
 
     graph = False if args.eager else None
     model.decode(args.warmup, use_graph=graph)      # captures the graph on first use
@@ -336,6 +333,10 @@ def main() -> int:
     model.decode(128, use_graph=graph)
     HipNative.synchronize()
     t_long = (time.perf_counter() - t0) / 128
+    model.reset()
+    model.prefill(prompt)
+    model.reset()
+    prefill_roof = prefill_roofline(model, args.prompt, max(1, args.table_iters // 2))
     model.reset()
     calibration_copy()
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg, args.prompt)
