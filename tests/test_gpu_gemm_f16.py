@@ -70,6 +70,40 @@ def test_plain_product_ragged_shapes(dev, m, k, n, tile):
     assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear M={m} K={k} N={n}")
 
 
+def test_random_shapes_both_tiles_and_shared_k(dev):
+    """Seeded random (M, K, N) over the kernel's whole domain - M not a multiple of 64, K not a multiple of 32, N only a
+    multiple of 4 - until each of the three ways the library takes a problem (128-row tiles, 64-row tiles, 64-row tiles
+    with K shared by several workgroups) has been exercised twice."""
+    rng = np.random.default_rng(20240607)
+    seen = {"128": 0, "64": 0, "64 shared": 0}
+    tries = 0
+    while min(seen.values()) < 2 and tries < 200:
+        tries += 1
+        m = int(rng.integers(256, 700))
+        k = int(rng.integers(64, 6000))
+        n = 4 * int(rng.integers(128, 4000))
+        tile = HipNative.q8GemmPath(m, k, n)
+        if tile == 0:
+            continue
+        cols = -(-n // 256)
+        shared = tile == 64 and -(-m // 64) * cols < 128
+        key = "64 shared" if shared else str(tile)
+        if seen[key] >= 2:
+            continue
+        seen[key] += 1
+        w = (rng.standard_normal((k, n)) * 0.03).astype(np.float32)
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        r = rng.standard_normal((m, n)).astype(np.float32)
+        wq, deq = quantised(dev, w)
+        exp = ref.add(r, ref.matmul(x, deq))
+        xb, rb, ob = dev.upload(x), dev.upload(r), dev.alloc(m * n)
+        Stream().q8_linear(xb, wq, ob, m, k, n, residual=rb).run()
+        got = dev.download(ob, (m, n))
+        dev.release(xb, rb, ob, wq)
+        assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear M={m} K={k} N={n} ({key})")
+    assert min(seen.values()) >= 2, seen
+
+
 def test_rows_spanning_twelve_decades_with_outliers(dev):
     """Each row gets its own power of two before the fp16 split: a row of 1e-6 magnitudes must come out as exact as a
     row of 1e6; inside a row, values 300 times the typical size and values 1e-4 of it share the row's scale."""
