@@ -186,11 +186,12 @@ def prefill_roofline(model, n: int, iters: int = 6):
         if code == op.OP_Q8_LINEAR and w[4] > 1 and t > 0:
             m, k, nn, flags = w[4], w[5], w[6], w[7]
             rows = 2 * nn if flags & op.LIN_SWIGLU else nn
-            tile = HipNative.q8GemmPath(m, k, rows)
+            tile, tile_cols, shares = HipNative.q8GemmTile(m, k, rows)
             f = 2.0 * m * k * rows
             e = table.setdefault(names.get((k, rows), f"{k}x{rows}"), {
                 "launches": 0, "us": 0.0, "flops": f,
-                "kernel": f"k_gemm_q8_f16 ({tile} x 256 tiles, fp16 x 2)" if tile else "k_gemm_q8 (bf16 x 3)"})
+                "kernel": (f"k_gemm_q8_f16 ({tile} x {tile_cols} tiles" + (f", K shared by {shares}" if shares > 1 else "") +
+                           ", fp16 x 2)") if tile else "k_gemm_q8 (bf16 x 3)"})
             e["launches"] += 1
             e["us"] += float(t)
             flops += f

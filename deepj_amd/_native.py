@@ -39,6 +39,8 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_prepared_floats.restype = C.c_int64
     lib.deepj_hip_q8_gemm_path.argtypes = [C.c_int32, C.c_int32, C.c_int32]
     lib.deepj_hip_q8_gemm_path.restype = C.c_int32
+    lib.deepj_hip_q8_gemm_tile.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
+    lib.deepj_hip_q8_gemm_tile.restype = None
     lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
     lib.deepj_hip_profile_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p, C.c_int32, _i32p]
     lib.deepj_hip_graph_capture.argtypes = [_i32p, C.c_int32, _i32p]
@@ -152,6 +154,13 @@ class HipNative:
     def q8PreparedFloats(k: int, rows: int) -> int:
         """Floats of the buffer OP_Q8_PREPARE fills for a Q8 weight of `rows` rows over k inputs."""
         return int(library().deepj_hip_q8_prepared_floats(k, rows))
+
+    @staticmethod
+    def q8GemmTile(m: int, k: int, rows: int):
+        """(tile rows, tile columns, workgroups sharing a tile's K) of the fp16 GEMM for this problem; rows 0: not taken."""
+        r, c, s = C.c_int32(), C.c_int32(), C.c_int32()
+        library().deepj_hip_q8_gemm_tile(m, k, rows, C.byref(r), C.byref(c), C.byref(s))
+        return r.value, c.value, s.value
 
     @staticmethod
     def q8GemmPath(m: int, k: int, rows: int) -> int:

@@ -86,20 +86,26 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int 
     return n_tile < n_tiles;
 }
 
-// One tile row of a wavefront's block: acc[tn][e] is C[row0 + 8 (e / 4) + 4 half + e % 4][col0 + 32 tn + l32].  The 32 x 128
-// floats go through 16 KB of LDS that belong to this wavefront alone and come back as rows of float4 (lane l32 + 32 half:
-// rows 2 i + half, columns 4 l32 ..), which get the row's power of two, bias / GELU / residual or the SwiGLU pairing.
-__device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stage_f, const float (&acc)[4][16], int row0, int col0, int half, int l32) {
+// One tile row of a wavefront's block: acc[tn][e] is C[row0 + 8 (e / 4) + 4 half + e % 4][col0 + 32 tn + l32], TNW tiles
+// wide.  The 32 x 32 TNW floats go through LDS that belongs to this wavefront alone (16 KB) and come back as rows of
+// float4 (8 TNW lanes per row, two rows per round), which get the row's power of two, bias / GELU / residual or the
+// SwiGLU pairing.
+template <int TNW>
+__device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stage_f, const float (&acc)[TNW][16], int row0, int col0, int lane) {
+    constexpr int W = 32 * TNW, LPR = 8 * TNW;                         // floats per row; lanes per row
     const GemmEpilogue &ep = a.ep;
     const int out_n = ep.swiglu ? a.n >> 1 : a.n;
+    const int half = lane >> 5, l32 = lane & 31;
 #pragma unroll
-    for (int tn = 0; tn < 4; tn++)
+    for (int tn = 0; tn < TNW; tn++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * 128 + 32 * tn + l32] = acc[tn][e];
+        for (int e = 0; e < 16; e++) stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * W + 32 * tn + l32] = acc[tn][e];
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    const int col = col0 + l32 * 4;                                    // first of this lane's four columns
+    const int rsel = lane / LPR, c4 = lane % LPR;                      // this lane's row of the pair, and its float4 in the row
+    const bool active = rsel < 2;
+    const int col = col0 + c4 * 4;                                     // first of this lane's four columns
     float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (ep.bias && col < a.n) {
+    if (active && ep.bias && col < a.n) {
         if (ep.interleaved_bias) {                                     // even column n: bias[n / 2], odd: bias2[n / 2]
             const float2 be = *reinterpret_cast<const float2 *>(ep.bias + (col >> 1)), bo = *reinterpret_cast<const float2 *>(ep.bias2 + (col >> 1));
             b4 = make_float4(be.x, bo.x, be.y, bo.y);
@@ -109,9 +115,9 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
     }
 #pragma unroll 4
     for (int i = 0; i < 16; i++) {
-        const int rl = i * 2 + half, row = row0 + rl;
-        float4 v = *reinterpret_cast<const float4 *>(stage_f + rl * 128 + l32 * 4);
-        if (row >= a.m || col >= a.n) continue;
+        const int rl = i * 2 + rsel, row = row0 + rl;
+        if (!active || row >= a.m || col >= a.n) continue;
+        float4 v = *reinterpret_cast<const float4 *>(stage_f + rl * W + c4 * 4);
         const float us = a.unscale[row];
         v.x = v.x * us; v.y = v.y * us; v.z = v.z * us; v.w = v.w * us;
         if (ep.bias) { v.x = v.x + b4.x; v.y = v.y + b4.y; v.z = v.z + b4.z; v.w = v.w + b4.w; }
@@ -265,40 +271,46 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) store_tile_row(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * 128, half, l32);
+    for (int tm = 0; tm < 2; tm++) store_tile_row<4>(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * 128, lane);
 }
 
-// The same product on a 64 x 256 workgroup tile, for problems whose 128-row tiles would leave most of the chip idle
-// (a 512-row prompt against 6144 output rows is 96 such tiles on 256 compute units, 192 of these).  A wavefront owns
-// one tile row (32 x 128, 64 accumulators), which leaves registers for two complete operand sets: everything step
-// s + 1 needs is read from its stage during step s, a stage is only ever read during the step before its own, and
-// the loads of step s + 3 go into the stage of step s at the top of step s, behind one barrier per step - two
-// steps of distance for the direct loads instead of one.  Stage: 8 KB of X (2 planes x 64 rows), 16 KB of W, scales.
+// The same product on a 64-row workgroup tile, 256 (TNW = 4) or 192 (TNW = 3) columns wide, for problems whose 128-row
+// tiles would leave most of the chip idle (a 512-row prompt against 6144 output rows is 96 such tiles on 256 compute
+// units, 192 of 64 x 256 and exactly 256 of 64 x 192).  A wavefront owns one tile row (32 rows x 32 TNW columns, 16 TNW
+// accumulators), which leaves registers for two complete operand sets: everything step s + 1 needs is read from its
+// stage during step s, a stage is only ever read during the step before its own, and the loads of step s + 3 go into
+// the stage of step s at the top of step s, behind one barrier per step - two steps of distance for the direct loads
+// instead of one.  Stage: 8 KB of X (2 planes x 64 rows), 4 TNW KB of W, 1 KB of scales (every wavefront fetches 64 of
+// them; with TNW = 3 the last 64 belong to the next column tile and are never read).
 constexpr int TM64 = 64;
 constexpr int kXs64 = 2 * TM64 * 64;
-constexpr int kStage64 = kXs64 + kWl + TN * 4;
-constexpr int kLoads64 = 7;                 // per wavefront per stage: 2 of X, 4 of W, 1 of scales
+constexpr int stage64_bytes(int tnw) { return kXs64 + 64 * tnw * 64 + 1024; }
 constexpr int kMinSplitSteps = 32;          // K steps a workgroup must at least have when several share a tile's K
 
+template <int TNW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16_m64(const GemmF16Args a) {
+    constexpr int kTn = 64 * TNW, kW = kTn * 64, kStage64 = stage64_bytes(TNW);
+    constexpr int kLoads64 = TNW + 3;           // per wavefront per stage: 2 of X, TNW of W, 1 of scales
+    constexpr int kReads = 4 + 3 * TNW, kSlots = 4 * TNW;
+    static_assert(TNW == 3 || TNW == 4, "the wait counts below are written out for these");
     extern __shared__ __align__(16) unsigned char lds[];
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
     int m_tile, n_tile;
     if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
-    const int m0 = m_tile * TM64, n0 = n_tile * TN;
+    const int m0 = m_tile * TM64, n0 = n_tile * kTn;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
-    float acc[4][16];
+    float acc[TNW][16];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < TNW; j++)
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[j][e] = 0.f;
 
     const int prow = lane >> 2, pchunk = (lane & 3) ^ ((prow >> 2) & 3);
     const uint32_t op_lane = (uint32_t)((prow * a.pitch + pchunk * 8) * 2), s_lane = lane * 4;
-    const unsigned char *x_base[2], *w_base[4];
-    uint32_t x_dst[2], w_dst[4];
+    const unsigned char *x_base[2], *w_base[TNW];
+    uint32_t x_dst[2], w_dst[TNW];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         const int blk = wave * 2 + i, pl = blk >> 2, rb = blk & 3;      // X: 2 planes x 4 row blocks
@@ -306,13 +318,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         x_dst[i] = pl * TM64 * 64 + rb * 1024;
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int blk = wave * 4 + i;                                   // W: 16 row blocks
+    for (int i = 0; i < TNW; i++) {
+        const int blk = wave * TNW + i;                                 // W: 4 TNW row blocks
         w_base[i] = reinterpret_cast<const unsigned char *>(a.w16) + (int64_t)(n0 + blk * 16) * a.pitch * 2;
         w_dst[i] = kXs64 + blk * 1024;
     }
     const unsigned char *s_base = reinterpret_cast<const unsigned char *>(a.scales_t) + (int64_t)(n0 + wave * 64) * 4;
-    const uint32_t s_dst = kXs64 + kWl + wave * 256;
+    const uint32_t s_dst = kXs64 + kW + wave * 256;
     // this workgroup's share of K: all of it, or split_steps steps from blockIdx.z * split_steps (a partial product)
     const int all_steps = a.kp / 32, first = a.split_steps ? (int)blockIdx.z * a.split_steps : 0;
     const int steps = a.split_steps ? min(a.split_steps, all_steps - first) : all_steps, last = first + steps - 1;
@@ -320,40 +332,43 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         const uint32_t sb = lds0 + stage * kStage64;
         step = min(first + step, last);
         if (i < 2) load_to_lds16(x_base[i] + (int64_t)step * 64, op_lane, sb + x_dst[i]);
-        else if (i < 6) load_to_lds16(w_base[i - 2] + (int64_t)step * 64, op_lane, sb + w_dst[i - 2]);
+        else if (i < 2 + TNW) load_to_lds16(w_base[i - 2] + (int64_t)step * 64, op_lane, sb + w_dst[i - 2]);
         else load_to_lds4(s_base + (int64_t)step * a.n_pad * 4, s_lane, sb + s_dst);
     };
 
     const int sw = (l32 >> 2) & 3;
     const int lane_sub0 = (l32 << 6) + (((0 + half) ^ sw) << 4), lane_sub1 = (l32 << 6) + (((2 + half) ^ sw) << 4);
-    const int x_wave = wm * 32 * 64, w_wave = kXs64 + wn * 128 * 64, s_wave = kXs64 + kWl + wn * 128 * 4 + l32 * 4;
+    const int x_wave = wm * 32 * 64, w_wave = kXs64 + wn * (32 * TNW) * 64, s_wave = kXs64 + kW + wn * (32 * TNW) * 4 + l32 * 4;
     const floatx16 z16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     halfx8 fx[2][2][2];                 // [set][K half][hi, lo]
-    halfx8 fw[2][2][4];                 // [set][K half][tile column]
-    float sc[2][4];                     // [set][tile column]
+    halfx8 fw[2][2][TNW];               // [set][K half][tile column]
+    float sc[2][TNW];                   // [set][tile column]
     floatx16 g[2] = {z16, z16};
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) sc[i][j] = 0.f;
-    // read n of the 16 LDS reads that fetch a step's operands, in the order of their first use
+        for (int j = 0; j < TNW; j++) sc[i][j] = 0.f;
+    // read n of the kReads LDS reads that fetch a step's operands, in the order of their first use
     auto read_one = [&](auto set_c, int n, const unsigned char *x0, const unsigned char *x1, const unsigned char *w0, const unsigned char *w1, const unsigned char *sp) {
         constexpr int set = decltype(set_c)::value;
         if (n < 4) fx[set][n >> 1][n & 1] = *reinterpret_cast<const halfx8 *>(((n >> 1) ? x1 : x0) + (n & 1) * TM64 * 64);
-        else if (n < 12) { const int tn = (n - 4) >> 1, sub = (n - 4) & 1; fw[set][sub][tn] = *reinterpret_cast<const halfx8 *>((sub ? w1 : w0) + tn * 2048); }
-        else sc[set][n - 12] = *reinterpret_cast<const float *>(sp + (n - 12) * 128);
+        else if (n < 4 + 2 * TNW) { const int tn = (n - 4) >> 1, sub = (n - 4) & 1; fw[set][sub][tn] = *reinterpret_cast<const halfx8 *>((sub ? w1 : w0) + tn * 2048); }
+        else sc[set][n - 4 - 2 * TNW] = *reinterpret_cast<const float *>(sp + (n - 4 - 2 * TNW) * 128);
     };
     auto k_step = [&](auto set_c, int step, int stage) {
         constexpr int set = decltype(set_c)::value;
-        asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory");   // step + 1 has landed (step + 2 may be in flight); this step's operands are in registers
+        // step + 1 has landed (step + 2 may be in flight); this step's operands are in registers
+        if (TNW == 4) asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         const int next = stage == 2 ? 0 : stage + 1;
         const unsigned char *nb = lds + next * kStage64;
         const unsigned char *x0 = nb + x_wave + lane_sub0, *x1 = nb + x_wave + lane_sub1, *w0 = nb + w_wave + lane_sub0, *w1 = nb + w_wave + lane_sub1, *sp = nb + s_wave;
 #pragma unroll
-        for (int tn = 0; tn < 4; tn++) {
-            const int par = tn & 1, ptn = (tn + 3) & 3, pset = tn == 0 ? 1 - set : set;
+        for (int tn = 0; tn < TNW; tn++) {
+            // the partial-sum registers alternate from tile to tile, across the step boundary as well
+            const int par = (set * TNW + tn) & 1, ptn = (tn + TNW - 1) % TNW, pset = tn == 0 ? 1 - set : set;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int sub = i >> 1, piece = i & 1, slot = tn * 4 + i;
@@ -361,7 +376,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 const int f0 = i <= 1 ? 0 : i == 2 ? 6 : 11, f1 = i == 0 ? 0 : i == 1 ? 6 : i == 2 ? 11 : 16;
 #pragma unroll
                 for (int f = f0; f < f1; f++) acc[ptn][f] = fmaf(g[1 - par][f], sc[pset][ptn], acc[ptn][f]);
-                read_one(std::integral_constant<int, 1 - set>{}, slot, x0, x1, w0, w1, sp);
+                // the next step's operands: two reads per slot at first, so that the last slots have none in flight
+                // when the next step begins by waiting for them
+                constexpr int kDouble = kReads - (kSlots - 4);         // slots that carry two reads
+                if (slot < kDouble) {
+                    read_one(std::integral_constant<int, 1 - set>{}, 2 * slot, x0, x1, w0, w1, sp);
+                    read_one(std::integral_constant<int, 1 - set>{}, 2 * slot + 1, x0, x1, w0, w1, sp);
+                } else if (slot < kSlots - 4) {
+                    read_one(std::integral_constant<int, 1 - set>{}, slot + kDouble, x0, x1, w0, w1, sp);
+                }
                 if ((slot & 1) && (slot >> 1) < kLoads64) load_one(slot >> 1, step + 3, stage);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -370,12 +393,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     for (int s = 0; s < 3; s++)
         for (int i = 0; i < kLoads64; i++) load_one(i, s, s);
-    asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+    if (TNW == 4) asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     {
         const unsigned char *x0 = lds + x_wave + lane_sub0, *x1 = lds + x_wave + lane_sub1, *w0 = lds + w_wave + lane_sub0, *w1 = lds + w_wave + lane_sub1, *sp = lds + s_wave;
-        for (int n = 0; n < 16; n++) read_one(std::integral_constant<int, 0>{}, n, x0, x1, w0, w1, sp);
+        for (int n = 0; n < kReads; n++) read_one(std::integral_constant<int, 0>{}, n, x0, x1, w0, w1, sp);
     }
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
@@ -387,11 +411,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         stage = st1 == 2 ? 0 : st1 + 1;
     }
     if (step < steps) k_step(S0{}, step, stage);
-    // the last tile's scaling: column 3 of the last step, whose set is the parity of that step
+    // the last tile's scaling: the last column of the last step, whose set (and partial-sum register) follow that step's parity
     {
         const bool odd = (steps - 1) & 1;
+        const bool in_g1 = ((odd ? TNW : 0) + TNW - 1) & 1;
 #pragma unroll
-        for (int e = 0; e < 16; e++) acc[3][e] = fmaf(g[1][e], odd ? sc[1][3] : sc[0][3], acc[3][e]);
+        for (int e = 0; e < 16; e++) acc[TNW - 1][e] = fmaf(in_g1 ? g[1][e] : g[0][e], odd ? sc[1][TNW - 1] : sc[0][TNW - 1], acc[TNW - 1][e]);
     }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -402,10 +427,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         GemmF16Args b = a;
         b.out = a.partial + (int64_t)blockIdx.z * a.m * a.n;
         b.ep = GemmEpilogue{nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0};
-        store_tile_row(b, stage_f, acc, m0 + wm * 32, n0 + wn * 128, half, l32);
+        store_tile_row<TNW>(b, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
         return;
     }
-    store_tile_row(a, stage_f, acc, m0 + wm * 32, n0 + wn * 128, half, l32);
+    store_tile_row<TNW>(a, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
 }
 
 // out = epilogue(sum over the splits of partial[z]) on float4s: bias, GELU, residual as in store_tile_row (a fixed order
@@ -583,39 +608,58 @@ __global__ void __launch_bounds__(256) k_q8_to_f16(const int8_t *__restrict__ wq
 
 }  // namespace
 
-// How these kernels take a problem: tile_rows 128 or 64 (0: not at all), and for the 64-row kernel the number of
-// workgroups that share K (1: none).  A compute unit runs one workgroup at a time, so what counts is how many of the
-// 256 a launch keeps busy and for how many rounds.
-struct GemmF16Plan { int tile_rows, splits; };
+// How these kernels take a problem: the workgroup tile (rows 128 or 64, columns 256 or 192; rows 0: not at all), and for
+// the 64-row kernel the number of workgroups that share K (1: none).  A compute unit runs one workgroup at a time, so
+// what counts is how many of the 256 a launch keeps busy and for how many rounds.
+struct GemmF16Plan { int tile_rows, tile_cols, splits; };
+
+constexpr int kNPad = 768;      // weight rows of a prepared buffer are padded to a multiple of both tile widths
 
 GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
-    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels, =64 / =128 forces a tile (for comparisons)
+    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels; =128, =64 or =192 force the 128 x 256, 64 x 256 or
+    // 64 x 192 tile (for comparisons)
     static const int forced = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return e ? atoi(e) : -1; }();
-    if (forced == 0) return {0, 1};
+    if (forced == 0) return {0, 0, 1};
     // four columns per lane in the epilogue need n_rows % 4 == 0
-    if (m < 256 || (n_rows & 3) != 0 || k < 64) return {0, 1};
-    const int64_t cols = (n_rows + TN - 1) / TN, t128 = (int64_t)((m + TM - 1) / TM) * cols, t64 = (int64_t)((m + TM64 - 1) / TM64) * cols;
-    if (forced == 128 || forced == 64) return {t64 >= 128 ? forced : 0, 1};
-    // measured on 512 rows x K 2048: 11264 output rows (176 / 352 tiles) 84 us with 128-row tiles, 91 us with 64-row
-    // ones; 6144 output rows (96 / 192 tiles) 76 us on the bf16 kernel, 53 us with 64-row tiles
-    if (t128 >= 160) return {128, 1};
-    if (t64 >= 128) return {64, 1};
+    if (m < 256 || (n_rows & 3) != 0 || k < 64) return {0, 0, 1};
+    const int64_t rows128 = (m + TM - 1) / TM, rows64 = (m + TM64 - 1) / TM64, cols256 = (n_rows + 255) / 256, cols192 = (n_rows + 191) / 192;
+    const int64_t t128 = rows128 * cols256, t64 = rows64 * cols256, t64n = rows64 * cols192;
+    if (forced == 128 || forced == 64 || forced == 192) {
+        if (t64 < 128) return {0, 0, 1};
+        return forced == 128 ? GemmF16Plan{128, 256, 1} : forced == 64 ? GemmF16Plan{64, 256, 1} : GemmF16Plan{64, 192, 1};
+    }
+    // Enough tiles for several rounds: the large tile.  Around one round the time is rounds x one tile's time, and a
+    // tile's time goes with its area over its efficiency (measured at 512 rows, K 2048: a 128 x 256 tile 58 us of K
+    // loop + 11 us of prologue and epilogue, 64 x 256 35 + 10, 64 x 192 27 + 9): take the cheapest.
+    if (t128 >= 512) return {128, 256, 1};
+    auto rounds = [](int64_t tiles) { return (tiles + 255) / 256; };
+    const double c128 = rounds(t128) * 1.00, c64 = rounds(t64) * 0.65, c64n = rounds(t64n) * 0.52;
+    if (t64 >= 128) {
+        if (t128 >= 160 && c128 <= c64 && c128 <= c64n) return {128, 256, 1};
+        return c64n < c64 ? GemmF16Plan{64, 192, 1} : GemmF16Plan{64, 256, 1};
+    }
     // few tiles but a long K (512 x 2048 output over K 5632: 64 tiles, 71 us on the bf16 kernel, 47 us as 4 x 64
     // workgroups): several workgroups per tile, each with a share of K of at least kMinSplitSteps steps, their partial
     // products summed by a second kernel.  With K 2048 (two shares) it is a tie with the bf16 kernel, which keeps it.
     const int steps = q8_padded_k(k) / 32;
     const int splits = (int)std::min<int64_t>(std::min<int64_t>(8, 256 / t64), steps / kMinSplitSteps);
-    if (t64 >= 32 && splits >= 3) return {64, splits};
-    return {0, 1};
+    if (t64 >= 32 && splits >= 3) return {64, 256, splits};
+    return {0, 0, 1};
 }
 
 int q8_gemm_f16_tile_rows(int m, int n_rows, int k) { return q8_gemm_f16_plan(m, n_rows, k).tile_rows; }
 bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) { return q8_gemm_f16_tile_rows(m, n_rows, k) != 0; }
+void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares) {
+    const GemmF16Plan p = q8_gemm_f16_plan(m, n_rows, k);
+    if (tile_rows) *tile_rows = p.tile_rows;
+    if (tile_cols) *tile_cols = p.tile_cols;
+    if (k_shares) *k_shares = p.splits;
+}
 
 // the weights in this kernel's layout: fp16 rows, then the transposed scales (each part 256-byte aligned)
 int64_t q8_prepared_floats(int k, int n_rows) {
-    const int64_t kp = q8_padded_k(k), pitch = kp + 64, n_pad = round_up(n_rows, TN);
-    return round_up(n_pad * pitch / 2, 64) + round_up((kp / 32) * n_pad, 64);
+    const int64_t kp = q8_padded_k(k), pitch = kp + 64, n_pad = round_up(n_rows, kNPad);
+    return round_up(n_pad * pitch / 2, 64) + round_up((kp / 32) * n_pad, 64) + 64;     // + the scale fetch's reach past the last tile
 }
 
 // floats of workspace: planes, row factors and, unless the caller holds prepared weights, those
@@ -628,7 +672,7 @@ int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared) {
 
 void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, float *prepared, int k, int n_rows) {
     if (k <= 0 || n_rows <= 0) return;
-    const int kp = q8_padded_k(k), pitch = kp + 64, n_pad = (int)round_up(n_rows, TN);
+    const int kp = q8_padded_k(k), pitch = kp + 64, n_pad = (int)round_up(n_rows, kNPad);
     uint16_t *w16 = reinterpret_cast<uint16_t *>(prepared);
     float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
     const int64_t items = (int64_t)n_rows * (kp / 8);
@@ -641,7 +685,7 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     if (!q8_gemm_f16_shape_ok(m, n_rows, k)) fail("q8_gemm_f16: shape outside this kernel's range");
     if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
-    const int kp = q8_padded_k(k), pitch = kp + 64, m_pad = (int)round_up(m, TM), n_pad = (int)round_up(n_rows, TN);
+    const int kp = q8_padded_k(k), pitch = kp + 64, m_pad = (int)round_up(m, TM), n_pad = (int)round_up(n_rows, kNPad);
     float *w = workspace;
     uint16_t *planes = reinterpret_cast<uint16_t *>(w); w += round_up((int64_t)m_pad * pitch, 64);
     float *unscale = w;                                  w += round_up(m_pad, 64);
@@ -659,18 +703,20 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     const uint16_t *w16 = reinterpret_cast<const uint16_t *>(prepared);
     const float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
     const int split_steps = plan.splits > 1 ? (kp / 32 + plan.splits - 1) / plan.splits : 0;
-    const int n_tiles = n_pad / TN, m_tiles = plan.tile_rows == 64 ? (m + TM64 - 1) / TM64 : m_pad / TM;
+    const int n_tiles = (n_rows + plan.tile_cols - 1) / plan.tile_cols, m_tiles = plan.tile_rows == 64 ? (m + TM64 - 1) / TM64 : m_pad / TM;
     const unsigned grid_x = (unsigned)((n_tiles + 7) / 8 * 8 * m_tiles);
     GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch, m_tiles, n_tiles,
                   GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}, split_steps, w};
     static bool configured = false;
     if (!configured) {
         hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
-        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage64), "hipFuncSetAttribute(k_gemm_q8_f16_m64)");
+        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4>)");
+        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3>)");
         configured = true;
     }
     if (plan.tile_rows == 64) {
-        launch_kernel(k_gemm_q8_f16_m64, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * kStage64, s, a);
+        if (plan.tile_cols == 192) launch_kernel(k_gemm_q8_f16_m64<3>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(3), s, a);
+        else launch_kernel(k_gemm_q8_f16_m64<4>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
         if (plan.splits > 1) {
             const int64_t mn4 = (int64_t)m * n_rows / 4;
             hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,

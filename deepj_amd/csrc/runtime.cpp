@@ -1089,6 +1089,14 @@ int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows) {
     return q8_gemm_f16_tile_rows(m, rows, k);
 }
 
+void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares) {
+    int tr = 0, tc = 0, ks = 1;
+    if (m > 1 && k > 0 && rows > 0) q8_gemm_f16_tile(m, rows, k, &tr, &tc, &ks);
+    if (tile_rows) *tile_rows = tr;
+    if (tile_cols) *tile_cols = tc;
+    if (k_shares) *k_shares = ks;
+}
+
 int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total) {
     return guarded([&] {
         ensure_init();

@@ -223,6 +223,8 @@ int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
  * No counterpart in the reference, whose weights are fp32 (J/layers/Linear.java:9-24). */
 int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows);
 int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);
+/* the same with the tile's columns (256 or 192) and the number of workgroups that share a tile's K (1: none) */
+void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares);
 
 /* ── host side: java.util.Random twin ─────────────────────────────────────
  * Tensor.random(rows, cols, Random) of the reference (J/tensor/cpu/CpuBackend.java:148-152)

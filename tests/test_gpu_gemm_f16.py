@@ -50,9 +50,14 @@ def test_path_query_matches_the_documented_rule():
     assert HipNative.q8GemmPath(512, 2048, 6144) == 64        # 96 such tiles would idle most of the chip: 192 of 64 x 256
     assert HipNative.q8GemmPath(512, 2048, 2048) == 0         # 64 even of those: the bf16 kernels' 64 x 64 tiles
     assert HipNative.q8GemmPath(512, 5632, 2048) == 64        # the same 64 tiles over a long K: four workgroups share each
+    assert HipNative.q8GemmTile(512, 5632, 2048) == (64, 256, 4)
+    assert HipNative.q8GemmTile(512, 2048, 6144) == (64, 192, 1)     # 256 tiles: one per compute unit
+    assert HipNative.q8GemmTile(512, 2048, 11264) == (128, 256, 1)
+    assert HipNative.q8GemmTile(8, 2048, 2048) == (0, 0, 1)
     assert HipNative.q8GemmPath(1, 2048, 32000) == 0          # the matvec's case
     assert HipNative.q8GemmPath(512, 2048, 11266) == 0        # four columns per lane in the epilogue
-    assert HipNative.q8PreparedFloats(2048, 11264) == (11264 * (2048 + 64)) // 2 + 64 * 11264
+    # fp16 rows padded to a multiple of 768 (both tile widths), the transposed scales, 64 floats of slack
+    assert HipNative.q8PreparedFloats(2048, 11264) == (11520 * (2048 + 64)) // 2 + 64 * 11520 + 64
 
 
 @pytest.mark.parametrize("m,k,n,tile", [(300, 1000, 13828, 128), (257, 96, 40964, 128), (640, 2048, 8192, 128),
