@@ -679,6 +679,14 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
     hipLaunchKernelGGL(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
 }
 
+// The kernels' LDS (three stages) is above the 64 KB a kernel gets without asking; called once per device at start-up
+// (not at the first launch, which may sit inside a graph capture).
+void q8_gemm_f16_configure() {
+    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
+    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4>)");
+    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3>)");
+}
+
 void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
                         const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
                         const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats) {
@@ -707,13 +715,6 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     const unsigned grid_x = (unsigned)((n_tiles + 7) / 8 * 8 * m_tiles);
     GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch, m_tiles, n_tiles,
                   GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}, split_steps, w};
-    static bool configured = false;
-    if (!configured) {
-        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
-        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4>)");
-        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3>)");
-        configured = true;
-    }
     if (plan.tile_rows == 64) {
         if (plan.tile_cols == 192) launch_kernel(k_gemm_q8_f16_m64<3>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(3), s, a);
         else launch_kernel(k_gemm_q8_f16_m64<4>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(4), s, a);

@@ -96,6 +96,7 @@ void ensure_init(int device = 0) {
     DJ_HIP(hipGetSymbolAddress((void **)&g.static_scratch, HIP_SYMBOL(scratch)));
     if (!g.static_scratch) fail("deepj_hip: the static scratch array has no device address");
     DJ_HIP(hipMemset(g.static_scratch, 0, kStaticCounterBytes));
+    q8_gemm_f16_configure();
     g.device = device;
     g.ready = true;
 }

@@ -234,3 +234,28 @@ def test_prepared_weights_give_the_same_bits_and_follow_the_weights(dev):
     with pytest.raises(RuntimeError, match="a buffer of its own"):
         Stream().q8_prepare(wq, wq, k, n).run()
     dev.release(src, wq, xb, ob)
+
+
+def test_graph_replays_of_the_gemm_match_eager_runs(dev):
+    """The three-kernel Q8_LINEAR (split, GEMM on shared K, sum of partial products) and the single-GEMM one captured into
+    a HIP graph: every replay, with eager work and synchronisation in between, gives the eager run's bits."""
+    for m, k, n in ((512, 5632, 2048), (300, 320, 20736)):
+        assert HipNative.q8GemmPath(m, k, n) != 0
+        x = JavaRandom(61).tensor(m, k, 1.0)
+        w = JavaRandom(62).tensor(k, n, 0.02)
+        r = JavaRandom(63).tensor(m, n, 1.0)
+        wq, _ = quantised(dev, w)
+        xb, rb, ob, scratch = dev.upload(x), dev.upload(r), dev.alloc(m * n), dev.alloc(m * n)
+        lin = Stream().q8_linear(xb, wq, ob, m, k, n, residual=rb)
+        lin.run()
+        eager = dev.download(ob, (m, n))
+        graph = HipNative.graphCapture(lin.array())
+        try:
+            for i in range(3):
+                Stream().fill(ob, 0, m * n).fill(scratch, i + 1, m * n).run()
+                HipNative.synchronize()
+                HipNative.graphLaunch(graph, 1)
+                assert np.array_equal(dev.download(ob, (m, n)).view(np.int32), eager.view(np.int32)), f"replay {i}"
+        finally:
+            HipNative.graphDestroy(graph)
+        dev.release(xb, rb, ob, scratch, wq)
