@@ -288,7 +288,7 @@ constexpr int stage64_bytes(int tnw) { return kXs64 + 64 * tnw * 64 + 1024; }
 constexpr int kMinSplitSteps = 32;          // K steps a workgroup must at least have when several share a tile's K
 
 template <int TNW>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16_m64(const GemmF16Args a) {
+__global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     constexpr int kTn = 64 * TNW, kW = kTn * 64, kStage64 = stage64_bytes(TNW);
     constexpr int kLoads64 = TNW + 3;           // per wavefront per stage: 2 of X, TNW of W, 1 of scales
     constexpr int kReads = 4 + 3 * TNW, kSlots = 4 * TNW;
