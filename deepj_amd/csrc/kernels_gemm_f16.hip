@@ -3,7 +3,8 @@
 // Arithmetic.  An int8 weight is exact in fp16.  A row of activations is multiplied by a power of two that brings its
 // largest magnitude into [2^14, 2^15) (exact, undone at the end) and every element is then written as hi + lo, two
 // fp16 numbers: hi = fp16(v) by round-to-nearest, lo = fp16(v - hi).  hi carries 11 significant bits and lo the next 11
-// (down to 2^-24 of the row's scale, where fp16 subnormals end), so hi + lo holds v to about 2^-23 relative - the fp32
+// (down to 2^-24 in the scaled units, i.e. 2^-38 of the row's largest value, where fp16 subnormals end), so hi + lo holds v to
+// about 2^-23 relative - the fp32
 // value itself for all practical rows - and x . q = hi . q + lo . q with exact products and fp32 accumulation: two
 // v_mfma_f32_32x32x16_f16 per 16 k instead of three bf16 ones.  The group scale multiplies the finished 32-k partial
 // sum, as in the reference's dequantise-then-multiply (Q8 layout: q8_format notes in dj_common.h).
@@ -12,6 +13,12 @@
 // planes of X (k_split_f16) and an fp16 copy of W with its scales transposed to [group][row] (k_q8_to_f16).  The GEMM
 // kernel then moves them with direct global -> LDS loads (global_load_lds_dwordx4: no vector registers, no LDS
 // store instructions), three stages deep, and spends its vector instructions on the per-group scaling only.
+//
+// Kernels.  k_gemm_q8_f16 (128 x 256 workgroup tile, described next) for problems with many tiles; k_gemm_q8_f16_m64
+// (64 x 256 or 64 x 192, further down) for those whose large tiles would leave compute units idle, optionally with a
+// tile's K shared by several workgroups and k_sum_partials adding their partial products in a fixed order;
+// q8_gemm_f16_plan chooses.  A workgroup's tile follows from its index so that the workgroups of one column tile
+// run on one XCD (tile_of_workgroup).
 //
 // Shape.  Workgroup tile 128 x 256, 256 threads = 4 wavefronts (2 x 2), one wavefront per SIMD; a wavefront owns
 // 64 x 128 of C = 8 MFMA tiles of 32 x 32 = 128 fp32 accumulators per lane, kept in ordinary vector registers because
