@@ -85,6 +85,25 @@ def test_q8_linear_full_width(sweep, idx, m):
     assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"Q8 linear M={m} {k}x{n}")
 
 
+@pytest.mark.parametrize("idx", range(4))
+def test_q8_linear_full_width_on_the_bf16_kernels(sweep, idx):
+    """The same 512-row products through the allocation-free entry point, whose fixed workspace keeps them on the bf16
+    matrix-core kernels (three-piece activations, 128 x 128 / 64 x 128 / 64 x 64 tiles) that the ordinary entry point
+    now leaves to the fp16 GEMM for most of these shapes: both kernels answer to the same oracle and gate."""
+    dev, mats, bufs, deq = sweep
+    k, n = mats[idx].shape
+    m = 512
+    x = activations(m, k)
+    exp = ref.matmul(x, deq[idx])
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    words = Stream().q8_linear(xb, bufs[idx], ob, m, k, n).array()
+    HipNative.flushOpsNoAlloc(words, words.size)
+    got = dev.download(ob, (m, n))
+    dev.release(xb, ob)
+    scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+    assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what=f"Q8 linear (bf16 kernels) M={m} {k}x{n}")
+
+
 @pytest.mark.parametrize("m", [1, 64, 512])
 @pytest.mark.parametrize("cols", [2048, 5632])
 def test_fused_rmsnorm_at_both_epsilons(sweep, m, cols):
