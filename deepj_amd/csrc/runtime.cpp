@@ -42,6 +42,9 @@ struct Graph {
     hipGraphExec_t exec = nullptr;
     std::vector<std::pair<int32_t, void *>> refs;
     float *workspace = nullptr;       // set when the stream needs workspace
+    // (weight id, prepared id) of every Q8_LINEAR that was captured reading a prepared copy the stream had not written
+    // itself: once the copy stops standing for the weights (they were written again) a replay would use stale weights
+    std::vector<std::pair<int32_t, int32_t>> prepared, self_prepared;
 };
 
 struct Runtime {
@@ -63,6 +66,7 @@ struct Runtime {
     unsigned char *static_scratch = nullptr;       // device address of `scratch` below on g.device
     bool no_alloc = false;                         // inside deepj_hip_flush_ops_noalloc: nothing may allocate
     std::vector<std::pair<int32_t, void *>> *track = nullptr;   // graph capture: buffers the dry pass resolves
+    Graph *capture_into = nullptr;                               // graph capture: the graph the run pass records for
     struct Prepared { int32_t id; int k, rows; };
     std::unordered_map<int32_t, Prepared> prepared;   // Q8 weight buffer -> its copy in the fp16 GEMM's layout (OP_Q8_PREPARE)
     void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
@@ -459,6 +463,11 @@ void exec_one(Cursor &c) {
                 auto pit = g.prepared.find(w[2]);
                 if (pit != g.prepared.end() && pit->second.k == k && pit->second.rows == rows)
                     p.prepared = buf(pit->second.id, q8_prepared_floats((int)k, (int)rows), op, "prepared weights");
+                if (p.prepared && run && g.capture_into) {
+                    const std::pair<int32_t, int32_t> pr(w[2], pit->second.id);
+                    auto &own = g.capture_into->self_prepared;
+                    if (std::find(own.begin(), own.end(), pr) == own.end()) g.capture_into->prepared.push_back(pr);
+                }
             }
             int64_t ws = g.no_alloc ? q8_linear_workspace_floats((int)m, (int)k, (int)n, flags)
                                     : q8_linear_preferred_workspace_floats((int)m, (int)k, (int)n, flags, p.prepared != nullptr);
@@ -768,6 +777,7 @@ void exec_one(Cursor &c) {
                 launch_q8_prepare(s, q, reinterpret_cast<const float *>(q + q8_scale_offset_bytes((int)k, (int)rows)), prep, (int)k, (int)rows);
                 forget_prepared(w[2]);
                 g.prepared[w[1]] = Runtime::Prepared{w[2], (int)k, (int)rows};
+                if (g.capture_into) g.capture_into->self_prepared.emplace_back(w[1], w[2]);   // every replay rewrites the copy
             }
             break;
         }
@@ -1201,16 +1211,19 @@ int deepj_hip_graph_capture(const int32_t *cmd, int32_t len, int32_t *handle) {
         DJ_HIP(hipStreamSynchronize(g.stream));
         DJ_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal));
         g.capturing = true;
+        g.capture_into = &gr;
         try {
             walk(cmd, len, false, nullptr);
         } catch (...) {
             g.capturing = false;
+            g.capture_into = nullptr;
             hipGraph_t tmp = nullptr;
             (void)hipStreamEndCapture(g.stream, &tmp);
             if (tmp) (void)hipGraphDestroy(tmp);
             throw;
         }
         g.capturing = false;
+        g.capture_into = nullptr;
         DJ_HIP(hipStreamEndCapture(g.stream, &gr.graph));
         hipError_t e = hipGraphInstantiate(&gr.exec, gr.graph, nullptr, nullptr, 0);
         if (e != hipSuccess) {
@@ -1238,6 +1251,12 @@ int deepj_hip_graph_launch(int32_t handle, int32_t times) {
         if (it->second.workspace && it->second.workspace != g.workspace)
             fail("graph_launch: the workspace was reallocated after graph " + std::to_string(handle) +
                  " was captured; capture the stream again");
+        for (const auto &pr : it->second.prepared) {
+            auto p = g.prepared.find(pr.first);
+            if (p == g.prepared.end() || p->second.id != pr.second)
+                fail("graph_launch: Q8 weights id=" + std::to_string(pr.first) + " were written after graph " + std::to_string(handle) +
+                     " was captured with their prepared copy id=" + std::to_string(pr.second) + "; capture the stream again");
+        }
         // Bounded run-ahead: at most kRing windows of kWindow replays are queued behind the one the
         // device is executing, so a long run never piles tens of thousands of dispatches (and their
         // kernel-argument blocks) into the queue; the device is never left idle by this.

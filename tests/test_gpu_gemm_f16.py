@@ -259,3 +259,39 @@ def test_graph_replays_of_the_gemm_match_eager_runs(dev):
         finally:
             HipNative.graphDestroy(graph)
         dev.release(xb, rb, ob, scratch, wq)
+
+
+def test_graph_with_prepared_weights_is_refused_once_the_weights_change(dev):
+    """A graph captured while a prepared copy stood for the weights replays that copy's address: once the weights are
+    written again the copy is stale and the replay must be refused, not run on the old weights.  A stream that prepares
+    the copy itself rewrites it on every replay and stays valid."""
+    m, k, n = 512, 512, 10240
+    x = JavaRandom(71).tensor(m, k, 1.0)
+    w1, w2 = JavaRandom(72).tensor(k, n, 0.02), JavaRandom(73).tensor(k, n, 0.02)
+    wq, _ = quantised(dev, w1)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    prep = dev.alloc(HipNative.q8PreparedFloats(k, n))
+    Stream().q8_prepare(wq, prep, k, n).run()
+    lin = Stream().q8_linear(xb, wq, ob, m, k, n)
+    lin.run()
+    first = dev.download(ob, (m, n))
+    uses_copy = HipNative.graphCapture(lin.array())
+    own_copy = HipNative.graphCapture(Stream().q8_prepare(wq, prep, k, n).q8_linear(xb, wq, ob, m, k, n).array())
+    try:
+        Stream().fill(ob, 0, m * n).run()
+        HipNative.graphLaunch(uses_copy, 1)
+        assert np.array_equal(dev.download(ob, (m, n)).view(np.int32), first.view(np.int32))
+        src = dev.upload(w2)
+        Stream().q8_quantize(src, wq, k, n).run()              # the copy no longer stands for wq
+        with pytest.raises(RuntimeError, match="were written after graph"):
+            HipNative.graphLaunch(uses_copy, 1)
+        lin.run()
+        second = dev.download(ob, (m, n))
+        assert not np.array_equal(second, first)
+        Stream().fill(ob, 0, m * n).run()
+        HipNative.graphLaunch(own_copy, 1)                      # converts the new weights, then multiplies
+        assert np.array_equal(dev.download(ob, (m, n)).view(np.int32), second.view(np.int32))
+    finally:
+        HipNative.graphDestroy(uses_copy)
+        HipNative.graphDestroy(own_copy)
+    dev.release(src, wq, xb, ob, prep)
