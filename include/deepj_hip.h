@@ -94,7 +94,9 @@ int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float 
 
 /* Captures a command stream into a HIP graph (no allocation may be pending:
  * every buffer it names must exist) and replays it.  Used for the per-token
- * decode stream, whose position and token live in device memory. */
+ * decode stream, whose position and token live in device memory.  A graph replays raw addresses: graph_launch fails,
+ * launching nothing, once a buffer the stream names was released or reallocated, the workspace it used was replaced, or
+ * Q8 weights it read through a prepared copy (DJ_OP_Q8_PREPARE) were written again - capture the stream again then. */
 int deepj_hip_graph_capture(const int32_t *cmd, int32_t len, int32_t *handle);
 int deepj_hip_graph_launch(int32_t handle, int32_t times);
 int deepj_hip_graph_destroy(int32_t handle);
