@@ -181,7 +181,10 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     float(*Kt)[HD][KT + 1] = reinterpret_cast<float(*)[HD][KT + 1]>(lds);              // [set][j][key]: transposed
     float(*Vs)[KT][HD] = reinterpret_cast<float(*)[KT][HD]>(lds + kKtFloats);          // [set][key][j]
 
-    const int h = blockIdx.x, qt = blockIdx.y;
+    // Causal work grows with the query tile.  The second half of the tiles is taken in reverse, so that the workgroups
+    // that become resident together on a compute unit (index i and i + half the grid) are a short and a long one.
+    const int h = blockIdx.x, y_half = gridDim.y >> 1;
+    const int qt = (int)blockIdx.y < y_half ? (int)blockIdx.y : (int)gridDim.y - 1 - ((int)blockIdx.y - y_half);
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, half = lane >> 5, l32 = lane & 31;
     const int qw = wave % QW, kset = wave / QW;
     const int d = a.H * HD;
