@@ -33,6 +33,7 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_last_error.restype = C.c_char_p
     lib.deepj_hip_pool_stats.argtypes = [C.POINTER(C.c_int64)]
     lib.deepj_hip_stream.restype = C.c_void_p
+    lib.deepj_hip_attn_record_splits.restype = C.c_int32
     lib.deepj_hip_q8_floats.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_q8_floats.restype = C.c_int64
     lib.deepj_hip_q8_prepared_floats.argtypes = [C.c_int32, C.c_int32]
@@ -149,6 +150,10 @@ class HipNative:
     @staticmethod
     def q8Floats(k: int, rows: int) -> int:
         return int(library().deepj_hip_q8_floats(k, rows))
+
+    @staticmethod
+    def attnRecordSplits() -> int:
+        return int(library().deepj_hip_attn_record_splits())
 
     @staticmethod
     def q8PreparedFloats(k: int, rows: int) -> int:

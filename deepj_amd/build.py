@@ -37,7 +37,6 @@ SOURCES = {
     "kernels_gemm_f16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "kernels_q8.hip": [],
     "kernels_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
-    "kernels_decode.hip": [],
     "runner.cpp": [],
     "host_random.cpp": [],
 }

@@ -112,6 +112,7 @@ struct Q8Linear {
     const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
     int m_extra = 0;
     const float *prepared = nullptr;  // the weights in the fp16 GEMM's layout (launch_q8_prepare), or null: converted per call
+    bool small_workspace_only = false; // the caller's workspace cannot grow: stay on the kernels that need M * K floats at most
 };
 void launch_q8_quantize(hipStream_t s, const float *w, int8_t *q, float *scales, int k, int n, int row_off,
                         int row_step);
@@ -162,7 +163,8 @@ void launch_attn_decode(hipStream_t s, const float *qkv, float *k_cache, float *
                         int max_seq, unsigned *counters);
 int64_t attn_decode_scratch_floats(int H, int hd);
 // Decode attention that stops at per-split records [H][kAttnRecordSplits][hd + 4] = {max, sum, -, -, o[hd]};
-// the consumer (Q8 matvec with the ATTN_MERGE prologue) merges them.
+// the consumer (Q8 matvec with the ATTN_MERGE prologue) merges them.  The maximum is in base-2 units (score *
+// log2(e)): both sides use the hardware exp2.
 constexpr int kAttnRecordSplits = 4;
 void launch_attn_decode_records(hipStream_t s, const float *qkv, float *k_cache, float *v_cache, float *records,
                                 const int32_t *state, const float *cos_t, const float *sin_t, int H, int hd,
@@ -170,33 +172,5 @@ void launch_attn_decode_records(hipStream_t s, const float *qkv, float *k_cache,
 void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
                         const float *table, float *x, int vocab, int d, int n_positions);
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq);
-
-// kernels_decode.hip: persistent greedy decode of the Llama block stack
-struct Q8Mat {
-    const int8_t *w; const float *sc;
-    int k, kp, rows;                       // rows = Q8 rows (gate/up: 2 * dFF, interleaved)
-};
-struct DecodeLayer {
-    Q8Mat qkv, wo, gu, down;
-    const float *g1, *g2, *bg, *bu, *bd;
-};
-struct DecodeParams {
-    int d, H, hd, dff, vocab, max_seq, L, steps, nsplit, capacity;
-    unsigned slot_count, xs_bytes;
-    const DecodeLayer *layers;             // device copy of the layer table
-    const DecodeLayer *layers_host;        // the same table on the host (launch-time checks only)
-    Q8Mat lm;
-    const float *gf, *blm, *emb, *cos_t, *sin_t;
-    float *kc, *vc;                        // [L][H][max_seq][hd]
-    float *x, *x2, *qkv, *att, *ff, *logits, *scratch, *argbuf;
-    int32_t *state, *tokens;
-    unsigned *sync;
-    float scale;
-    unsigned long long *timing;            // debug: phase time stamps of workgroup 0 (null = off)
-};
-int64_t llama_decode_sync_words();
-void llama_decode_plan(int H, int hd, int *grid, int *nsplit, int64_t *scratch_floats, int64_t *argbuf_floats);
-bool llama_decode_supported(int d, int dff);
-void launch_llama_decode(hipStream_t s, DecodeParams &p);
 
 }  // namespace dj

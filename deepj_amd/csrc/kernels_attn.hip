@@ -480,16 +480,42 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     }
 }
 
-// Splits per head for the fused decode op: about two workgroups per CU in total.
 // ── decode attention that leaves the split merge to its consumer ───────────
 // Same work as the fused kernel above (rotate q and the new key, append the new row, online softmax over this
-// split's keys) with kRecSplits splits per head and 1024 threads per workgroup, but it stops at the per-split
-// record [max, sum, -, -, o[hd]]: merging records across workgroups inside one kernel costs a store
-// acknowledgement, an atomic and a reload - three trips to memory in a row - while the next kernel reads them
-// across the kernel boundary for free (the Q8 matvec's ATTN_MERGE prologue does the merge while its weight rows
-// are in flight).
-constexpr int kRecThreads = 1024;
+// split's keys), but it stops at the per-split record [max, sum, -, -, o[hd]]: merging records across workgroups
+// inside one kernel costs a store acknowledgement, an atomic and a reload - three trips to memory in a row - while
+// the next kernel reads them across the kernel boundary for free (the Q8 matvec's ATTN_MERGE prologue does the
+// merge while its weight rows are in flight).
+//
+// What the kernel is built around: a launch of this size is bound by memory round trips and by its own serial
+// tail, not by bytes.
+//  * Keys are dealt to the kAttnRecordSplits splits of a head in TILES of kRecWaves * (64 / LPK) consecutive keys,
+//    tile t to split t % splits: every split has work from the first tiles on, whatever the position.
+//  * The running softmax is updated once per round of kRecU keys, not once per key: one maximum, one correction,
+//    kRecU weights - and in base 2 with the hardware exponential (scores are multiplied by log2(e), the records hold
+//    the maximum in that unit): a dozen instructions per round where the library expf took sixty.
+//  * Four splits of 512 threads: eight splits shorten this kernel by 0.9 us at 1500 keys and cost the Wo matvec,
+//    every workgroup of which reads all records, 0.7 us.  (Requesting the first tiles before the position is known
+//    - rows past it are readable, being inside the cache buffer - gained nothing: measured 2435 against 2443 tok/s.)
+#ifndef DJ_REC_THREADS
+#define DJ_REC_THREADS 512
+#endif
+constexpr int kRecThreads = DJ_REC_THREADS;
 constexpr int kRecWaves = kRecThreads / 64;
+#ifndef DJ_REC_U
+#define DJ_REC_U 4
+#endif
+constexpr int kRecU = DJ_REC_U;   // key tiles a workgroup requests per round
+
+// Timeline of one launch, for tuning builds only (-DDJ_TRACE; never in the shipped library).
+#ifdef DJ_TRACE
+__device__ unsigned long long g_at_trace[8 * 8192];
+#define DJ_STAMP(i) do { if (lane == 0) g_at_trace[((blockIdx.y * gridDim.x + blockIdx.x) * kRecWaves + wave) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define DJ_STAMP(i) do {} while (0)
+#endif
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }   // exp2(-inf) = 0
 
 // Separate scalar arguments, the ones the first loads need in front (they can reach a wavefront in registers at
 // launch; a by-value struct is always fetched from the argument buffer first).
@@ -499,96 +525,107 @@ k_attn_decode_records(const int32_t *a_state, float *a_k_cache, float *a_v_cache
                       const float *a_cos_t, const float *a_sin_t, int a_max_seq, int a_H, float *a_records,
                       float a_scale) {
     constexpr int HD = LPK * 4;
-    DecodeArgs a;
-    a.qkv = a_qkv; a.k_cache = a_k_cache; a.v_cache = a_v_cache; a.tok_stride = HD;
-    a.head_stride = (int64_t)a_max_seq * HD; a.out = nullptr; a.state = a_state; a.scratch = a_records;
-    a.cos_t = a_cos_t; a.sin_t = a_sin_t; a.H = a_H; a.hd = HD; a.max_seq = a_max_seq; a.nsplit = kAttnRecordSplits;
-    a.scale = a_scale; a.counters = nullptr;
     constexpr int KPW = 64 / LPK;                  // keys a wavefront handles at a time
-    constexpr int STRIDE = kRecWaves * KPW;        // keys per workgroup round
-    constexpr int U = 4;
+    constexpr int TILE = kRecWaves * KPW;          // consecutive keys of one tile
+    constexpr float kLog2e = 1.44269504088896340736f;
+    constexpr int U = kRecU;
+    constexpr int NS = kAttnRecordSplits;
     __shared__ float s_m[kRecWaves], s_l[kRecWaves];
     __shared__ __align__(16) float s_o[kRecWaves][HD];
 
     const int h = blockIdx.x, split = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane / LPK, dl = lane % LPK;
-    const int d = a.H * HD, half = HD / 2;
+    const int d = a_H * HD, half = HD / 2;
+    const int64_t head_stride = (int64_t)a_max_seq * HD;
+    DJ_STAMP(0);
 
-    int pos = a.state[0];
+    float *kb = a_k_cache + (int64_t)h * head_stride + dl * 4;
+    float *vb = a_v_cache + (int64_t)h * head_stride + dl * 4;
+    const int key0 = split * TILE + wave * KPW + sub;          // this lane group's key in tile 0 of the split
+    const int row_cap = a_max_seq - 1;
+    int pos = a_state[0];
     if (pos < 0) pos = 0;
-    if (pos >= a.max_seq) pos = a.max_seq - 1;             // the host never lets this happen; stay in bounds
-    const int n_keys = pos + 1;
-    const int per = (n_keys + a.nsplit - 1) / a.nsplit;
-    const int k_begin = split * per;
-    const int k_end = k_begin + per < n_keys ? k_begin + per : n_keys;
-
-    float *kb = a.k_cache + (int64_t)h * a.head_stride + dl * 4;
-    float *vb = a.v_cache + (int64_t)h * a.head_stride + dl * 4;
-    float4 kk[U], vv[U];
-    auto load_tile = [&](int base) {
+    if (pos > row_cap) pos = row_cap;                      // the host never lets this happen; stay in bounds
+    DJ_STAMP(1);
+    // Round r of a split: tiles r * U .. r * U + U - 1 of its own, i.e. keys key0 + (r * U + u) * NS * TILE.  Loads are
+    // unconditional (row 0 for keys past the position: an L2 hit), so waits for them are counted ones.
+    auto load_round = [&](float4 (&K)[U], float4 (&V)[U], int t0) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int key = base + u * STRIDE;
-            const int row = (key < k_end && key != pos) ? key : 0;      // row 0 always exists; unused rows are masked
-            kk[u] = *reinterpret_cast<const float4 *>(kb + (int64_t)row * a.tok_stride);
-            vv[u] = *reinterpret_cast<const float4 *>(vb + (int64_t)row * a.tok_stride);
+            const int key = key0 + (t0 + u) * NS * TILE;
+            const int row = key < pos ? key : 0;
+            K[u] = *reinterpret_cast<const float4 *>(kb + (int64_t)row * HD);
+            V[u] = *reinterpret_cast<const float4 *>(vb + (int64_t)row * HD);
         }
     };
-    // The small operands (L2 hits) go out first and the first round of keys and values right behind them, all
-    // unconditional: the rotation below then waits for the small ones only (a counted wait) while the key/value
-    // rows are on their way from HBM.
-    const float2 c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
-    const float2 s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
-    float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
-    const float4 k0 = *reinterpret_cast<const float4 *>(a.qkv + d + h * HD + dl * 4);
-    const float4 nv = *reinterpret_cast<const float4 *>(a.qkv + 2 * d + h * HD + dl * 4);
-    const int base0 = k_begin + wave * KPW + sub;
-    load_tile(base0);
+    auto has_keys = [&](int t0) { return (t0 * NS + split) * TILE <= pos; };    // workgroup-uniform
+    // The small operands (L2 hits) go out first and the first two rounds of keys and values right behind them: the
+    // rotation below then waits for the small ones only while the key/value rows are on their way from HBM.
+    const float2 c2 = *reinterpret_cast<const float2 *>(a_cos_t + (int64_t)pos * half + dl * 2);
+    const float2 s2 = *reinterpret_cast<const float2 *>(a_sin_t + (int64_t)pos * half + dl * 2);
+    float4 q0 = *reinterpret_cast<const float4 *>(a_qkv + h * HD + dl * 4);
+    const float4 k0 = *reinterpret_cast<const float4 *>(a_qkv + d + h * HD + dl * 4);
+    const float4 nv = *reinterpret_cast<const float4 *>(a_qkv + 2 * d + h * HD + dl * 4);
+    float4 ka[U], va[U];
+    load_round(ka, va, 0);
     asm volatile("" ::: "memory");
     asm volatile("" : "+v"(q0.x), "+v"(q0.y), "+v"(q0.z), "+v"(q0.w));
-    const float4 qv = make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
+    const float4 qr = make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
                                   q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y);
     const float4 nk = make_float4(k0.x * c2.x - k0.y * s2.x, k0.x * s2.x + k0.y * c2.x,
                                   k0.z * c2.y - k0.w * s2.y, k0.z * s2.y + k0.w * c2.y);
 
     float m = -INFINITY, l = 0.0f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int off = 0;; ) {                                  // every lane runs the same number of rounds
-        const int base = base0 + off;
+    auto compute_round = [&](float4 (&K)[U], float4 (&V)[U], int t0) {
+        float sc[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            int key = base + u * STRIDE;
-            bool valid = key < k_end;                       // uniform over the LPK lanes of a key
-            if (valid && key == pos) {
-                kk[u] = nk; vv[u] = nv;
-                *reinterpret_cast<float4 *>(kb + (int64_t)key * a.tok_stride) = nk;
-                *reinterpret_cast<float4 *>(vb + (int64_t)key * a.tok_stride) = nv;
+            const int key = key0 + (t0 + u) * NS * TILE;
+            const bool valid = key <= pos;                  // uniform over the LPK lanes of a key
+            if (key == pos) {                               // the new row: used from registers, and appended
+                K[u] = nk; V[u] = nv;
+                *reinterpret_cast<float4 *>(kb + (int64_t)key * HD) = nk;
+                *reinterpret_cast<float4 *>(vb + (int64_t)key * HD) = nv;
             }
-            float s = group_sum<LPK>(qv.x * kk[u].x + qv.y * kk[u].y + qv.z * kk[u].z + qv.w * kk[u].w);
-            if (valid) {
-                s *= a.scale;
-                float mn = fmaxf(m, s);
-                float corr = expf(m - mn);
-                float p = expf(s - mn);
-                l = l * corr + p;
-                o.x = o.x * corr + p * vv[u].x; o.y = o.y * corr + p * vv[u].y;
-                o.z = o.z * corr + p * vv[u].z; o.w = o.w * corr + p * vv[u].w;
-                m = mn;
-            }
+            // (q.k) * scale as the reference computes it (HeadOps.java:96-99), then the change of base
+            const float dot = group_sum<LPK>(qr.x * K[u].x + qr.y * K[u].y + qr.z * K[u].z + qr.w * K[u].w);
+            sc[u] = valid ? (dot * a_scale) * kLog2e : -INFINITY;
+            if (!valid) V[u] = make_float4(0.f, 0.f, 0.f, 0.f);       // whatever the row held, it adds nothing
         }
-        off += U * STRIDE;
-        if (off >= per) break;                              // workgroup-uniform
-        load_tile(base0 + off);
+        float mn = m;
+#pragma unroll
+        for (int u = 0; u < U; u++) mn = fmaxf(mn, sc[u]);
+        if (mn > -INFINITY) {
+            const float corr = fast_exp2(m - mn);           // m = -inf: 0
+            l *= corr; o.x *= corr; o.y *= corr; o.z *= corr; o.w *= corr;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float p = fast_exp2(sc[u] - mn);
+                l += p;
+                o.x += p * V[u].x; o.y += p * V[u].y; o.z += p * V[u].z; o.w += p * V[u].w;
+            }
+            m = mn;
+        }
+    };
+    // (Requesting round r + 1 before round r is used - two register sets in turn - was slower: 2419 against 2441 tok/s.)
+    for (int t0 = 0;;) {
+        compute_round(ka, va, t0);
+        if (t0 == 0) DJ_STAMP(2);
+        t0 += U;
+        if (!has_keys(t0)) break;
+        load_round(ka, va, t0);
     }
+    DJ_STAMP(3);
     // the KPW lane groups of a wavefront first (shuffles), then the wavefronts (LDS)
 #pragma unroll
     for (int off = LPK; off < 64; off <<= 1) {
-        float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
-        float4 o2 = make_float4(__shfl_xor(o.x, off, 64), __shfl_xor(o.y, off, 64), __shfl_xor(o.z, off, 64),
-                                __shfl_xor(o.w, off, 64));
-        float mn = fmaxf(m, m2);
-        float w1 = m == -INFINITY ? 0.0f : expf(m - mn), w2 = m2 == -INFINITY ? 0.0f : expf(m2 - mn);
+        const float m2 = __shfl_xor(m, off, 64), l2 = __shfl_xor(l, off, 64);
+        const float4 o2 = make_float4(__shfl_xor(o.x, off, 64), __shfl_xor(o.y, off, 64), __shfl_xor(o.z, off, 64),
+                                      __shfl_xor(o.w, off, 64));
+        const float mn = fmaxf(m, m2);
+        const float w1 = mn == -INFINITY ? 0.0f : fast_exp2(m - mn), w2 = mn == -INFINITY ? 0.0f : fast_exp2(m2 - mn);
         l = l * w1 + l2 * w2;
         o.x = o.x * w1 + o2.x * w2; o.y = o.y * w1 + o2.y * w2; o.z = o.z * w1 + o2.z * w2; o.w = o.w * w1 + o2.w * w2;
         m = mn;
@@ -596,6 +633,7 @@ k_attn_decode_records(const int32_t *a_state, float *a_k_cache, float *a_v_cache
     if (lane == 0) { s_m[wave] = m; s_l[wave] = l; }
     if (sub == 0) *reinterpret_cast<float4 *>(&s_o[wave][dl * 4]) = o;
     __syncthreads();
+    DJ_STAMP(4);
     if (tid < HD) {
         float M = -INFINITY, L = 0.0f, O = 0.0f;
 #pragma unroll
@@ -603,15 +641,16 @@ k_attn_decode_records(const int32_t *a_state, float *a_k_cache, float *a_v_cache
         if (M != -INFINITY) {
 #pragma unroll
             for (int i = 0; i < kRecWaves; i++) {
-                float w = expf(s_m[i] - M);
+                const float w = fast_exp2(s_m[i] - M);
                 L += s_l[i] * w;
                 O += s_o[i][tid] * w;
             }
         }
-        float *rec = a.scratch + ((int64_t)h * a.nsplit + split) * (HD + 4);
+        float *rec = a_records + ((int64_t)h * NS + split) * (HD + 4);
         rec[4 + tid] = O;
         if (tid == 0) { rec[0] = M; rec[1] = L; }
     }
+    DJ_STAMP(5);
 }
 
 
@@ -752,5 +791,11 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
         default: fail("attention: head dim must be 32, 64 or 128");
     }
 }
+
+#ifdef DJ_TRACE
+extern "C" int deepj_hip_debug_attn_trace(unsigned long long *out, int n) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_at_trace), (size_t)n * sizeof(unsigned long long));
+}
+#endif
 
 }  // namespace dj

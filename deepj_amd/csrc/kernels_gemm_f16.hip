@@ -74,13 +74,19 @@ struct GemmF16Args {
     float *partial;             // [gridDim.z][m][n] partial products when split_steps > 0
 };
 
-// 64 lanes x 16 bytes from base + off[lane] into LDS bytes [dst, dst + 1024), lane order
+// 64 lanes x 16 bytes from base + off[lane] into LDS bytes [dst, dst + 1024), lane order.  The statements write M0
+// and say so in their clobber lists, so that the compiler never carries a value of its own in M0 across them (it
+// initialises M0 itself for some LDS and message instructions); clang notes that M0 is a reserved register, which
+// is the point of listing it.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_to_lds16(const void *base, uint32_t off, uint32_t dst) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void load_to_lds4(const void *base, uint32_t off, uint32_t dst) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // Workgroup -> tile.  Workgroups go to the eight XCDs (each with its own L2) round-robin by their linear index, so index L
 // runs on XCD L % 8.  All row tiles of one column tile get indices that agree mod 8: the column tile's weights - the

@@ -35,6 +35,15 @@ using namespace dev;
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 
+// Timeline of one launch, for tuning builds only (-DDJ_TRACE; never in the shipped library): every wavefront leaves
+// 100 MHz time stamps at fixed points of the decode matvec.
+#ifdef DJ_TRACE
+__device__ unsigned long long g_mv_trace[8 * 16384];
+#define DJ_STAMP(i) do { if (lane == 0 && wave_global < 16384) g_mv_trace[wave_global * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define DJ_STAMP(i) do {} while (0)
+#endif
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -260,6 +269,7 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
     const int o_end = p.n_out;
     const int o_begin = wave_global * B;
     const int o_step = wave_count * B;
+    DJ_STAMP(0);
 
     RowBatch<NC, R> ba, bb;
     bool deferred_norm = false;
@@ -319,7 +329,7 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
 #pragma unroll
             for (int sp = 0; sp < NS; sp++) {
                 const float ms = sp == 0 ? m0 : rml[j][sp].x;
-                const float w = ms == -INFINITY ? 0.0f : expf(ms - mx);     // a split without keys
+                const float w = __builtin_amdgcn_exp2f(ms - mx);            // base-2 maxima; a split without keys: exp2(-inf) = 0
                 lsum += rml[j][sp].y * w;
                 acc.x += rov[j][sp].x * w; acc.y += rov[j][sp].y * w; acc.z += rov[j][sp].z * w; acc.w += rov[j][sp].w * w;
             }
@@ -429,7 +439,9 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
             for (int i = tid; i < p.k; i += kThreads) xs[xs_at(i)] = (xs[xs_at(i)] / rms) * p.gamma[i];
         }
     }
+    DJ_STAMP(1);
     lds_barrier();
+    DJ_STAMP(2);
     if (!has_work) return;
     float rms = 1.0f;
     if (deferred_norm) {
@@ -450,13 +462,16 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
         }
     }
 
+    DJ_STAMP(3);
     for (int o0 = o_begin; o0 < o_end; o0 += 2 * o_step) {
         if (o0 + o_step < o_end) { load_batch<NC, R>(bb, p, (o0 + o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(bb, p, o0 + o_step); }
         finish_batch<NC, B, SWIGLU, GELU>(ba, xr, p, o0, o_end, lane, rms);
+        if (o0 == o_begin) DJ_STAMP(4);
         if (o0 + o_step >= o_end) break;
         if (o0 + 2 * o_step < o_end) { load_batch<NC, R>(ba, p, (o0 + 2 * o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(ba, p, o0 + 2 * o_step); }
         finish_batch<NC, B, SWIGLU, GELU>(bb, xr, p, o0 + o_step, o_end, lane, rms);
     }
+    DJ_STAMP(5);
 }
 
 constexpr int kMvGridCap = 768;          // three workgroups per CU
@@ -627,7 +642,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     // many rows and enough tiles: the fp16 kernel, when the caller's workspace also holds its prepared operands; the
     // normalisation happens on the rows' way into that layout
     const int n_rows = swiglu ? 2 * p.n : p.n;
-    if (!p.m_dev && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
+    if (!p.m_dev && !p.small_workspace_only && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
         launch_q8_gemm_f16(s, p.x, gamma, beta, p.wq, p.scales, p.prepared, p.out, p.m, p.k, n_rows, bias, swiglu ? bias2 : nullptr,
                            swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, workspace, workspace_floats);
         return;
@@ -647,5 +662,11 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
         launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0, p.m_dev, p.m_extra, gelu, 0);
     }
 }
+
+#ifdef DJ_TRACE
+extern "C" int deepj_hip_debug_mv_trace(unsigned long long *out, int n) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mv_trace), (size_t)n * sizeof(unsigned long long));
+}
+#endif
 
 }  // namespace dj

@@ -81,9 +81,6 @@ struct Runner {
     int32_t state = -1, tokens = -1, scratch = -1, logits = -1, last_x = -1;
     int32_t records = -1;                                  // decode attention records (merged by the Wo matvec)
     int32_t latent = -1, kv_all = -1;                      // latent cache [L][maxSeq][kvRank]; re-expanded [maxSeq][K | V] of one layer
-    int32_t p_scratch = -1, p_argbuf = -1, p_sync = -1;   // persistent decode kernel (Llama)
-    int64_t p_sync_floats = 0;
-    bool p_pending = false;                                // a persistent launch has not been checked yet
     std::vector<int32_t> prepared;                         // the weights in the many-row GEMM's layout (first long prompt)
     bool prepared_done = false;
     Acts dec, pre;
@@ -358,7 +355,7 @@ void finalize(Runner &r) {
     int ns = std::max(1, std::min(16, 512 / c.heads));
     int64_t sf = (int64_t)c.heads * ns * (hd + 4);           // split-attention records (S = 1 paths)
     r.scratch = r.alloc(sf);
-    r.records = r.alloc((int64_t)c.heads * 4 * (hd + 4));
+    r.records = r.alloc((int64_t)c.heads * deepj_hip_attn_record_splits() * (hd + 4));
     Stream s;
     emit(s, DJ_OP_FILL, r.state, 0, 4);
     r.run(s);
@@ -572,64 +569,15 @@ void warm_up(Runner &r) {
     reset(r);
 }
 
-// The persistent decode kernel (experimental: about half the speed of the replayed graph) gets its buffers on first use.
-void ensure_persistent(Runner &r) {
-    if (r.p_sync >= 0) return;
-    const Config &c = r.cfg;
-    int64_t psf = 0, paf = 0;
-    hip(deepj_hip_llama_decode_plan(c.heads, r.hd(), nullptr, nullptr, &psf, &paf));
-    r.p_scratch = r.alloc(psf);
-    r.p_argbuf = r.alloc(paf);
-    r.p_sync_floats = deepj_hip_llama_decode_sync_floats();
-    r.p_sync = r.alloc(r.p_sync_floats);
-    Stream s;
-    emit(s, DJ_OP_FILL, r.p_sync, 0, r.p_sync_floats);
-    r.run(s);
-}
-
-// All `steps` tokens in one launch of the persistent decode kernel.
-Stream persistent_stream(Runner &r, int steps) {
-    const Config &c = r.cfg;
-    ensure_persistent(r);
-    Stream s;
-    emit(s, DJ_OP_LLAMA_DECODE, 29 + 9 * c.layers, steps, c.d, c.heads, c.dff, c.vocab, c.max_seq, c.layers, c.max_seq,
-         r.emb, r.cos_t, r.sin_t, r.kc, r.vc, r.state, r.tokens, r.dec.x, r.dec.x2, r.dec.qkv, r.dec.att, r.dec.ff,
-         r.logits, r.p_scratch, r.p_argbuf, r.p_sync, r.gf, r.wlm, r.blm);
-    for (const Layer &L : r.layers) emit(s, L.wqkv, L.wo, L.wgu, L.wd, L.g1, L.g2, L.bg, L.bu, L.bd);
-    return s;
-}
-
-// After a persistent launch: state[3] != 0 means a grid barrier timed out and the result is void.
-void check_persistent(Runner &r) {
-    if (!r.p_pending) return;
-    r.p_pending = false;
-    int32_t st[4] = {0, 0, 0, 0};
-    hip(deepj_hip_download(r.state, reinterpret_cast<float *>(st), 4));
-    if (st[3] != 0) {
-        Stream s;
-        emit(s, DJ_OP_FILL, r.p_sync, 0, r.p_sync_floats);
-        r.run(s);
-        st[3] = 0;
-        hip(deepj_hip_upload(r.state, reinterpret_cast<const float *>(st), 4));
-        throw Error("persistent decode: a grid barrier timed out (were all compute units available?); the sequence "
-                    "state is invalid, reset and run again");
-    }
-}
-
 // Greedy steps on the device: each consumes state[1] at position state[0] and appends the argmax.
-// mode 0: the per-token stream, eagerly; 1: the same stream as a replayed HIP graph; 2: persistent kernel.
+// mode 0: the per-token stream, eagerly; 1: the same stream as a replayed HIP graph.
 void decode_greedy(Runner &r, int steps, int mode) {
     const Config &c = r.cfg;
     if (steps <= 0) return;
     if (r.pos + steps > c.max_seq)
         throw Error("context of " + std::to_string(r.pos + steps) + " tokens exceeds maxSeqLen " + std::to_string(c.max_seq));
-    if (mode == 2 && c.kind != 0) throw Error("the persistent decode kernel covers the Llama block only");
     const bool use_graph = mode == 1;
-    if (mode == 2) {
-        check_persistent(r);
-        r.run(persistent_stream(r, steps));
-        r.p_pending = true;
-    } else if (use_graph) {
+    if (use_graph) {
         // A replay costs a few microseconds of its own on top of its kernels: long runs go through a graph
         // that holds kGraphUnroll consecutive tokens, the remainder through the one-token graph.
         const int runs = steps / kGraphUnroll, rest = steps % kGraphUnroll;
@@ -741,7 +689,6 @@ void generate(Runner &r, const int32_t *prompt, int n_prompt, int max_new, float
         if (cached > 0 && greedy) {
             prefill(r, prompt, n_prompt, nullptr, true);
             decode_greedy(r, cached - 1, mode);
-            check_persistent(r);
             hip(deepj_hip_download(r.tokens, reinterpret_cast<float *>(out + n_prompt), cached));
         } else if (cached > 0) {
             Stream fwd = decode_stream(r, false);
@@ -818,7 +765,7 @@ void deepj_runner_destroy(void *h) {
                            L.bu, L.wd, L.bd})
             add(id);
     for (int32_t id : {r->emb, r->gf, r->wlm, r->blm, r->cos_t, r->sin_t, r->kc, r->vc, r->state,
-                       r->tokens, r->scratch, r->records, r->logits, r->last_x, r->p_scratch, r->p_argbuf, r->p_sync,
+                       r->tokens, r->scratch, r->records, r->logits, r->last_x,
                        r->pos_table, r->bf, r->latent, r->kv_all})
         add(id);
     for (Acts *a : {&r->dec, &r->pre})
@@ -871,7 +818,7 @@ int deepj_runner_prefill(void *h, const int32_t *ids, int32_t n, float *all_logi
 int deepj_runner_decode(void *h, int32_t steps, int32_t mode) {
     auto *r = static_cast<Runner *>(h);
     return guarded(r, [&] {
-        if (mode < 0 || mode > 2) throw Error("decode: mode must be 0 (eager), 1 (graph) or 2 (persistent kernel)");
+        if (mode < 0 || mode > 1) throw Error("decode: mode must be 0 (eager) or 1 (graph)");
         decode_greedy(*r, steps, mode);
     });
 }
@@ -884,7 +831,6 @@ int deepj_runner_step(void *h, int32_t token) {
 int deepj_runner_last_logits(void *h, float *out) {
     auto *r = static_cast<Runner *>(h);
     return guarded(r, [&] {
-        check_persistent(*r);
         hip(deepj_hip_download(r->logits, out, r->cfg.vocab));
     });
 }
@@ -893,7 +839,6 @@ int deepj_runner_last_logits(void *h, float *out) {
 int deepj_runner_tokens(void *h, int32_t *out, int32_t capacity, int32_t *n) {
     auto *r = static_cast<Runner *>(h);
     return guarded(r, [&] {
-        check_persistent(*r);
         int32_t count = std::min(r->generated, capacity);
         if (count > 0) hip(deepj_hip_download(r->tokens, reinterpret_cast<float *>(out), count));
         else hip(deepj_hip_synchronize());
@@ -905,7 +850,7 @@ int deepj_runner_generate(void *h, const int32_t *prompt, int32_t n_prompt, int3
                           int32_t top_k, int64_t seed, int32_t mode, int32_t *out) {
     auto *r = static_cast<Runner *>(h);
     return guarded(r, [&] {
-        if (mode < 0 || mode > 2) throw Error("generate: mode must be 0 (eager), 1 (graph) or 2 (persistent kernel)");
+        if (mode < 0 || mode > 1) throw Error("generate: mode must be 0 (eager) or 1 (graph)");
         generate(*r, prompt, n_prompt, max_new, temperature, top_k, seed, out, mode);
     });
 }

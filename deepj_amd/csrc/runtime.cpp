@@ -69,8 +69,6 @@ struct Runtime {
     Graph *capture_into = nullptr;                               // graph capture: the graph the run pass records for
     struct Prepared { int32_t id; int k, rows; };
     std::unordered_map<int32_t, Prepared> prepared;   // Q8 weight buffer -> its copy in the fp16 GEMM's layout (OP_Q8_PREPARE)
-    void *decode_table = nullptr;                  // device copy of LLAMA_DECODE's layer table
-    std::vector<int64_t> decode_table_key;
 };
 
 Runtime g;
@@ -233,7 +231,6 @@ int stride_of(int op) {
         case DJ_OP_ATTN_DECODE: return 13;
         case DJ_OP_APPEND_ROWS: return 8;
         case DJ_OP_Q8_LINEAR_DYN: return 10;
-        case DJ_OP_LLAMA_DECODE: return 0;      // variable: word 1
         case DJ_OP_LAYERNORM: return 7;
         case DJ_OP_ATTN_DECODE_RECORDS: return 12;
         case DJ_OP_ADD_POSITIONS: return 7;
@@ -472,6 +469,9 @@ void exec_one(Cursor &c) {
             int64_t ws = g.no_alloc ? q8_linear_workspace_floats((int)m, (int)k, (int)n, flags)
                                     : q8_linear_preferred_workspace_floats((int)m, (int)k, (int)n, flags, p.prepared != nullptr);
             if (c.dry) c.ws_need = std::max(c.ws_need, ws);
+            // One rule for the allocation-free entry point, whatever happens to fit its fixed array: the many-row
+            // fp16 GEMM (whose operands live in a workspace sized by the shape) is never taken there.
+            p.small_workspace_only = g.no_alloc;
             if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
             break;
         }
@@ -683,80 +683,6 @@ void exec_one(Cursor &c) {
             if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
             break;
         }
-        case DJ_OP_LLAMA_DECODE: {
-            const int len = w[1];
-            if (len < 29) fail("OP_LLAMA_DECODE: length word below the 29 header words");    // before any of them is read
-            if (g.no_alloc) fail("OP_LLAMA_DECODE keeps a device copy of its layer table and cannot run allocation-free");
-            const int64_t steps = w[2], d = w[3], H = w[4], dff = w[5], vocab = w[6], max_seq = w[7], L = w[8], cap = w[9];
-            if (steps < 0 || d <= 0 || H <= 0 || dff <= 0 || vocab <= 0 || max_seq <= 0 || L <= 0 || cap < 0 || d % H)
-                fail("OP_LLAMA_DECODE: bad shape");
-            if (len != 29 + 9 * L) fail("OP_LLAMA_DECODE: length word does not match the layer count");
-            if (g.capturing) fail("OP_LLAMA_DECODE cannot be captured into a graph");
-            const int64_t hd = d / H;
-            int grid = 0, ns = 0; int64_t sf = 0, af = 0;
-            llama_decode_plan((int)H, (int)hd, &grid, &ns, &sf, &af);
-            auto q8 = [&](int32_t id, int64_t k, int64_t rows, const char *role) {
-                const float *base = buf(id, (q8_bytes((int)k, (int)rows) + 3) / 4, op, role);
-                Q8Mat m;
-                m.w = reinterpret_cast<const int8_t *>(base);
-                m.sc = reinterpret_cast<const float *>(m.w + q8_scale_offset_bytes((int)k, (int)rows));
-                m.k = (int)k; m.kp = q8_padded_k((int)k); m.rows = (int)rows;
-                return m;
-            };
-            DecodeParams p{};
-            p.d = (int)d; p.H = (int)H; p.hd = (int)hd; p.dff = (int)dff; p.vocab = (int)vocab; p.max_seq = (int)max_seq;
-            p.L = (int)L; p.steps = (int)steps; p.capacity = (int)cap;
-            p.emb = buf(w[10], vocab * d, op, "embedding");
-            p.cos_t = buf(w[11], max_seq * (hd / 2), op, "cos");
-            p.sin_t = buf(w[12], max_seq * (hd / 2), op, "sin");
-            p.kc = buf(w[13], L * max_seq * d, op, "k cache");
-            p.vc = buf(w[14], L * max_seq * d, op, "v cache");
-            p.state = reinterpret_cast<int32_t *>(buf(w[15], 4, op, "state"));
-            p.tokens = reinterpret_cast<int32_t *>(buf(w[16], cap, op, "tokens"));
-            p.x = buf(w[17], d, op, "x"); p.x2 = buf(w[18], d, op, "x2"); p.qkv = buf(w[19], 3 * d, op, "qkv");
-            p.att = buf(w[20], d, op, "att"); p.ff = buf(w[21], dff, op, "ff"); p.logits = buf(w[22], vocab, op, "logits");
-            p.scratch = buf(w[23], sf, op, "scratch"); p.argbuf = buf(w[24], af, op, "argbuf");
-            p.sync = reinterpret_cast<unsigned *>(buf(w[25], llama_decode_sync_words(), op, "sync"));
-            p.gf = buf(w[26], d, op, "final norm gain");
-            p.lm = q8(w[27], d, vocab, "lm head");
-            p.blm = buf(w[28], vocab, op, "lm bias");
-            std::vector<DecodeLayer> table((size_t)L);
-            for (int64_t l = 0; l < L; l++) {
-                const int32_t *q = w + 29 + 9 * l;
-                DecodeLayer &T = table[(size_t)l];
-                T.qkv = q8(q[0], d, 3 * d, "wqkv"); T.wo = q8(q[1], d, d, "wo");
-                T.gu = q8(q[2], d, 2 * dff, "wgu"); T.down = q8(q[3], dff, d, "wd");
-                T.g1 = buf(q[4], d, op, "g1"); T.g2 = buf(q[5], d, op, "g2");
-                T.bg = buf(q[6], dff, op, "bg"); T.bu = buf(q[7], dff, op, "bu"); T.bd = buf(q[8], d, op, "bd");
-            }
-            if (!llama_decode_supported((int)d, (int)dff))
-                fail("OP_LLAMA_DECODE: dModel above 2048 or dFF above 6144 is not supported by the persistent kernel");
-            if (run && steps > 0) {
-                // device copy of the layer table, rebuilt only when a pointer in it changes
-                const size_t bytes = table.size() * sizeof(DecodeLayer);
-                std::vector<int64_t> key;
-                for (const DecodeLayer &T : table) {
-                    for (const Q8Mat *m : {&T.qkv, &T.wo, &T.gu, &T.down}) {
-                        key.push_back((int64_t)(intptr_t)m->w); key.push_back((int64_t)(intptr_t)m->sc);
-                        key.push_back(m->k); key.push_back(m->rows);
-                    }
-                    for (const float *q : {T.g1, T.g2, T.bg, T.bu, T.bd}) key.push_back((int64_t)(intptr_t)q);
-                }
-                if (key != g.decode_table_key) {
-                    DJ_HIP(hipStreamSynchronize(g.stream));
-                    if (g.decode_table) DJ_HIP(hipFree(g.decode_table));
-                    g.decode_table = nullptr;
-                    DJ_HIP(hipMalloc(&g.decode_table, bytes));
-                    DJ_HIP(hipMemcpy(g.decode_table, table.data(), bytes, hipMemcpyHostToDevice));
-                    g.decode_table_key = key;
-                    g.driver_allocs++;
-                }
-                p.layers = static_cast<const DecodeLayer *>(g.decode_table);
-                p.layers_host = table.data();
-                launch_llama_decode(s, p);
-            }
-            break;
-        }
         case DJ_OP_COPY: {
             int64_t n = w[3], so = w[4], dof = w[5];
             if (n < 0 || so < 0 || dof < 0) fail("OP_COPY: bad range");
@@ -868,7 +794,6 @@ const char *op_name(int op) {
         case DJ_OP_ATTN_DECODE: return "OP_ATTN_DECODE";
         case DJ_OP_APPEND_ROWS: return "OP_APPEND_ROWS";
         case DJ_OP_Q8_LINEAR_DYN: return "OP_Q8_LINEAR_DYN";
-        case DJ_OP_LLAMA_DECODE: return "OP_LLAMA_DECODE";
         case DJ_OP_STREAM_READ: return "OP_STREAM_READ";
         case DJ_OP_NOP: return "OP_NOP";
         case DJ_OP_Q8_PREPARE: return "OP_Q8_PREPARE";
@@ -1048,8 +973,7 @@ int deepj_hip_shutdown(void) {
         g.workspace = nullptr; g.workspace_floats = 0;
         if (g.attn_counters) (void)hipFree(g.attn_counters);
         g.attn_counters = nullptr;
-        if (g.decode_table) (void)hipFree(g.decode_table);
-        g.decode_table = nullptr; g.decode_table_key.clear();
+        g.prepared.clear();      // the association names buffer ids; a later session may reuse them for other things
         if (g.staging) (void)hipHostFree(g.staging);
         g.staging = nullptr;
         (void)hipStreamDestroy(g.stream);
@@ -1071,19 +995,7 @@ int deepj_hip_pool_stats(int64_t out[4]) {
 
 void *deepj_hip_stream(void) { return g.ready ? (void *)g.stream : nullptr; }
 
-int deepj_hip_llama_decode_plan(int32_t heads, int32_t head_dim, int32_t *grid, int32_t *nsplit,
-                                int64_t *scratch_floats, int64_t *argbuf_floats) {
-    return guarded([&] {
-        ensure_init();
-        if (heads <= 0 || head_dim <= 0) fail("llama_decode_plan: bad shape");
-        int gr = 0, ns = 0;
-        llama_decode_plan(heads, head_dim, &gr, &ns, scratch_floats, argbuf_floats);
-        if (grid) *grid = gr;
-        if (nsplit) *nsplit = ns;
-    });
-}
-
-int64_t deepj_hip_llama_decode_sync_floats(void) { return llama_decode_sync_words(); }
+int32_t deepj_hip_attn_record_splits(void) { return kAttnRecordSplits; }
 
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows) {
     if (k <= 0 || rows <= 0) return 0;

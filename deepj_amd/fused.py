@@ -169,7 +169,7 @@ def attn_decode_scratch_floats(H: int, hd: int) -> int:
 
 def attn_record_floats(H: int, hd: int) -> int:
     """Floats of the records buffer ATTN_DECODE_RECORDS writes and the ATTN_MERGE prologue reads."""
-    return H * op.ATTN_RECORD_SPLITS * (hd + 4)
+    return H * HipNative.attnRecordSplits() * (hd + 4)
 
 
 def attention_scratch_floats(H: int, hd: int, max_seq: int = 0) -> int:

@@ -28,7 +28,7 @@ final class HipRunnerNative {
     /** Logits {@code [ids.length x vocab]} of a fresh sequence, row-major (DecoderOnlyModel.forward). */
     static native float[] forward(long handle, int[] ids, int vocab);
 
-    /** TextGenerator.generate on token ids: returns prompt + maxNewTokens ids.  mode 0 eager, 1 graph, 2 persistent. */
+    /** TextGenerator.generate on token ids: returns prompt + maxNewTokens ids.  mode 0 eager, 1 graph. */
     static native int[] generate(long handle, int[] prompt, int maxNewTokens, float temperature, int topK, long seed,
                                  int mode);
 }

@@ -221,15 +221,12 @@ class _DecoderOnlyModel:
         self._check(_lib().deepj_runner_prefill(self._h, ids.ctypes.data_as(_i32p), len(ids), None,
                                                 1 if choose_next else 0))
 
-    def _mode(self, use_graph, persistent) -> int:
-        """0 eager per-token stream, 1 the stream as a replayed HIP graph (default), 2 the persistent
-        decode kernel (Llama with dModel <= 2048 and dFF <= 6144)."""
-        if persistent:
-            return 2
+    def _mode(self, use_graph) -> int:
+        """0 eager per-token stream, 1 the stream as a replayed HIP graph (default)."""
         return 0 if use_graph is False else 1
 
-    def decode(self, steps: int, use_graph: bool | None = None, persistent: bool | None = None) -> None:
-        self._check(_lib().deepj_runner_decode(self._h, steps, self._mode(use_graph, persistent)))
+    def decode(self, steps: int, use_graph: bool | None = None) -> None:
+        self._check(_lib().deepj_runner_decode(self._h, steps, self._mode(use_graph)))
 
     def step(self, token: int) -> None:
         """Feed one caller-chosen token through the single-row (cached) path; see lastLogits()."""
@@ -294,11 +291,10 @@ class TextGenerator:
 
     @staticmethod
     def generate(model: _DecoderOnlyModel, prompt_ids, max_new_tokens: int, temperature: float = 1.0,
-                 top_k: int = 1, seed: int = 0, use_graph: bool | None = None,
-                 persistent: bool | None = None) -> np.ndarray:
+                 top_k: int = 1, seed: int = 0, use_graph: bool | None = None) -> np.ndarray:
         prompt = np.ascontiguousarray(np.asarray(prompt_ids, dtype=np.int32))
         out = np.empty(len(prompt) + max(max_new_tokens, 0), dtype=np.int32)
         model._check(_lib().deepj_runner_generate(model._h, prompt.ctypes.data_as(_i32p), len(prompt),
                                                   max_new_tokens, temperature, top_k, seed,
-                                                  model._mode(use_graph, persistent), out.ctypes.data_as(_i32p)))
+                                                  model._mode(use_graph), out.ctypes.data_as(_i32p)))
         return out

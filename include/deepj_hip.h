@@ -53,14 +53,17 @@ int deepj_hip_release(const int32_t *ids, int32_t count);
 int deepj_hip_flush_ops(const int32_t *cmd, int32_t len);
 
 /* deepj_hip_flush_ops for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same streams, same
- * kernels, same results; the device scratch those kernels need - the workspace that Q8_LINEAR with a norm
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same streams and
+ * the same kernels and bits as deepj_hip_flush_ops, with ONE exception: a Q8_LINEAR of 256 rows or more that
+ * flush_ops runs on the fp16 GEMM (operands in a workspace sized by the shape) always runs on the bf16 GEMM here,
+ * prepared weights or not - both meet the per-op tolerance against the CPU backend, their bits differ.  The
+ * device scratch the kernels need - the workspace that Q8_LINEAR with a norm
  * prologue and M > 1 writes its normalised rows to, and the arrival counters of the split decode attention
  * (ATTENTION / ATTENTION_KV with S = 1, ATTN_DECODE) - is a fixed array inside the library's code object instead
  * of memory the runtime allocates and grows.  The call never calls hipMalloc or hipFree: it fails when the
  * runtime is not initialised yet (deepj_hip_init allocates), when the stream needs more than
- * DEEPJ_HIP_NOALLOC_WORKSPACE_FLOATS floats of workspace (M * K of the largest such Q8_LINEAR), and on
- * LLAMA_DECODE.  Every buffer the stream names must already exist.  All calls on a GPU share the one array,
+ * DEEPJ_HIP_NOALLOC_WORKSPACE_FLOATS floats of workspace (M * K of the largest such Q8_LINEAR).
+ * Every buffer the stream names must already exist.  All calls on a GPU share the one array,
  * which keeps the previous call's contents (the counters are cleared by a kernel at the start of each call);
  * calls that overlap on one GPU would race - the single-caller rule above already excludes that. */
 #define DEEPJ_HIP_NOALLOC_WORKSPACE_FLOATS (2 << 20)
@@ -168,21 +171,10 @@ enum {
      * Q8_LINEAR_DYN [op, x, w, out, Mmax, K, N, state, extraRows, xOff]
      *     Q8_LINEAR (no prologue/epilogue) on rows [0, min(Mmax, state[0]+extraRows)) of x + xOff: the row count
      *     lives on the device, so the op can sit in a replayed graph while a cache grows
-     * LLAMA_DECODE  [op, len, steps, d, H, dFF, vocab, maxSeq, L, capacity,
-     *                emb, cosT, sinT, kCache, vCache, state, tokens, x, x2, qkv, att, ff, logits, scratch, argbuf, sync,
-     *                gf, wlm, blm,  then per layer: wqkv, wo, wgu, wd, g1, g2, bg, bu, bd]      (len = 29 + 9 L words)
-     *     `steps` greedy tokens of the whole Llama block stack (LlamaTransformerBlock.java:50-53,
-     *     DecoderOnlyModel.java:58-64, TextGenerator.java:91-114 with topK = 1) in ONE persistent launch: the
-     *     phases of a token are separated by grid-wide barriers instead of kernel boundaries and the Q8 rows of
-     *     the next phase stream into LDS while the current one finishes.  Starts from state[0] (positions in the
-     *     cache) and state[1] (token to process); appends to kCache/vCache and tokens, leaves the last logits in
-     *     `logits`, advances state[0..2]; state[3] != 0 afterwards means a grid barrier timed out (result invalid).
-     *     wqkv [3d x d], wgu interleaved [2 dFF x d], all weights Q8.  scratch >= H*nsplit*(hd+4) floats, argbuf >=
-     *     2*grid floats (deepj_hip_llama_decode_plan), sync = deepj_hip_llama_decode_sync_floats() floats, zero-filled
-     *     once.  Not capturable into a graph; calls that overlap on one device are not supported.
      * ATTN_DECODE_RECORDS [op, qkv, kCache, vCache, records, state, cosT, sinT, H, hd, maxSeq, layer]
-     *     ATTN_DECODE that stops before the merge of its key splits: records holds H * 4 * (hd + 4) floats,
-     *     per (head, split) {max, sum, -, -, o[hd]}; a Q8_LINEAR with the ATTN_MERGE prologue consumes them.
+     *     ATTN_DECODE that stops before the merge of its key splits: records holds
+     *     H * deepj_hip_attn_record_splits() * (hd + 4) floats, per (head, split) {max, sum, -, -, o[hd]} with the
+     *     maximum in base-2 units (score * log2 e); a Q8_LINEAR with the ATTN_MERGE prologue consumes them.
      *     (Merging across workgroups inside one kernel costs three dependent trips to memory; across the
      *     kernel boundary it is free.)
      * LAYERNORM     [op, x, gamma, beta, out, rows, cols]      J/layers/transformer/norm/LayerNorm1D.java:34-66
@@ -203,18 +195,15 @@ enum {
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
-    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, DJ_OP_LLAMA_DECODE = 82, DJ_OP_LAYERNORM = 83,
+    DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, /* 82 unused */ DJ_OP_LAYERNORM = 83,
     DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85, DJ_OP_STREAM_READ = 86, DJ_OP_NOP = 87, DJ_OP_Q8_PREPARE = 88
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8, DJ_LIN_LAYERNORM = 16,
        DJ_LIN_GELU = 32, DJ_LIN_ATTN_MERGE = 64 };
 
-/* Buffer sizes LLAMA_DECODE needs on this device: workgroups launched, key splits per head, floats of
- * `scratch` and `argbuf`; and the floats of its `sync` buffer. */
-int deepj_hip_llama_decode_plan(int32_t heads, int32_t head_dim, int32_t *grid, int32_t *nsplit,
-                                int64_t *scratch_floats, int64_t *argbuf_floats);
-int64_t deepj_hip_llama_decode_sync_floats(void);
+/* Key splits per head of ATTN_DECODE_RECORDS: its records buffer holds H * splits * (hd + 4) floats. */
+int32_t deepj_hip_attn_record_splits(void);
 
 /* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
@@ -265,7 +254,7 @@ int deepj_runner_finalize(void *runner);
 int deepj_runner_reset(void *runner);
 int deepj_runner_prefill(void *runner, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next);
 /* Greedy decode of `steps` tokens on the device.  mode 0: the per-token stream, launched eagerly; 1: the same
- * stream replayed as a HIP graph; 2: one launch of the persistent kernel (LLAMA_DECODE; Llama only). */
+ * stream replayed as a HIP graph. */
 int deepj_runner_decode(void *runner, int32_t steps, int32_t mode);
 int deepj_runner_step(void *runner, int32_t token);     /* one caller-chosen token through the S=1 path */
 int deepj_runner_last_logits(void *runner, float *out);

@@ -158,8 +158,6 @@ def test_gpt_greedy_64_tokens_identical_to_oracle(g1):
         got = TextGenerator.generate(gpu, prompt, 64, top_k=1, **kw)
         assert np.array_equal(got, exp), f"{kw}: first mismatch at {int(np.argmax(got != exp))}"
         assert float(np.max(np.abs(gpu.lastLogits() - exp_logits[-1]))) <= 1e-3
-    with pytest.raises(RuntimeError, match="Llama block only"):
-        TextGenerator.generate(gpu, prompt, 4, top_k=1, persistent=True)
 
 
 def test_gpt_decode_row_equals_prefill_row_and_positions_advance(g1):

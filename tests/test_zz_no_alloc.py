@@ -94,6 +94,51 @@ def test_noalloc_flush_matches_flush_on_two_calls_the_second_smaller():
         dev.release_all()
 
 
+def test_noalloc_flush_with_256_rows_and_more_stays_on_the_small_workspace_kernels():
+    """From 256 rows on flush_ops may run a Q8_LINEAR on the fp16 GEMM, whose operands live in a workspace sized by the
+    shape; the allocation-free entry point never does, whether the fp16 kernel's need would happen to fit the fixed
+    array (prepared weights: about 1.1 M floats here) or not (unprepared: about 7.6 M).  Both entry points are
+    held to the oracle at the per-op tolerance; the allocation-free result is the same bits with and without a
+    prepared copy of the weights (the copy is not used there), which the fp16 kernel's would not be against the
+    bf16 kernel's."""
+    HipNative.init(0)
+    dev = DeviceBuffers()
+    try:
+        m, k, n = 512, 2048, 6144
+        w = gaussian(k, n, 31, 0.02)
+        x = gaussian(m, k, 32)
+        gamma = 1.0 + gaussian(1, k, 33, 0.02)
+        src = dev.upload(w)
+        wq = dev.alloc(HipNative.q8Floats(k, n))
+        Stream().q8_quantize(src, wq, k, n).run()
+        dev.release(src)
+        xb, gb, out = dev.upload(x), dev.upload(gamma), dev.alloc(m * n)
+        exp = ref.matmul(ref.rmsnorm(x, gamma), ref.q8_roundtrip(w))
+        scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+        words = Stream().q8_linear(xb, wq, out, m, k, n, gamma=gb).array()
+
+        def noalloc():
+            dev.write(out, np.zeros(m * n, np.float32))
+            before = HipNative.poolStats()["driver_allocs"]
+            HipNative.flushOpsNoAlloc(words, words.size)
+            got = dev.download(out, (m, n))
+            assert HipNative.poolStats()["driver_allocs"] == before, "the allocation-free entry point allocated"
+            assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what="noalloc GEMM vs oracle")
+            return got
+
+        plain = noalloc()
+        HipNative.nativeFlushOps(words, words.size)
+        assert_close(exp, dev.download(out, (m, n)), atol=1e-4 * scale, rtol=1e-4, what="flush_ops GEMM vs oracle")
+        prepared = dev.alloc(HipNative.q8PreparedFloats(k, n))
+        Stream().q8_prepare(wq, prepared, k, n).run()
+        assert np.array_equal(noalloc().view(np.int32), plain.view(np.int32)), \
+            "a prepared copy of the weights changed the allocation-free result"
+        HipNative.nativeFlushOps(words, words.size)
+        assert_close(exp, dev.download(out, (m, n)), atol=1e-4 * scale, rtol=1e-4, what="flush_ops GEMM (prepared) vs oracle")
+    finally:
+        dev.release_all()
+
+
 def test_noalloc_flush_rejects_what_it_cannot_serve():
     HipNative.init(0)
     dev = DeviceBuffers()
