@@ -213,6 +213,182 @@ def prefill_roofline(model, n: int, iters: int = 6):
             "timing": "mean kernel duration (start/stop events on each dispatch, whole prompt in order)"}
 
 
+C2_SHAPES = [(2048, 2048), (2048, 5632), (5632, 2048), (4096, 11008)]     # K x N of the isolated linear-op sweep
+C2_ROTATION_BYTES = 512 << 20      # distinct Q8 copies a cache-cold row rotates over: twice the 256 MB Infinity Cache
+
+
+def _best_of(fn, reps: int) -> float:
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def c2_sweep(iters: int = 10, cpu: bool = True):
+    """The isolated linear-op sweep as a measurement: the four weight shapes at M = 1 (decode matvec; cache-cold
+    over a rotation of distinct Q8 copies and cache-warm on one copy), M = 64 and M = 512 (prompt GEMM), and the
+    fused RMSNorm / SiLU-times-up / RoPE-and-cache-append ops on [M x 2048] and [M x 5632] rows; next to each row
+    the CPU oracle's matmul, RMSNorm or SiLU-times-up on the same shape (best of a few runs after a warm-up, like the
+    reference's own harness: MetalBackendAllOpsPerformanceTest.java:85-107).  Weight VALUES come from numpy here
+    (a timing does not depend on them; the parity of this sweep, on the java.util.Random streams the baseline
+    states, is tests/test_gpu_c2_sweep.py).  GPU times are launch periods of back-to-back launches (HIP events
+    around the whole run, every helper kernel of an op included)."""
+    from deepj_amd import HipNative
+    from deepj_amd.fused import DeviceBuffers, Stream
+    rng = np.random.default_rng(1)
+    dev = DeviceBuffers()
+    ref = None
+    threads = 1
+    if cpu:
+        from oracle import cpu_ref as ref
+        threads = ref.default_threads()
+        ref.set_threads(threads)
+        ref.set_column_parallel(False)
+    linear, fused = [], []
+
+    def period_us(stream, launches, n_iters=iters):
+        stream.time(2)
+        return stream.time(n_iters) * 1e3 / (n_iters * launches)
+
+    for k, n in C2_SHAPES:
+        w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+        q_floats = HipNative.q8Floats(k, n)
+        nbytes = q8_linear_bytes(k, n)
+        copies = max(2, -(-C2_ROTATION_BYTES // (4 * q_floats)))
+        src = dev.upload(w)
+        qs = [dev.alloc(q_floats) for _ in range(copies)]
+        Stream().q8_quantize(src, qs[0], k, n).run()
+        dev.release(src)
+        dup = Stream()
+        for q in qs[1:]:
+            dup.copy(qs[0], q, q_floats)
+        dup.run()
+        for m in (1, 64, 512):
+            x_host = rng.standard_normal((m, k)).astype(np.float32)
+            x, out = dev.upload(x_host), dev.alloc(m * n)
+            row = {"K": k, "N": n, "M": m}
+            if m == 1:
+                cold, warm = Stream(), Stream()
+                for q in qs:
+                    cold.q8_linear(x, q, out, 1, k, n)
+                    warm.q8_linear(x, qs[0], out, 1, k, n)
+                cold.profile(2)
+                ev = float(np.mean(cold.profile(iters)))
+                cold_us, warm_us = period_us(cold, copies), period_us(warm, copies)
+                row.update({"kernel": "k_q8_matvec", "bytes": nbytes, "rotation_copies": copies,
+                            "cold_us": round(cold_us, 3), "cold_GBs": round(nbytes / cold_us / 1e3, 1),
+                            "cold_frac_of_hbm_peak": round(nbytes / cold_us / 1e3 / HBM_PEAK_GBS, 4),
+                            "cold_kernel_us": round(ev, 3),
+                            "cold_kernel_frac_of_hbm_peak": round(nbytes / ev / 1e3 / HBM_PEAK_GBS, 4),
+                            "warm_us": round(warm_us, 3), "warm_GBs": round(nbytes / warm_us / 1e3, 1)})
+            else:
+                tile, tile_cols, shares = HipNative.q8GemmTile(m, k, n)
+                flops = 2.0 * m * k * n
+                use = qs[:min(copies, 4)]
+                plain = Stream()
+                for q in use:
+                    plain.q8_linear(x, q, out, m, k, n)
+                us = period_us(plain, len(use))
+                row.update({"kernel": (f"k_gemm_q8_f16 ({tile} x {tile_cols} tiles" + (f", K shared by {shares}" if shares > 1 else "") +
+                                       ", fp16 x 2) + k_split_f16 + k_q8_to_f16") if tile else "k_gemm_q8 (bf16 x 3)",
+                            "flops": flops, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                            "frac_of_mfma_peak": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4)})
+                if tile:
+                    # with the weight kept in the GEMM's own layout (OP_Q8_PREPARE), as the decode driver keeps them
+                    prep = [dev.alloc(HipNative.q8PreparedFloats(k, n)) for _ in use[:2]]
+                    ps = Stream()
+                    for q, pb in zip(use, prep):
+                        ps.q8_prepare(q, pb, k, n)
+                    ps.run()
+                    prepared = Stream()
+                    for q in use[:2]:
+                        prepared.q8_linear(x, q, out, m, k, n)
+                    pus = period_us(prepared, len(use[:2]))
+                    row.update({"prepared_us": round(pus, 2), "prepared_TFLOPs": round(flops / pus / 1e6, 1),
+                                "prepared_frac_of_mfma_peak": round(flops / pus / 1e6 / MFMA_PEAK_TFLOPS, 4)})
+                    dev.release(*prep)       # releasing a prepared copy ends its association with the weight
+            if ref is not None:
+                reps = 1 if m * k * n > 2e9 else 3      # (the oracle multiplies the fp32 weights, as CpuBackend.matmul does)
+                if reps > 1:
+                    ref.matmul(x_host, w)
+                t = _best_of(lambda: ref.matmul(x_host, w), reps)
+                row["cpu_us"] = round(t * 1e6, 1)
+                row["cpu_threads"] = 1 if m == 1 else min(threads, m)
+            dev.release(x, out)
+            linear.append(row)
+        dev.release(*qs)
+
+    # fused element-wise and norm ops: rows rotate over enough buffers that the larger ones come from HBM
+    H, hd = 32, 64
+    for d in (2048, 5632):
+        for m in (1, 64, 512):
+            n_el = m * d
+            x_host = rng.standard_normal((m, d)).astype(np.float32)
+            g_host = (1.0 + 0.02 * rng.standard_normal((1, d))).astype(np.float32)
+            rot = int(max(2, min(48, -(-C2_ROTATION_BYTES // (12 * n_el)))))
+            xs = [dev.upload(x_host) for _ in range(rot)]
+            ys = [dev.upload(x_host) for _ in range(rot)]
+            outs = [dev.alloc(n_el) for _ in range(rot)]
+            gam = dev.upload(g_host)
+            s1, s2 = Stream(), Stream()
+            for a, b, o in zip(xs, ys, outs):
+                s1.rmsnorm(a, gam, o, m, d)
+                s2.silu_mul(a, b, o, n_el)
+            for name, st, nbytes in (("rmsnorm", s1, 4 * (2 * n_el + d)), ("silu_mul", s2, 12 * n_el)):
+                us = period_us(st, rot)
+                st.profile(2)
+                ev = float(np.mean(st.profile(iters)))
+                row = {"op": name, "M": m, "cols": d, "bytes": nbytes, "rotation_buffers": rot, "us": round(us, 3),
+                       "GBs": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                       "kernel_us": round(ev, 3), "kernel_frac_of_hbm_peak": round(nbytes / ev / 1e3 / HBM_PEAK_GBS, 4)}
+                if ref is not None:
+                    fn = (lambda: ref.rmsnorm(x_host, g_host)) if name == "rmsnorm" else (lambda: ref.multiply(ref.silu(x_host), x_host))
+                    fn()
+                    row["cpu_us"] = round(_best_of(fn, 3) * 1e6, 1)
+                    row["cpu_threads"] = min(threads, m)
+                fused.append(row)
+            dev.release(*xs, *ys, *outs, gam)
+    # RoPE on Q and K with the append of K and V to the cache (ROPE_KV_STORE), d = 2048 as 32 heads of 64
+    d = H * hd
+    theta = np.arange(2048, dtype=np.float64)[:, None] / np.power(10000.0, 2.0 * np.arange(hd // 2) / hd)[None, :]
+    cos, sin = np.cos(theta).astype(np.float32), np.sin(theta).astype(np.float32)
+    cos_b, sin_b = dev.upload(cos), dev.upload(sin)
+    state = dev.upload(np.zeros(4, np.int32))
+    for m in (1, 64, 512):
+        rot = int(max(2, min(32, -(-C2_ROTATION_BYTES // (40 * m * d)))))
+        qkvs = [dev.upload(rng.standard_normal((m, 3 * d)).astype(np.float32)) for _ in range(rot)]
+        qo = [dev.alloc(m * d) for _ in range(rot)]
+        kc, vc = dev.alloc(2048 * d), dev.alloc(2048 * d)
+        st = Stream()
+        for a, o in zip(qkvs, qo):
+            st.rope_kv_store(a, o, kc, vc, state, cos_b, sin_b, m, H, hd, 2048, 0)
+        us = period_us(st, rot)
+        st.profile(2)
+        ev = float(np.mean(st.profile(iters)))
+        nbytes = 16 * m * d                      # Q and K read and written; the V rows' move to the cache is extra
+        moved = 24 * m * d + 2 * 4 * m * (hd // 2)
+        fused.append({"op": "rope_kv_store", "M": m, "cols": d, "bytes": nbytes, "bytes_moved": moved,
+                      "rotation_buffers": rot, "us": round(us, 3), "GBs": round(nbytes / us / 1e3, 1),
+                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "kernel_us": round(ev, 3),
+                      "kernel_frac_of_hbm_peak": round(nbytes / ev / 1e3 / HBM_PEAK_GBS, 4),
+                      "moved_frac_of_hbm_peak": round(moved / ev / 1e3 / HBM_PEAK_GBS, 4)})
+        dev.release(*qkvs, *qo, kc, vc)
+    dev.release_all()
+    if ref is not None:
+        ref.set_threads(1)
+    return {"workload": "isolated Q8 linear-op sweep: 2048x2048, 2048x5632, 5632x2048, 4096x11008 at M = 1 / 64 / 512; "
+                        "fused RMSNorm, SiLU x up and RoPE + cache append on [M x 2048] and [M x 5632]",
+            "timing": "launch period of back-to-back launches (HIP events around the run; an op's helper kernels "
+                      "included); *kernel_us: mean begin-to-end time of the dispatch alone; cold = rotation over "
+                      f"{C2_ROTATION_BYTES >> 20} MiB of distinct buffers, warm = one buffer",
+            "hbm_peak_GBs": HBM_PEAK_GBS, "mfma_peak_TFLOPs": MFMA_PEAK_TFLOPS,
+            "cpu": "C restatement of CpuBackend (not the JVM): matmul parallel over rows of A like DeepJExecutor.forRange, "
+                   f"{threads} threads available" if ref is not None else None,
+            "linear": linear, "fused": fused}
+
+
 def calibration_copy(mib: int = 256, repeats: int = 3) -> None:
     """A plain device copy of known size (reads `mib` MiB, writes `mib` MiB per launch), so that a
     hardware-counter run of this script has a kernel (k_copy) whose FETCH_SIZE / WRITE_SIZE readings
@@ -277,6 +453,9 @@ def main() -> int:
                     help="decode without the HIP graph (same kernels, launched one by one): for runs under a tracer")
     ap.add_argument("--prefill-only", action="store_true",
                     help="stop after the prompt: prints the prefill object alone (short runs under a counter-collecting profiler)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="only the isolated linear-op sweep (four weight shapes x M = 1 / 64 / 512, fused norm and element-wise ops)")
+    ap.add_argument("--no-sweep", action="store_true", help="leave the sweep out of the default line")
     ap.add_argument("--table-iters", type=int, default=12,
                     help="passes behind the per-kernel tables; counter-collecting profilers serialise every dispatch, 1 keeps such runs short")
     args = ap.parse_args()
@@ -286,6 +465,12 @@ def main() -> int:
 
     from deepj_amd import HipNative, JavaRandom, LlamaConfig, LlamaModel
 
+    if args.sweep:
+        HipNative.init(0)
+        sw = c2_sweep(max(2, args.table_iters), cpu=not args.no_cpu_baseline)
+        print(json.dumps({"metric": "Q8 matvec HBM GB/s vs peak; Q8 GEMM TFLOP/s vs peak (isolated linear-op sweep)",
+                          "n_gpus": 1, "sweep": sw}))
+        return 0
     cfg = LlamaConfig(vocabSize=32000, maxSeqLen=2048, dModel=2048, nHeads=32, nLayers=16, dFF=5632)
     if args.prompt + args.warmup + args.steps > cfg.maxSeqLen:
         print("bench.py: prompt + warmup + steps exceeds maxSeq 2048", file=sys.stderr)
@@ -341,6 +526,7 @@ def main() -> int:
     model.reset()
     calibration_copy()
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg, args.prompt)
+    sweep = None if args.no_sweep else c2_sweep(max(2, args.table_iters), cpu=not args.no_cpu_baseline)
 
     # per-token algorithmic bytes at the mean decoded position (weights + fp32 KV read)
     weights = sum(q8_linear_bytes(k, n) for k, n in
@@ -364,6 +550,7 @@ def main() -> int:
                        "first_prefill_ms": round(t_first_prefill * 1e3, 2), "model_build_s": round(t_build, 1),
                        "decode_tok_s_at_context_1536": round(1.0 / t_long, 1)},
         "prefill": prefill_roof,
+        "sweep": sweep,
     }
     print(json.dumps(line))
     model.close()

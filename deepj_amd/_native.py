@@ -43,7 +43,7 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_gemm_tile.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
     lib.deepj_hip_q8_gemm_tile.restype = None
     lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
-    lib.deepj_hip_profile_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p, C.c_int32, _i32p]
+    lib.deepj_hip_profile_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p, C.c_int32, _i32p, _f32p, _i32p]
     lib.deepj_hip_graph_capture.argtypes = [_i32p, C.c_int32, _i32p]
     lib.deepj_hip_graph_launch.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_graph_destroy.argtypes = [C.c_int32]
@@ -181,13 +181,20 @@ class HipNative:
         return float(ms.value)
 
     @staticmethod
-    def profileOps(cmd_stream, iters: int, max_ops: int = 4096) -> np.ndarray:
-        """Mean kernel duration (microseconds, start/stop events on each op's dispatch) of every op of the stream."""
+    def profileOps(cmd_stream, iters: int, max_ops: int = 4096, detail: bool = False):
+        """Mean kernel time (microseconds) of every op of the stream: a start and a stop event on each of the op's
+        dispatches, summed per op.  detail=True also returns the op's longest dispatch (its main kernel) and its
+        number of dispatches."""
         cmd = _ids(cmd_stream)
         out = np.empty(max_ops, dtype=np.float32)
+        top = np.empty(max_ops, dtype=np.float32)
+        cnt = np.empty(max_ops, dtype=np.int32)
         n = C.c_int32()
         _check(library().deepj_hip_profile_ops(cmd.ctypes.data_as(_i32p), cmd.size, iters,
-                                               out.ctypes.data_as(_f32p), max_ops, C.byref(n)))
+                                               out.ctypes.data_as(_f32p), max_ops, C.byref(n),
+                                               top.ctypes.data_as(_f32p), cnt.ctypes.data_as(_i32p)))
+        if detail:
+            return out[: n.value].copy(), top[: n.value].copy(), cnt[: n.value].copy()
         return out[: n.value].copy()
 
     @staticmethod

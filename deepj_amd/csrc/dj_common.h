@@ -36,21 +36,23 @@ inline int64_t q8_bytes(int k, int rows) {
     return q8_scale_offset_bytes(k, rows) + (int64_t)rows * (q8_padded_k(k) / kQ8Group) * 4;
 }
 
-// Per-kernel timing for deepj_hip_profile_ops: while `armed`, the next kernel that goes through launch_kernel()
-// is launched with a start and a stop event attached to that one dispatch (its begin and end time stamps on the
-// device, the quantity a kernel trace reports); every other launch is an ordinary one.
+// Per-kernel timing for deepj_hip_profile_ops: while `armed`, every kernel that goes through launch_kernel() is
+// launched with a start and a stop event of its own attached to that one dispatch (its begin and end time stamps on
+// the device, the quantity a kernel trace reports), up to kMaxTimedLaunches per op; every other launch is an
+// ordinary one.
+constexpr int kMaxTimedLaunches = 6;
 struct LaunchTiming {
-    hipEvent_t start = nullptr, stop = nullptr;
+    hipEvent_t *pairs = nullptr;     // 2 * kMaxTimedLaunches events of the op being run: start, stop, start, stop ...
+    int used = 0;                    // dispatches of the op that carried events so far
     bool armed = false;
 };
 extern LaunchTiming g_launch_timing;
 
 template <typename... Params, typename... Args>
 inline void launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds, hipStream_t s, Args... args) {
-    if (g_launch_timing.armed) {
-        g_launch_timing.armed = false;
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, g_launch_timing.start, g_launch_timing.stop, 0,
-                              static_cast<Params>(args)...);
+    if (g_launch_timing.armed && g_launch_timing.used < kMaxTimedLaunches) {
+        hipEvent_t *pair = g_launch_timing.pairs + 2 * g_launch_timing.used++;
+        hipExtLaunchKernelGGL(kernel, grid, block, lds, s, pair[0], pair[1], 0, static_cast<Params>(args)...);
     } else {
         hipLaunchKernelGGL(kernel, grid, block, lds, s, static_cast<Params>(args)...);
     }

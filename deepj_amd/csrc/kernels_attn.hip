@@ -681,7 +681,7 @@ void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *
     if (total <= 0) return;
     int64_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(k_rope_rows, dim3((int)blocks), dim3(kThreads), 0, s, x, out, state, cos_t, sin_t, rows, H, hd,
+    launch_kernel(k_rope_rows, dim3((int)blocks), dim3(kThreads), 0, s, x, out, state, cos_t, sin_t, rows, H, hd,
                        max_seq, pos_from_row, row_stride > 0 ? row_stride : H * hd, live_extra);
 }
 
@@ -699,9 +699,9 @@ static void launch_decode_kernels(hipStream_t s, DecodeArgs &a) {
     a.scale = (float)(1.0 / sqrt((double)a.hd));
     dim3 grid(a.H, a.nsplit);
     switch (a.hd) {
-        case 32: hipLaunchKernelGGL((k_attn_decode_partial<8, FUSED>), grid, dim3(kThreads), 0, s, a); break;
-        case 64: hipLaunchKernelGGL((k_attn_decode_partial<16, FUSED>), grid, dim3(kThreads), 0, s, a); break;
-        case 128: hipLaunchKernelGGL((k_attn_decode_partial<32, FUSED>), grid, dim3(kThreads), 0, s, a); break;
+        case 32: launch_kernel((k_attn_decode_partial<8, FUSED>), grid, dim3(kThreads), 0, s, a); break;
+        case 64: launch_kernel((k_attn_decode_partial<16, FUSED>), grid, dim3(kThreads), 0, s, a); break;
+        case 128: launch_kernel((k_attn_decode_partial<32, FUSED>), grid, dim3(kThreads), 0, s, a); break;
         default: fail("attention: head dim must be 32, 64 or 128");
     }
 }
@@ -785,9 +785,9 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
     }
     dim3 grid(p.h, p.s);
     switch (p.hd) {
-        case 32: hipLaunchKernelGGL(k_attention<8>, grid, dim3(kThreads), 0, s, a); break;
-        case 64: hipLaunchKernelGGL(k_attention<16>, grid, dim3(kThreads), 0, s, a); break;
-        case 128: hipLaunchKernelGGL(k_attention<32>, grid, dim3(kThreads), 0, s, a); break;
+        case 32: launch_kernel(k_attention<8>, grid, dim3(kThreads), 0, s, a); break;
+        case 64: launch_kernel(k_attention<16>, grid, dim3(kThreads), 0, s, a); break;
+        case 128: launch_kernel(k_attention<32>, grid, dim3(kThreads), 0, s, a); break;
         default: fail("attention: head dim must be 32, 64 or 128");
     }
 }

@@ -289,7 +289,7 @@ __global__ void k_decode_advance(int32_t *state, const int32_t *token, int32_t *
 }  // namespace
 
 #define DJ_LAUNCH(kernel, grid, block, stream, ...) \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, __VA_ARGS__)
+    launch_kernel(kernel, dim3(grid), dim3(block), 0, stream, __VA_ARGS__)
 
 void launch_binary(hipStream_t s, int op, const float *a, const float *b, float *out, int64_t n) {
     if (n <= 0) return;
@@ -358,7 +358,7 @@ void launch_broadcast(hipStream_t s, int op, const float *a, const float *v, flo
 void launch_transpose(hipStream_t s, const float *a, float *out, int rows, int cols) {
     if (rows <= 0 || cols <= 0) return;
     dim3 grid((cols + 31) / 32, (rows + 31) / 32);
-    hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, s, a, out, rows, cols);
+    launch_kernel(k_transpose, grid, dim3(256), 0, s, a, out, rows, cols);
 }
 
 void launch_adamw(hipStream_t s, float *w, const float *g, float *mt, float *vt, int64_t n, float lr, float beta1,

@@ -689,7 +689,7 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
     uint16_t *w16 = reinterpret_cast<uint16_t *>(prepared);
     float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
     const int64_t items = (int64_t)n_rows * (kp / 8);
-    hipLaunchKernelGGL(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
+    launch_kernel(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
 }
 
 // The kernels' LDS (three stages) is above the 64 KB a kernel gets without asking; called once per device at start-up
@@ -713,7 +713,7 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     // gamma alone: RMSNorm of the rows first; gamma and beta: LayerNorm
     auto split = !gamma ? k_split_f16<0> : beta ? k_split_f16<2> : k_split_f16<1>;
     // (the helpers are ordinary launches: per-kernel timing of this op, launch_kernel's business, is the GEMM's)
-    hipLaunchKernelGGL(split, dim3(m), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
+    launch_kernel(split, dim3(m), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
     if (!prepared) {
         launch_q8_prepare(s, wq, scales, w, k, n_rows);
         prepared = w;
@@ -733,7 +733,7 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
         else launch_kernel(k_gemm_q8_f16_m64<4>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
         if (plan.splits > 1) {
             const int64_t mn4 = (int64_t)m * n_rows / 4;
-            hipLaunchKernelGGL(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
+            launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
                                mn4, n_rows / 4, bias, residual, gelu);
         }
     } else

@@ -508,11 +508,11 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
     GemmEpilogue ep{nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0};
     if (use_big_tile(m, n)) {
         dim3 grid2((n + BN2 - 1) / BN2, (m + BM2 - 1) / BM2);
-        hipLaunchKernelGGL(k_gemm128, grid2, dim3(256), 0, s, a, b, out, m, n, k, ep);
+        launch_kernel(k_gemm128, grid2, dim3(256), 0, s, a, b, out, m, n, k, ep);
         return;
     }
     dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM);
-    hipLaunchKernelGGL(k_gemm, grid, dim3(256), 0, s, a, b, out, m, n, k, ep);
+    launch_kernel(k_gemm, grid, dim3(256), 0, s, a, b, out, m, n, k, ep);
 }
 
 // Q8 GEMM used by launch_q8_linear for M > 1.  n_rows is the number of Q8 rows

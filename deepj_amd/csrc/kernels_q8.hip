@@ -571,7 +571,7 @@ void launch_q8_quantize(hipStream_t s, const float *w, int8_t *q, float *scales,
     if (k <= 0 || n <= 0) return;
     int kp = q8_padded_k(k);
     dim3 grid((n + 63) / 64, kp / kQ8Group);
-    hipLaunchKernelGGL(k_q8_quantize, grid, dim3(kThreads), 0, s, w, q, scales, k, n, kp, row_off, row_step);
+    launch_kernel(k_q8_quantize, grid, dim3(kThreads), 0, s, w, q, scales, k, n, kp, row_off, row_step);
 }
 
 void launch_q8_dequantize(hipStream_t s, const int8_t *q, const float *scales, float *w, int k, int n, int row_off,
@@ -580,7 +580,7 @@ void launch_q8_dequantize(hipStream_t s, const int8_t *q, const float *scales, f
     if (total <= 0) return;
     int64_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(k_q8_dequantize, dim3((int)blocks), dim3(kThreads), 0, s, q, scales, w, k, n,
+    launch_kernel(k_q8_dequantize, dim3((int)blocks), dim3(kThreads), 0, s, q, scales, w, k, n,
                        q8_padded_k(k), row_off, row_step);
 }
 

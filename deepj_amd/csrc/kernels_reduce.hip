@@ -205,12 +205,13 @@ __global__ void __launch_bounds__(kThreads) k_cross_entropy(const float *__restr
 
 // out = gamma * (x / sqrt(mean(x*x) + 1e-6)) in one pass over the row
 // (RMSNorm1D.java:46-57 folds six primitive ops and five temporaries into this).
+// NV: 128-bit words a thread keeps of one row (rows of up to 1024 * NV floats stay in registers between the sum of
+// squares and the scaling: one pass over memory); NV = 0: any width, two passes with scalar accesses.
+template <int NV>
 __global__ void __launch_bounds__(kThreads) k_rmsnorm(const float *__restrict__ x, const float *__restrict__ gamma,
                                                       float *__restrict__ out, int rows, int cols) {
     __shared__ float lds[kWaves];
-    constexpr int NV = 4;                                        // 128-bit words a thread keeps of one row
-    if ((cols & 3) == 0 && cols <= kThreads * 4 * NV) {
-        // the row stays in registers between the sum of squares and the scaling: one pass over memory
+    if constexpr (NV > 0) {
         const int n4 = cols >> 2;
         for (int r = blockIdx.x; r < rows; r += gridDim.x) {
             const float4 *row4 = reinterpret_cast<const float4 *>(x + (int64_t)r * cols);
@@ -234,16 +235,16 @@ __global__ void __launch_bounds__(kThreads) k_rmsnorm(const float *__restrict__ 
                                           (v[j].w / rms) * g[j].w);
             }
         }
-        return;
-    }
-    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
-        const float *row = x + (int64_t)r * cols;
-        float *orow = out + (int64_t)r * cols;
-        float s = 0.0f;
-        for (int c = threadIdx.x; c < cols; c += kThreads) { float v = row[c]; s += v * v; }
-        s = block_sum(s, lds);
-        float rms = sqrtf(s * (1.0f / (float)cols) + kRmsEps);
-        for (int c = threadIdx.x; c < cols; c += kThreads) orow[c] = (row[c] / rms) * gamma[c];
+    } else {
+        for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+            const float *row = x + (int64_t)r * cols;
+            float *orow = out + (int64_t)r * cols;
+            float s = 0.0f;
+            for (int c = threadIdx.x; c < cols; c += kThreads) { float v = row[c]; s += v * v; }
+            s = block_sum(s, lds);
+            float rms = sqrtf(s * (1.0f / (float)cols) + kRmsEps);
+            for (int c = threadIdx.x; c < cols; c += kThreads) orow[c] = (row[c] / rms) * gamma[c];
+        }
     }
 }
 
@@ -401,38 +402,38 @@ void launch_row_reduce(hipStream_t s, int op, const float *a, float *out, int ro
     if (rows <= 0) return;
     dim3 grid(row_grid(rows)), block(kThreads);
     switch (op) {
-        case DJ_OP_SUM_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_SUM_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
-        case DJ_OP_MEAN_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_MEAN_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
-        case DJ_OP_VARIANCE_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_VARIANCE_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
-        case DJ_OP_MAX_ALONG_ROWS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_MAX_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
-        case DJ_OP_SUM_ABS: hipLaunchKernelGGL(k_row_reduce<DJ_OP_SUM_ABS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_SUM_ALONG_ROWS: launch_kernel(k_row_reduce<DJ_OP_SUM_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_MEAN_ALONG_ROWS: launch_kernel(k_row_reduce<DJ_OP_MEAN_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_VARIANCE_ALONG_ROWS: launch_kernel(k_row_reduce<DJ_OP_VARIANCE_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_MAX_ALONG_ROWS: launch_kernel(k_row_reduce<DJ_OP_MAX_ALONG_ROWS>, grid, block, 0, s, a, out, rows, cols); break;
+        case DJ_OP_SUM_ABS: launch_kernel(k_row_reduce<DJ_OP_SUM_ABS>, grid, block, 0, s, a, out, rows, cols); break;
         default: fail("launch_row_reduce: bad op");
     }
 }
 
 void launch_sum_rows(hipStream_t s, const float *a, float *out, int rows, int cols) {
     if (cols <= 0) return;
-    hipLaunchKernelGGL(k_sum_rows, dim3((cols + 63) / 64), dim3(kThreads), 0, s, a, out, rows, cols);
+    launch_kernel(k_sum_rows, dim3((cols + 63) / 64), dim3(kThreads), 0, s, a, out, rows, cols);
 }
 
 void launch_sum_scalar(hipStream_t s, const float *a, float *out, int64_t n) {
-    hipLaunchKernelGGL(k_sum_scalar, dim3(1), dim3(1024), 0, s, a, out, n);
+    launch_kernel(k_sum_scalar, dim3(1), dim3(1024), 0, s, a, out, n);
 }
 
 void launch_softmax_rows(hipStream_t s, const float *a, float *out, int rows, int cols) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(k_softmax_rows, dim3(row_grid(rows)), dim3(kThreads), 0, s, a, out, rows, cols);
+    launch_kernel(k_softmax_rows, dim3(row_grid(rows)), dim3(kThreads), 0, s, a, out, rows, cols);
 }
 
 void launch_softmax_backward(hipStream_t s, const float *g, const float *sm, float *out, int rows, int cols) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(k_softmax_backward, dim3(row_grid(rows)), dim3(kThreads), 0, s, g, sm, out, rows, cols);
+    launch_kernel(k_softmax_backward, dim3(row_grid(rows)), dim3(kThreads), 0, s, g, sm, out, rows, cols);
 }
 
 void launch_layernorm_backward(hipStream_t s, const float *dxhat, const float *xhat, const float *stdv, float *out,
                                int rows, int cols) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(k_layernorm_backward, dim3(row_grid(rows)), dim3(kThreads), 0, s, dxhat, xhat, stdv, out, rows,
+    launch_kernel(k_layernorm_backward, dim3(row_grid(rows)), dim3(kThreads), 0, s, dxhat, xhat, stdv, out, rows,
                        cols);
 }
 
@@ -440,22 +441,28 @@ void launch_cross_entropy(hipStream_t s, bool gradient, const float *logits, con
                           int rows, int cols) {
     if (rows <= 0) return;
     if (gradient)
-        hipLaunchKernelGGL(k_cross_entropy<true>, dim3(row_grid(rows)), dim3(kThreads), 0, s, logits, targets, out,
+        launch_kernel(k_cross_entropy<true>, dim3(row_grid(rows)), dim3(kThreads), 0, s, logits, targets, out,
                            rows, cols);
     else
-        hipLaunchKernelGGL(k_cross_entropy<false>, dim3(row_grid(rows)), dim3(kThreads), 0, s, logits, targets, out,
+        launch_kernel(k_cross_entropy<false>, dim3(row_grid(rows)), dim3(kThreads), 0, s, logits, targets, out,
                            rows, cols);
 }
 
 void launch_rmsnorm(hipStream_t s, const float *x, const float *gamma, float *out, int rows, int cols) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(k_rmsnorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, out, rows, cols);
+    const dim3 grid(row_grid(rows)), block(kThreads);
+    const int need = (cols & 3) == 0 ? (cols + 4 * kThreads - 1) / (4 * kThreads) : 0;     // 128-bit words per thread
+    if (need >= 1 && need <= 2) launch_kernel(k_rmsnorm<2>, grid, block, 0, s, x, gamma, out, rows, cols);
+    else if (need >= 3 && need <= 4) launch_kernel(k_rmsnorm<4>, grid, block, 0, s, x, gamma, out, rows, cols);
+    else if (need >= 5 && need <= 6) launch_kernel(k_rmsnorm<6>, grid, block, 0, s, x, gamma, out, rows, cols);
+    else if (need >= 7 && need <= 11) launch_kernel(k_rmsnorm<11>, grid, block, 0, s, x, gamma, out, rows, cols);
+    else launch_kernel(k_rmsnorm<0>, grid, block, 0, s, x, gamma, out, rows, cols);
 }
 
 void launch_layernorm(hipStream_t s, const float *x, const float *gamma, const float *beta, float *out, int rows,
                       int cols) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(k_layernorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, beta, out, rows, cols);
+    launch_kernel(k_layernorm, dim3(row_grid(rows)), dim3(kThreads), 0, s, x, gamma, beta, out, rows, cols);
 }
 
 void launch_add_positions(hipStream_t s, float *x, const float *table, const int32_t *state, int rows, int d,
@@ -464,7 +471,7 @@ void launch_add_positions(hipStream_t s, float *x, const float *table, const int
     if (total <= 0) return;
     int64_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(k_add_positions, dim3((int)blocks), dim3(kThreads), 0, s, x, table, state, rows, d, max_seq);
+    launch_kernel(k_add_positions, dim3((int)blocks), dim3(kThreads), 0, s, x, table, state, rows, d, max_seq);
 }
 
 void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int32_t *tokens, int capacity,
@@ -475,7 +482,7 @@ void launch_decode_next(hipStream_t s, const float *logits, int32_t *state, int3
 
 void launch_argmax_rows(hipStream_t s, const float *a, int32_t *out, int rows, int cols) {
     if (rows <= 0) return;
-    hipLaunchKernelGGL(k_argmax_rows, dim3(row_grid(rows)), dim3(kThreads), 0, s, a, out, rows, cols);
+    launch_kernel(k_argmax_rows, dim3(row_grid(rows)), dim3(kThreads), 0, s, a, out, rows, cols);
 }
 
 }  // namespace dj

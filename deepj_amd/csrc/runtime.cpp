@@ -738,10 +738,6 @@ void walk(const int32_t *cmd, int32_t len, bool dry, int64_t *ws_need) {
         int op = cmd[c.pos];
         int stride = stride_of(op);
         if (stride < 0) fail("Unknown op code in graph: " + std::to_string(op));
-        if (stride == 0) {                      // the op carries its own length
-            if (c.pos + 1 >= len || cmd[c.pos + 1] < 2) fail(std::string(op_name(op)) + ": bad length word");
-            stride = cmd[c.pos + 1];
-        }
         if (c.pos + stride > len)
             fail(std::string(op_name(op)) + ": command stream truncated at word " + std::to_string(c.pos));
         exec_one(c);
@@ -1042,11 +1038,13 @@ int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms
     });
 }
 
-// Per-op kernel durations: every op of the stream is launched with a start and a stop event on its (first) kernel
-// dispatch, the stream runs `iters` times in order, and us_per_op[i] receives the mean begin-to-end time of op i's
-// kernel on the device in microseconds (-1 for an op none of whose launches can carry events).
+// Per-op kernel durations: every kernel dispatch of every op of the stream carries a start and a stop event, the
+// stream runs `iters` times in order, and us_per_op[i] receives the mean over the passes of the summed begin-to-end
+// times of op i's dispatches in microseconds (-1 for an op that launched nothing).  Optional outputs of the same
+// length: us_longest[i], the longest single dispatch of the op (its main kernel), and dispatches[i], how many
+// dispatches the op made (at most kMaxTimedLaunches of them are timed).
 int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float *us_per_op, int32_t capacity,
-                          int32_t *n_ops) {
+                          int32_t *n_ops, float *us_longest, int32_t *dispatches) {
     return guarded([&] {
         ensure_init();
         if (iters <= 0 || !us_per_op || capacity < 0) fail("profile_ops: bad arguments");
@@ -1054,17 +1052,14 @@ int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float 
         walk(cmd, len, true, &ws);
         ensure_workspace(ws);
         std::vector<int32_t> starts;                 // word offset of every op
-        for (int32_t pos = 0; pos < len;) {
-            starts.push_back(pos);
-            int stride = stride_of(cmd[pos]);
-            pos += stride == 0 ? cmd[pos + 1] : stride;
-        }
+        for (int32_t pos = 0; pos < len; pos += stride_of(cmd[pos])) starts.push_back(pos);
         const int n = (int)starts.size();
         if (n_ops) *n_ops = n;
         if (n > capacity) fail("profile_ops: the stream holds " + std::to_string(n) + " ops, the output only " + std::to_string(capacity));
-        std::vector<hipEvent_t> ev((size_t)2 * n, nullptr);
-        std::vector<double> sum((size_t)n, 0.0);
-        std::vector<int> count((size_t)n, 0);
+        constexpr int per_op = 2 * kMaxTimedLaunches;
+        std::vector<hipEvent_t> ev((size_t)per_op * n, nullptr);
+        std::vector<double> sum((size_t)n, 0.0), longest((size_t)n, 0.0);
+        std::vector<int> count((size_t)n, 0), launches((size_t)n, 0);
         auto cleanup = [&] {
             g_launch_timing = LaunchTiming{};
             for (hipEvent_t e : ev) if (e) (void)hipEventDestroy(e);
@@ -1072,22 +1067,27 @@ int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float 
         try {
             for (auto &e : ev) DJ_HIP(hipEventCreate(&e));
             for (int it = 0; it < iters; it++) {
-                std::vector<char> timed((size_t)n, 0);
                 for (int i = 0; i < n; i++) {
                     Cursor c{cmd, len, starts[(size_t)i], false, 0};
-                    g_launch_timing.start = ev[(size_t)2 * i];
-                    g_launch_timing.stop = ev[(size_t)2 * i + 1];
+                    g_launch_timing.pairs = ev.data() + (size_t)per_op * i;
+                    g_launch_timing.used = 0;
                     g_launch_timing.armed = true;
                     exec_one(c);
-                    timed[(size_t)i] = !g_launch_timing.armed;
+                    launches[(size_t)i] = g_launch_timing.used;
                     g_launch_timing.armed = false;
                 }
                 DJ_HIP(hipStreamSynchronize(g.stream));
                 for (int i = 0; i < n; i++) {
-                    if (!timed[(size_t)i]) continue;
-                    float ms = 0.0f;
-                    DJ_HIP(hipEventElapsedTime(&ms, ev[(size_t)2 * i], ev[(size_t)2 * i + 1]));
-                    sum[(size_t)i] += (double)ms * 1e3;
+                    if (!launches[(size_t)i]) continue;
+                    double total = 0.0, top = 0.0;
+                    for (int j = 0; j < launches[(size_t)i]; j++) {
+                        float ms = 0.0f;
+                        DJ_HIP(hipEventElapsedTime(&ms, ev[(size_t)per_op * i + 2 * j], ev[(size_t)per_op * i + 2 * j + 1]));
+                        total += (double)ms * 1e3;
+                        top = std::max(top, (double)ms * 1e3);
+                    }
+                    sum[(size_t)i] += total;
+                    longest[(size_t)i] += top;
                     count[(size_t)i]++;
                 }
             }
@@ -1096,7 +1096,12 @@ int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float 
             throw;
         }
         cleanup();
-        for (int i = 0; i < n; i++) us_per_op[i] = count[(size_t)i] ? (float)(sum[(size_t)i] / count[(size_t)i]) : -1.0f;
+        for (int i = 0; i < n; i++) {
+            const bool ok = count[(size_t)i] > 0;
+            us_per_op[i] = ok ? (float)(sum[(size_t)i] / count[(size_t)i]) : -1.0f;
+            if (us_longest) us_longest[i] = ok ? (float)(longest[(size_t)i] / count[(size_t)i]) : -1.0f;
+            if (dispatches) dispatches[i] = launches[(size_t)i];
+        }
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) fail(std::string("kernel launch failed: ") + hipGetErrorString(e));
     });

@@ -87,13 +87,14 @@ void *deepj_hip_stream(void);
  * recorded on the library's stream; *ms_total receives the elapsed time. */
 int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total);
 
-/* Runs a validated stream `iters` times in order with a start and a stop event attached to each op's (first)
- * kernel dispatch: us_per_op[i] receives the mean begin-to-end time of op i's kernel on the device, in
- * microseconds - the duration a kernel trace reports for it (-1 for ops whose launches carry no events: every
- * decode-path op does - Q8_LINEAR with M = 1, ATTN_DECODE_RECORDS, DECODE_NEXT, STREAM_READ, NOP).  *n_ops = ops in
- * the stream; fails when capacity is smaller. */
+/* Runs a validated stream `iters` times in order with a start and a stop event attached to every kernel dispatch
+ * of every op: us_per_op[i] receives the mean over the passes of the summed begin-to-end times of op i's
+ * dispatches on the device, in microseconds - the durations a kernel trace reports, helpers of the op included
+ * (-1 for an op that launched nothing).  us_longest (optional, same length): the op's longest single dispatch, its
+ * main kernel; dispatches (optional): how many the op made.  *n_ops = ops in the stream; fails when capacity is
+ * smaller. */
 int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float *us_per_op, int32_t capacity,
-                          int32_t *n_ops);
+                          int32_t *n_ops, float *us_longest, int32_t *dispatches);
 
 /* Captures a command stream into a HIP graph (no allocation may be pending:
  * every buffer it names must exist) and replays it.  Used for the per-token
