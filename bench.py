@@ -534,6 +534,7 @@ def main() -> int:
     mean_pos = args.prompt + args.warmup + args.steps / 2
     kv = cfg.nLayers * 2 * mean_pos * cfg.dModel * 4
     tok_s = args.steps / elapsed
+    mem, prepared_bytes = HipNative.poolStats(), model.preparedBytes()
     line = {
         "metric": "decode tok/s, Q8 Llama d=2048 L=16, 1 GPU; Q8 matvec HBM GB/s vs peak",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -548,6 +549,11 @@ def main() -> int:
                        "frac_of_hbm_peak": round((weights + kv) * tok_s / 1e9 / HBM_PEAK_GBS, 4),
                        "prefill_tok_s": round(args.prompt / t_prefill, 1),
                        "first_prefill_ms": round(t_first_prefill * 1e3, 2), "model_build_s": round(t_build, 1),
+                       # device memory: everything the library holds for this model, the Q8 weights (1.125 B/weight), and
+                       # the fp16 copies of the projections the prompt GEMM reads (2 B/weight; LlamaModel.setPreparedBudget
+                       # bounds them, 0 = none at about 40 us per layer and prompt)
+                       "device_bytes_live": int(mem["live_bytes"]), "q8_weight_bytes": int(weights),
+                       "prepared_weight_bytes": prepared_bytes,
                        "decode_tok_s_at_context_1536": round(1.0 / t_long, 1)},
         "prefill": prefill_roof,
         "sweep": sweep,

@@ -83,6 +83,8 @@ struct Runner {
     int32_t latent = -1, kv_all = -1;                      // latent cache [L][maxSeq][kvRank]; re-expanded [maxSeq][K | V] of one layer
     std::vector<int32_t> prepared;                         // the weights in the many-row GEMM's layout (first long prompt)
     bool prepared_done = false;
+    int64_t prepared_budget = -1;                          // bytes such copies may take in all; -1: no limit
+    int64_t prepared_bytes = 0;
     Acts dec, pre;
     int32_t graph = 0, graph_unrolled = 0;                 // one token per replay / kGraphUnroll tokens per replay
     bool finalized = false;
@@ -460,18 +462,23 @@ Stream decode_stream(Runner &r, bool sample_on_device) {
 
 // A long prompt runs its projections on the GEMM that loads fp16 weights straight into LDS.  The first such prompt
 // writes the weights once in that layout (about 2 bytes per weight more, kept until the runner goes) instead of every
-// call converting them into the workspace.  (finalize()'s warm-up pass runs long prompts when maxSeqLen allows them, so
-// with the warm-up on the copies exist from the start.)
+// call converting them into the workspace - layer by layer while the byte budget lasts; the layers past it convert on
+// every call (same results, 40 us or so per layer and prompt slower).  (finalize()'s warm-up pass runs long prompts
+// when maxSeqLen allows them, so with the warm-up on the copies exist from the start.)
 void ensure_prepared(Runner &r, int n) {
     if (r.prepared_done || n < 256) return;
     r.prepared_done = true;
     const Config &c = r.cfg;
     const int d = c.d;
     Stream s;
+    bool room = true;
     auto prepare = [&](int32_t w, int k, int rows) {
-        if (w < 0 || !deepj_hip_q8_gemm_path(c.max_seq, k, rows)) return;
-        int32_t p = r.alloc(deepj_hip_q8_prepared_floats(k, rows));
+        if (!room || w < 0 || !deepj_hip_q8_gemm_path(c.max_seq, k, rows)) return;
+        const int64_t floats = deepj_hip_q8_prepared_floats(k, rows);
+        if (r.prepared_budget >= 0 && r.prepared_bytes + 4 * floats > r.prepared_budget) { room = false; return; }
+        int32_t p = r.alloc(floats);
         r.prepared.push_back(p);
+        r.prepared_bytes += 4 * floats;
         emit(s, DJ_OP_Q8_PREPARE, w, p, k, rows);
     };
     for (const Layer &L : r.layers) {
@@ -481,6 +488,13 @@ void ensure_prepared(Runner &r, int n) {
         prepare(L.wd, c.dff, d);
     }
     if (!s.empty()) r.run(s);
+}
+
+void release_prepared(Runner &r) {
+    for (int32_t &id : r.prepared) r.release(id);
+    r.prepared.clear();
+    r.prepared_bytes = 0;
+    r.prepared_done = false;
 }
 
 void check_ids(const Config &c, const int32_t *ids, int n) {
@@ -798,6 +812,21 @@ int deepj_runner_init_seeded_gpt(void *h, int64_t seed, float init_scale, int32_
         init_seeded(*r, seed, threads, init_scale);
     });
 }
+
+// Bytes the runner may spend on fp16 copies of its weights for the many-row (prompt) GEMM: -1 no limit (every layer:
+// + 2 bytes per weight), 0 none (every call converts into the workspace), otherwise layers in order while the budget
+// lasts.  Copies held under an earlier budget are released; the next long prompt prepares anew.  Results do not
+// depend on it.
+int deepj_runner_set_prepared_budget(void *h, int64_t bytes) {
+    auto *r = static_cast<Runner *>(h);
+    return guarded(r, [&] {
+        if (bytes < -1) throw Error("prepared-weight budget must be -1 (no limit) or a byte count");
+        release_prepared(*r);
+        r->prepared_budget = bytes;
+    });
+}
+
+int64_t deepj_runner_prepared_bytes(void *h) { return h ? static_cast<Runner *>(h)->prepared_bytes : 0; }
 
 int deepj_runner_finalize(void *h) {
     auto *r = static_cast<Runner *>(h);

@@ -35,6 +35,9 @@ def _lib():
         lib.deepj_runner_init_seeded.argtypes = [C.c_void_p, C.c_int64, C.c_int32]
         lib.deepj_runner_init_seeded_gpt.argtypes = [C.c_void_p, C.c_int64, C.c_float, C.c_int32]
         lib.deepj_runner_finalize.argtypes = [C.c_void_p]
+        lib.deepj_runner_set_prepared_budget.argtypes = [C.c_void_p, C.c_int64]
+        lib.deepj_runner_prepared_bytes.argtypes = [C.c_void_p]
+        lib.deepj_runner_prepared_bytes.restype = C.c_int64
         lib.deepj_runner_reset.argtypes = [C.c_void_p]
         lib.deepj_runner_prefill.argtypes = [C.c_void_p, _i32p, C.c_int32, C.c_void_p, C.c_int32]
         lib.deepj_runner_decode.argtypes = [C.c_void_p, C.c_int32, C.c_int32]
@@ -203,6 +206,15 @@ class _DecoderOnlyModel:
 
     def finalize(self) -> None:
         self._check(_lib().deepj_runner_finalize(self._h))
+
+    def setPreparedBudget(self, nbytes: int | None) -> None:
+        """Bytes the model may spend on fp16 copies of its weights for the prompt GEMM (2 bytes per weight when every
+        layer has one): None = no limit, 0 = none (every call converts), otherwise layers in order while it lasts.
+        Same results whatever the budget."""
+        self._check(_lib().deepj_runner_set_prepared_budget(self._h, -1 if nbytes is None else int(nbytes)))
+
+    def preparedBytes(self) -> int:
+        return int(_lib().deepj_runner_prepared_bytes(self._h))
 
     # inference ----------------------------------------------------------------
     def reset(self) -> None:

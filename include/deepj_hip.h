@@ -251,6 +251,12 @@ int deepj_runner_set_weight(void *runner, const char *name, const float *data, i
 int deepj_runner_init_seeded(void *runner, int64_t seed, int32_t threads);  /* new LlamaModel(cfg, seed) */
 /* new GPTModel(cfg, seed) with GPTConfig.initScale = init_scale (J/models/gpt/GPTModel.java:27-46,76-81) */
 int deepj_runner_init_seeded_gpt(void *runner, int64_t seed, float init_scale, int32_t threads);
+/* Bytes a runner may spend on fp16 copies of its weights for the many-row (prompt) GEMM, which reads them in that
+ * form: -1 (default) no limit - a copy of every layer, written at the first prompt of 256 rows or more (+ 2 bytes
+ * per weight); 0 none - every call converts into the workspace; otherwise layers in order while the budget lasts.
+ * Results are bit-identical whatever the budget.  deepj_runner_prepared_bytes: what the copies take now. */
+int deepj_runner_set_prepared_budget(void *runner, int64_t bytes);
+int64_t deepj_runner_prepared_bytes(void *runner);
 int deepj_runner_finalize(void *runner);
 int deepj_runner_reset(void *runner);
 int deepj_runner_prefill(void *runner, const int32_t *ids, int32_t n, float *all_logits, int32_t choose_next);

@@ -236,6 +236,37 @@ def test_prepared_weights_give_the_same_bits_and_follow_the_weights(dev):
     dev.release(src, wq, xb, ob)
 
 
+def test_runner_prepared_weight_budgets_give_identical_logits_and_tokens():
+    """Whatever a runner may spend on fp16 copies of its weights for the prompt GEMM - every layer, the first two,
+    none - the arithmetic is the same: identical logits, bit for bit, and identical tokens; the bytes held follow
+    the budget."""
+    from deepj_amd import LlamaConfig, LlamaModel, TextGenerator
+    cfg = LlamaConfig(vocabSize=512, maxSeqLen=384, dModel=1024, nHeads=16, nLayers=4, dFF=3328)
+    assert HipNative.q8GemmPath(320, 1024, 2 * 3328) != 0        # the gate/up projection takes the fp16 GEMM at this size
+    prompt = JavaRandom(5).ints(320, 512)
+    model = LlamaModel(cfg, 42)
+    try:
+        full = model.preparedBytes()
+        assert full > 0                                          # the warm-up pass prepared every layer
+        results, held = {}, {}
+        for name, budget in (("all", None), ("two layers", full // 2), ("none", 0), ("all again", None)):
+            model.setPreparedBudget(budget)
+            assert model.preparedBytes() == 0                    # released; the next long prompt prepares anew
+            logits = model.forward(prompt)
+            toks = TextGenerator.generate(model, prompt, 8, top_k=1)
+            held[name] = model.preparedBytes()
+            results[name] = (logits, toks)
+        for name in ("two layers", "none", "all again"):
+            assert np.array_equal(results[name][0].view(np.int32), results["all"][0].view(np.int32)), name
+            assert np.array_equal(results[name][1], results["all"][1]), name
+        assert held["none"] == 0 and held["all"] == held["all again"] == full
+        assert 0 < held["two layers"] <= full // 2
+        with pytest.raises(ValueError, match="budget must be"):
+            model.setPreparedBudget(-5)
+    finally:
+        model.close()
+
+
 def test_graph_replays_of_the_gemm_match_eager_runs(dev):
     """The three-kernel Q8_LINEAR (split, GEMM on shared K, sum of partial products) and the single-GEMM one captured into
     a HIP graph: every replay, with eager work and synchronisation in between, gives the eager run's bits."""
