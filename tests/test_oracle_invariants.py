@@ -255,6 +255,32 @@ def test_llama_init_order_and_forward_matches_layers():
         m.forward([0, 256])                              # Embedding.java:30-32
 
 
+def test_deepseek_init_order_and_forward_matches_layers():
+    """DeepSeekModel.forward as the composition of the separately pinned layer functions
+    (DeepSeekTransformerBlock.java:54-57: x2 = x + mla(norm1(x)); x2 + mlp(norm2(x2));
+    DecoderOnlyModel.java:58-64), and the parameter order of one shared Random across the blocks
+    (DeepSeekTransformerBuilder.java:56-68, MultiHeadLatentAttention.java:81-86)."""
+    cfg = dict(TINY, q_rank=16, kv_rank=8)
+    m = ref.Model(seed=42, **cfg)
+    r = ref.JavaRandom(42)
+    for name, shape in [("L0.wdq", (32, 16)), ("L0.wuq", (16, 32)), ("L0.wdkv", (32, 8)), ("L0.wuk", (8, 32)),
+                        ("L0.wuv", (8, 32)), ("L0.wo", (32, 32)), ("L0.wg", (32, 88)), ("L0.wu", (32, 88)),
+                        ("L0.wd", (88, 32)), ("L1.wdq", (32, 16))]:
+        assert np.array_equal(m.weight(name), r.tensor(*shape)), name
+    assert np.array_equal(m.weight("wlm"), ref.JavaRandom(43).tensor(32, 256))
+    ids = ref.JavaRandom(7).ints(6, 256)
+    x = ref.slice_rows(m.weight("emb"), ids)
+    cos, sin = ref.rope_tables(8, 16)
+    for l in range(2):
+        w = lambda n: m.weight(f"L{l}.{n}")
+        att = ref.mla_forward(ref.rmsnorm(x, w("g1")), w("wdq"), w("wuq"), w("wdkv"), w("wuk"), w("wuv"), w("wo"), 4, cos, sin)
+        x2 = ref.add(x, att)
+        x = ref.add(x2, ref.swiglu(ref.rmsnorm(x2, w("g2")), w("wg"), w("bg"), w("wu"), w("bu"), w("wd"), w("bd")))
+        assert np.array_equal(m.hidden(ids, l + 1), x), f"state after block {l}"
+    exp = ref.linear(ref.rmsnorm(x, m.weight("gf")), m.weight("wlm"), m.weight("blm"))
+    assert np.array_equal(m.forward(ids), exp)
+
+
 def test_cached_forward_is_bit_identical_to_full_context():
     for cfg in (dict(TINY), dict(TINY, q_rank=16, kv_rank=8)):
         m = ref.Model(seed=42, **cfg)
