@@ -468,6 +468,7 @@ def main() -> int:
     if args.sweep:
         HipNative.init(0)
         sw = c2_sweep(max(2, args.table_iters), cpu=not args.no_cpu_baseline)
+        calibration_copy()
         print(json.dumps({"metric": "Q8 matvec HBM GB/s vs peak; Q8 GEMM TFLOP/s vs peak (isolated linear-op sweep)",
                           "n_gpus": 1, "sweep": sw}))
         return 0

@@ -13,7 +13,11 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdeepj_hip.so")
+# DEEPJ_HIP_LIBRARY: another build of the library (python -m deepj_amd.build --no-kernarg-preload writes one for runs
+# under a counter-collecting profiler); a relative path is taken from the package's parent directory
+LIB_PATH = os.environ.get("DEEPJ_HIP_LIBRARY") or os.path.join(_HERE, "libdeepj_hip.so")
+if not os.path.isabs(LIB_PATH):
+    LIB_PATH = os.path.join(os.path.dirname(_HERE), LIB_PATH)
 
 _i32p = C.POINTER(C.c_int32)
 _f32p = C.POINTER(C.c_float)

@@ -22,8 +22,14 @@ ARCH = "gfx950"
 # wavefront in registers at launch instead of through a load from the argument buffer that every other load of the
 # kernel would have to wait for.  The latency-bound decode kernels take their operands as separate arguments,
 # the first-needed ones in front, for this reason.
-COMMON = ["-x", "hip", f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-kernarg-preload-count=16"]
+BASE = ["-x", "hip", f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
+COMMON = BASE + PRELOAD
+# A second build of the same sources without kernarg preload, for runs under a hardware-counter profiler (the
+# counter-collecting rocprofv3 crashed on the host at the first dispatch of a kernel with preloaded arguments; the
+# bytes a kernel moves do not depend on how its arguments arrive).  DEEPJ_HIP_LIBRARY selects it at run time.
+LIB_NO_PRELOAD = os.path.join(HERE, "libdeepj_hip_nopreload.so")
 
 # Kernels whose results are compared element by element with the CPU backend keep
 # a*b+c unfused (the CPU never fuses); the contraction kernels use fma on purpose.
@@ -83,9 +89,9 @@ def verify_packed_fp32_off() -> None:
 
 
 def _compile(item):
-    src, extra = item
-    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *COMMON, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    src, extra, common, obj_dir = item
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *common, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     out = "\n".join(l for l in (r.stdout + r.stderr).splitlines() if l.strip() != _HOST_PASS_NOTE)
     if r.returncode != 0:
@@ -93,23 +99,26 @@ def _compile(item):
     return obj, out
 
 
-def build(verbose: bool = False) -> str:
-    os.makedirs(OBJ, exist_ok=True)
+def build(verbose: bool = False, kernarg_preload: bool = True) -> str:
+    obj_dir = OBJ if kernarg_preload else OBJ + "_nopreload"
+    lib = LIB if kernarg_preload else LIB_NO_PRELOAD
+    common = COMMON if kernarg_preload else BASE
+    os.makedirs(obj_dir, exist_ok=True)
     verify_packed_fp32_off()
-    present = {s: e for s, e in SOURCES.items() if os.path.exists(os.path.join(CSRC, s))}
+    present = [(s, e, common, obj_dir) for s, e in SOURCES.items() if os.path.exists(os.path.join(CSRC, s))]
     with ThreadPoolExecutor(max_workers=min(8, len(present))) as ex:
-        results = list(ex.map(_compile, present.items()))
+        results = list(ex.map(_compile, present))
     if verbose:
         for _, out in results:
             if out.strip():
                 print(out)
     objs = [o for o, _ in results]
-    cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB, *objs, "-lpthread"]
+    cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", lib, *objs, "-lpthread"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, kernarg_preload="--no-kernarg-preload" not in sys.argv))

@@ -753,7 +753,10 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
     a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
     a.S = p.s; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
     a.scale = (float)(1.0 / sqrt((double)p.hd));
-    if (p.s >= 16) {                     // enough rows to share key tiles: matrix-core kernel
+#ifndef DJ_TILED_FROM
+#define DJ_TILED_FROM 16
+#endif
+    if (p.s >= DJ_TILED_FROM) {                     // enough rows to share key tiles: matrix-core kernel
         dim3 tg(p.h, (p.s + 127) / 128);
         if ((int64_t)tg.x * tg.y * 2 < kAttnFullGrid) {  // far too few workgroups for the chip: 32 rows each, keys in four sets
             dim3 tg4(p.h, (p.s + 31) / 32);

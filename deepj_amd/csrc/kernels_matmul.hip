@@ -15,6 +15,7 @@
 // finished 32-k partial sums (one scale per accumulator column per step).  Tile shapes (64 x 64, 64 x 128,
 // 128 x 128), scale groups per step and wavefront sets per workgroup are template arguments chosen per problem
 // shape by launch_q8_gemm; the epilogue adds bias / GELU / residual or pairs interleaved gate/up columns (SwiGLU).
+#include <cstdlib>
 #include "dj_common.h"
 #include "gemm_epilogue.h"
 
@@ -278,7 +279,8 @@ __device__ __forceinline__ float top_bits(float x) {      // the leading 8 signi
 template <int WTM, int WTN, int G, int KS>
 __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ A, const int8_t *__restrict__ Bq,
                                                  const float *__restrict__ Bs, float *__restrict__ C, int M,
-                                                 const int N, const int K, const int kp, GemmEpilogue ep) {
+                                                 const int N, const int K, const int kp, GemmEpilogue ep,
+                                                 const int split_k, float *__restrict__ partial) {
     constexpr int TM = 64 * WTM, TN = 64 * WTN;
     constexpr int QBK = kQ8Group * G;        // k per step
     constexpr int LDK = QBK + 8;             // LDS row: the step's bf16 payload + 8 of padding (16-byte aligned, spreads banks)
@@ -385,11 +387,15 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
         if (s_kb % kQ8Group == 0) Ss[s_kb / kQ8Group][s_col] = qsc;
     };
 
-    if (K > 0) fetch(0);
-    for (int k0 = 0; k0 < K; k0 += QBK) {
+    // split_k > 0: gridDim.z workgroups share a tile's K, this one takes [k_begin, k_end) (split_k is a multiple of the
+    // step) and leaves its bare sums in its own slab of `partial`; k_sum_partials_q8 adds the slabs in a fixed order
+    const int k_begin = split_k > 0 ? (int)blockIdx.z * split_k : 0;
+    const int k_end = split_k > 0 && k_begin + split_k < K ? k_begin + split_k : K;
+    if (k_begin < k_end) fetch(k_begin);
+    for (int k0 = k_begin; k0 < k_end; k0 += QBK) {
         stage();
         __syncthreads();
-        if (k0 + QBK < K) fetch(k0 + QBK);     // next step's global loads fly while this step multiplies
+        if (k0 + QBK < k_end) fetch(k0 + QBK);     // next step's global loads fly while this step multiplies
 
         // (a run-time loop on purpose: unrolled, the products of consecutive groups get interleaved and the kernel
         // measured 4-10 % slower)
@@ -456,6 +462,22 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
     }
 
     // epilogue: acc[i][jn][e] is C[32*i + 8*(e/4) + 4*(lane/32) + e%4][32*jn + lane%32] of the wavefront's block
+    if (split_k > 0) {
+        float *slab = partial + (int64_t)blockIdx.z * M * N;
+#pragma unroll
+        for (int jn = 0; jn < WTN; jn++) {
+            const int col = n0 + wn * 32 * WTN + 32 * jn + l32;
+            if (col >= N) continue;
+#pragma unroll
+            for (int i = 0; i < WTM; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int row = m0 + wm * 32 * WTM + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                    if (row < M) slab[(int64_t)row * N + col] = acc[i][jn][e];
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int jn = 0; jn < WTN; jn++) {
         const int col = n0 + wn * 32 * WTN + 32 * jn + l32;
@@ -491,6 +513,38 @@ __global__ void __launch_bounds__(256 * KS) k_gemm_q8(const float *__restrict__ 
     }
 }
 
+// C = epilogue(sum over the splits of partial[z]) for the K-sharing launches of k_gemm_q8: the same bias / GELU /
+// residual / SwiGLU steps, in the same order, as the kernel's own epilogue (a fixed order of additions, so a run
+// repeats bit for bit - which adding into C with atomics would not).  One thread per column pair of a row.
+__global__ void __launch_bounds__(256) k_sum_partials_q8(const float *__restrict__ partial, float *__restrict__ C, int splits,
+                                                        int M, int N, GemmEpilogue ep) {
+    const int64_t pairs = (int64_t)M * (N >> 1), mn = (int64_t)M * N;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < pairs; i += (int64_t)gridDim.x * 256) {
+        const int row = (int)(i / (N >> 1)), col = (int)(i % (N >> 1)) * 2;
+        const int64_t at = (int64_t)row * N + col;
+        float2 v = *reinterpret_cast<const float2 *>(partial + at);
+        for (int z = 1; z < splits; z++) {
+            const float2 p = *reinterpret_cast<const float2 *>(partial + (int64_t)z * mn + at);
+            v.x += p.x; v.y += p.y;
+        }
+        if (ep.bias) {
+            if (ep.interleaved_bias) { v.x = v.x + ep.bias[col >> 1]; v.y = v.y + ep.bias2[col >> 1]; }
+            else { v.x = v.x + ep.bias[col]; v.y = v.y + ep.bias[col + 1]; }
+        }
+        if (ep.swiglu) {                        // SiLU.java:20-24, SwiGLULayer.java:69
+            const float sg = v.x * (1.0f / (1.0f + expf(-v.x)));
+            C[(int64_t)row * (N >> 1) + (col >> 1)] = sg * v.y;
+            continue;
+        }
+        if (ep.gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); }
+        if (ep.residual) {
+            const float2 r = *reinterpret_cast<const float2 *>(ep.residual + at);
+            v.x = r.x + v.x; v.y = r.y + v.y;
+        }
+        *reinterpret_cast<float2 *>(C + at) = v;
+    }
+}
+
 constexpr int kFewTiles = 512, kGroupsFew = 4, kSetsFew = 4;
 constexpr int kSetsBig = 1;
 constexpr int kGroupsSmall = 2, kGroupsBig = 1;    // measured: 4 and 2 are slower (LDS per workgroup, registers)
@@ -515,11 +569,35 @@ void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out
     launch_kernel(k_gemm, grid, dim3(256), 0, s, a, b, out, m, n, k, ep);
 }
 
+// Few tiles over a long K: how many workgroups share a tile's K (1: none).  A 64 x 64 tile's workgroup (1024 threads,
+// its four wavefront sets already dividing every 128-k step) streams 64 weight rows; with fewer such workgroups than
+// compute units the launch is as long as one workgroup's walk through K (64 rows x 2048 x 2048: 32 workgroups, 23 us,
+// for 4.7 MB of weights; 11 us as 8 x 32).  Shares of at least two steps; one workgroup per compute unit at most (a
+// second round of workgroups costs what the shorter walk saves: 64 x 5632 x 2048 16.1 us with 176 workgroups, 18.7 with 352).
+int q8_gemm_k_shares(int m, int n_rows, int k) {
+    if (n_rows & 1) return 1;
+    if (use_big_tile(m, n_rows)) return 1;
+    const int64_t tiles = (int64_t)((n_rows + BN - 1) / BN) * ((m + BM - 1) / BM);
+    const int steps = (q8_padded_k(k) + kQ8Group * kGroupsFew - 1) / (kQ8Group * kGroupsFew);
+    if (tiles > 128 || steps < 4) return 1;
+    int shares = (int)std::min<int64_t>(std::min<int64_t>(8, 256 / tiles), steps / 2);
+    if (shares < 2) return 1;
+    const int per = (steps + shares - 1) / shares;
+    return (steps + per - 1) / per;
+}
+
+int64_t q8_gemm_workspace_floats(int m, int n_rows, int k) {
+    const int shares = q8_gemm_k_shares(m, n_rows, k);
+    return shares > 1 ? (int64_t)shares * m * n_rows : 0;
+}
+
 // Q8 GEMM used by launch_q8_linear for M > 1.  n_rows is the number of Q8 rows
-// (= output columns of this launch; 2N for an interleaved gate/up weight).
+// (= output columns of this launch; 2N for an interleaved gate/up weight).  workspace: room for the partial products
+// of a K-sharing launch (q8_gemm_workspace_floats), or less - then no K is shared.
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu, int swiglu) {
+                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu, int swiglu, float *workspace,
+                    int64_t workspace_floats) {
     if (m <= 0 || n_rows <= 0) return;
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
     GemmEpilogue ep{bias, bias2, residual, interleaved_bias, m_dev, m_extra, gelu, swiglu};
@@ -531,18 +609,30 @@ void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float
         const int64_t tiles = (int64_t)grid2.x * grid2.y, rounds = (tiles + 511) / 512;
         if (tiles * 100 < rounds * 512 * 85) {
             dim3 gridw(grid2.x, (m + 63) / 64);
-            launch_kernel((k_gemm_q8<1, 2, 2, 1>), gridw, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+            launch_kernel((k_gemm_q8<1, 2, 2, 1>), gridw, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep, 0, nullptr);
             return;
         }
-        launch_kernel((k_gemm_q8<2, 2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        launch_kernel((k_gemm_q8<2, 2, kGroupsBig, kSetsBig>), grid2, dim3(256 * kSetsBig), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep, 0, nullptr);
         return;
     }
     dim3 grid((n_rows + BN - 1) / BN, (m + BM - 1) / BM);
+    const int shares = m_dev ? 1 : q8_gemm_k_shares(m, n_rows, k);
+    if (shares > 1 && workspace && workspace_floats >= (int64_t)shares * m * n_rows) {
+        constexpr int step = kQ8Group * kGroupsFew;
+        const int steps = (q8_padded_k(k) + step - 1) / step, per = (steps + shares - 1) / shares;
+        grid.z = shares;
+        launch_kernel((k_gemm_q8<1, 1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep,
+                      per * step, workspace);
+        const int64_t pairs = (int64_t)m * (n_rows / 2);
+        launch_kernel(k_sum_partials_q8, dim3((unsigned)std::min<int64_t>((pairs + 255) / 256, 4096)), dim3(256), 0, s, (const float *)workspace, out,
+                      shares, m, n_rows, ep);
+        return;
+    }
     // few tiles (about one per CU): a workgroup brings its own second wavefront per SIMD
     if ((int64_t)grid.x * grid.y <= kFewTiles)
-        launch_kernel((k_gemm_q8<1, 1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        launch_kernel((k_gemm_q8<1, 1, kGroupsFew, kSetsFew>), grid, dim3(256 * kSetsFew), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep, 0, nullptr);
     else
-        launch_kernel((k_gemm_q8<1, 1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep);
+        launch_kernel((k_gemm_q8<1, 1, kGroupsSmall, 1>), grid, dim3(256), 0, s, x, wq, scales, out, m, n_rows, k, q8_padded_k(k), ep, 0, nullptr);
 }
 
 }  // namespace dj

@@ -27,7 +27,9 @@ namespace dj {
 
 void launch_q8_gemm(hipStream_t s, const float *x, const int8_t *wq, const float *scales, float *out, int m,
                     int k, int n_rows, const float *bias, const float *bias2, const float *residual,
-                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu, int swiglu);
+                    int interleaved_bias, const int32_t *m_dev, int m_extra, int gelu, int swiglu, float *workspace,
+                    int64_t workspace_floats);
+int64_t q8_gemm_workspace_floats(int m, int n_rows, int k);
 
 namespace {
 using namespace dev;
@@ -600,6 +602,7 @@ int64_t q8_linear_preferred_workspace_floats(int m, int k, int n, int flags, boo
     const int n_rows = (flags & DJ_LIN_SWIGLU) ? 2 * n : n;
     const bool mv = (m == 1) && matvec_supported(k);
     if (!mv && q8_gemm_f16_shape_ok(m, n_rows, k)) return std::max(ws, q8_gemm_f16_workspace_floats(m, n_rows, k, prepared));
+    if (!mv) return ws + q8_gemm_workspace_floats(m, n_rows, k);      // the partial products of a K-sharing launch
     return ws;
 }
 
@@ -655,11 +658,15 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
         x = ws;
         ws += (int64_t)p.m * p.k;
     }
+    // what is left of the workspace takes the partial products when a few tiles share their K among several workgroups
+    // (never with a workspace that cannot grow: one rule for the allocation-free entry point)
+    float *part = p.small_workspace_only ? nullptr : ws;
+    const int64_t part_floats = p.small_workspace_only ? 0 : workspace_floats - (ws - workspace);
     if (swiglu) {
         // the GEMM's epilogue pairs the interleaved gate/up columns, so the 2N-wide product never reaches memory
-        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, 2 * p.n, bias, bias2, nullptr, 1, nullptr, 0, 0, 1);
+        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, 2 * p.n, bias, bias2, nullptr, 1, nullptr, 0, 0, 1, part, part_floats);
     } else {
-        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0, p.m_dev, p.m_extra, gelu, 0);
+        launch_q8_gemm(s, x, p.wq, p.scales, p.out, p.m, p.k, p.n, bias, nullptr, residual, 0, p.m_dev, p.m_extra, gelu, 0, part, part_floats);
     }
 }
 

@@ -54,9 +54,10 @@ int deepj_hip_flush_ops(const int32_t *cmd, int32_t len);
 
 /* deepj_hip_flush_ops for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same streams and
- * the same kernels and bits as deepj_hip_flush_ops, with ONE exception: a Q8_LINEAR of 256 rows or more that
- * flush_ops runs on the fp16 GEMM (operands in a workspace sized by the shape) always runs on the bf16 GEMM here,
- * prepared weights or not - both meet the per-op tolerance against the CPU backend, their bits differ.  The
+ * the same kernels and bits as deepj_hip_flush_ops, with ONE exception: a Q8_LINEAR of more than one row always
+ * runs as a single launch of the bf16 GEMM here, where flush_ops - with a workspace sized by the shape - takes
+ * the fp16 GEMM (256 rows and more, enough tiles) or lets several workgroups share a tile's K (few tiles, long K),
+ * prepared weights or not; both meet the per-op tolerance against the CPU backend, their bits differ.  The
  * device scratch the kernels need - the workspace that Q8_LINEAR with a norm
  * prologue and M > 1 writes its normalised rows to, and the arrival counters of the split decode attention
  * (ATTENTION / ATTENTION_KV with S = 1, ATTN_DECODE) - is a fixed array inside the library's code object instead

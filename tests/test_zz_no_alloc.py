@@ -71,7 +71,9 @@ def test_noalloc_flush_matches_flush_on_two_calls_the_second_smaller():
     try:
         # the second case is smaller in every dimension: its workspace rows and its counters lie inside what
         # the first call used
-        cases = [Case(dev, 192, 2048, 320, 32, 64, 515, 100), Case(dev, 40, 1024, 96, 8, 32, 70, 200)]
+        # (GEMM shapes that flush_ops runs as ONE launch of the bf16 kernel, as the allocation-free entry point always
+        # does: 288 tiles of 64 x 64, and a K of three steps - too many tiles, too short a K, for workgroups to share it)
+        cases = [Case(dev, 192, 2048, 6144, 32, 64, 515, 100), Case(dev, 40, 384, 96, 8, 32, 70, 200)]
         expected = [c.run(noalloc=False) for c in cases]
         # the oracle on the first case's GEMM: the comparison below is between two HIP paths, this pins one of them
         c = cases[0]
@@ -90,6 +92,36 @@ def test_noalloc_flush_matches_flush_on_two_calls_the_second_smaller():
             for name, w, g in zip(("gemm", "attention", "k cache", "v cache"), want, got):
                 assert np.array_equal(w.view(np.int32), g.view(np.int32)), f"{name} differs between the entry points"
         assert HipNative.poolStats()["driver_allocs"] >= allocs_before
+    finally:
+        dev.release_all()
+
+
+def test_noalloc_flush_never_shares_k_among_workgroups():
+    """A few-tile, long-K product (64 rows x 2048 x 2048: 32 tiles) runs under flush_ops as eight workgroups per tile
+    with their partial products in the workspace; the allocation-free entry point runs it as one launch.  Both are
+    held to the oracle at the per-op tolerance."""
+    HipNative.init(0)
+    dev = DeviceBuffers()
+    try:
+        m, k, n = 64, 2048, 2048
+        w = gaussian(k, n, 41, 0.02)
+        x = gaussian(m, k, 42)
+        src = dev.upload(w)
+        wq = dev.alloc(HipNative.q8Floats(k, n))
+        Stream().q8_quantize(src, wq, k, n).run()
+        dev.release(src)
+        xb, out = dev.upload(x), dev.alloc(m * n)
+        exp = ref.matmul(x, ref.q8_roundtrip(w))
+        scale = float(np.sqrt(np.mean(exp.astype(np.float64) ** 2)))
+        words = Stream().q8_linear(xb, wq, out, m, k, n).array()
+        HipNative.nativeFlushOps(words, words.size)
+        assert_close(exp, dev.download(out, (m, n)), atol=1e-4 * scale, rtol=1e-4, what="flush_ops (K shared) vs oracle")
+        dev.write(out, np.zeros(m * n, np.float32))
+        before = HipNative.poolStats()["driver_allocs"]
+        HipNative.flushOpsNoAlloc(words, words.size)
+        got = dev.download(out, (m, n))
+        assert HipNative.poolStats()["driver_allocs"] == before
+        assert_close(exp, got, atol=1e-4 * scale, rtol=1e-4, what="noalloc (one launch) vs oracle")
     finally:
         dev.release_all()
 
