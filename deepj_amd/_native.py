@@ -38,6 +38,8 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_pool_stats.argtypes = [C.POINTER(C.c_int64)]
     lib.deepj_hip_stream.restype = C.c_void_p
     lib.deepj_hip_attn_record_splits.restype = C.c_int32
+    lib.deepj_hip_attention_scratch_floats.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    lib.deepj_hip_attention_scratch_floats.restype = C.c_int64
     lib.deepj_hip_q8_floats.argtypes = [C.c_int32, C.c_int32]
     lib.deepj_hip_q8_floats.restype = C.c_int64
     lib.deepj_hip_q8_prepared_floats.argtypes = [C.c_int32, C.c_int32]
@@ -154,6 +156,10 @@ class HipNative:
     @staticmethod
     def q8Floats(k: int, rows: int) -> int:
         return int(library().deepj_hip_q8_floats(k, rows))
+
+    @staticmethod
+    def attentionScratchFloats(S: int, H: int, hd: int, max_seq: int) -> int:
+        return int(library().deepj_hip_attention_scratch_floats(S, H, hd, max_seq))
 
     @staticmethod
     def attnRecordSplits() -> int:

@@ -97,6 +97,7 @@ struct AttnKernelArgs {
     int64_t tok_stride, head_stride;
     int S, H, hd, max_seq;
     float scale;
+    float *partial = nullptr;   // key-sharing launches of the tiled kernel: records [row][head][share][hd + 4]
 };
 
 template <int LPK>
@@ -170,7 +171,11 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // KSETS = 2 or 4 (for grids that would leave CUs idle): a workgroup takes 64 or 32 query rows; its wavefronts are
 // 2 or 4 sets that walk every KSETS-th key tile for the SAME queries, KSETS tiles are staged per round, and the
 // sets' partial soft-max states are merged through LDS at the end - more workgroups and fewer rounds.
-template <int HD, int KSETS>
+// SHARE: the gridDim.z workgroups of a (head, query tile) take the rounds of key tiles in turn (round r goes to
+// r % gridDim.z, so the shares are even whatever the position, which only the device knows) and leave their
+// unnormalised states as records; k_attention_merge_shares finishes the rows.  For a handful of query rows over a
+// long context, where (head, query tile) alone are far fewer workgroups than compute units.
+template <int HD, int KSETS, bool SHARE = false>
 __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     constexpr int KT = 32, NT = HD / 32;
     constexpr int QW = 4 / KSETS;                           // wavefronts that hold distinct query rows
@@ -220,7 +225,9 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 
     const float *kbase = a.k + (int64_t)h * a.head_stride;
     const float *vbase = a.v + (int64_t)h * a.head_stride;
-    for (int k0 = 0; k0 <= wg_last; k0 += KT * KSETS) {
+    const int k_first = SHARE ? (int)blockIdx.z * KT * KSETS : 0;
+    const int k_stride = SHARE ? (int)gridDim.z * KT * KSETS : KT * KSETS;
+    for (int k0 = k_first; k0 <= wg_last; k0 += k_stride) {
 #pragma unroll
         for (int ks = 0; ks < KSETS; ks++) {
             // stage the key tile transposed and the value tile; rows past the last key repeat it (masked below)
@@ -314,6 +321,17 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
         }
     }
     l += __shfl_xor(l, 32, 64);
+    if constexpr (SHARE) {
+        if (q_ok) {
+            float *rec = a.partial + (((int64_t)qi * a.H + h) * gridDim.z + blockIdx.z) * (HD + 4);
+            if (half == 0) { rec[0] = m; rec[1] = l; }
+#pragma unroll
+            for (int i = 0; i < NT; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) rec[4 + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3)] = acc[i][e];
+        }
+        return;
+    }
     if (q_ok) {
         float *orow = a.out + (int64_t)qi * d + h * HD;
 #pragma unroll
@@ -321,6 +339,26 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; e++) orow[32 * i + 8 * (e >> 2) + 4 * half + (e & 3)] = acc[i][e] / l;
     }
+}
+
+// out[row, h, :] = sum_z w_z o_z / sum_z w_z l_z,  w_z = exp(m_z - max m), over the `shares` records of (row, head);
+// grid (H, S), one thread per output element.  A share without keys left m = -inf, l = 0.
+__global__ void __launch_bounds__(128) k_attention_merge_shares(const float *__restrict__ partial, float *__restrict__ out, int H,
+                                                               int hd, int shares) {
+    const int h = blockIdx.x, row = blockIdx.y, j = threadIdx.x;
+    if (j >= hd) return;
+    const float *rec = partial + ((int64_t)row * H + h) * shares * (hd + 4);
+    float M = -INFINITY;
+    for (int z = 0; z < shares; z++) M = fmaxf(M, rec[(int64_t)z * (hd + 4)]);
+    float L = 0.0f, O = 0.0f;
+    for (int z = 0; z < shares; z++) {
+        const float *r = rec + (int64_t)z * (hd + 4);
+        if (r[0] == -INFINITY) continue;
+        const float w = expf(r[0] - M);
+        L += r[1] * w;
+        O += r[4 + j] * w;
+    }
+    out[((int64_t)row * H + h) * hd + j] = O / L;
 }
 
 // ── fused decode attention ──────────────────────────────────────────────────
@@ -335,7 +373,8 @@ struct DecodeArgs {
     const float *cos_t, *sin_t;
     int H, hd, max_seq, nsplit;
     float scale;
-    unsigned *counters;        // one arrival counter per head, zero between launches
+    unsigned *counters;        // one arrival counter per (query row, head), zero between launches
+    int64_t q_row_stride = 0;  // floats between the q rows when one launch serves several (grid z)
 };
 
 // FUSED: rotate q and the new key in registers and append the new key/value row to the cache.
@@ -347,12 +386,12 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     __shared__ float s_m[NSUB], s_l[NSUB];
     __shared__ __align__(16) float s_o[NSUB][HD];
 
-    const int h = blockIdx.x, split = blockIdx.y;
+    const int h = blockIdx.x, split = blockIdx.y, qrow = blockIdx.z;     // qrow: query row (a few rows of a prompt; 0 in decode)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane / LPK, dl = lane % LPK;
     const int d = a.H * HD, half = HD / 2;
 
-    int pos = a.state[0];
+    int pos = a.state[0] + qrow;
     if (pos < 0) pos = 0;
     if (pos >= a.max_seq) pos = a.max_seq - 1;             // the host never lets this happen; stay in bounds
     const int n_keys = pos + 1;
@@ -366,7 +405,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
         c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
         s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
     }
-    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
+    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + (int64_t)qrow * a.q_row_stride + h * HD + dl * 4);
     const float4 qv = FUSED ? make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
                                           q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y)
                             : q0;
@@ -436,7 +475,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
         }
         // The record is written through to memory (agent-scope stores) so that the split that
         // finishes last can read every record of its head without a cache flush.
-        float *rec = a.scratch + ((int64_t)h * a.nsplit + split) * (HD + 4);
+        float *rec = a.scratch + (((int64_t)qrow * a.H + h) * a.nsplit + split) * (HD + 4);
         __hip_atomic_store(rec + 4 + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (tid == 0) {
             __hip_atomic_store(rec, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -448,14 +487,15 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     __builtin_amdgcn_s_waitcnt(0x0f70);            // vmcnt(0): this workgroup's record and appended row are in memory
     __syncthreads();
     if (tid == 0) {
-        unsigned old = __hip_atomic_fetch_add(a.counters + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned *counter = a.counters + qrow * a.H + h;
+        unsigned old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         bool last = old + 1 == (unsigned)a.nsplit;
-        if (last) __hip_atomic_store(a.counters + h, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = last ? 1 : 0;
     }
     __syncthreads();
     if (s_last && tid < HD) {
-        const float *base = a.scratch + (int64_t)h * a.nsplit * (HD + 4);
+        const float *base = a.scratch + ((int64_t)qrow * a.H + h) * a.nsplit * (HD + 4);
         float m[16], l[16], o[16];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -476,7 +516,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
                 O += o[i] * w;
             }
         }
-        a.out[h * HD + tid] = O / L;
+        a.out[(int64_t)qrow * d + h * HD + tid] = O / L;
     }
 }
 
@@ -685,19 +725,29 @@ void launch_rope_rows(hipStream_t s, const float *x, float *out, const int32_t *
                        max_seq, pos_from_row, row_stride > 0 ? row_stride : H * hd, live_extra);
 }
 
-// S = 1 uses the split kernels (scratch: attn_decode_scratch_floats); S > 1 needs no scratch.
+// One row uses the split decode kernel (scratch: attn_decode_scratch_floats); 2 to kAttnShareRows rows - a short
+// continuation of a cached prefix - the matrix-core kernel with the key rounds dealt to kAttnKeyShares workgroups
+// (scratch: their records); more rows need no scratch.
+constexpr int kAttnShareRows = 32;
+int attention_key_shares(int S, int H) {
+    if (S < 2 || S > kAttnShareRows) return 1;
+    int z = 256 / H;                                   // about one workgroup per compute unit
+    return z < 1 ? 1 : (z > 8 ? 8 : z);
+}
 int64_t attention_scratch_floats(int S, int H, int hd, int max_seq) {
     (void)max_seq;
-    return S == 1 ? attn_decode_scratch_floats(H, hd) : 0;
+    if (S == 1) return attn_decode_scratch_floats(H, hd);
+    const int z = attention_key_shares(S, H);
+    return z > 1 ? (int64_t)S * H * z * (hd + 4) : 0;
 }
 
 int64_t attn_decode_scratch_floats(int H, int hd) { return (int64_t)H * fused_decode_splits(H) * (hd + 4); }
 
 template <bool FUSED>
-static void launch_decode_kernels(hipStream_t s, DecodeArgs &a) {
+static void launch_decode_kernels(hipStream_t s, DecodeArgs &a, int rows = 1) {
     a.nsplit = fused_decode_splits(a.H);
     a.scale = (float)(1.0 / sqrt((double)a.hd));
-    dim3 grid(a.H, a.nsplit);
+    dim3 grid(a.H, a.nsplit, rows);
     switch (a.hd) {
         case 32: launch_kernel((k_attn_decode_partial<8, FUSED>), grid, dim3(kThreads), 0, s, a); break;
         case 64: launch_kernel((k_attn_decode_partial<16, FUSED>), grid, dim3(kThreads), 0, s, a); break;
@@ -753,10 +803,25 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
     a.tok_stride = p.k_tok_stride; a.head_stride = p.k_head_stride;
     a.S = p.s; a.H = p.h; a.hd = p.hd; a.max_seq = p.max_seq;
     a.scale = (float)(1.0 / sqrt((double)p.hd));
-#ifndef DJ_TILED_FROM
-#define DJ_TILED_FROM 16
-#endif
-    if (p.s >= DJ_TILED_FROM) {                     // enough rows to share key tiles: matrix-core kernel
+    const int shares = attention_key_shares(p.s, p.h);
+    if (shares > 1) {
+        // A handful of rows after a long prefix: one 32-row query tile per head, its key rounds dealt to `shares`
+        // workgroups.  (32 heads of 64, 2 to 31 rows after 1500 cached ones: 15 to 17 us with the merge, against 34 us
+        // for one workgroup per row (2 to 15 rows) and 55 us for the unshared matrix-core kernel (16 to 31); after 500:
+        // 10 to 12 us against 13 and 25.  A fresh prompt of so few rows pays 6 us for it.)
+        if (p.scratch_floats < attention_scratch_floats(p.s, p.h, p.hd, p.max_seq)) fail("attention: scratch buffer too small");
+        a.partial = p.scratch;
+        dim3 tgz(p.h, 1, shares);
+        switch (p.hd) {
+            case 32: launch_kernel((k_attention_tiled<32, 4, true>), tgz, dim3(256), 0, s, a); break;
+            case 64: launch_kernel((k_attention_tiled<64, 4, true>), tgz, dim3(256), 0, s, a); break;
+            case 128: launch_kernel((k_attention_tiled<128, 4, true>), tgz, dim3(256), 0, s, a); break;
+            default: fail("attention: head dim must be 32, 64 or 128");
+        }
+        launch_kernel(k_attention_merge_shares, dim3(p.h, p.s), dim3(128), 0, s, (const float *)p.scratch, p.out, p.h, p.hd, shares);
+        return;
+    }
+    if (p.s >= 16) {                     // enough rows to share key tiles: matrix-core kernel
         dim3 tg(p.h, (p.s + 127) / 128);
         if ((int64_t)tg.x * tg.y * 2 < kAttnFullGrid) {  // far too few workgroups for the chip: 32 rows each, keys in four sets
             dim3 tg4(p.h, (p.s + 31) / 32);

@@ -355,7 +355,9 @@ void finalize(Runner &r) {
     r.logits = r.alloc(c.vocab);
     r.last_x = r.alloc(c.d);
     int ns = std::max(1, std::min(16, 512 / c.heads));
-    int64_t sf = (int64_t)c.heads * ns * (hd + 4);           // split-attention records (S = 1 paths)
+    // attention scratch: the split records of one row (decode paths) or of a short prompt whose key rounds are shared
+    int64_t sf = (int64_t)c.heads * ns * (hd + 4);
+    for (int rows = 2; rows <= 32; rows++) sf = std::max(sf, deepj_hip_attention_scratch_floats(rows, c.heads, hd, c.max_seq));
     r.scratch = r.alloc(sf);
     r.records = r.alloc((int64_t)c.heads * deepj_hip_attn_record_splits() * (hd + 4));
     Stream s;

@@ -993,6 +993,11 @@ void *deepj_hip_stream(void) { return g.ready ? (void *)g.stream : nullptr; }
 
 int32_t deepj_hip_attn_record_splits(void) { return kAttnRecordSplits; }
 
+int64_t deepj_hip_attention_scratch_floats(int32_t S, int32_t H, int32_t hd, int32_t max_seq) {
+    if (S <= 0 || H <= 0 || hd <= 0) return 0;
+    return attention_scratch_floats(S, H, hd, max_seq);
+}
+
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows) {
     if (k <= 0 || rows <= 0) return 0;
     return (q8_bytes(k, rows) + 3) / 4;

@@ -173,5 +173,6 @@ def attn_record_floats(H: int, hd: int) -> int:
 
 
 def attention_scratch_floats(H: int, hd: int, max_seq: int = 0) -> int:
-    """Floats the scratch buffer of ATTENTION / ATTENTION_KV must hold when S = 1."""
-    return attn_decode_scratch_floats(H, hd)
+    """Floats a scratch buffer of ATTENTION / ATTENTION_KV must hold to serve any S (one row and short prompts of up to
+    32 rows use it)."""
+    return max(HipNative.attentionScratchFloats(S, H, hd, max_seq) for S in range(1, 34))

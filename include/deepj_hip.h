@@ -152,7 +152,9 @@ enum {
      * ROPE_KV_STORE [op, qkv, qOut, kCache, vCache, state, cosT, sinT, S, H, hd, maxSeq, layer]
      *     qkv [S x 3d]; rows sit at positions state[0]..state[0]+S-1
      * ATTENTION     [op, q, kCache, vCache, out, state, scratch, S, H, hd, maxSeq, layer]
-     *     scratch is only used when S = 1 (H * min(16, max(1, 512/H)) * (hd+4) floats, no initialisation)
+     *     scratch (deepj_hip_attention_scratch_floats(S, H, hd, maxSeq) floats, no initialisation) is used by one
+     *     row, whose keys are split over workgroups, and by 2 to 32 rows, whose key tiles are dealt to several
+     *     workgroups per head (a short continuation of a long cached prefix would otherwise leave most of the chip idle)
      * ARGMAX_ROWS   [op, logits, out, rows, cols]      out int32 words, ties -> lowest index
      * DECODE_ADVANCE[op, state, token, tokens, capacity, nPos]
      *     state (int32 words): [0] positions held in the cache, [1] current token, [2] tokens generated;
@@ -206,6 +208,9 @@ enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU =
 
 /* Key splits per head of ATTN_DECODE_RECORDS: its records buffer holds H * splits * (hd + 4) floats. */
 int32_t deepj_hip_attn_record_splits(void);
+
+/* Floats the scratch buffer of ATTENTION / ATTENTION_KV must hold for S query rows (0: none needed). */
+int64_t deepj_hip_attention_scratch_floats(int32_t S, int32_t H, int32_t hd, int32_t max_seq);
 
 /* Floats a Q8 weight buffer with `rows` output rows over K inputs must hold. */
 int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);

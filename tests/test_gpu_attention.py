@@ -31,7 +31,13 @@ def oracle_attention(q, k, v, H, cos, sin):
                                                  # two-key-set and one-key-set variants (the small shapes above use four)
                                                  (32, 64, 1200, [1100, 1, 20]), (64, 32, 1150, [1100, 1]),
                                                  # ragged chunks around the 16-row threshold and the 32-row query tile
-                                                 (4, 64, 200, [17, 1, 33, 15, 16, 65]), (3, 128, 150, [31, 97])])
+                                                 (4, 64, 200, [17, 1, 33, 15, 16, 65]), (3, 128, 150, [31, 97]),
+                                                 # short continuations of a cached prefix (2 to 32 rows: the key rounds
+                                                 # of a head are dealt to several workgroups whose records a second
+                                                 # kernel merges), ragged, after prefixes of less than one round of
+                                                 # keys and of many; with few heads (eight shares) and with 256 (one)
+                                                 (32, 64, 2048, [515, 2, 7, 15, 8, 32, 1, 31, 900, 5]), (4, 128, 700, [600, 7, 2, 8, 15]),
+                                                 (8, 32, 300, [2, 3, 31, 7, 130, 9]), (256, 32, 40, [20, 3, 8, 4, 5])])
 def test_rope_store_attention_prefill_and_decode(H, hd, max_seq, chunks):
     d = H * hd
     total = sum(chunks)
