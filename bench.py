@@ -170,47 +170,68 @@ MFMA_PEAK_TFLOPS = 2500.0       # MI355X dense fp16 / bf16 matrix-core peak
 
 
 def prefill_roofline(model, n: int, iters: int = 6):
-    """Per-kernel durations of the n-token prompt's command stream, measured live like the decode table (a start and a
-    stop event on each op's main dispatch; the small helpers of a Q8_LINEAR - the activation split, the sum of partial
-    products - are inside the whole-prompt time but not in the per-kernel figure).  A projection's algorithmic work is
-    one multiply-add per weight per row, 2 M K N flops; the fp16 kernels issue two matrix-core products for it (hi and
-    lo halves of the activation), the bf16 kernels three - `issued` counts those against the same peak."""
+    """Per-op durations of the n-token prompt's command stream, measured live like the decode table: a start and a stop
+    event on EVERY dispatch of every op, summed per op - so a projection's figure holds its GEMM and the helpers the
+    op cannot do without (the split of the activations into fp16 planes, with the norm; the sum of partial products
+    when workgroups share K; the per-call conversion of the weights when the runner holds no fp16 copy).  `gemm_us` is
+    the op's longest dispatch alone.  A projection's algorithmic work is one multiply-add per weight per row,
+    2 M K N flops; the fp16 kernels issue two matrix-core products for it (hi and lo halves of the activation), the
+    bf16 kernels three - `issued` counts those against the same peak."""
     from deepj_amd import HipNative, opcodes as op
     stream = model.prefillStream(n)
     ops = decode_ops(stream)
     HipNative.profileOps(stream, 2)
-    us = HipNative.profileOps(stream, iters)
+    us, top, count = HipNative.profileOps(stream, iters, detail=True)
     names = {(2048, 6144): "qkv", (2048, 2048): "wo", (2048, 11264): "gate_up", (5632, 2048): "down"}
-    table, flops, gemm_us, issued = {}, 0.0, 0.0, 0.0
-    for (code, w), t in zip(ops, us):
-        if code == op.OP_Q8_LINEAR and w[4] > 1 and t > 0:
+    other_names = {op.OP_ROPE_KV_STORE: "rope_kv_store", op.OP_EMBED_GATHER: "embed_gather", op.OP_DECODE_NEXT: "decode_next",
+                   op.OP_COPY: "copy_last_row"}
+    table, flops, gemm_us, issued, all_us = {}, 0.0, 0.0, 0.0, 0.0
+    for (code, w), t, t_top, c in zip(ops, us, top, count):
+        if t <= 0:
+            continue
+        all_us += float(t)
+        if code == op.OP_Q8_LINEAR and w[4] > 1:
             m, k, nn, flags = w[4], w[5], w[6], w[7]
             rows = 2 * nn if flags & op.LIN_SWIGLU else nn
             tile, tile_cols, shares = HipNative.q8GemmTile(m, k, rows)
             f = 2.0 * m * k * rows
             e = table.setdefault(names.get((k, rows), f"{k}x{rows}"), {
-                "launches": 0, "us": 0.0, "flops": f,
+                "launches": 0, "us": 0.0, "gemm_us": 0.0, "dispatches_per_op": int(c), "flops": f,
                 "kernel": (f"k_gemm_q8_f16 ({tile} x {tile_cols} tiles" + (f", K shared by {shares}" if shares > 1 else "") +
                            ", fp16 x 2)") if tile else "k_gemm_q8 (bf16 x 3)"})
             e["launches"] += 1
             e["us"] += float(t)
+            e["gemm_us"] += float(t_top)
             flops += f
             gemm_us += float(t)
             issued += f * (2 if tile else 3)
-        elif code == op.OP_ATTENTION and t > 0:
+        elif code == op.OP_ATTENTION:
             e = table.setdefault("attention", {"launches": 0, "us": 0.0, "kernel": "k_attention_tiled (fp32 matrix cores)"})
+            e["launches"] += 1
+            e["us"] += float(t)
+        elif code in other_names or (code == op.OP_Q8_LINEAR and w[4] == 1):
+            e = table.setdefault(other_names.get(code, "lm_head_last_row"), {"launches": 0, "us": 0.0})
             e["launches"] += 1
             e["us"] += float(t)
     for e in table.values():
         e["us"] = round(e["us"] / e["launches"], 2)
+        if "gemm_us" in e:
+            e["gemm_us"] = round(e["gemm_us"] / e["launches"], 2)
         if "flops" in e:
             e["TFLOPs"] = round(e.pop("flops") / e["us"] / 1e6, 1)
             e["frac"] = round(e["TFLOPs"] / MFMA_PEAK_TFLOPS, 4)
+    # HBM-bound helpers of the prompt against the HBM peak: RoPE + cache append moves 24 bytes per element of [n x d]
+    d = model.cfg.dModel
+    if "rope_kv_store" in table:
+        e = table["rope_kv_store"]
+        e["bytes"] = 24 * n * d
+        e["frac_of_hbm_peak"] = round(e["bytes"] / e["us"] / 1e3 / HBM_PEAK_GBS, 4)
     achieved = flops / gemm_us / 1e6
     return {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "issued_frac": round(issued / gemm_us / 1e6 / MFMA_PEAK_TFLOPS, 4),
-            "kernel": "Q8 GEMM of the prompt's projections", "rows": n, "per_kernel": table,
-            "timing": "mean kernel duration (start/stop events on each dispatch, whole prompt in order)"}
+            "kernel": "Q8_LINEAR ops of the prompt's projections (GEMM + their helper kernels)", "rows": n,
+            "kernel_time_us_all_ops": round(all_us, 1), "per_kernel": table,
+            "timing": "per op: sum of the begin-to-end times of all its dispatches (start/stop events on each, whole prompt in order)"}
 
 
 C2_SHAPES = [(2048, 2048), (2048, 5632), (5632, 2048), (4096, 11008)]     # K x N of the isolated linear-op sweep
