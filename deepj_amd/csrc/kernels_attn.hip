@@ -373,8 +373,7 @@ struct DecodeArgs {
     const float *cos_t, *sin_t;
     int H, hd, max_seq, nsplit;
     float scale;
-    unsigned *counters;        // one arrival counter per (query row, head), zero between launches
-    int64_t q_row_stride = 0;  // floats between the q rows when one launch serves several (grid z)
+    unsigned *counters;        // one arrival counter per head, zero between launches
 };
 
 // FUSED: rotate q and the new key in registers and append the new key/value row to the cache.
@@ -386,12 +385,12 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     __shared__ float s_m[NSUB], s_l[NSUB];
     __shared__ __align__(16) float s_o[NSUB][HD];
 
-    const int h = blockIdx.x, split = blockIdx.y, qrow = blockIdx.z;     // qrow: query row (a few rows of a prompt; 0 in decode)
+    const int h = blockIdx.x, split = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane / LPK, dl = lane % LPK;
     const int d = a.H * HD, half = HD / 2;
 
-    int pos = a.state[0] + qrow;
+    int pos = a.state[0];
     if (pos < 0) pos = 0;
     if (pos >= a.max_seq) pos = a.max_seq - 1;             // the host never lets this happen; stay in bounds
     const int n_keys = pos + 1;
@@ -405,7 +404,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
         c2 = *reinterpret_cast<const float2 *>(a.cos_t + (int64_t)pos * half + dl * 2);
         s2 = *reinterpret_cast<const float2 *>(a.sin_t + (int64_t)pos * half + dl * 2);
     }
-    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + (int64_t)qrow * a.q_row_stride + h * HD + dl * 4);
+    const float4 q0 = *reinterpret_cast<const float4 *>(a.qkv + h * HD + dl * 4);
     const float4 qv = FUSED ? make_float4(q0.x * c2.x - q0.y * s2.x, q0.x * s2.x + q0.y * c2.x,
                                           q0.z * c2.y - q0.w * s2.y, q0.z * s2.y + q0.w * c2.y)
                             : q0;
@@ -475,7 +474,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
         }
         // The record is written through to memory (agent-scope stores) so that the split that
         // finishes last can read every record of its head without a cache flush.
-        float *rec = a.scratch + (((int64_t)qrow * a.H + h) * a.nsplit + split) * (HD + 4);
+        float *rec = a.scratch + ((int64_t)h * a.nsplit + split) * (HD + 4);
         __hip_atomic_store(rec + 4 + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (tid == 0) {
             __hip_atomic_store(rec, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -487,7 +486,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     __builtin_amdgcn_s_waitcnt(0x0f70);            // vmcnt(0): this workgroup's record and appended row are in memory
     __syncthreads();
     if (tid == 0) {
-        unsigned *counter = a.counters + qrow * a.H + h;
+        unsigned *counter = a.counters + h;
         unsigned old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         bool last = old + 1 == (unsigned)a.nsplit;
         if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -495,7 +494,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
     }
     __syncthreads();
     if (s_last && tid < HD) {
-        const float *base = a.scratch + ((int64_t)qrow * a.H + h) * a.nsplit * (HD + 4);
+        const float *base = a.scratch + (int64_t)h * a.nsplit * (HD + 4);
         float m[16], l[16], o[16];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -516,7 +515,7 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
                 O += o[i] * w;
             }
         }
-        a.out[(int64_t)qrow * d + h * HD + tid] = O / L;
+        a.out[h * HD + tid] = O / L;
     }
 }
 
@@ -537,15 +536,9 @@ __global__ void __launch_bounds__(kThreads) k_attn_decode_partial(DecodeArgs a) 
 //  * Four splits of 512 threads: eight splits shorten this kernel by 0.9 us at 1500 keys and cost the Wo matvec,
 //    every workgroup of which reads all records, 0.7 us.  (Requesting the first tiles before the position is known
 //    - rows past it are readable, being inside the cache buffer - gained nothing: measured 2435 against 2443 tok/s.)
-#ifndef DJ_REC_THREADS
-#define DJ_REC_THREADS 512
-#endif
-constexpr int kRecThreads = DJ_REC_THREADS;
+constexpr int kRecThreads = 512;
 constexpr int kRecWaves = kRecThreads / 64;
-#ifndef DJ_REC_U
-#define DJ_REC_U 4
-#endif
-constexpr int kRecU = DJ_REC_U;   // key tiles a workgroup requests per round
+constexpr int kRecU = 4;          // key tiles a workgroup requests per round (2: 2437, 4: 2443, 8: 2411 tok/s)
 
 // Timeline of one launch, for tuning builds only (-DDJ_TRACE; never in the shipped library).
 #ifdef DJ_TRACE
@@ -744,10 +737,10 @@ int64_t attention_scratch_floats(int S, int H, int hd, int max_seq) {
 int64_t attn_decode_scratch_floats(int H, int hd) { return (int64_t)H * fused_decode_splits(H) * (hd + 4); }
 
 template <bool FUSED>
-static void launch_decode_kernels(hipStream_t s, DecodeArgs &a, int rows = 1) {
+static void launch_decode_kernels(hipStream_t s, DecodeArgs &a) {
     a.nsplit = fused_decode_splits(a.H);
     a.scale = (float)(1.0 / sqrt((double)a.hd));
-    dim3 grid(a.H, a.nsplit, rows);
+    dim3 grid(a.H, a.nsplit);
     switch (a.hd) {
         case 32: launch_kernel((k_attn_decode_partial<8, FUSED>), grid, dim3(kThreads), 0, s, a); break;
         case 64: launch_kernel((k_attn_decode_partial<16, FUSED>), grid, dim3(kThreads), 0, s, a); break;

@@ -298,7 +298,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 constexpr int TM64 = 64;
 constexpr int kXs64 = 2 * TM64 * 64;
 constexpr int stage64_bytes(int tnw) { return kXs64 + 64 * tnw * 64 + 1024; }
-constexpr int kMinSplitSteps = 32;          // K steps a workgroup must at least have when several share a tile's K
+constexpr int kMinSplitSteps = 16;          // K steps a workgroup must at least have when several share a tile's K
 
 template <int TNW>
 __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
@@ -653,7 +653,8 @@ GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
     }
     // few tiles but a long K (512 x 2048 output over K 5632: 64 tiles, 71 us on the bf16 kernel, 47 us as 4 x 64
     // workgroups): several workgroups per tile, each with a share of K of at least kMinSplitSteps steps, their partial
-    // products summed by a second kernel.  With K 2048 (two shares) it is a tie with the bf16 kernel, which keeps it.
+    // products summed by a second kernel.  (512 x 2048 over K 2048, 64 tiles: four shares of 16 steps, GEMM 18.4 us,
+    // 27.4 with the activation split and the sum, against 30.3 on the bf16 kernel; three shares 29.4, two a tie.)
     const int steps = q8_padded_k(k) / 32;
     const int splits = (int)std::min<int64_t>(std::min<int64_t>(8, 256 / t64), steps / kMinSplitSteps);
     if (t64 >= 32 && splits >= 3) return {64, 256, splits};

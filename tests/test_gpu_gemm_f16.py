@@ -48,7 +48,8 @@ def test_path_query_matches_the_documented_rule():
     assert HipNative.q8GemmPath(512, 2048, 11264) == 128      # 4 x 44 tiles of 128 x 256
     assert HipNative.q8GemmPath(2048, 4096, 4096) == 128      # 16 x 16
     assert HipNative.q8GemmPath(512, 2048, 6144) == 64        # 96 such tiles would idle most of the chip: 192 of 64 x 256
-    assert HipNative.q8GemmPath(512, 2048, 2048) == 0         # 64 even of those: the bf16 kernels' 64 x 64 tiles
+    assert HipNative.q8GemmPath(512, 2048, 2048) == 64        # 64 even of those: four workgroups share each tile's K
+    assert HipNative.q8GemmPath(512, 1024, 2048) == 0         # ... when K is long enough for shares of 16 steps: else the bf16 kernels
     assert HipNative.q8GemmPath(512, 5632, 2048) == 64        # the same 64 tiles over a long K: four workgroups share each
     assert HipNative.q8GemmTile(512, 5632, 2048) == (64, 256, 4)
     assert HipNative.q8GemmTile(512, 2048, 6144) == (64, 192, 1)     # 256 tiles: one per compute unit
