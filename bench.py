@@ -36,10 +36,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-# HBM bytes read + written per matvec launch (mean over the 65 launches of one token), from rocprofv3
-# FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
-# (profiles/q8_matvec_llama_d2048_decode_hbm_traffic.txt); algorithmic bytes are 15.40 MB.
-MATVEC_TRAFFIC_BYTES_PER_LAUNCH = 15_800_000
+# HBM bytes read + written per matvec launch (mean over the 65 launches of one token).  rocprofv3 cannot collect
+# counters over the decode stream on this build (profiles/README.md), so the figure is the algorithmic 15.40 MB times
+# the fetched / algorithmic ratios its FETCH_SIZE counter gives for the same kernel on buffers of the same sizes in the
+# isolated sweep (profiles/q8_matvec_c2_sweep_hbm_traffic.txt: 1.032 at 4.7 MB, 1.014-1.024 at 13 MB, 1.010 at 51 MB).
+MATVEC_TRAFFIC_BYTES_PER_LAUNCH = 15_700_000
 
 
 def q8_linear_bytes(k: int, n_rows: int) -> int:
@@ -150,8 +151,9 @@ def matvec_roofline(model, position: int, iters: int = 12):
     dev.release_all()
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MATVEC_TRAFFIC_BYTES_PER_LAUNCH,
-            "traffic_source": "profiles/q8_matvec_llama_d2048_decode_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
-                              "WRITE_SIZE, scaled by k_copy)",
+            "traffic_source": "not measured in this run: algorithmic bytes x the fetched / algorithmic ratio of the same kernel "
+                              "in profiles/q8_matvec_c2_sweep_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over "
+                              "bench.py --sweep, scaled by k_copy)",
             "kernel": "k_q8_matvec", "launches_per_token": launches, "bytes_per_launch": lin_bytes // launches,
             "avg_launch_us": round(lin_us / launches, 3),
             "timing": "mean kernel duration (start/stop events on each dispatch, whole token in order, HBM-cold); "
