@@ -9,8 +9,7 @@ from .hip_backend import HipBackend, HipGpuRuntime
 from .tensor import Tensor
 from .models import (DeepSeekConfig, DeepSeekModel, GPTConfig, GPTModel, JavaRandom, LlamaConfig, LlamaModel,
                      TextGenerator)
-from . import dropin
 from .persistence import ModelSerializer, parameter_names, parameter_shapes
 
-__all__ = ["ModelSerializer", "parameter_names", "parameter_shapes", "opcodes", "dropin", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor",
+__all__ = ["ModelSerializer", "parameter_names", "parameter_shapes", "opcodes", "HipNative", "LIB_PATH", "ComputeGraph", "GpuBuffer", "HipBackend", "HipGpuRuntime", "Tensor",
            "LlamaConfig", "LlamaModel", "GPTConfig", "GPTModel", "DeepSeekConfig", "DeepSeekModel", "TextGenerator", "JavaRandom"]

@@ -48,6 +48,8 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_gemm_path.restype = C.c_int32
     lib.deepj_hip_q8_gemm_tile.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
     lib.deepj_hip_q8_gemm_tile.restype = None
+    lib.deepj_hip_q8_gemm_f16_extents.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+    lib.deepj_hip_q8_gemm_f16_extents.restype = C.c_int32
     lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
     lib.deepj_hip_profile_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p, C.c_int32, _i32p, _f32p, _i32p]
     lib.deepj_hip_graph_capture.argtypes = [_i32p, C.c_int32, _i32p]
@@ -176,6 +178,14 @@ class HipNative:
         r, c, s = C.c_int32(), C.c_int32(), C.c_int32()
         library().deepj_hip_q8_gemm_tile(m, k, rows, C.byref(r), C.byref(c), C.byref(s))
         return r.value, c.value, s.value
+
+    @staticmethod
+    def q8GemmF16Extents(m: int, k: int, rows: int, tile_rows: int = 0, tile_cols: int = 0):
+        """(verdict, reach, size): bytes the fp16 GEMM's direct loads reach in (planes, fp16 weights, scales) against the
+        bytes those hold; verdict 1 inside, 0 outside, -1 not a shape of these kernels.  Host arithmetic, no GPU call."""
+        reach, size = (C.c_int64 * 3)(), (C.c_int64 * 3)()
+        ok = int(library().deepj_hip_q8_gemm_f16_extents(m, k, rows, tile_rows, tile_cols, reach, size))
+        return ok, list(reach), list(size)
 
     @staticmethod
     def q8GemmPath(m: int, k: int, rows: int) -> int:

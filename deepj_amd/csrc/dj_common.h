@@ -130,6 +130,9 @@ int64_t q8_linear_preferred_workspace_floats(int m, int k, int n, int flags, boo
 bool q8_gemm_f16_shape_ok(int m, int n_rows, int k);
 int q8_gemm_f16_tile_rows(int m, int n_rows, int k);   // 128 or 64 rows per workgroup tile, 0: not for these kernels
 void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares);
+// bytes the direct loads of a launch with this tile reach in {planes, fp16 weights, transposed scales} and bytes those
+// hold; false when any load would pass its buffer
+bool q8_gemm_f16_extents(int m, int n_rows, int k, int tile_rows, int tile_cols, int64_t reach[3], int64_t size[3]);
 void q8_gemm_f16_configure();   // once per device, before the first launch
 int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared);
 // floats of the weights in that kernel's layout: fp16 [rows up to a multiple of 256][Kp + 64], then the scales as

@@ -474,8 +474,9 @@ __global__ void __launch_bounds__(256) k_sum_partials(const float *__restrict__ 
 // and unfused multiply-adds as the stand-alone kernels), the largest magnitude of the result, then the two fp16 planes
 // of it times 2^s.  Rows of up to 8192 floats stay in registers in between; longer or ragged ones are read three or four
 // times, from L2 after the first.  Columns [k, kp) are written as zeros
-// (the weights' padding is zero as well, but 0 x garbage could be a NaN); rows [m, m_pad) are left alone: they only
-// feed output rows that are never stored.
+// (the weights' padding is zero as well, but 0 x garbage could be a NaN).  The grid covers the rows the GEMM's tiles
+// read, which may go past m: those rows only feed output rows that are never stored, and are written as zeros so that
+// the GEMM never multiplies what an earlier user of the workspace left there.
 template <int NORM>
 __global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
                                                    uint16_t *__restrict__ planes, float *__restrict__ unscale, int m, int k, int kp, int pitch,
@@ -483,6 +484,12 @@ __global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, 
 #pragma clang fp contract(off)
     __shared__ float red[4];
     const int row = blockIdx.x, t = threadIdx.x;
+    if (row >= m) {
+        uint32_t *hi32 = reinterpret_cast<uint32_t *>(planes + (int64_t)row * pitch), *lo32 = hi32 + plane_elems / 2;
+        for (int c = t; c < kp / 2; c += 256) { hi32[c] = 0u; lo32[c] = 0u; }
+        if (t == 0) unscale[row] = 0.f;
+        return;
+    }
     const float *xr = x + (int64_t)row * k;
     auto block_reduce = [&](float v, bool is_max) {
 #pragma unroll
@@ -599,13 +606,19 @@ __global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, 
     }
 }
 
-// int8 weights [rows x kp] -> fp16 [rows x pitch] (8 per thread), scales [rows x groups] -> [groups x n_pad]
+// int8 weights [rows x kp] -> fp16 [rows x pitch] (8 per thread), scales [rows x groups] -> [groups x n_pad]; rows
+// [rows, rows_read) - what a last column tile of either width reads past the weight - become zeros
 __global__ void __launch_bounds__(256) k_q8_to_f16(const int8_t *__restrict__ wq, const float *__restrict__ scales, uint16_t *__restrict__ w16,
-                                                   float *__restrict__ scales_t, int rows, int kp, int pitch, int n_pad) {
+                                                   float *__restrict__ scales_t, int rows, int rows_read, int kp, int pitch, int n_pad) {
     const int chunks = kp >> 3;
-    const int64_t total = (int64_t)rows * chunks;
+    const int64_t total = (int64_t)rows_read * chunks;
     for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
         const int row = (int)(idx / chunks), c = (int)(idx % chunks);
+        if (row >= rows) {                                   // rows the last column tile reads past the weight: zeros
+            *reinterpret_cast<uint4 *>(w16 + (int64_t)row * pitch + c * 8) = make_uint4(0u, 0u, 0u, 0u);
+            if ((c & 3) == 0) scales_t[(int64_t)(c >> 2) * n_pad + row] = 0.f;
+            continue;
+        }
         const int2 q = *reinterpret_cast<const int2 *>(wq + (int64_t)row * kp + c * 8);
         uint32_t o[4];
 #pragma unroll
@@ -670,6 +683,9 @@ void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, 
     if (k_shares) *k_shares = p.splits;
 }
 
+// weight rows a column tile of either width (256 or 192) may read: the prepared buffer holds zeros from n_rows up to here
+static int q8_prepared_rows_read(int n_rows) { return (int)std::max(round_up(n_rows, 256), round_up(n_rows, 192)); }
+
 // the weights in this kernel's layout: fp16 rows, then the transposed scales (each part 256-byte aligned)
 int64_t q8_prepared_floats(int k, int n_rows) {
     const int64_t kp = q8_padded_k(k), pitch = kp + 64, n_pad = round_up(n_rows, kNPad);
@@ -684,13 +700,34 @@ int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared) {
            (splits > 1 ? round_up((int64_t)splits * m * n_rows, 64) : 0);
 }
 
+// What the direct global -> LDS loads of one launch reach, against what the buffers hold, in bytes from the start of
+// the planes, of the fp16 weights and of the transposed scales.  A lane's load is 16 bytes (4 for a scale) at
+// base + lane offset + step * 64: the last one of the activations is plane 1, the last row of the last row tile, the
+// last K step; of the weights the last row of the last column tile; of the scales the 256 floats that the four
+// wavefronts fetch from the last column tile's first row on (with 192-column tiles the last 64 of them lie past the
+// tile, are fetched and never read).  Loads past a workgroup's last step are clamped to it, so the last step bounds
+// every address.  Pure host arithmetic: a CPU test runs it over the shape space, and every launch checks it.
+bool q8_gemm_f16_extents(int m, int n_rows, int k, int tile_rows, int tile_cols, int64_t reach[3], int64_t size[3]) {
+    const int64_t kp = q8_padded_k(k), pitch = kp + 64, m_pad = round_up(m, TM), n_pad = round_up(n_rows, kNPad), steps = kp / 32;
+    const int64_t m_read = round_up(m, tile_rows), n_read = round_up(n_rows, tile_cols);
+    reach[0] = 2 * (m_pad * pitch + (m_read - 1) * pitch + kp);
+    size[0] = 2 * 2 * m_pad * pitch;
+    reach[1] = 2 * ((n_read - 1) * pitch + kp);
+    size[1] = 2 * std::min<int64_t>(n_pad, q8_prepared_rows_read(n_rows)) * pitch;      // the rows that hold weights or zeros
+    reach[2] = 4 * ((steps - 1) * n_pad + (n_read - tile_cols) + 256);
+    size[2] = 4 * (round_up(steps * n_pad, 64) + 64);
+    return m_read <= m_pad && reach[0] <= size[0] && reach[1] <= size[1] && reach[2] <= size[2];
+}
+
 void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, float *prepared, int k, int n_rows) {
     if (k <= 0 || n_rows <= 0) return;
     const int kp = q8_padded_k(k), pitch = kp + 64, n_pad = (int)round_up(n_rows, kNPad);
     uint16_t *w16 = reinterpret_cast<uint16_t *>(prepared);
     float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
-    const int64_t items = (int64_t)n_rows * (kp / 8);
-    launch_kernel(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, kp, pitch, n_pad);
+    const int rows_read = q8_prepared_rows_read(n_rows);
+    if (rows_read > n_pad) fail("q8_prepare: the column tiles reach past the padded rows");
+    const int64_t items = (int64_t)rows_read * (kp / 8);
+    launch_kernel(k_q8_to_f16, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 8192)), dim3(256), 0, s, wq, scales, w16, scales_t, n_rows, rows_read, kp, pitch, n_pad);
 }
 
 // The kernels' LDS (three stages) is above the 64 KB a kernel gets without asking; called once per device at start-up
@@ -708,19 +745,22 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
     const int kp = q8_padded_k(k), pitch = kp + 64, m_pad = (int)round_up(m, TM), n_pad = (int)round_up(n_rows, kNPad);
+    const GemmF16Plan plan = q8_gemm_f16_plan(m, n_rows, k);
+    int64_t reach[3], size[3];
+    if (!q8_gemm_f16_extents(m, n_rows, k, plan.tile_rows, plan.tile_cols, reach, size)) fail("q8_gemm_f16: a tile's loads would reach past its buffer");
+    const int m_read = (int)round_up(m, plan.tile_rows);                // rows the row tiles read: [m, m_read) are zeros
     float *w = workspace;
     uint16_t *planes = reinterpret_cast<uint16_t *>(w); w += round_up((int64_t)m_pad * pitch, 64);
     float *unscale = w;                                  w += round_up(m_pad, 64);
     // gamma alone: RMSNorm of the rows first; gamma and beta: LayerNorm
     auto split = !gamma ? k_split_f16<0> : beta ? k_split_f16<2> : k_split_f16<1>;
     // (the helpers are ordinary launches: per-kernel timing of this op, launch_kernel's business, is the GEMM's)
-    launch_kernel(split, dim3(m), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
+    launch_kernel(split, dim3(m_read), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
     if (!prepared) {
         launch_q8_prepare(s, wq, scales, w, k, n_rows);
         prepared = w;
         w += q8_prepared_floats(k, n_rows);
     }
-    const GemmF16Plan plan = q8_gemm_f16_plan(m, n_rows, k);
     if (plan.splits > 1 && swiglu) fail("q8_gemm_f16: no SwiGLU epilogue on partial products");
     const uint16_t *w16 = reinterpret_cast<const uint16_t *>(prepared);
     const float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);

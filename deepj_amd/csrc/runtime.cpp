@@ -1021,6 +1021,14 @@ void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_ro
     if (k_shares) *k_shares = ks;
 }
 
+int32_t deepj_hip_q8_gemm_f16_extents(int32_t m, int32_t k, int32_t rows, int32_t tile_rows, int32_t tile_cols, int64_t *reach3, int64_t *size3) {
+    if (m <= 1 || k <= 0 || rows <= 0 || !reach3 || !size3) return -1;
+    int tr = tile_rows, tc = tile_cols;
+    if (tr == 0) q8_gemm_f16_tile(m, rows, k, &tr, &tc, nullptr);
+    if (!((tr == 128 && tc == 256) || (tr == 64 && (tc == 256 || tc == 192)))) return -1;
+    return q8_gemm_f16_extents(m, rows, k, tr, tc, reach3, size3) ? 1 : 0;
+}
+
 int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms_total) {
     return guarded([&] {
         ensure_init();

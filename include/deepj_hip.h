@@ -192,8 +192,9 @@ enum {
      *     its own) as fp16 rows plus scales transposed to [group][row], the layout the many-row GEMM loads straight
      *     into LDS, and lets `prepared` stand for `weight` in later Q8_LINEARs with M > 1 (they otherwise convert the
      *     weights into the workspace on every call).  The association ends when either buffer is released, uploaded
-     *     to, or the destination of Q8_QUANTIZE / COPY / FILL; a graph captured before that keeps the copy it was
-     *     captured with.  Results are the same with and without it.
+     *     to, or the destination of Q8_QUANTIZE / COPY / FILL - the ways Q8 data gets into a buffer; an op that writes
+     *     floats over a Q8 weight (which no longer is one then) does not end it.  A graph captured before that keeps the
+     *     copy it was captured with.  Results are the same with and without it.
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
@@ -223,6 +224,12 @@ int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows);
 int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);
 /* the same with the tile's columns (256 or 192) and the number of workgroups that share a tile's K (1: none) */
 void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares);
+/* Host arithmetic only (no GPU call): the last byte + 1 that the fp16 GEMM's direct global -> LDS loads reach in its three
+ * operand buffers {activation planes, fp16 weights, transposed scales} for a tile of tile_rows x tile_cols (128 x 256,
+ * 64 x 256 or 64 x 192; tile_rows 0: the tile the library would choose), and the bytes those buffers hold.  Returns 1
+ * when every load stays inside, 0 when one does not (a launch then fails instead of running), -1 when the shape is not
+ * one of these kernels'.  Every launch runs the same check. */
+int32_t deepj_hip_q8_gemm_f16_extents(int32_t m, int32_t k, int32_t rows, int32_t tile_rows, int32_t tile_cols, int64_t *reach3, int64_t *size3);
 
 /* ── host side: java.util.Random twin ─────────────────────────────────────
  * Tensor.random(rows, cols, Random) of the reference (J/tensor/cpu/CpuBackend.java:148-152)

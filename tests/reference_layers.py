@@ -1,4 +1,4 @@
-"""The drop-in path as a model: Python twins of the reference's layer COMPOSITIONS, written over Tensor exactly as
+"""Test scaffolding, not part of the library: the drop-in path as a model - Python twins of the reference's layer COMPOSITIONS, written over Tensor exactly as
 the Java classes are, so that with Tensor.setBackend(HipBackend()) a whole LlamaModel forward runs through the 42
 primitive opcodes, the lazy ComputeGraph and the five GpuRuntime calls - the way an unmodified DeepJ model would.
 
@@ -18,8 +18,8 @@ import math
 
 import numpy as np
 
-from .models import JavaRandom, LlamaConfig
-from .tensor import Tensor
+from deepj_amd.models import JavaRandom, LlamaConfig
+from deepj_amd.tensor import Tensor
 
 
 class Parameter:

@@ -1,4 +1,4 @@
-"""The drop-in path as a whole model: the reference's layer compositions (deepj_amd/dropin.py, twins of LlamaModel,
+"""The drop-in path as a whole model: the reference's layer compositions (tests/reference_layers.py, twins of LlamaModel,
 LlamaTransformerBlock, RoPEMultiHeadSelfAttention, HeadOps, RotaryEmbedding, RMSNorm1D, SwiGLULayer, Linear,
 Embedding, TextGenerator) over Tensor + HipBackend: every tensor op is one of the 42 primitive opcodes recorded by the
 lazy ComputeGraph and executed through the five GpuRuntime calls of the C ABI, with the reference's host loops
@@ -11,7 +11,8 @@ baseline's tiny Llama (vocab 256, dModel 256, 4 layers, 8 heads, dFF 688, maxSeq
 import numpy as np
 import pytest
 
-from deepj_amd import HipBackend, HipGpuRuntime, LlamaConfig, Tensor, dropin
+import reference_layers as dropin
+from deepj_amd import HipBackend, HipGpuRuntime, LlamaConfig, Tensor
 from oracle import cpu_ref as ref
 
 pytestmark = pytest.mark.gpu
