@@ -446,23 +446,37 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     store_tile_row<TNW>(a, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
 }
 
-// out = epilogue(sum over the splits of partial[z]) on float4s: bias, GELU, residual as in store_tile_row (a fixed order
-// of additions, so a run repeats bit for bit - which adding into C with atomics would not)
+// out = epilogue(sum over the splits of partial[z]) on float4s: bias, GELU, residual or the SwiGLU pairing as in
+// store_tile_row (a fixed order of additions, so a run repeats bit for bit - which adding into C with atomics would not)
 __global__ void __launch_bounds__(256) k_sum_partials(const float *__restrict__ partial, float *__restrict__ out, int splits, int64_t mn4, int n4,
-                                                     const float *__restrict__ bias, const float *__restrict__ residual, int gelu) {
+                                                     const GemmEpilogue ep) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < mn4; i += (int64_t)gridDim.x * 256) {
         float4 v = reinterpret_cast<const float4 *>(partial)[i];
         for (int z = 1; z < splits; z++) {
             const float4 p = reinterpret_cast<const float4 *>(partial)[(int64_t)z * mn4 + i];
             v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
         }
-        if (bias) {
-            const float4 b = reinterpret_cast<const float4 *>(bias)[i % n4];
+        const int c4 = (int)(i % n4);                                   // this float4's place in its row
+        if (ep.bias) {
+            float4 b;
+            if (ep.interleaved_bias) {                                  // even column n: bias[n / 2], odd: bias2[n / 2]
+                const float2 be = reinterpret_cast<const float2 *>(ep.bias)[c4], bo = reinterpret_cast<const float2 *>(ep.bias2)[c4];
+                b = make_float4(be.x, bo.x, be.y, bo.y);
+            } else {
+                b = reinterpret_cast<const float4 *>(ep.bias)[c4];
+            }
             v.x = v.x + b.x; v.y = v.y + b.y; v.z = v.z + b.z; v.w = v.w + b.w;
         }
-        if (gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
-        if (residual) {
-            const float4 r = reinterpret_cast<const float4 *>(residual)[i];
+        if (ep.swiglu) {                                                // (gate, up) pairs in neighbouring columns
+            float2 o;
+            o.x = v.x * (1.0f / (1.0f + expf(-v.x))) * v.y;
+            o.y = v.z * (1.0f / (1.0f + expf(-v.z))) * v.w;
+            reinterpret_cast<float2 *>(out)[i] = o;                     // row * (n / 2) + col / 2 = 2 i floats in
+            continue;
+        }
+        if (ep.gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
+        if (ep.residual) {
+            const float4 r = reinterpret_cast<const float4 *>(ep.residual)[i];
             v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
         }
         reinterpret_cast<float4 *>(out)[i] = v;
@@ -761,7 +775,6 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
         prepared = w;
         w += q8_prepared_floats(k, n_rows);
     }
-    if (plan.splits > 1 && swiglu) fail("q8_gemm_f16: no SwiGLU epilogue on partial products");
     const uint16_t *w16 = reinterpret_cast<const uint16_t *>(prepared);
     const float *scales_t = prepared + round_up((int64_t)n_pad * pitch / 2, 64);
     const int split_steps = plan.splits > 1 ? (kp / 32 + plan.splits - 1) / plan.splits : 0;
@@ -775,7 +788,7 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
         if (plan.splits > 1) {
             const int64_t mn4 = (int64_t)m * n_rows / 4;
             launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
-                               mn4, n_rows / 4, bias, residual, gelu);
+                               mn4, n_rows / 4, a.ep);
         }
     } else
         launch_kernel(k_gemm_q8_f16, dim3(grid_x), dim3(256), (size_t)kStages * kStage, s, a);

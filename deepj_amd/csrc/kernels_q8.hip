@@ -10,12 +10,16 @@
 //
 // Decode (M = 1): every weight byte is read from HBM exactly once.  One
 // wavefront owns an output row at a time; its 64 lanes read the row with 128-bit
-// loads (1 KiB per wave-load, fully coalesced), convert int8 -> fp32 in registers,
-// multiply with the activation slice the lane keeps in VGPRs for the whole kernel,
-// and reduce across the wavefront with DPP row operations.  The activation vector is staged
-// once per workgroup through LDS, where the optional prologue is applied (RMSNorm,
-// LayerNorm, or the merge of the decode attention's per-split records), so norm +
-// projection (+ bias, + GELU, + residual, or the SwiGLU gate) is one launch.
+// loads (1 KiB per wave-load, fully coalesced), multiply them with the activation
+// slice the lane keeps in VGPRs for the whole kernel, and reduce across the wavefront
+// with DPP row operations.  The activation vector is staged once per workgroup through
+// LDS, where the optional prologue is applied (RMSNorm, LayerNorm, or the merge of the
+// decode attention's per-split records), so norm + projection (+ bias, + GELU,
+// + residual, or the SwiGLU gate) is one launch.  The staged form is three planes of
+// signed bytes per value (a 23-bit integer times a power of two per 16 values, XSlice
+// below) that go into v_dot4_i32_i8 with the int8 weights as they are: the work left
+// behind the last weight bytes to arrive is 19 instead of 33 instructions per 16 weights
+// (decode 2430 -> 2448 tokens/s), at an error of 2^-23 of a slice's largest value.
 // M > 1 goes to the MFMA GEMM in kernels_matmul.hip.
 #include <cstdlib>
 #include <type_traits>
@@ -168,8 +172,33 @@ __device__ __forceinline__ void load_batch(RowBatch<NC, R> &b, const MatvecArgs 
     }
 }
 
-template <int NC, int B, bool SWIGLU, bool GELU>
-__device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 : 1)> &b, const float (&xr)[NC][16],
+// The activations of a lane's slice (16 consecutive k of each 1 KiB chunk) in the form the inner product wants.
+// DIGITS: each value is t * 2^-shift of its slice with an integer |t| <= 2^22, held as three signed bytes
+// t = d0 + 256 d1 + 65536 d2 (d0, d1 in [-128, 127], |d2| <= 64): one dword per four values and digit, so that
+// v_dot4_i32_i8 multiplies four int8 weights by four digits at a time - 12 integer instructions per 16 weights and
+// digit set, against 16 conversions and 16 multiply-adds on floats.  The integer sums are exact; they are put
+// together in fp32 (k[0..2] = 2^-shift x {1, 256, 65536}).  A value is off by at most 2^-23 of its slice's largest.
+template <int NC, bool DIGITS> struct XSlice;
+template <int NC> struct XSlice<NC, false> { float f[NC][16]; };
+template <int NC> struct XSlice<NC, true> { int d[NC][12]; float k[NC][3]; };
+
+template <int NC>
+__device__ __forceinline__ float dot_slice(const int4 &w, const XSlice<NC, false> &x, int c) { return dot16(w, x.f[c]); }
+template <int NC>
+__device__ __forceinline__ float dot_slice(const int4 &w, const XSlice<NC, true> &x, int c) {
+    const int wd[4] = {w.x, w.y, w.z, w.w};
+    int a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        a0 = __builtin_amdgcn_sdot4(wd[i], x.d[c][i], a0, false);
+        a1 = __builtin_amdgcn_sdot4(wd[i], x.d[c][4 + i], a1, false);
+        a2 = __builtin_amdgcn_sdot4(wd[i], x.d[c][8 + i], a2, false);
+    }
+    return fmaf((float)a2, x.k[c][2], fmaf((float)a1, x.k[c][1], (float)a0 * x.k[c][0]));
+}
+
+template <int NC, int B, bool SWIGLU, bool GELU, bool DIGITS>
+__device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 : 1)> &b, const XSlice<NC, DIGITS> &xr,
                                              const MatvecArgs &p, int o0, int o_end, int lane, float rms) {
     constexpr int R = B * (SWIGLU ? 2 : 1);
     float acc[R];
@@ -177,7 +206,7 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
     for (int u = 0; u < R; u++) {
         float a = 0.0f;
 #pragma unroll
-        for (int c = 0; c < NC; c++) a = fmaf(dot16(b.w[u][c], xr[c]), b.sc[u][c], a);
+        for (int c = 0; c < NC; c++) a = fmaf(dot_slice<NC>(b.w[u][c], xr, c), b.sc[u][c], a);
         acc[u] = wave_sum_dpp(a) / rms;        // rms = 1 unless the RMSNorm scale was deferred to here
     }
     float eb[B], eb2[B], er[B];
@@ -211,18 +240,61 @@ __device__ __forceinline__ void finish_batch(const RowBatch<NC, B *(SWIGLU ? 2 :
     }
 }
 
-// LDS layout of the staged activation row.  A lane multiplies the 16 consecutive activations of "its" 16-byte
-// weight chunk (chunk = 64 * c + lane) and reads them as four 128-bit words; stored in order, consecutive lanes
-// would be 64 bytes apart and four of every sixteen lanes would hit the same banks on every read.  So the row is
-// kept as planes: plane 4 * c + q holds the q-th word of every lane's slice of chunk row c, lane after lane
-// (conflict free to read), and a plane is padded by 16 floats so that the staging writes - consecutive threads
-// write the four words of one slice, i.e. to four planes - spread over the banks as well.
+// LDS layout of the staged activation row, float form (rows whose length is not a multiple of 4).  A lane multiplies
+// the 16 consecutive activations of "its" 16-byte weight chunk (chunk = 64 * c + lane) and reads them as four 128-bit
+// words; stored in order, consecutive lanes would be 64 bytes apart and four of every sixteen lanes would hit the
+// same banks on every read.  So the row is kept as planes: plane 4 * c + q holds the q-th word of every lane's slice
+// of chunk row c, lane after lane (conflict free to read), and a plane is padded by 16 floats so that the staging
+// writes - consecutive threads write the four words of one slice, i.e. to four planes - spread over the banks as well.
 constexpr int kXsPlane = 64 * 4 + 16;                              // floats per plane
 __host__ __device__ inline int xs_floats(int kp) { return ((kp + 1023) / 1024) * 4 * kXsPlane; }
 // offset of activation e (any e < Kp rounded up to 1024)
 __device__ __forceinline__ int xs_at(int e) {
     const int chunk = e >> 4, q = (e >> 2) & 3;
     return ((chunk >> 6) * 4 + q) * kXsPlane + (chunk & 63) * 4 + (e & 3);
+}
+
+// Digit form (XSlice<NC, true>), in the same LDS bytes: for chunk row c three planes of 256 dwords - plane
+// 3 * c + digit holds, for slice l of the row (the one lane l multiplies), the four dwords of that digit at
+// [4 l, 4 l + 4) - and behind all planes one shift per slice.  Thread t of the workgroup holds values
+// 4 t .. 4 t + 3 of chunk row c, i.e. the dword t of each of its planes: writes and reads are both lane-consecutive.
+// The four threads of a quad hold one slice; its shift puts the largest magnitude of the slice in [2^21, 2^22).
+__device__ __forceinline__ int xd_plane(int c, int digit) { return (c * 3 + digit) * 256; }
+template <int NC> __device__ __forceinline__ int xd_shift(int c) { return NC * 768 + c * 64; }
+static_assert(768 + 64 <= 4 * kXsPlane, "the digit form fits in the float form's bytes");
+
+__device__ __forceinline__ void stage_digits(float *xs, int plane0, int shift_at, int tid, float4 v) {
+    // largest magnitude of the quad's 16 values, as bit patterns: an infinity or a NaN compares above every number
+    uint32_t m = max(max(__float_as_uint(v.x) & 0x7fffffffu, __float_as_uint(v.y) & 0x7fffffffu),
+                     max(__float_as_uint(v.z) & 0x7fffffffu, __float_as_uint(v.w) & 0x7fffffffu));
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, false));      // quad_perm [1,0,3,2]
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, false));      // quad_perm [2,3,0,1]
+    // m = f * 2^e, f in [0.5, 1): values times 2^(22 - e) are below 2^22 in magnitude.  The shift stays where
+    // 2^shift and 2^-shift are normal numbers (slices below 2^-98 keep fewer digits, of values that small).
+    const int e = __builtin_amdgcn_frexp_expf(__uint_as_float(m));
+    const int shift = min(22 - e, 120);
+    const float up = ldexpf(1.0f, shift);
+    // v * 2^shift + 1.5 * 2^23 rounds to an integer (to nearest even) and leaves it, as C + t with C = 0x4B400000,
+    // in the bits of the sum.  t = b0 + 256 t1 with b0 the signed low byte means t1 = (t + 128) >> 8, and the same
+    // once more for t1: the three digits are byte 0 of t, byte 1 of t + 128 and byte 2 of t + 128 + 32768 - and C
+    // has no bits in its two low bytes, so only the last needs C taken off.
+    const float magic = 12582912.0f;
+    const uint32_t b[4] = {__float_as_uint(fmaf(v.x, up, magic)), __float_as_uint(fmaf(v.y, up, magic)),
+                           __float_as_uint(fmaf(v.z, up, magic)), __float_as_uint(fmaf(v.w, up, magic))};
+    uint32_t u[4], w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { u[i] = b[i] + 128u; w[i] = b[i] + (32896u - 0x400000u); }
+    // __builtin_amdgcn_perm(hi, lo, sel): result byte i is byte sel_i of the eight bytes {lo: 0-3, hi: 4-7}
+    const uint32_t d0 = __builtin_amdgcn_perm(__builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu), __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u), 0x07060100u);
+    const uint32_t d1 = __builtin_amdgcn_perm(__builtin_amdgcn_perm(u[3], u[2], 0x05010c0cu), __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0501u), 0x07060100u);
+    const uint32_t d2 = __builtin_amdgcn_perm(__builtin_amdgcn_perm(w[3], w[2], 0x06020c0cu), __builtin_amdgcn_perm(w[1], w[0], 0x0c0c0602u), 0x07060100u);
+    uint32_t *xd = reinterpret_cast<uint32_t *>(xs);
+    xd[plane0 + tid] = d0;
+    xd[plane0 + 256 + tid] = d1;
+    xd[plane0 + 512 + tid] = d2;
+    // a slice with an infinity or a NaN in it: the sums of this slice become NaN (the float form would give NaN or
+    // an infinity there)
+    if ((tid & 3) == 0) xs[shift_at + (tid >> 2)] = m >= 0x7f800000u ? __uint_as_float(0x7fc00000u) : ldexpf(1.0f, -shift);
 }
 
 // NC: 1 KiB chunks of one row a lane visits (ceil(Kp/1024)); B: outputs per batch.
@@ -387,7 +459,8 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
             float4 y;
             y.x = (xv[j].x / sd) * gv[j].x + bv[j].x; y.y = (xv[j].y / sd) * gv[j].y + bv[j].y;
             y.z = (xv[j].z / sd) * gv[j].z + bv[j].z; y.w = (xv[j].w / sd) * gv[j].w + bv[j].w;
-            if (e < p.kp) *reinterpret_cast<float4 *>(xs + xs_at(e)) = y;      // e >= k: x, gamma and beta are all zero
+            (void)e;
+            stage_digits(xs, xd_plane(j, 0), xd_shift<NC>(j), tid, y);         // e >= k: x, gamma and beta are all zero
         }
     } else if (vec) {
         if (PRO == 1) {
@@ -407,10 +480,7 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
             }
         }
 #pragma unroll
-        for (int j = 0; j < NC; j++) {
-            int e = (tid + kThreads * j) * 4;
-            if (e < p.kp) *reinterpret_cast<float4 *>(xs + xs_at(e)) = xv[j];
-        }
+        for (int j = 0; j < NC; j++) stage_digits(xs, xd_plane(j, 0), xd_shift<NC>(j), tid, xv[j]);
     } else {
         float ss = 0.0f;
         for (int i = tid; i < p.kp; i += kThreads) {
@@ -452,26 +522,37 @@ k_q8_matvec(const float *a_x, const int8_t *a_wq, const float *a_scales, float *
     }
 
     // this lane's activation slice: 16 consecutive k of each 1 KiB chunk
-    float xr[NC][16];
+    XSlice<NC, VEC> xr;
 #pragma unroll
     for (int c = 0; c < NC; c++) {
-        int kb = (c * 64 + lane) * 16;
-        bool active = kb < p.kp;
+        if constexpr (VEC) {
+            const uint32_t *xd = reinterpret_cast<const uint32_t *>(xs);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float4 v = active ? *reinterpret_cast<const float4 *>(xs + (c * 4 + j) * kXsPlane + lane * 4) : make_float4(0, 0, 0, 0);
-            xr[c][4 * j] = v.x; xr[c][4 * j + 1] = v.y; xr[c][4 * j + 2] = v.z; xr[c][4 * j + 3] = v.w;
+            for (int g = 0; g < 3; g++) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(xd + xd_plane(c, g) + lane * 4);
+                xr.d[c][4 * g] = (int)v.x; xr.d[c][4 * g + 1] = (int)v.y; xr.d[c][4 * g + 2] = (int)v.z; xr.d[c][4 * g + 3] = (int)v.w;
+            }
+            const float unit = xs[xd_shift<NC>(c) + lane];
+            xr.k[c][0] = unit; xr.k[c][1] = unit * 256.0f; xr.k[c][2] = unit * 65536.0f;
+        } else {
+            int kb = (c * 64 + lane) * 16;
+            bool active = kb < p.kp;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float4 v = active ? *reinterpret_cast<const float4 *>(xs + (c * 4 + j) * kXsPlane + lane * 4) : make_float4(0, 0, 0, 0);
+                xr.f[c][4 * j] = v.x; xr.f[c][4 * j + 1] = v.y; xr.f[c][4 * j + 2] = v.z; xr.f[c][4 * j + 3] = v.w;
+            }
         }
     }
 
     DJ_STAMP(3);
     for (int o0 = o_begin; o0 < o_end; o0 += 2 * o_step) {
         if (o0 + o_step < o_end) { load_batch<NC, R>(bb, p, (o0 + o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(bb, p, o0 + o_step); }
-        finish_batch<NC, B, SWIGLU, GELU>(ba, xr, p, o0, o_end, lane, rms);
+        finish_batch<NC, B, SWIGLU, GELU, VEC>(ba, xr, p, o0, o_end, lane, rms);
         if (o0 == o_begin) DJ_STAMP(4);
         if (o0 + o_step >= o_end) break;
         if (o0 + 2 * o_step < o_end) { load_batch<NC, R>(ba, p, (o0 + 2 * o_step) * RPO, row_last, lane, groups); load_epilogue<NC, R, B, SWIGLU>(ba, p, o0 + 2 * o_step); }
-        finish_batch<NC, B, SWIGLU, GELU>(bb, xr, p, o0 + o_step, o_end, lane, rms);
+        finish_batch<NC, B, SWIGLU, GELU, VEC>(bb, xr, p, o0 + o_step, o_end, lane, rms);
     }
     DJ_STAMP(5);
 }

@@ -205,6 +205,32 @@ def test_swiglu_and_norm_prologues(dev, norm, dff, tile):
     assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"{norm}-norm prologue")
 
 
+def test_swiglu_on_partial_products_of_a_shared_k(dev):
+    """A few-tile gate/up projection over a long K runs as several workgroups per tile; the kernel that adds their
+    partial products applies the interleaved biases and the SwiGLU pairing (a DeepSeek block at 256 rows has this
+    shape)."""
+    m, d, dff = 256, 2048, 1024
+    assert HipNative.q8GemmTile(m, d, 2 * dff) == (64, 256, 4)
+    x = JavaRandom(51).tensor(m, d, 1.0)
+    gamma = (1.0 + JavaRandom(52).tensor(1, d, 0.1)).astype(np.float32)
+    wg, wu = JavaRandom(53).tensor(d, dff, 0.03), JavaRandom(54).tensor(d, dff, 0.03)
+    bg, bu = JavaRandom(55).tensor(1, dff, 0.2), JavaRandom(56).tensor(1, dff, 0.2)
+    h = ref.rmsnorm(x, gamma)
+    exp = ref.multiply(ref.silu(ref.add_row_vector(ref.matmul(h, ref.q8_roundtrip(wg)), bg)),
+                       ref.add_row_vector(ref.matmul(h, ref.q8_roundtrip(wu)), bu))
+    wgu = dev.alloc(HipNative.q8Floats(d, 2 * dff))
+    for w, off in ((wg, 0), (wu, 1)):
+        src = dev.upload(w)
+        Stream().q8_quantize(src, wgu, d, dff, off, 2, 2 * dff).run()
+        dev.release(src)
+    xb, gb, ob = dev.upload(x), dev.upload(gamma), dev.alloc(m * dff)
+    bgb, bub = dev.upload(bg), dev.upload(bu)
+    Stream().q8_linear(xb, wgu, ob, m, d, dff, gamma=gb, bias=bgb, bias2=bub, swiglu=True).run()
+    got = dev.download(ob, (m, dff))
+    dev.release(wgu, ob, xb, gb, bgb, bub)
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what="SwiGLU over shared K")
+
+
 def test_prepared_weights_give_the_same_bits_and_follow_the_weights(dev):
     m, k, n = 512, 512, 10240
     assert HipNative.q8GemmPath(m, k, n) == 128
