@@ -56,10 +56,7 @@ namespace {
 
 constexpr int TM = 128, TN = 256;
 constexpr int kXs = 2 * TM * 64;            // bytes of the two activation planes of one stage: [plane][row][32 k] fp16
-constexpr int kWl = TN * 64;                // bytes of the weights of one stage: [row][32 k] fp16
-constexpr int kStage = kXs + kWl + TN * 4;  // + one scale per weight row
 constexpr int kStages = 3;
-constexpr int kLoads = 9;                   // direct loads per wavefront per stage: 4 of X, 4 of W, 1 of scales
 
 struct GemmF16Args {
     const uint16_t *planes;     // [2][m_pad][pitch] fp16: hi plane, lo plane
@@ -152,20 +149,30 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                  // the rows are in registers before anything overwrites them
 }
 
+// TNW: 32-column MFMA tiles per wavefront along N - 4 (workgroup tile 128 x 256, the shape described at the top) or 3
+// (128 x 192: 512 rows against 11264 output rows are 176 tiles of the former on 256 compute units, 236 of the latter).
+// A K step is 2 TNW passes; the schedule below places the same kinds of work in both.
+constexpr int stage128_bytes(int tnw) { return kXs + 64 * tnw * 64 + 1024; }     // X planes, W rows, 256 scales
+
+template <int TNW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16(const GemmF16Args a) {
+    static_assert(TNW == 3 || TNW == 4, "the slots of the schedule are written out for these");
+    constexpr int kTn = 64 * TNW, kW = kTn * 64, kStageB = stage128_bytes(TNW);
+    constexpr int kPasses = 2 * TNW;
+    constexpr int kLoadsB = 5 + TNW;            // direct loads per wavefront per stage: 4 of X, TNW of W, 1 of scales
     extern __shared__ __align__(16) unsigned char lds[];
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
     int m_tile, n_tile;
     if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
-    const int m0 = m_tile * TM, n0 = n_tile * TN;
+    const int m0 = m_tile * TM, n0 = n_tile * kTn;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
-    float acc[2][4][16];
+    float acc[2][TNW][16];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < TNW; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
@@ -175,41 +182,46 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // offset is the same in every block; a block's origin is wave-uniform.
     const int prow = lane >> 2, pchunk = (lane & 3) ^ ((prow >> 2) & 3);
     const uint32_t op_lane = (uint32_t)((prow * a.pitch + pchunk * 8) * 2), s_lane = lane * 4;
-    const unsigned char *x_base[4], *w_base[4];
-    uint32_t x_dst[4], w_dst[4];
+    const unsigned char *x_base[4], *w_base[TNW];
+    uint32_t x_dst[4], w_dst[TNW];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int blk = wave * 4 + i, pl = blk >> 3, rb = blk & 7;      // X: 2 planes x 8 row blocks; W: 16 row blocks
+        const int blk = wave * 4 + i, pl = blk >> 3, rb = blk & 7;      // X: 2 planes x 8 row blocks
         x_base[i] = reinterpret_cast<const unsigned char *>(a.planes) + (pl * plane_elems + (int64_t)(m0 + rb * 16) * a.pitch) * 2;
         x_dst[i] = pl * TM * 64 + rb * 1024;
+    }
+#pragma unroll
+    for (int i = 0; i < TNW; i++) {
+        const int blk = wave * TNW + i;                                 // W: 4 TNW row blocks
         w_base[i] = reinterpret_cast<const unsigned char *>(a.w16) + (int64_t)(n0 + blk * 16) * a.pitch * 2;
         w_dst[i] = kXs + blk * 1024;
     }
+    // every wavefront fetches 64 scales; with TNW = 3 the last 64 belong to the next column tile and are never read
     const unsigned char *s_base = reinterpret_cast<const unsigned char *>(a.scales_t) + (int64_t)(n0 + wave * 64) * 4;
-    const uint32_t s_dst = kXs + kWl + wave * 256;
+    const uint32_t s_dst = kXs + kW + wave * 256;
     const int steps = a.kp / 32, last = steps - 1;
     auto load_one = [&](int i, int step, int stage) {
-        const uint32_t sb = lds0 + stage * kStage;
+        const uint32_t sb = lds0 + stage * kStageB;
         step = min(step, last);
         if (i < 4) load_to_lds16(x_base[i] + (int64_t)step * 64, op_lane, sb + x_dst[i]);
-        else if (i < 8) load_to_lds16(w_base[i - 4] + (int64_t)step * 64, op_lane, sb + w_dst[i - 4]);
+        else if (i < 4 + TNW) load_to_lds16(w_base[i - 4] + (int64_t)step * 64, op_lane, sb + w_dst[i - 4]);
         else load_to_lds4(s_base + (int64_t)step * a.n_pad * 4, s_lane, sb + s_dst);
     };
 
     // MFMA operand addresses: lane l32 + 32 * half reads row l32, K chunk 2 * sub + half of its tile
     const int sw = (l32 >> 2) & 3;
     const int lane_sub0 = (l32 << 6) + (((0 + half) ^ sw) << 4), lane_sub1 = (l32 << 6) + (((2 + half) ^ sw) << 4);
-    const int x_wave = wm * 64 * 64, w_wave = kXs + wn * 128 * 64, s_wave = kXs + kWl + wn * 128 * 4 + l32 * 4;
+    const int x_wave = wm * 64 * 64, w_wave = kXs + wn * (32 * TNW) * 64, s_wave = kXs + kW + wn * (32 * TNW) * 4 + l32 * 4;
     const floatx16 z16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     halfx8 fx[2][2][2];                 // [tile row][K half][hi, lo]
-    halfx8 fw[2][4];                    // [K half][tile column]
-    float sc[4];                        // [tile column]
+    halfx8 fw[2][TNW];                  // [K half][tile column]
+    float sc[TNW];                      // [tile column]
     floatx16 g[2] = {z16, z16};         // partial sums of the tile in flight and of the one being scaled
 #pragma unroll
-    for (int j = 0; j < 4; j++) sc[j] = 0.f;
+    for (int j = 0; j < TNW; j++) sc[j] = 0.f;
     struct Addr { const unsigned char *x0, *x1, *w0, *w1, *s; };
     auto addr_of = [&](int stage) {
-        const unsigned char *sb = lds + stage * kStage;
+        const unsigned char *sb = lds + stage * kStageB;
         return Addr{sb + x_wave + lane_sub0, sb + x_wave + lane_sub1, sb + w_wave + lane_sub0, sb + w_wave + lane_sub1, sb + s_wave};
     };
     auto read_x = [&](int tm, int q, const Addr &ad) {      // q = K half * 2 + piece
@@ -221,15 +233,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto k_step = [&](int step, int stage) {
         const int sy = stage == 2 ? 0 : stage + 1, sz = sy == 2 ? 0 : sy + 1;
         const Addr ax = addr_of(stage);
-        const int dy = (sy - stage) * kStage;
+        const int dy = (sy - stage) * kStageB;
         __builtin_amdgcn_s_barrier();                                  // every wavefront has left stage sz
         asm volatile("" ::: "memory");
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int tm = k >> 2, tn = k & 3, par = k & 1;
-            const int pk = (k + 7) & 7, ptm = pk >> 2, ptn = pk & 3;   // the tile finished by the previous pass
-            if (k == 4) {
-                asm volatile("s_waitcnt vmcnt(9)" ::: "memory");      // this wavefront's loads of step + 1 have landed ...
+        for (int k = 0; k < kPasses; k++) {
+            const int tm = k / TNW, tn = k % TNW, par = k & 1;
+            const int pk = (k + kPasses - 1) % kPasses, ptm = pk / TNW, ptn = pk % TNW;   // the tile finished by the previous pass
+            if (k == TNW) {
+                // this wavefront's loads of step + 1 have landed (all but the kLoadsB of step + 2 it has issued since) ...
+                if (TNW == 4) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
                 __builtin_amdgcn_s_barrier();                          // ... and so have everyone's
                 asm volatile("" ::: "memory");
             }
@@ -242,41 +256,52 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 const int f0 = i <= 1 ? 0 : i == 2 ? 6 : 11, f1 = i == 0 ? 0 : i == 1 ? 6 : i == 2 ? 11 : 16;
 #pragma unroll
                 for (int f = f0; f < f1; f++) acc[ptm][ptn][f] = fmaf(g[1 - par][f], sc[ptn], acc[ptm][ptn][f]);
-                // column 3 of this step (operands, scale) in pass 0; columns 0-2 of the next step as this step leaves them
-                if (k == 0 && i < 2) read_w(i, 3, ax);
-                if (k >= 5 && i < 2) read_w(i, k - 5, ay);
-                if (k == 0 && i == 3) sc[3] = *reinterpret_cast<const float *>(ax.s + 3 * 128);
-                if (k >= 5 && i == 3) sc[k - 5] = *reinterpret_cast<const float *>(ay.s + (k - 5) * 128);
-                // the second tile row of this step in passes 0-3, the first tile row of the next step in passes 4-7
-                if (k < 4 && i == 2) read_x(1, k, ax);
-                if (k >= 4 && i == 2) read_x(0, k - 4, ay);
-                // the loads of step + 2
-                if (k < 4 && (i == 1 || i == 3)) load_one(k * 2 + (i >> 1), step + 2, sz);
-                if (k == 3 && i == 0) load_one(8, step + 2, sz);
+                // the last column of this step (operands, scale) in pass 0 - its registers were in use until the end of the
+                // previous step; the other columns of the next step as this step leaves them, from pass TNW + 1 on
+                if (k == 0 && i < 2) read_w(i, TNW - 1, ax);
+                if (k >= TNW + 1 && i < 2) read_w(i, k - (TNW + 1), ay);
+                if (k == 0 && i == 3) sc[TNW - 1] = *reinterpret_cast<const float *>(ax.s + (TNW - 1) * 128);
+                if (k >= TNW + 1 && i == 3) sc[k - (TNW + 1)] = *reinterpret_cast<const float *>(ay.s + (k - (TNW + 1)) * 128);
+                // the four operand reads of this step's second tile row in its first half, of the next step's first
+                // tile row in its second half; the loads of step + 2 in the first half
+                if constexpr (TNW == 4) {
+                    if (k < 4 && i == 2) read_x(1, k, ax);
+                    if (k >= 4 && i == 2) read_x(0, k - 4, ay);
+                    if (k < 4 && (i == 1 || i == 3)) load_one(k * 2 + (i >> 1), step + 2, sz);
+                    if (k == 3 && i == 0) load_one(8, step + 2, sz);
+                } else {
+                    if (k < 3 && i == 2) read_x(1, k, ax);
+                    if (k == 2 && i == 0) read_x(1, 3, ax);
+                    if (k >= 3 && i == 2) read_x(0, k - 3, ay);
+                    if (k == 3 && i == 0) read_x(0, 3, ay);
+                    if (k < 3 && (i == 1 || i == 3)) load_one(k * 2 + (i >> 1), step + 2, sz);
+                    if (k == 1 && i == 0) load_one(6, step + 2, sz);
+                    if (k == 2 && i == 2) load_one(7, step + 2, sz);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
 
     for (int s = 0; s < 2; s++)
-        for (int i = 0; i < kLoads; i++) load_one(i, s, s);
+        for (int i = 0; i < kLoadsB; i++) load_one(i, s, s);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     {
         const Addr a0 = addr_of(0);
         for (int q = 0; q < 4; q++) read_x(0, q, a0);
-        for (int tn = 0; tn < 3; tn++) { read_w(0, tn, a0); read_w(1, tn, a0); }
-        for (int tn = 0; tn < 3; tn++) sc[tn] = *reinterpret_cast<const float *>(a0.s + tn * 128);
+        for (int tn = 0; tn < TNW - 1; tn++) { read_w(0, tn, a0); read_w(1, tn, a0); }
+        for (int tn = 0; tn < TNW - 1; tn++) sc[tn] = *reinterpret_cast<const float *>(a0.s + tn * 128);
     }
     int stage = 0;
     for (int step = 0; step < steps; step++) {
         k_step(step, stage);
         stage = stage == 2 ? 0 : stage + 1;
     }
-    // the last tile's scaling; its scale (column 3 of the last step) is still in place
+    // the last tile's scaling; its scale (the last column of the last step) is still in place
 #pragma unroll
-    for (int e = 0; e < 16; e++) acc[1][3][e] = fmaf(g[1][e], sc[3], acc[1][3][e]);
+    for (int e = 0; e < 16; e++) acc[1][TNW - 1][e] = fmaf(g[1][e], sc[TNW - 1], acc[1][TNW - 1][e]);
     // no direct load may still be writing LDS when the epilogue reuses it or the workgroup ends
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -284,7 +309,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) store_tile_row<4>(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * 128, lane);
+    for (int tm = 0; tm < 2; tm++) store_tile_row<TNW>(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * (32 * TNW), lane);
 }
 
 // The same product on a 64-row workgroup tile, 256 (TNW = 4) or 192 (TNW = 3) columns wide, for problems whose 128-row
@@ -656,25 +681,28 @@ struct GemmF16Plan { int tile_rows, tile_cols, splits; };
 constexpr int kNPad = 768;      // weight rows of a prepared buffer are padded to a multiple of both tile widths
 
 GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
-    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels; =128, =64 or =192 force the 128 x 256, 64 x 256 or
-    // 64 x 192 tile (for comparisons)
+    // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels; =128, =128192, =64 or =192 force the 128 x 256,
+    // 128 x 192, 64 x 256 or 64 x 192 tile (for comparisons)
     static const int forced = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return e ? atoi(e) : -1; }();
     if (forced == 0) return {0, 0, 1};
     // four columns per lane in the epilogue need n_rows % 4 == 0
     if (m < 256 || (n_rows & 3) != 0 || k < 64) return {0, 0, 1};
     const int64_t rows128 = (m + TM - 1) / TM, rows64 = (m + TM64 - 1) / TM64, cols256 = (n_rows + 255) / 256, cols192 = (n_rows + 191) / 192;
-    const int64_t t128 = rows128 * cols256, t64 = rows64 * cols256, t64n = rows64 * cols192;
-    if (forced == 128 || forced == 64 || forced == 192) {
+    const int64_t t128 = rows128 * cols256, t128n = rows128 * cols192, t64 = rows64 * cols256, t64n = rows64 * cols192;
+    if (forced == 128 || forced == 128192 || forced == 64 || forced == 192) {
         if (t64 < 128) return {0, 0, 1};
-        return forced == 128 ? GemmF16Plan{128, 256, 1} : forced == 64 ? GemmF16Plan{64, 256, 1} : GemmF16Plan{64, 192, 1};
+        return forced == 128 ? GemmF16Plan{128, 256, 1} : forced == 128192 ? GemmF16Plan{128, 192, 1} : forced == 64 ? GemmF16Plan{64, 256, 1} : GemmF16Plan{64, 192, 1};
     }
     // Enough tiles for several rounds: the large tile.  Around one round the time is rounds x one tile's time, and a
     // tile's time goes with its area over its efficiency (measured at 512 rows, K 2048: a 128 x 256 tile 58 us of K
-    // loop + 11 us of prologue and epilogue, 64 x 256 35 + 10, 64 x 192 27 + 9): take the cheapest.
+    // loop + 11 us of prologue and epilogue, 64 x 256 35 + 10, 64 x 192 27 + 9; a 128 x 192 tile takes almost as long as
+    // a 128 x 256 one - 236 of them 66.2 us where 176 of those take 67.6 - so it only wins where it saves a round or
+    // fills idle compute units): take the cheapest.
     if (t128 >= 512) return {128, 256, 1};
     auto rounds = [](int64_t tiles) { return (tiles + 255) / 256; };
-    const double c128 = rounds(t128) * 1.00, c64 = rounds(t64) * 0.65, c64n = rounds(t64n) * 0.52;
+    const double c128 = rounds(t128) * 1.00, c128n = rounds(t128n) * 0.98, c64 = rounds(t64) * 0.65, c64n = rounds(t64n) * 0.52;
     if (t64 >= 128) {
+        if (t128n >= 160 && c128n < c128 && c128n < c64 && c128n < c64n) return {128, 192, 1};
         if (t128 >= 160 && c128 <= c64 && c128 <= c64n) return {128, 256, 1};
         return c64n < c64 ? GemmF16Plan{64, 192, 1} : GemmF16Plan{64, 256, 1};
     }
@@ -747,7 +775,8 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
 // The kernels' LDS (three stages) is above the 64 KB a kernel gets without asking; called once per device at start-up
 // (not at the first launch, which may sit inside a graph capture).
 void q8_gemm_f16_configure() {
-    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * kStage), "hipFuncSetAttribute(k_gemm_q8_f16)");
+    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage128_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16<4>)");
+    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage128_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16<3>)");
     hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4>)");
     hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3>)");
 }
@@ -790,8 +819,10 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
             launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
                                mn4, n_rows / 4, a.ep);
         }
-    } else
-        launch_kernel(k_gemm_q8_f16, dim3(grid_x), dim3(256), (size_t)kStages * kStage, s, a);
+    } else if (plan.tile_cols == 192)
+        launch_kernel(k_gemm_q8_f16<3>, dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(3), s, a);
+    else
+        launch_kernel(k_gemm_q8_f16<4>, dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(4), s, a);
 }
 
 }  // namespace dj

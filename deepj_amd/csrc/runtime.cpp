@@ -1025,7 +1025,7 @@ int32_t deepj_hip_q8_gemm_f16_extents(int32_t m, int32_t k, int32_t rows, int32_
     if (m <= 1 || k <= 0 || rows <= 0 || !reach3 || !size3) return -1;
     int tr = tile_rows, tc = tile_cols;
     if (tr == 0) q8_gemm_f16_tile(m, rows, k, &tr, &tc, nullptr);
-    if (!((tr == 128 && tc == 256) || (tr == 64 && (tc == 256 || tc == 192)))) return -1;
+    if (!((tr == 128 || tr == 64) && (tc == 256 || tc == 192))) return -1;
     return q8_gemm_f16_extents(m, rows, k, tr, tc, reach3, size3) ? 1 : 0;
 }
 

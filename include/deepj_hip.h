@@ -225,8 +225,8 @@ int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);
 /* the same with the tile's columns (256 or 192) and the number of workgroups that share a tile's K (1: none) */
 void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares);
 /* Host arithmetic only (no GPU call): the last byte + 1 that the fp16 GEMM's direct global -> LDS loads reach in its three
- * operand buffers {activation planes, fp16 weights, transposed scales} for a tile of tile_rows x tile_cols (128 x 256,
- * 64 x 256 or 64 x 192; tile_rows 0: the tile the library would choose), and the bytes those buffers hold.  Returns 1
+ * operand buffers {activation planes, fp16 weights, transposed scales} for a tile of tile_rows x tile_cols (128 or 64 rows
+ * by 256 or 192 columns; tile_rows 0: the tile the library would choose), and the bytes those buffers hold.  Returns 1
  * when every load stays inside, 0 when one does not (a launch then fails instead of running), -1 when the shape is not
  * one of these kernels'.  Every launch runs the same check. */
 int32_t deepj_hip_q8_gemm_f16_extents(int32_t m, int32_t k, int32_t rows, int32_t tile_rows, int32_t tile_cols, int64_t *reach3, int64_t *size3);

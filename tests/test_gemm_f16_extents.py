@@ -12,7 +12,7 @@ import pytest
 
 from deepj_amd import HipNative
 
-TILES = [(128, 256), (64, 256), (64, 192)]
+TILES = [(128, 256), (128, 192), (64, 256), (64, 192)]
 
 
 def enumerate_reach(m, k, n, tile_rows, tile_cols):
@@ -80,5 +80,5 @@ def test_buffer_sizes_agree_with_the_prepared_weight_and_workspace_queries():
 def test_tiles_the_kernels_do_not_have_and_single_rows_are_not_answered():
     assert HipNative.q8GemmF16Extents(512, 2048, 2048, 64, 192)[0] == 1
     assert HipNative.q8GemmF16Extents(512, 2048, 2048, 96, 256)[0] == -1
-    assert HipNative.q8GemmF16Extents(512, 2048, 2048, 128, 192)[0] == -1
+    assert HipNative.q8GemmF16Extents(512, 2048, 2048, 128, 128)[0] == -1
     assert HipNative.q8GemmF16Extents(1, 2048, 2048)[0] == -1

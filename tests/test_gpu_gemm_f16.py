@@ -45,7 +45,7 @@ def gate(exp):
 
 
 def test_path_query_matches_the_documented_rule():
-    assert HipNative.q8GemmPath(512, 2048, 11264) == 128      # 4 x 44 tiles of 128 x 256
+    assert HipNative.q8GemmPath(512, 2048, 11264) == 128      # 4 x 59 tiles of 128 x 192 (4 x 44 of 128 x 256 leave 80 compute units idle)
     assert HipNative.q8GemmPath(2048, 4096, 4096) == 128      # 16 x 16
     assert HipNative.q8GemmPath(512, 2048, 6144) == 64        # 96 such tiles would idle most of the chip: 192 of 64 x 256
     assert HipNative.q8GemmPath(512, 2048, 2048) == 64        # 64 even of those: four workgroups share each tile's K
@@ -53,7 +53,8 @@ def test_path_query_matches_the_documented_rule():
     assert HipNative.q8GemmPath(512, 5632, 2048) == 64        # the same 64 tiles over a long K: four workgroups share each
     assert HipNative.q8GemmTile(512, 5632, 2048) == (64, 256, 4)
     assert HipNative.q8GemmTile(512, 2048, 6144) == (64, 192, 1)     # 256 tiles: one per compute unit
-    assert HipNative.q8GemmTile(512, 2048, 11264) == (128, 256, 1)
+    assert HipNative.q8GemmTile(512, 2048, 11264) == (128, 192, 1)
+    assert HipNative.q8GemmTile(2048, 4096, 12288) == (128, 256, 1)  # several rounds of tiles: the large one
     assert HipNative.q8GemmTile(8, 2048, 2048) == (0, 0, 1)
     assert HipNative.q8GemmPath(1, 2048, 32000) == 0          # the matvec's case
     assert HipNative.q8GemmPath(512, 2048, 11266) == 0        # four columns per lane in the epilogue
@@ -137,11 +138,12 @@ def test_rows_spanning_twelve_decades_with_outliers(dev):
     assert worst <= 1e-4
 
 
-@pytest.mark.parametrize("k,n,tile", [(256, 14336, 128), (256, 9216, 64), (4000, 2052, 64)])   # the last: K shared by four workgroups
+@pytest.mark.parametrize("k,n,tile", [(256, 16384, (128, 256, 1)), (256, 14336, (128, 192, 1)), (256, 9216, (64, 256, 1)),
+                                      (256, 7680, (64, 192, 1)), (4000, 2052, (64, 256, 4))])   # the last: K shared by four workgroups
 @pytest.mark.parametrize("epilogue", ["bias", "bias_gelu", "bias_residual", "residual"])
 def test_epilogues(dev, epilogue, k, n, tile):
     m = 384
-    assert HipNative.q8GemmPath(m, k, n) == tile
+    assert HipNative.q8GemmTile(m, k, n) == tile
     x = JavaRandom(31).tensor(m, k, 1.0)
     w = JavaRandom(32).tensor(k, n, 0.05)
     b = JavaRandom(33).tensor(1, n, 0.3)
