@@ -426,6 +426,70 @@ def calibration_copy(mib: int = 256, repeats: int = 3) -> None:
     dev.release_all()
 
 
+def clock_probe():
+    """The shader clock under the library's own kernels: a one-wavefront sampler on a second stream reads the shader
+    clock counter against the 100 MHz wall clock every few microseconds while a stream runs (deepj_hip_clock_probe).
+    Workloads: nothing (idle), a pure read of 1 GiB (STREAM_READ), the prompt's gate/up GEMM at 512 rows, a
+    2048 x 12288 x 4096 GEMM (prepared weights), and the empty kernel.  Reported: median / 10th / 90th percentile of the clock
+    over the sampling intervals that lie inside the stream's runs, and how long the runs took."""
+    from deepj_amd import HipNative
+    from deepj_amd.fused import DeviceBuffers, Stream
+    rng = np.random.default_rng(5)
+    dev = DeviceBuffers()
+    rows = []
+
+    def measure(name, stream, iters, samples):
+        if iters:
+            stream.run()
+            HipNative.synchronize()
+        mhz, t, win = HipNative.clockProbe(stream.array(), iters, samples, 1)
+        inside = mhz[(t > win[0] + 20.0) & (t < win[1] - 5.0)] if iters else mhz
+        if inside.size == 0:
+            inside = mhz
+        rows.append({"workload": name, "run_us": round(win[1] - win[0], 1) if iters else 0.0, "intervals": int(inside.size),
+                     "interval_us": round(float(np.median(np.diff(t))), 2),
+                     "clock_MHz_median": round(float(np.median(inside)), 0), "clock_MHz_p10": round(float(np.percentile(inside, 10)), 0),
+                     "clock_MHz_p90": round(float(np.percentile(inside, 90)), 0)})
+
+    measure("idle (sampler alone)", Stream().nop(1), 0, 400)
+    measure("empty kernels back to back", Stream().nop(768), 4000, 1500)
+    n = 1 << 28
+    big, sink = dev.alloc(n), dev.alloc(64)
+    Stream().fill(big, 0x3F800000, n).run()
+    measure("pure read of 1 GiB (STREAM_READ)", Stream().stream_read(big, sink, n), 24, 1500)
+    dev.release(big, sink)
+    k, nn = 2048, 5632                       # the decode matvec over a rotation of distinct weight copies (HBM-cold)
+    wf = dev.upload((rng.standard_normal((k, nn)) * 0.02).astype(np.float32))
+    q_floats = HipNative.q8Floats(k, nn)
+    qs = [dev.alloc(q_floats) for _ in range(40)]
+    Stream().q8_quantize(wf, qs[0], k, nn).run()
+    dup = Stream()
+    for q in qs[1:]:
+        dup.copy(qs[0], q, q_floats)
+    dup.run()
+    x, out = dev.upload(rng.standard_normal((1, k)).astype(np.float32)), dev.alloc(nn)
+    mv = Stream()
+    for q in qs:
+        mv.q8_linear(x, q, out, 1, k, nn)
+    measure("Q8 matvec 2048 x 5632, 40 distinct copies in turn", mv, 40, 1500)
+    dev.release(wf, x, out, *qs)
+    for m, k, nn, iters in ((512, 2048, 11264, 96), (2048, 4096, 12288, 14)):
+        x = dev.upload(rng.standard_normal((m, k)).astype(np.float32))
+        wf = dev.upload((rng.standard_normal((k, nn)) * 0.02).astype(np.float32))
+        wq = dev.alloc(HipNative.q8Floats(k, nn))
+        Stream().q8_quantize(wf, wq, k, nn).run()
+        dev.release(wf)
+        prep = dev.alloc(HipNative.q8PreparedFloats(k, nn))
+        Stream().q8_prepare(wq, prep, k, nn).run()
+        out = dev.alloc(m * nn)
+        tile = HipNative.q8GemmTile(m, k, nn)
+        measure(f"Q8 GEMM {m} x {nn} x {k} (fp16 x 2, {tile[0]} x {tile[1]} tiles)", Stream().q8_linear(x, wq, out, m, k, nn), iters, 2000)
+        dev.release(x, wq, prep, out)
+    return {"method": "one wavefront on a second stream samples s_memtime (shader clock counter) against s_memrealtime (100 MHz) "
+                      "while the workload runs on the library's stream; clock = counter difference / wall difference x 100 MHz "
+                      "per sampling interval; intervals inside the workload's runs only", "rows": rows}
+
+
 def cpu_baseline(cfg, ctx: int, tokens: int = 12):
     """Oracle timing, like for like: the whole 16-layer model, S = 1 with a KV cache at context `ctx`.
 
@@ -479,6 +543,8 @@ def main() -> int:
     ap.add_argument("--sweep", action="store_true",
                     help="only the isolated linear-op sweep (four weight shapes x M = 1 / 64 / 512, fused norm and element-wise ops)")
     ap.add_argument("--no-sweep", action="store_true", help="leave the sweep out of the default line")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="only sample the shader clock under a pure read and under the prompt GEMMs (one JSON line)")
     ap.add_argument("--table-iters", type=int, default=12,
                     help="passes behind the per-kernel tables; counter-collecting profilers serialise every dispatch, 1 keeps such runs short")
     args = ap.parse_args()
@@ -488,6 +554,10 @@ def main() -> int:
 
     from deepj_amd import HipNative, JavaRandom, LlamaConfig, LlamaModel
 
+    if args.clock_probe:
+        HipNative.init(0)
+        print(json.dumps({"metric": "shader clock under load, MHz", "n_gpus": 1, "clock_probe": clock_probe()}))
+        return 0
     if args.sweep:
         HipNative.init(0)
         sw = c2_sweep(max(2, args.table_iters), cpu=not args.no_cpu_baseline)

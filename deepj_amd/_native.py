@@ -48,6 +48,8 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_gemm_path.restype = C.c_int32
     lib.deepj_hip_q8_gemm_tile.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
     lib.deepj_hip_q8_gemm_tile.restype = None
+    lib.deepj_hip_clock_probe.argtypes = [_i32p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+    lib.deepj_hip_clock_probe.restype = C.c_int
     lib.deepj_hip_q8_gemm_f16_extents.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     lib.deepj_hip_q8_gemm_f16_extents.restype = C.c_int32
     lib.deepj_hip_time_ops.argtypes = [_i32p, C.c_int32, C.c_int32, _f32p]
@@ -216,6 +218,23 @@ class HipNative:
         if detail:
             return out[: n.value].copy(), top[: n.value].copy(), cnt[: n.value].copy()
         return out[: n.value].copy()
+
+    @staticmethod
+    def clockProbe(cmd_stream, iters: int, samples: int, sleep_reps: int = 1):
+        """Runs the stream `iters` times while a one-wavefront kernel on a second stream samples the shader clock.
+        Returns (MHz per sampling interval, wall time of each interval's end in microseconds from the first sample,
+        (begin, end) of the stream's runs on the same time axis)."""
+        cmd = _ids(cmd_stream)
+        pairs = np.zeros(2 * samples, dtype=np.uint64)
+        window = np.zeros(2, dtype=np.uint64)
+        _check(library().deepj_hip_clock_probe(cmd.ctypes.data_as(_i32p), cmd.size, iters, samples, sleep_reps,
+                                               pairs.ctypes.data_as(C.POINTER(C.c_uint64)), window.ctypes.data_as(C.POINTER(C.c_uint64))))
+        clk, wall = pairs[0::2].astype(np.int64), pairs[1::2].astype(np.int64)
+        dw = np.maximum(np.diff(wall), 1)
+        mhz = np.diff(clk) / dw * 100.0
+        t = (wall[1:] - wall[0]) / 100.0
+        win = ((int(window[0]) - int(wall[0])) / 100.0, (int(window[1]) - int(wall[0])) / 100.0)
+        return mhz, t, win
 
     @staticmethod
     def graphCapture(cmd_stream) -> int:

@@ -76,6 +76,8 @@ void launch_copy(hipStream_t s, const float *src, float *dst, int64_t n);
 // measurement floors: a pure streaming read of n floats (nothing kept), and an empty kernel of `grid` workgroups
 void launch_stream_read(hipStream_t s, const float *src, float *sink, int64_t n);
 void launch_nop(hipStream_t s, int grid);
+void launch_clock_probe(hipStream_t s, unsigned long long *out, int samples, int sleep_reps);
+void launch_wall_stamp(hipStream_t s, unsigned long long *out);
 void launch_silu_mul(hipStream_t s, const float *gate, const float *up, float *out, int64_t n);
 void launch_append_rows(hipStream_t s, const float *src, float *dst, const int32_t *state, int rows, int row_floats,
                         int max_rows);

@@ -399,6 +399,26 @@ void launch_stream_read(hipStream_t s, const float *src, float *sink, int64_t n)
     }
 }
 
+// One wavefront that writes (shader clock counter, 100 MHz wall clock) pairs, `samples` of them, with naps of
+// sleep_reps x 127 x 64 clocks in between: run beside other work, the pairs give the shader clock over time.  Both
+// loops are bounded by arguments; nothing waits for anyone.
+__global__ void __launch_bounds__(64) k_clock_probe(unsigned long long *out, int samples, int sleep_reps) {
+    if (threadIdx.x != 0) return;
+    for (int i = 0; i < samples; i++) {
+        const unsigned long long c = clock64(), w = wall_clock64();
+        __hip_atomic_store(out + 2 * i, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(out + 2 * i + 1, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int j = 0; j < sleep_reps; j++) __builtin_amdgcn_s_sleep(127);
+    }
+}
+// the wall clock at this point of a stream
+__global__ void k_wall_stamp(unsigned long long *out) { if (threadIdx.x == 0) *out = wall_clock64(); }
+
+void launch_clock_probe(hipStream_t s, unsigned long long *out, int samples, int sleep_reps) {
+    hipLaunchKernelGGL(k_clock_probe, dim3(1), dim3(64), 0, s, out, samples, sleep_reps);
+}
+void launch_wall_stamp(hipStream_t s, unsigned long long *out) { hipLaunchKernelGGL(k_wall_stamp, dim3(1), dim3(64), 0, s, out); }
+
 void launch_nop(hipStream_t s, int grid) {
     launch_kernel(k_nop, dim3(grid < 1 ? 1 : grid), dim3(kThreads), 0, s);
 }

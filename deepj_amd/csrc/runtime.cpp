@@ -1051,6 +1051,41 @@ int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms
     });
 }
 
+// The shader clock while a stream runs: a one-wavefront kernel on a second stream (default priority) samples
+// (shader clock counter, 100 MHz wall clock) pairs while `cmd` runs `iters` times on the library's stream, bracketed by
+// wall-clock stamps.  pairs receives 2 * samples counters, window the wall clock before and after the runs.  The
+// sampler sleeps sleep_reps x 127 x 64 clocks between samples and ends by itself after `samples` of them.
+int deepj_hip_clock_probe(const int32_t *cmd, int32_t len, int32_t iters, int32_t samples, int32_t sleep_reps,
+                          uint64_t *pairs, uint64_t *window) {
+    return guarded([&] {
+        ensure_init();
+        if (iters < 0 || samples <= 0 || samples > (1 << 20) || sleep_reps < 0 || sleep_reps > 4096 || !pairs || !window)
+            fail("clock_probe: bad arguments");
+        int64_t ws = 0;
+        if (len > 0) walk(cmd, len, true, &ws);
+        ensure_workspace(ws);
+        hipStream_t side = nullptr;
+        unsigned long long *d = nullptr;
+        DJ_HIP(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
+        const size_t bytes = ((size_t)2 * samples + 2) * sizeof(unsigned long long);
+        hipError_t e = hipMalloc((void **)&d, bytes);
+        if (e != hipSuccess) { (void)hipStreamDestroy(side); fail(std::string("clock_probe: hipMalloc: ") + hipGetErrorString(e)); }
+        (void)hipMemset(d, 0, bytes);
+        DJ_HIP(hipDeviceSynchronize());
+        launch_clock_probe(side, d, samples, sleep_reps);
+        launch_wall_stamp(g.stream, d + 2 * samples);
+        for (int i = 0; i < iters && len > 0; i++) walk(cmd, len, false, nullptr);
+        launch_wall_stamp(g.stream, d + 2 * samples + 1);
+        e = hipStreamSynchronize(g.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(side);
+        if (e == hipSuccess) e = hipMemcpy(pairs, d, (size_t)2 * samples * sizeof(unsigned long long), hipMemcpyDeviceToHost);
+        if (e == hipSuccess) e = hipMemcpy(window, d + 2 * samples, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost);
+        (void)hipFree(d);
+        (void)hipStreamDestroy(side);
+        if (e != hipSuccess) fail(std::string("clock_probe: ") + hipGetErrorString(e));
+    });
+}
+
 // Per-op kernel durations: every kernel dispatch of every op of the stream carries a start and a stop event, the
 // stream runs `iters` times in order, and us_per_op[i] receives the mean over the passes of the summed begin-to-end
 // times of op i's dispatches in microseconds (-1 for an op that launched nothing).  Optional outputs of the same

@@ -96,6 +96,13 @@ int deepj_hip_time_ops(const int32_t *cmd, int32_t len, int32_t iters, float *ms
  * smaller. */
 int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float *us_per_op, int32_t capacity,
                           int32_t *n_ops, float *us_longest, int32_t *dispatches);
+/* Measurement aid, no counterpart in the reference: the shader clock while a stream runs.  A one-wavefront kernel on a
+ * second stream writes `samples` pairs (shader clock counter, 100 MHz wall clock) into pairs[2 * samples], sleeping
+ * sleep_reps x 127 x 64 clocks between two samples, while `cmd` runs `iters` times on the library's stream;
+ * window[0..1] are the wall clock before and after those runs.  Clock over an interval = counter difference / wall
+ * difference x 100 MHz.  The sampler ends by itself; the call returns when both streams are idle. */
+int deepj_hip_clock_probe(const int32_t *cmd, int32_t len, int32_t iters, int32_t samples, int32_t sleep_reps,
+                          uint64_t *pairs, uint64_t *window);
 
 /* Captures a command stream into a HIP graph (no allocation may be pending:
  * every buffer it names must exist) and replays it.  Used for the per-token
