@@ -451,12 +451,44 @@ def clock_probe():
                      "clock_MHz_median": round(float(np.median(inside)), 0), "clock_MHz_p10": round(float(np.percentile(inside, 10)), 0),
                      "clock_MHz_p90": round(float(np.percentile(inside, 90)), 0)})
 
+    smi = []
+
+    def smi_during(name, stream, iters):
+        """The driver's own view beside the sampler's: rocm-smi's sclk, read a few times while the stream loops for a
+        second or two (None where the tool is not there or prints no clock)."""
+        import re, subprocess, threading
+        reads = []
+
+        def poll():
+            for _ in range(6):
+                try:
+                    r = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20)
+                except (OSError, subprocess.SubprocessError):
+                    return
+                found = re.search(r"sclk clock level: *\d+: *\((\d+)Mhz\)", r.stdout)
+                if found:
+                    reads.append((time.perf_counter(), int(found.group(1))))
+                time.sleep(0.2)
+
+        stream.run()
+        HipNative.synchronize()
+        th = threading.Thread(target=poll)
+        t0 = time.perf_counter()
+        th.start()
+        ms = stream.time(iters)
+        t1 = time.perf_counter()
+        th.join()
+        inside = [mhz for t, mhz in reads if t0 + 0.3 < t < t1]
+        return {"workload": name, "loop_s": round(t1 - t0, 2), "us_per_launch": round(ms * 1e3 / iters, 1),
+                "rocm_smi_sclk_MHz": inside or None}
+
     measure("idle (sampler alone)", Stream().nop(1), 0, 400)
     measure("empty kernels back to back", Stream().nop(768), 4000, 1500)
     n = 1 << 28
     big, sink = dev.alloc(n), dev.alloc(64)
     Stream().fill(big, 0x3F800000, n).run()
     measure("pure read of 1 GiB (STREAM_READ)", Stream().stream_read(big, sink, n), 24, 1500)
+    smi.append(smi_during("pure read of 1 GiB (STREAM_READ)", Stream().stream_read(big, sink, n), 10000))
     dev.release(big, sink)
     k, nn = 2048, 5632                       # the decode matvec over a rotation of distinct weight copies (HBM-cold)
     wf = dev.upload((rng.standard_normal((k, nn)) * 0.02).astype(np.float32))
@@ -483,11 +515,15 @@ def clock_probe():
         Stream().q8_prepare(wq, prep, k, nn).run()
         out = dev.alloc(m * nn)
         tile = HipNative.q8GemmTile(m, k, nn)
-        measure(f"Q8 GEMM {m} x {nn} x {k} (fp16 x 2, {tile[0]} x {tile[1]} tiles)", Stream().q8_linear(x, wq, out, m, k, nn), iters, 2000)
+        gemm = Stream().q8_linear(x, wq, out, m, k, nn)
+        measure(f"Q8 GEMM {m} x {nn} x {k} (fp16 x 2, {tile[0]} x {tile[1]} tiles)", gemm, iters, 2000)
+        if m == 2048:
+            smi.append(smi_during(f"Q8 GEMM {m} x {nn} x {k}", gemm, 4000))
         dev.release(x, wq, prep, out)
     return {"method": "one wavefront on a second stream samples s_memtime (shader clock counter) against s_memrealtime (100 MHz) "
                       "while the workload runs on the library's stream; clock = counter difference / wall difference x 100 MHz "
-                      "per sampling interval; intervals inside the workload's runs only", "rows": rows}
+                      "per sampling interval; intervals inside the workload's runs only", "rows": rows,
+            "rocm_smi": smi}
 
 
 def cpu_baseline(cfg, ctx: int, tokens: int = 12):
