@@ -168,6 +168,11 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 // beyond every query of a wavefront is skipped by it.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// The hardware's base-2 exponential (exp2(-inf) = 0).  Soft-max weights are exp2((s - max) log2 e): scores are carried
+// multiplied by log2(e), one instruction per weight where the library's expf takes some twenty.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+constexpr float kLog2e = 1.44269504088896340736f;
+
 // KSETS = 2 or 4 (for grids that would leave CUs idle): a workgroup takes 64 or 32 query rows; its wavefronts are
 // 2 or 4 sets that walk every KSETS-th key tile for the SAME queries, KSETS tiles are staged per round, and the
 // sets' partial soft-max states are merged through LDS at the end - more workgroups and fewer rounds.
@@ -262,17 +267,17 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 int key = kb0 + 8 * (e >> 2) + 4 * half + (e & 3);
-                float sv = (q_ok && key <= qpos) ? st[e] * a.scale : -INFINITY;      // scale after the product
+                float sv = (q_ok && key <= qpos) ? (st[e] * a.scale) * kLog2e : -INFINITY;      // scale after the product, then the change of base
                 st[e] = sv;
                 tmax = fmaxf(tmax, sv);
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
             const float mn = fmaxf(m, tmax);
-            const float corr = (mn == -INFINITY) ? 1.0f : expf(m - mn);
+            const float corr = (mn == -INFINITY) ? 1.0f : fast_exp2(m - mn);
             float psum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-                float p = (st[e] == -INFINITY) ? 0.0f : expf(st[e] - mn);
+                float p = (st[e] == -INFINITY) ? 0.0f : fast_exp2(st[e] - mn);
                 st[e] = p;
                 psum += p;
             }
@@ -311,7 +316,7 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
             const float *mg = lds + (int64_t)(((ks - 1) * QW + qw) * 64 + lane) * REC;
             const float m1 = mg[0], l1 = mg[1];
             const float mn = fmaxf(m, m1);
-            const float w0 = (m == -INFINITY) ? 0.0f : expf(m - mn), w1 = (m1 == -INFINITY) ? 0.0f : expf(m1 - mn);
+            const float w0 = (m == -INFINITY) ? 0.0f : fast_exp2(m - mn), w1 = (m1 == -INFINITY) ? 0.0f : fast_exp2(m1 - mn);
             l = l * w0 + l1 * w1;
             m = mn;
 #pragma unroll
@@ -341,7 +346,7 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     }
 }
 
-// out[row, h, :] = sum_z w_z o_z / sum_z w_z l_z,  w_z = exp(m_z - max m), over the `shares` records of (row, head);
+// out[row, h, :] = sum_z w_z o_z / sum_z w_z l_z,  w_z = exp2(m_z - max m) (the maxima are in base-2 units), over the `shares` records of (row, head);
 // grid (H, S), one thread per output element.  A share without keys left m = -inf, l = 0.
 __global__ void __launch_bounds__(128) k_attention_merge_shares(const float *__restrict__ partial, float *__restrict__ out, int H,
                                                                int hd, int shares) {
@@ -354,7 +359,7 @@ __global__ void __launch_bounds__(128) k_attention_merge_shares(const float *__r
     for (int z = 0; z < shares; z++) {
         const float *r = rec + (int64_t)z * (hd + 4);
         if (r[0] == -INFINITY) continue;
-        const float w = expf(r[0] - M);
+        const float w = fast_exp2(r[0] - M);
         L += r[1] * w;
         O += r[4 + j] * w;
     }
@@ -548,8 +553,6 @@ __device__ unsigned long long g_at_trace[8 * 8192];
 #define DJ_STAMP(i) do {} while (0)
 #endif
 
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }   // exp2(-inf) = 0
-
 // Separate scalar arguments, the ones the first loads need in front (they can reach a wavefront in registers at
 // launch; a by-value struct is always fetched from the argument buffer first).
 template <int LPK>
@@ -560,7 +563,6 @@ k_attn_decode_records(const int32_t *a_state, float *a_k_cache, float *a_v_cache
     constexpr int HD = LPK * 4;
     constexpr int KPW = 64 / LPK;                  // keys a wavefront handles at a time
     constexpr int TILE = kRecWaves * KPW;          // consecutive keys of one tile
-    constexpr float kLog2e = 1.44269504088896340736f;
     constexpr int U = kRecU;
     constexpr int NS = kAttnRecordSplits;
     __shared__ float s_m[kRecWaves], s_l[kRecWaves];
