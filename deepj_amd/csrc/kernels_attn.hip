@@ -158,15 +158,33 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 
 // ── attention, many query rows: tiled on the matrix cores ────────────────────
 // grid (H, ceil(S / 128)): a workgroup takes one head and 128 query rows, 32 per wavefront, and walks the
-// keys in tiles of 32 that all four wavefronts share through LDS (K transposed, V as is).  Per tile and
-// wavefront two products run on v_mfma_f32_32x32x2_f32:
-//     S^T = K . Q^T      32 keys x 32 queries; a lane ends up with ONE query column and 16 of its keys, so
-//                        the running soft-max state (max, sum) is one scalar pair per lane
-//     O^T += V^T . P     P is consumed straight from the accumulator registers of the first product: the
+// keys in tiles of 32 that all four wavefronts share through LDS (K as three bf16 planes, V as is).  Per tile and
+// wavefront two products run on the matrix cores:
+//     S^T = K . Q^T      v_mfma_f32_32x32x16_bf16 on split planes (split3 above): 32 keys x 32 queries; a lane ends up
+//                        with ONE query column and 16 of its keys, so the running soft-max state (max, sum) is one
+//                        scalar pair per lane.  A key row is HD bf16 values per plane, its 16-byte chunks XOR-ed with
+//                        the key's low bits so that the 32 rows an operand read touches spread over all banks
+//     O^T += V^T . P     v_mfma_f32_32x32x2_f32; P is consumed straight from the accumulator registers of the first product: the
 //                        key order of the contraction is chosen to be the order in which a lane holds them
 // Causal masking (HeadOps.java:105-126) excludes key j for query position p when j > p; a tile that lies
 // beyond every query of a wavefront is skipped by it.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// An fp32 value is the exact sum of three bf16 pieces: its leading 8 significant bits, the next 8, the last 8 (each by
+// truncation; the remainders are exact).  A product of two such values on the bf16 matrix cores takes the six piece
+// products whose weights reach 2^-24 of the largest - hi.hi, hi.mid, mid.hi, hi.lo, lo.hi, mid.mid - accumulated in
+// fp32: fp32 accuracy at three eighths of the fp32 matrix instructions' time (32 x 32 x 16 in 32 cycles against
+// 32 x 32 x 2 in 64).
+__device__ __forceinline__ float top_bits(float x) { return __uint_as_float(__float_as_uint(x) & 0xffff0000u); }
+// bf16(a) | bf16(b) << 16 of values that are bf16 numbers already
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) { return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u); }
+__device__ __forceinline__ void split3(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+    const float h0 = top_bits(x0), h1 = top_bits(x1);
+    const float r0 = x0 - h0, r1 = x1 - h1;
+    const float c0 = top_bits(r0), c1 = top_bits(r1);
+    hi = pack_bf16(h0, h1); mid = pack_bf16(c0, c1); lo = pack_bf16(r0 - c0, r1 - c1);
+}
 
 // The hardware's base-2 exponential (exp2(-inf) = 0).  Soft-max weights are exp2((s - max) log2 e): scores are carried
 // multiplied by log2(e), one instruction per weight where the library's expf takes some twenty.
@@ -185,10 +203,12 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     constexpr int KT = 32, NT = HD / 32;
     constexpr int QW = 4 / KSETS;                           // wavefronts that hold distinct query rows
     constexpr int QWG = 32 * QW;                            // query rows per workgroup
-    constexpr int kKtFloats = KSETS * HD * (KT + 1), kVsFloats = KSETS * KT * HD;
+    constexpr int KSTEPS = HD / 16;                         // bf16 matrix instructions (K = 16) along the head dimension
+    constexpr int CH = HD / 8;                              // 16-byte chunks of a key row of one plane
+    constexpr int kKtFloats = KSETS * 3 * KT * HD / 2, kVsFloats = KSETS * KT * HD;
     constexpr int kMergeFloats = (KSETS - 1) * QW * 64 * (NT * 16 + 2);
     __shared__ __align__(16) float lds[kKtFloats + kVsFloats > kMergeFloats ? kKtFloats + kVsFloats : kMergeFloats];
-    float(*Kt)[HD][KT + 1] = reinterpret_cast<float(*)[HD][KT + 1]>(lds);              // [set][j][key]: transposed
+    uint16_t(*Kb)[3][KT][HD] = reinterpret_cast<uint16_t(*)[3][KT][HD]>(lds);          // [set][plane][key][j], chunks swizzled
     float(*Vs)[KT][HD] = reinterpret_cast<float(*)[KT][HD]>(lds + kKtFloats);          // [set][key][j]
 
     // Causal work grows with the query tile.  The second half of the tiles is taken in reverse, so that the workgroups
@@ -211,14 +231,21 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     if (wg_last >= a.max_seq) wg_last = a.max_seq - 1;
     const int wave_last = q_end_wave > q_wave0 ? pos0 + q_end_wave - 1 : -1;
 
-    // this lane's query row: the elements of parity `half`
-    float qreg[HD / 2];
+    // this lane's query row as the B operand of the score products: for step s its eight k slots are the elements
+    // 16 s + 8 half .. + 7 (the same numbering the key operand uses), three planes
+    bf16x8 qv[3][KSTEPS];
     {
         const float *qrow = a.q + (int64_t)(q_ok ? qi : 0) * d + h * HD;
 #pragma unroll
-        for (int kk = 0; kk < HD / 2; kk++) {
-            float2 v = *reinterpret_cast<const float2 *>(qrow + 2 * kk);
-            qreg[kk] = half ? v.y : v.x;
+        for (int sidx = 0; sidx < KSTEPS; sidx++) {
+            const float4 v0 = *reinterpret_cast<const float4 *>(qrow + 16 * sidx + 8 * half);
+            const float4 v1 = *reinterpret_cast<const float4 *>(qrow + 16 * sidx + 8 * half + 4);
+            uint32_t hi[4], mid[4], lo[4];
+            split3(v0.x, v0.y, hi[0], mid[0], lo[0]); split3(v0.z, v0.w, hi[1], mid[1], lo[1]);
+            split3(v1.x, v1.y, hi[2], mid[2], lo[2]); split3(v1.z, v1.w, hi[3], mid[3], lo[3]);
+            qv[0][sidx] = __builtin_bit_cast(bf16x8, make_uint4(hi[0], hi[1], hi[2], hi[3]));
+            qv[1][sidx] = __builtin_bit_cast(bf16x8, make_uint4(mid[0], mid[1], mid[2], mid[3]));
+            qv[2][sidx] = __builtin_bit_cast(bf16x8, make_uint4(lo[0], lo[1], lo[2], lo[3]));
         }
     }
     floatx16 acc[NT];
@@ -235,7 +262,7 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     for (int k0 = k_first; k0 <= wg_last; k0 += k_stride) {
 #pragma unroll
         for (int ks = 0; ks < KSETS; ks++) {
-            // stage the key tile transposed and the value tile; rows past the last key repeat it (masked below)
+            // stage the key tile as bf16 planes and the value tile; rows past the last key repeat it (masked below)
             constexpr int PART = HD / 8;
             int key = k0 + ks * KT + (t & 31);
             if (key > wg_last) key = wg_last;
@@ -243,8 +270,13 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 #pragma unroll
             for (int j = 0; j < PART; j += 4) {
                 float4 v = *reinterpret_cast<const float4 *>(kr + j);
-                int c = (t >> 5) * PART + j;
-                Kt[ks][c][t & 31] = v.x; Kt[ks][c + 1][t & 31] = v.y; Kt[ks][c + 2][t & 31] = v.z; Kt[ks][c + 3][t & 31] = v.w;
+                const int c = (t >> 5) * PART + j;                                       // first of four elements of the row
+                const int at = ((((c >> 3) ^ (t & 31)) & (CH - 1)) << 3) + (c & 7);       // chunk c / 8 lives at (c / 8) ^ key
+                uint32_t hi[2], mid[2], lo[2];
+                split3(v.x, v.y, hi[0], mid[0], lo[0]); split3(v.z, v.w, hi[1], mid[1], lo[1]);
+                *reinterpret_cast<uint2 *>(&Kb[ks][0][t & 31][at]) = make_uint2(hi[0], hi[1]);
+                *reinterpret_cast<uint2 *>(&Kb[ks][1][t & 31][at]) = make_uint2(mid[0], mid[1]);
+                *reinterpret_cast<uint2 *>(&Kb[ks][2][t & 31][at]) = make_uint2(lo[0], lo[1]);
             }
             int vkey = k0 + ks * KT + (t >> 3);
             if (vkey > wg_last) vkey = wg_last;
@@ -260,8 +292,19 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; e++) st[e] = 0.0f;
 #pragma unroll
-            for (int kk = 0; kk < HD / 2; kk++)
-                st = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[kset][2 * kk + half][l32], qreg[kk], st, 0, 0, 0);
+            for (int sidx = 0; sidx < KSTEPS; sidx++) {
+                const int at = (((2 * sidx + half) ^ l32) & (CH - 1)) << 3;
+                const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&Kb[kset][0][l32][at]);
+                const bf16x8 k_mid = *reinterpret_cast<const bf16x8 *>(&Kb[kset][1][l32][at]);
+                const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&Kb[kset][2][l32][at]);
+                // the small terms first
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_lo, qv[0][sidx], st, 0, 0, 0);
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_hi, qv[2][sidx], st, 0, 0, 0);
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_mid, qv[1][sidx], st, 0, 0, 0);
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_mid, qv[0][sidx], st, 0, 0, 0);
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_hi, qv[1][sidx], st, 0, 0, 0);
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_hi, qv[0][sidx], st, 0, 0, 0);
+            }
             // st[e] = q . k for key kb0 + 8*(e/4) + 4*half + e%4 and this lane's query
             float tmax = -INFINITY;
 #pragma unroll
