@@ -208,7 +208,7 @@ def prefill_roofline(model, n: int, iters: int = 6):
             gemm_us += float(t)
             issued += f * (2 if tile else 3)
         elif code == op.OP_ATTENTION:
-            e = table.setdefault("attention", {"launches": 0, "us": 0.0, "kernel": "k_attention_tiled (scores: bf16 x 6 on split planes; values: fp32 matrix instructions)"})
+            e = table.setdefault("attention", {"launches": 0, "us": 0.0, "kernel": "k_attention_tiled (scores: bf16 x 6 on split planes; values: fp32 matrix instructions at this shape)"})
             e["launches"] += 1
             e["us"] += float(t)
         elif code in other_names or (code == op.OP_Q8_LINEAR and w[4] == 1):

@@ -17,6 +17,9 @@
 // graph stays valid as the cache grows) over gridDim.y workgroups per head so the
 // HBM-bound KV read is spread over all CUs, and a second tiny kernel merges the
 // per-split (max, sum, weighted V) records.
+#include <cstdlib>
+#include <type_traits>
+
 #include "dj_common.h"
 #include "dj_device.h"
 
@@ -164,7 +167,9 @@ __global__ void __launch_bounds__(kThreads) k_attention(AttnKernelArgs a) {
 //                        with ONE query column and 16 of its keys, so the running soft-max state (max, sum) is one
 //                        scalar pair per lane.  A key row is HD bf16 values per plane, its 16-byte chunks XOR-ed with
 //                        the key's low bits so that the 32 rows an operand read touches spread over all banks
-//     O^T += V^T . P     v_mfma_f32_32x32x2_f32; P is consumed straight from the accumulator registers of the first product: the
+//     O^T += V^T . P     either v_mfma_f32_32x32x2_f32 with P consumed straight from the accumulator registers of the first
+//                        product, or (PVB) the bf16 instruction again on split planes of P and of the value tile, which is
+//                        staged transposed - [element][key slot] - into the bytes the key planes have just left: the
 //                        key order of the contraction is chosen to be the order in which a lane holds them
 // Causal masking (HeadOps.java:105-126) excludes key j for query position p when j > p; a tile that lies
 // beyond every query of a wavefront is skipped by it.
@@ -198,18 +203,23 @@ constexpr float kLog2e = 1.44269504088896340736f;
 // r % gridDim.z, so the shares are even whatever the position, which only the device knows) and leave their
 // unnormalised states as records; k_attention_merge_shares finishes the rows.  For a handful of query rows over a
 // long context, where (head, query tile) alone are far fewer workgroups than compute units.
-template <int HD, int KSETS, bool SHARE = false>
+template <int HD, int KSETS, bool SHARE = false, bool PVB = false>
 __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
     constexpr int KT = 32, NT = HD / 32;
     constexpr int QW = 4 / KSETS;                           // wavefronts that hold distinct query rows
     constexpr int QWG = 32 * QW;                            // query rows per workgroup
     constexpr int KSTEPS = HD / 16;                         // bf16 matrix instructions (K = 16) along the head dimension
     constexpr int CH = HD / 8;                              // 16-byte chunks of a key row of one plane
-    constexpr int kKtFloats = KSETS * 3 * KT * HD / 2, kVsFloats = KSETS * KT * HD;
+    constexpr int VP = KT + 8;                              // bf16 values per row of the transposed value tile: 32 keys + 16 bytes
+    constexpr int kKbFloats = KSETS * 3 * KT * HD / 2, kVtFloats = KSETS * 3 * HD * VP / 2, kVsFloats = KSETS * KT * HD;
+    // PVB: the key planes and the value planes use the same bytes in turn (scores first, then values); else the value
+    // tile sits behind the key planes as fp32 rows
+    constexpr int kStageFloats = PVB ? (kKbFloats > kVtFloats ? kKbFloats : kVtFloats) : kKbFloats + kVsFloats;
     constexpr int kMergeFloats = (KSETS - 1) * QW * 64 * (NT * 16 + 2);
-    __shared__ __align__(16) float lds[kKtFloats + kVsFloats > kMergeFloats ? kKtFloats + kVsFloats : kMergeFloats];
+    __shared__ __align__(16) float lds[kStageFloats > kMergeFloats ? kStageFloats : kMergeFloats];
     uint16_t(*Kb)[3][KT][HD] = reinterpret_cast<uint16_t(*)[3][KT][HD]>(lds);          // [set][plane][key][j], chunks swizzled
-    float(*Vs)[KT][HD] = reinterpret_cast<float(*)[KT][HD]>(lds + kKtFloats);          // [set][key][j]
+    uint16_t(*Vt)[3][HD][VP] = reinterpret_cast<uint16_t(*)[3][HD][VP]>(lds);          // PVB: [set][plane][j][key slot], transposed
+    float(*Vs)[KT][HD] = reinterpret_cast<float(*)[KT][HD]>(lds + kKbFloats);          // else: [set][key][j]
 
     // Causal work grows with the query tile.  The second half of the tiles is taken in reverse, so that the workgroups
     // that become resident together on a compute unit (index i and i + half the grid) are a short and a long one.
@@ -257,6 +267,15 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
 
     const float *kbase = a.k + (int64_t)h * a.head_stride;
     const float *vbase = a.v + (int64_t)h * a.head_stride;
+    // Value staging: a thread takes a pair of neighbouring keys (2 vkp, 2 vkp + 1) and four elements 4 vq .. 4 vq + 3 of
+    // their rows, and writes each element's pair - neighbours in the transposed row - as one dword per plane.  Slot of key
+    // kk in a row: the order in which the lanes hold their 16 scores of a tile (key 8 (e / 4) + 4 half + e % 4 in st[e]),
+    // product mm = e / 8 taking slots 16 mm + 8 half + e % 8.  (Thread bits chosen so that the writes of a wavefront
+    // spread over the banks two to a bank; an 80-byte row pitch makes the operand reads conflict free.)
+    constexpr int VREP = HD >= 64 ? HD / 64 : 1;
+    const int vq = (t & 3) | ((t >> 6) << 2), vkp = (t >> 2) & 15;
+    const bool v_ok = 4 * vq < HD;
+    const int vslot = 16 * (vkp >> 3) + 8 * ((vkp >> 1) & 1) + 4 * ((vkp >> 2) & 1) + 2 * (vkp & 1);
     const int k_first = SHARE ? (int)blockIdx.z * KT * KSETS : 0;
     const int k_stride = SHARE ? (int)gridDim.z * KT * KSETS : KT * KSETS;
     for (int k0 = k_first; k0 <= wg_last; k0 += k_stride) {
@@ -278,17 +297,38 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
                 *reinterpret_cast<uint2 *>(&Kb[ks][1][t & 31][at]) = make_uint2(mid[0], mid[1]);
                 *reinterpret_cast<uint2 *>(&Kb[ks][2][t & 31][at]) = make_uint2(lo[0], lo[1]);
             }
-            int vkey = k0 + ks * KT + (t >> 3);
-            if (vkey > wg_last) vkey = wg_last;
-            const float *vr = vbase + (int64_t)vkey * a.tok_stride + (t & 7) * PART;
+        }
+        // PVB: the value rows are requested now and fly while the scores are computed; else the value tile is staged as it is
+        float4 va[PVB ? KSETS : 1][VREP], vb[PVB ? KSETS : 1][VREP];
+        if constexpr (!PVB) {
 #pragma unroll
-            for (int j = 0; j < PART; j += 4)
-                *reinterpret_cast<float4 *>(&Vs[ks][t >> 3][(t & 7) * PART + j]) = *reinterpret_cast<const float4 *>(vr + j);
+            for (int ks = 0; ks < KSETS; ks++) {
+                constexpr int PART = HD / 8;
+                int vkey = k0 + ks * KT + (t >> 3);
+                if (vkey > wg_last) vkey = wg_last;
+                const float *vr = vbase + (int64_t)vkey * a.tok_stride + (t & 7) * PART;
+#pragma unroll
+                for (int j = 0; j < PART; j += 4)
+                    *reinterpret_cast<float4 *>(&Vs[ks][t >> 3][(t & 7) * PART + j]) = *reinterpret_cast<const float4 *>(vr + j);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < (PVB ? KSETS : 0); ks++) {
+            int key_a = k0 + ks * KT + 2 * vkp, key_b = key_a + 1;
+            if (key_a > wg_last) key_a = wg_last;
+            if (key_b > wg_last) key_b = wg_last;
+#pragma unroll
+            for (int rep = 0; rep < VREP; rep++) {
+                const int j0 = v_ok ? 4 * (vq + 16 * rep) : 0;
+                va[ks][rep] = *reinterpret_cast<const float4 *>(vbase + (int64_t)key_a * a.tok_stride + j0);
+                vb[ks][rep] = *reinterpret_cast<const float4 *>(vbase + (int64_t)key_b * a.tok_stride + j0);
+            }
         }
         __syncthreads();
         const int kb0 = k0 + kset * KT;                     // this wavefront's tile of the round
-        if (kb0 <= wave_last) {                             // wave-uniform
-            floatx16 st;
+        const bool active = kb0 <= wave_last;               // wave-uniform
+        floatx16 st;
+        if (active) {
 #pragma unroll
             for (int e = 0; e < 16; e++) st[e] = 0.0f;
 #pragma unroll
@@ -330,12 +370,61 @@ __global__ void __launch_bounds__(256) k_attention_tiled(AttnKernelArgs a) {
             for (int i = 0; i < NT; i++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][e] *= corr;
+            if constexpr (!PVB) {
+                // O^T += V^T . P on the fp32 matrix instruction, P straight from the registers the scores arrived in
 #pragma unroll
-            for (int kk = 0; kk < 16; kk++) {
-                const int key = 8 * (kk >> 2) + 4 * half + (kk & 3);
+                for (int kk = 0; kk < 16; kk++) {
+                    const int key = 8 * (kk >> 2) + 4 * half + (kk & 3);
 #pragma unroll
-                for (int i = 0; i < NT; i++)
-                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[kset][key][32 * i + l32], st[kk], acc[i], 0, 0, 0);
+                    for (int i = 0; i < NT; i++)
+                        acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[kset][key][32 * i + l32], st[kk], acc[i], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();                                    // every wavefront has read its keys (PVB: the bytes now take the values)
+        if constexpr (!PVB) continue;
+#pragma unroll
+        for (int ks = 0; ks < (PVB ? KSETS : 0); ks++) {
+            if (!v_ok) break;
+#pragma unroll
+            for (int rep = 0; rep < VREP; rep++) {
+                const float ca[4] = {va[ks][rep].x, va[ks][rep].y, va[ks][rep].z, va[ks][rep].w};
+                const float cb[4] = {vb[ks][rep].x, vb[ks][rep].y, vb[ks][rep].z, vb[ks][rep].w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t hi, mid, lo;                   // (key, key + 1) of one element: neighbours in the row
+                    split3(ca[i], cb[i], hi, mid, lo);
+                    const int j = 4 * (vq + 16 * rep) + i;
+                    *reinterpret_cast<uint32_t *>(&Vt[ks][0][j][vslot]) = hi;
+                    *reinterpret_cast<uint32_t *>(&Vt[ks][1][j][vslot]) = mid;
+                    *reinterpret_cast<uint32_t *>(&Vt[ks][2][j][vslot]) = lo;
+                }
+            }
+        }
+        __syncthreads();
+        if (active) {
+            // O^T += V^T . P: the k slots of product mm are the keys the lane holds in st[8 mm .. 8 mm + 7]
+#pragma unroll
+            for (int mm = 0; mm < 2; mm++) {
+                uint32_t ph[4], pm[4], pl[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) split3(st[8 * mm + 2 * i], st[8 * mm + 2 * i + 1], ph[i], pm[i], pl[i]);
+                const bf16x8 p_hi = __builtin_bit_cast(bf16x8, make_uint4(ph[0], ph[1], ph[2], ph[3]));
+                const bf16x8 p_mid = __builtin_bit_cast(bf16x8, make_uint4(pm[0], pm[1], pm[2], pm[3]));
+                const bf16x8 p_lo = __builtin_bit_cast(bf16x8, make_uint4(pl[0], pl[1], pl[2], pl[3]));
+#pragma unroll
+                for (int i = 0; i < NT; i++) {
+                    const int j = 32 * i + l32, at = 16 * mm + 8 * half;
+                    const bf16x8 v_hi = *reinterpret_cast<const bf16x8 *>(&Vt[kset][0][j][at]);
+                    const bf16x8 v_mid = *reinterpret_cast<const bf16x8 *>(&Vt[kset][1][j][at]);
+                    const bf16x8 v_lo = *reinterpret_cast<const bf16x8 *>(&Vt[kset][2][j][at]);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_lo, p_hi, acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_hi, p_lo, acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_mid, p_mid, acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_mid, p_hi, acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_hi, p_mid, acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_hi, p_hi, acc[i], 0, 0, 0);
+                }
             }
         }
         __syncthreads();
@@ -860,33 +949,32 @@ void launch_attention(hipStream_t s, const AttnArgs &p) {
         return;
     }
     if (p.s >= 16) {                     // enough rows to share key tiles: matrix-core kernel
+        // the value products on bf16 planes (PVB) or on the fp32 matrix instruction: DEEPJ_HIP_ATTN_PVB=0 / 1 forces one
+        static const int forced = [] { const char *e = getenv("DEEPJ_HIP_ATTN_PVB"); return e ? atoi(e) : -1; }();
+        auto go = [&](auto hd_tag, auto sets_tag, dim3 grid, bool pvb) {
+            constexpr int HD = decltype(hd_tag)::value, KSETS = decltype(sets_tag)::value;
+            if (pvb) launch_kernel((k_attention_tiled<HD, KSETS, false, true>), grid, dim3(256), 0, s, a);
+            else launch_kernel((k_attention_tiled<HD, KSETS, false, false>), grid, dim3(256), 0, s, a);
+        };
+        auto by_hd = [&](auto sets_tag, dim3 grid) {
+            constexpr int KSETS = decltype(sets_tag)::value;
+            // measured: wide heads gain from the bf16 value products (2048 rows, 128-wide: 328 -> 294 us per block); 64-wide
+            // heads with four key sets lose (20.9 -> 23.8 us at 512 rows: the second staging pass and its barriers)
+            const bool pvb = forced >= 0 ? forced != 0 : (p.hd == 128 || KSETS == 1);
+            switch (p.hd) {
+                case 32: go(std::integral_constant<int, 32>{}, sets_tag, grid, pvb); break;
+                case 64: go(std::integral_constant<int, 64>{}, sets_tag, grid, pvb); break;
+                case 128: go(std::integral_constant<int, 128>{}, sets_tag, grid, pvb); break;
+                default: fail("attention: head dim must be 32, 64 or 128");
+            }
+        };
         dim3 tg(p.h, (p.s + 127) / 128);
-        if ((int64_t)tg.x * tg.y * 2 < kAttnFullGrid) {  // far too few workgroups for the chip: 32 rows each, keys in four sets
-            dim3 tg4(p.h, (p.s + 31) / 32);
-            switch (p.hd) {
-                case 32: launch_kernel((k_attention_tiled<32, 4>), tg4, dim3(256), 0, s, a); break;
-                case 64: launch_kernel((k_attention_tiled<64, 4>), tg4, dim3(256), 0, s, a); break;
-                case 128: launch_kernel((k_attention_tiled<128, 4>), tg4, dim3(256), 0, s, a); break;
-                default: fail("attention: head dim must be 32, 64 or 128");
-            }
-            return;
-        }
-        if ((int64_t)tg.x * tg.y < kAttnFullGrid) {      // too few: 64 rows each, keys in two sets
-            dim3 tg2(p.h, (p.s + 63) / 64);
-            switch (p.hd) {
-                case 32: launch_kernel((k_attention_tiled<32, 2>), tg2, dim3(256), 0, s, a); break;
-                case 64: launch_kernel((k_attention_tiled<64, 2>), tg2, dim3(256), 0, s, a); break;
-                case 128: launch_kernel((k_attention_tiled<128, 2>), tg2, dim3(256), 0, s, a); break;
-                default: fail("attention: head dim must be 32, 64 or 128");
-            }
-            return;
-        }
-        switch (p.hd) {
-            case 32: launch_kernel((k_attention_tiled<32, 1>), tg, dim3(256), 0, s, a); break;
-            case 64: launch_kernel((k_attention_tiled<64, 1>), tg, dim3(256), 0, s, a); break;
-            case 128: launch_kernel((k_attention_tiled<128, 1>), tg, dim3(256), 0, s, a); break;
-            default: fail("attention: head dim must be 32, 64 or 128");
-        }
+        if ((int64_t)tg.x * tg.y * 2 < kAttnFullGrid)        // far too few workgroups for the chip: 32 rows each, keys in four sets
+            by_hd(std::integral_constant<int, 4>{}, dim3(p.h, (p.s + 31) / 32));
+        else if ((int64_t)tg.x * tg.y < kAttnFullGrid)      // too few: 64 rows each, keys in two sets
+            by_hd(std::integral_constant<int, 2>{}, dim3(p.h, (p.s + 63) / 64));
+        else
+            by_hd(std::integral_constant<int, 1>{}, tg);
         return;
     }
     dim3 grid(p.h, p.s);

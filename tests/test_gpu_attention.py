@@ -30,6 +30,9 @@ def oracle_attention(q, k, v, H, cos, sin):
                                                  # grids of 288 and 576 workgroups at 128 rows each: the prefill kernel's
                                                  # two-key-set and one-key-set variants (the small shapes above use four)
                                                  (32, 64, 1200, [1100, 1, 20]), (64, 32, 1150, [1100, 1]),
+                                                 # the value products on bf16 planes: one key set at 64-wide heads, two at
+                                                 # 128-wide ones (narrower heads with two or four sets keep the fp32 form)
+                                                 (64, 64, 1100, [1050, 1, 17]), (32, 128, 1150, [1100, 3]),
                                                  # ragged chunks around the 16-row threshold and the 32-row query tile
                                                  (4, 64, 200, [17, 1, 33, 15, 16, 65]), (3, 128, 150, [31, 97]),
                                                  # short continuations of a cached prefix (2 to 32 rows: the key rounds
