@@ -192,15 +192,16 @@ def prefill_roofline(model, n: int, iters: int = 6):
         if t <= 0:
             continue
         all_us += float(t)
-        if code == op.OP_Q8_LINEAR and w[4] > 1:
-            m, k, nn, flags = w[4], w[5], w[6], w[7]
+        if (code == op.OP_Q8_LINEAR and w[4] > 1) or code == op.OP_Q8_LINEAR_ROPE:
+            fused_rope = code == op.OP_Q8_LINEAR_ROPE
+            m, k, nn, flags = w[4], w[5], (3 * w[6] if fused_rope else w[6]), w[7]
             rows = 2 * nn if flags & op.LIN_SWIGLU else nn
             tile, tile_cols, shares = HipNative.q8GemmTile(m, k, rows)
             f = 2.0 * m * k * rows
-            e = table.setdefault(names.get((k, rows), f"{k}x{rows}"), {
+            e = table.setdefault(names.get((k, rows), f"{k}x{rows}") + ("_rope_kv_store" if fused_rope else ""), {
                 "launches": 0, "us": 0.0, "gemm_us": 0.0, "dispatches_per_op": int(c), "flops": f,
                 "kernel": (f"k_gemm_q8_f16 ({tile} x {tile_cols} tiles" + (f", K shared by {shares}" if shares > 1 else "") +
-                           ", fp16 x 2)") if tile else "k_gemm_q8 (bf16 x 3)"})
+                           ", fp16 x 2" + (", RoPE + cache append as the epilogue)" if fused_rope else ")")) if tile else "k_gemm_q8 (bf16 x 3)"})
             e["launches"] += 1
             e["us"] += float(t)
             e["gemm_us"] += float(t_top)

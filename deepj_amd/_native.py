@@ -48,6 +48,8 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_gemm_path.restype = C.c_int32
     lib.deepj_hip_q8_gemm_tile.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
     lib.deepj_hip_q8_gemm_tile.restype = None
+    lib.deepj_hip_q8_linear_rope_ok.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+    lib.deepj_hip_q8_linear_rope_ok.restype = C.c_int32
     lib.deepj_hip_clock_probe.argtypes = [_i32p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
     lib.deepj_hip_clock_probe.restype = C.c_int
     lib.deepj_hip_q8_gemm_f16_extents.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
@@ -188,6 +190,11 @@ class HipNative:
         reach, size = (C.c_int64 * 3)(), (C.c_int64 * 3)()
         ok = int(library().deepj_hip_q8_gemm_f16_extents(m, k, rows, tile_rows, tile_cols, reach, size))
         return ok, list(reach), list(size)
+
+    @staticmethod
+    def q8LinearRopeOk(m: int, k: int, d: int) -> bool:
+        """Whether OP_Q8_LINEAR_ROPE takes a projection of m rows over k inputs to 3 d outputs."""
+        return bool(library().deepj_hip_q8_linear_rope_ok(m, k, d))
 
     @staticmethod
     def q8GemmPath(m: int, k: int, rows: int) -> int:

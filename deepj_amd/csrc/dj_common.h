@@ -10,6 +10,7 @@
 #include <string>
 
 #include "../../include/deepj_hip.h"
+#include "gemm_epilogue.h"
 
 namespace dj {
 
@@ -116,6 +117,7 @@ struct Q8Linear {
     const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
     int m_extra = 0;
     const float *prepared = nullptr;  // the weights in the fp16 GEMM's layout (launch_q8_prepare), or null: converted per call
+    RopeStore rope;                   // fp16 GEMM only: out = nullptr, the q | k | v row goes through RoPE to q and the caches
     bool small_workspace_only = false; // the caller's workspace cannot grow: stay on the kernels that need M * K floats at most
 };
 void launch_q8_quantize(hipStream_t s, const float *w, int8_t *q, float *scales, int k, int n, int row_off,
@@ -144,7 +146,9 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
 // gamma (and beta): the rows are RMS- (Layer-) normalised on their way into the kernel's layout
 void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
                         const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
-                        const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats);
+                        const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats,
+                        const RopeStore *rope = nullptr);
+bool q8_gemm_f16_rope_ok(int m, int d, int k);
 
 // kernels_attn.hip
 struct AttnArgs {

@@ -100,7 +100,7 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int 
 // wide.  The 32 x 32 TNW floats go through LDS that belongs to this wavefront alone (16 KB) and come back as rows of
 // float4 (8 TNW lanes per row, two rows per round), which get the row's power of two, bias / GELU / residual or the
 // SwiGLU pairing.
-template <int TNW>
+template <int TNW, bool ROPE = false>
 __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stage_f, const float (&acc)[TNW][16], int row0, int col0, int lane) {
     constexpr int W = 32 * TNW, LPR = 8 * TNW;                         // floats per row; lanes per row
     const GemmEpilogue &ep = a.ep;
@@ -123,7 +123,19 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
             b4 = *reinterpret_cast<const float4 *>(ep.bias + col);
         }
     }
-#pragma unroll 4
+    constexpr bool rope = ROPE;      // (a compile-time variant: its sixteen table entries would cost every other launch registers)
+    RopeColumn rc{0, 0, 0, 0};
+    int pos0 = 0;
+    float4 tab[ROPE ? 16 : 1];                                         // the rotation's table entries of the lane's 16 rows, requested together
+    if (rope && active && col < a.n) {
+        rc = rope_column(ep.rope, col);
+        pos0 = ep.rope.state[0];
+        if (rc.region < 2) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) tab[i] = rope_table(ep.rope, rc, min(row0 + i * 2 + rsel, a.m - 1), pos0);
+        }
+    }
+#pragma unroll(ROPE ? 16 : 4)
     for (int i = 0; i < 16; i++) {
         const int rl = i * 2 + rsel, row = row0 + rl;
         if (!active || row >= a.m || col >= a.n) continue;
@@ -131,6 +143,7 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
         const float us = a.unscale[row];
         v.x = v.x * us; v.y = v.y * us; v.z = v.z * us; v.w = v.w * us;
         if (ep.bias) { v.x = v.x + b4.x; v.y = v.y + b4.y; v.z = v.z + b4.z; v.w = v.w + b4.w; }
+        if constexpr (ROPE) { rope_store(ep.rope, rc, v, row, pos0, tab[i]); continue; }
         if (ep.swiglu) {
             // (gate, up) pairs in neighbouring columns (SiLU.java:20-24, SwiGLULayer.java:69)
             float2 o;
@@ -154,7 +167,7 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
 // A K step is 2 TNW passes; the schedule below places the same kinds of work in both.
 constexpr int stage128_bytes(int tnw) { return kXs + 64 * tnw * 64 + 1024; }     // X planes, W rows, 256 scales
 
-template <int TNW>
+template <int TNW, bool ROPE = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) k_gemm_q8_f16(const GemmF16Args a) {
     static_assert(TNW == 3 || TNW == 4, "the slots of the schedule are written out for these");
     constexpr int kTn = 64 * TNW, kW = kTn * 64, kStageB = stage128_bytes(TNW);
@@ -309,7 +322,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) store_tile_row<TNW>(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * (32 * TNW), lane);
+    for (int tm = 0; tm < 2; tm++) store_tile_row<TNW, ROPE>(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * (32 * TNW), lane);
 }
 
 // The same product on a 64-row workgroup tile, 256 (TNW = 4) or 192 (TNW = 3) columns wide, for problems whose 128-row
@@ -325,7 +338,7 @@ constexpr int kXs64 = 2 * TM64 * 64;
 constexpr int stage64_bytes(int tnw) { return kXs64 + 64 * tnw * 64 + 1024; }
 constexpr int kMinSplitSteps = 16;          // K steps a workgroup must at least have when several share a tile's K
 
-template <int TNW>
+template <int TNW, bool ROPE = false>
 __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     constexpr int kTn = 64 * TNW, kW = kTn * 64, kStage64 = stage64_bytes(TNW);
     constexpr int kLoads64 = TNW + 3;           // per wavefront per stage: 2 of X, TNW of W, 1 of scales
@@ -468,7 +481,7 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
         store_tile_row<TNW>(b, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
         return;
     }
-    store_tile_row<TNW>(a, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
+    store_tile_row<TNW, ROPE>(a, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
 }
 
 // out = epilogue(sum over the splits of partial[z]) on float4s: bias, GELU, residual or the SwiGLU pairing as in
@@ -717,6 +730,11 @@ GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
 }
 
 int q8_gemm_f16_tile_rows(int m, int n_rows, int k) { return q8_gemm_f16_plan(m, n_rows, k).tile_rows; }
+// the fused q | k | v projection with RoPE and the cache append as its epilogue: on these kernels, K not shared
+bool q8_gemm_f16_rope_ok(int m, int d, int k) {
+    const GemmF16Plan p = q8_gemm_f16_plan(m, 3 * d, k);
+    return p.tile_rows != 0 && p.splits == 1;
+}
 bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) { return q8_gemm_f16_tile_rows(m, n_rows, k) != 0; }
 void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares) {
     const GemmF16Plan p = q8_gemm_f16_plan(m, n_rows, k);
@@ -775,20 +793,28 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
 // The kernels' LDS (three stages) is above the 64 KB a kernel gets without asking; called once per device at start-up
 // (not at the first launch, which may sit inside a graph capture).
 void q8_gemm_f16_configure() {
-    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage128_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16<4>)");
-    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage128_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16<3>)");
-    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(4)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4>)");
-    hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3>), hipFuncAttributeMaxDynamicSharedMemorySize, kStages * stage64_bytes(3)), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3>)");
+    auto lds = [](const void *kernel, int bytes, const char *what) { hip_check(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes), what); };
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16<4>), kStages * stage128_bytes(4), "hipFuncSetAttribute(k_gemm_q8_f16<4>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16<3>), kStages * stage128_bytes(3), "hipFuncSetAttribute(k_gemm_q8_f16<3>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16<4, true>), kStages * stage128_bytes(4), "hipFuncSetAttribute(k_gemm_q8_f16<4, rope>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16<3, true>), kStages * stage128_bytes(3), "hipFuncSetAttribute(k_gemm_q8_f16<3, rope>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4>), kStages * stage64_bytes(4), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3>), kStages * stage64_bytes(3), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<4, true>), kStages * stage64_bytes(4), "hipFuncSetAttribute(k_gemm_q8_f16_m64<4, rope>)");
+    lds(reinterpret_cast<const void *>(k_gemm_q8_f16_m64<3, true>), kStages * stage64_bytes(3), "hipFuncSetAttribute(k_gemm_q8_f16_m64<3, rope>)");
 }
 
 void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
                         const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
-                        const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats) {
+                        const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats,
+                        const RopeStore *rope) {
     if (!q8_gemm_f16_shape_ok(m, n_rows, k)) fail("q8_gemm_f16: shape outside this kernel's range");
     if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
     const int kp = q8_padded_k(k), pitch = kp + 64, m_pad = (int)round_up(m, TM), n_pad = (int)round_up(n_rows, kNPad);
     const GemmF16Plan plan = q8_gemm_f16_plan(m, n_rows, k);
+    if (rope && (plan.splits > 1 || swiglu || gelu || residual || n_rows != 3 * rope->d || (rope->hd & 3) || rope->d % rope->hd))
+        fail("q8_gemm_f16: the RoPE epilogue needs an unshared K, N = 3 d and no other epilogue than a bias");
     int64_t reach[3], size[3];
     if (!q8_gemm_f16_extents(m, n_rows, k, plan.tile_rows, plan.tile_cols, reach, size)) fail("q8_gemm_f16: a tile's loads would reach past its buffer");
     const int m_read = (int)round_up(m, plan.tile_rows);                // rows the row tiles read: [m, m_read) are zeros
@@ -810,19 +836,29 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     const int n_tiles = (n_rows + plan.tile_cols - 1) / plan.tile_cols, m_tiles = plan.tile_rows == 64 ? (m + TM64 - 1) / TM64 : m_pad / TM;
     const unsigned grid_x = (unsigned)((n_tiles + 7) / 8 * 8 * m_tiles);
     GemmF16Args a{planes, w16, scales_t, unscale, out, m, n_rows, m_pad, n_pad, kp, pitch, m_tiles, n_tiles,
-                  GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu}, split_steps, w};
+                  GemmEpilogue{bias, bias2, residual, interleaved_bias, nullptr, 0, gelu, swiglu, rope ? *rope : RopeStore{}}, split_steps, w};
+    const bool roped = rope != nullptr;
     if (plan.tile_rows == 64) {
-        if (plan.tile_cols == 192) launch_kernel(k_gemm_q8_f16_m64<3>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(3), s, a);
-        else launch_kernel(k_gemm_q8_f16_m64<4>, dim3(grid_x, 1, plan.splits), dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
+        const dim3 grid(grid_x, 1, plan.splits);
+        if (plan.tile_cols == 192) {
+            if (roped) launch_kernel((k_gemm_q8_f16_m64<3, true>), grid, dim3(256), (size_t)kStages * stage64_bytes(3), s, a);
+            else launch_kernel((k_gemm_q8_f16_m64<3>), grid, dim3(256), (size_t)kStages * stage64_bytes(3), s, a);
+        } else {
+            if (roped) launch_kernel((k_gemm_q8_f16_m64<4, true>), grid, dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
+            else launch_kernel((k_gemm_q8_f16_m64<4>), grid, dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
+        }
         if (plan.splits > 1) {
             const int64_t mn4 = (int64_t)m * n_rows / 4;
             launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
                                mn4, n_rows / 4, a.ep);
         }
-    } else if (plan.tile_cols == 192)
-        launch_kernel(k_gemm_q8_f16<3>, dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(3), s, a);
-    else
-        launch_kernel(k_gemm_q8_f16<4>, dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(4), s, a);
+    } else if (plan.tile_cols == 192) {
+        if (roped) launch_kernel((k_gemm_q8_f16<3, true>), dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(3), s, a);
+        else launch_kernel((k_gemm_q8_f16<3>), dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(3), s, a);
+    } else {
+        if (roped) launch_kernel((k_gemm_q8_f16<4, true>), dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(4), s, a);
+        else launch_kernel((k_gemm_q8_f16<4>), dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(4), s, a);
+    }
 }
 
 }  // namespace dj

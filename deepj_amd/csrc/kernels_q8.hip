@@ -700,6 +700,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     const int kp = q8_padded_k(p.k);
 
     if (p.m == 1 && !p.m_dev && matvec_supported(p.k)) {
+        if (p.rope.q) fail("q8_linear: the RoPE epilogue exists on the fp16 GEMM only (deepj_hip_q8_linear_rope_ok says for which shapes)");
         const int rec_hd = (p.flags & DJ_LIN_ATTN_MERGE) ? p.rec_hd : 0;
         MatvecArgs a{p.x, p.wq, p.scales, p.out, p.k, kp, p.n, gamma, bias, bias2, residual, beta, rec_hd};
         int nc = (kp + 1023) / 1024;
@@ -726,11 +727,14 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     // many rows and enough tiles: the fp16 kernel, when the caller's workspace also holds its prepared operands; the
     // normalisation happens on the rows' way into that layout
     const int n_rows = swiglu ? 2 * p.n : p.n;
+    const bool rope = p.rope.q != nullptr;
     if (!p.m_dev && !p.small_workspace_only && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
         launch_q8_gemm_f16(s, p.x, gamma, beta, p.wq, p.scales, p.prepared, p.out, p.m, p.k, n_rows, bias, swiglu ? bias2 : nullptr,
-                           swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, workspace, workspace_floats);
+                           swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, workspace, workspace_floats,
+                           rope ? &p.rope : nullptr);
         return;
     }
+    if (rope) fail("q8_linear: the RoPE epilogue exists on the fp16 GEMM only (deepj_hip_q8_linear_rope_ok says for which shapes)");
     const float *x = p.x;
     float *ws = workspace;
     if (gamma) {

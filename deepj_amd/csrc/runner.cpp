@@ -377,7 +377,9 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     const Config &c = r.cfg;
     const Layer &L = r.layers[l];
     const int d = c.d, H = c.heads, hd = r.hd();
-    bool wo_done = false;
+    bool wo_done = false, rope_fused = false;
+    // a prompt's q | k | v projection takes RoPE and the cache append as its epilogue where the library has that kernel
+    auto fuse_rope = [&](int k_in) { return !c.latent && !(S == 1 && &a == &r.dec) && S > 1 && deepj_hip_q8_linear_rope_ok(S, k_in, d) != 0; };
     // x2 = x + Wo . attention(RoPE(split(norm1(x) . [Wq|Wk|Wv])))      LlamaTransformerBlock.java:51
     // GPT: LayerNorm instead of RMSNorm and no rotation                  GPTTransformerBlock.java:66-68
     // DeepSeek: [Q|K|V] = ([cQ|cKV] = norm1(x).[Wdq|Wdkv]) . blockdiag(Wuq, [Wuk|Wuv])   MultiHeadLatentAttention.java:92-123
@@ -400,11 +402,14 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
     } else if (c.kind == 1) {
         const int k2 = r.latent_width();
         q8_linear(s, a.x, L.wdown, a.cq, S, d, k2, DJ_LIN_RMSNORM, L.g1);
-        q8_linear(s, a.cq, L.wup, a.qkv, S, k2, 3 * d, 0);
+        if (!(rope_fused = fuse_rope(k2))) q8_linear(s, a.cq, L.wup, a.qkv, S, k2, 3 * d, 0);
+        else emit(s, DJ_OP_Q8_LINEAR_ROPE, a.cq, L.wup, a.q, S, k2, d, 0, -1, -1, -1, r.kc, r.vc, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
     } else if (c.kind == 2) {
-        q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1);
+        if (!(rope_fused = fuse_rope(d))) q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1);
+        else emit(s, DJ_OP_Q8_LINEAR_ROPE, a.x, L.wqkv, a.q, S, d, d, DJ_LIN_LAYERNORM, L.g1, -1, L.be1, r.kc, r.vc, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
     } else {
-        q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
+        if (!(rope_fused = fuse_rope(d))) q8_linear(s, a.x, L.wqkv, a.qkv, S, d, 3 * d, DJ_LIN_RMSNORM, L.g1);
+        else emit(s, DJ_OP_Q8_LINEAR_ROPE, a.x, L.wqkv, a.q, S, d, d, DJ_LIN_RMSNORM, L.g1, -1, -1, r.kc, r.vc, r.state, r.cos_t, r.sin_t, H, hd, c.max_seq, l);
     }
     if (c.latent) {
         // attention and Wo were emitted above
@@ -414,7 +419,7 @@ void block_stream(Runner &r, Stream &s, Acts &a, int l, int S) {
         emit(s, DJ_OP_Q8_LINEAR, r.records, L.wo, a.x2, 1, d, d, DJ_LIN_RESIDUAL | DJ_LIN_ATTN_MERGE, hd, -1, -1, a.x);
         wo_done = true;
     } else {
-        emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
+        if (!rope_fused) emit(s, DJ_OP_ROPE_KV_STORE, a.qkv, a.q, r.kc, r.vc, r.state, r.cos_t, r.sin_t, S, H, hd, c.max_seq, l);
         emit(s, DJ_OP_ATTENTION, a.q, r.kc, r.vc, a.att, r.state, r.scratch, S, H, hd, c.max_seq, l);
     }
     if (!wo_done) q8_linear(s, a.att, L.wo, a.x2, S, d, d, DJ_LIN_RESIDUAL, -1, -1, -1, a.x);

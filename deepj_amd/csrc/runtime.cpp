@@ -237,6 +237,7 @@ int stride_of(int op) {
         case DJ_OP_STREAM_READ: return 4;
         case DJ_OP_NOP: return 2;
         case DJ_OP_Q8_PREPARE: return 5;
+        case DJ_OP_Q8_LINEAR_ROPE: return 20;
         default: return -1;
     }
 }
@@ -472,6 +473,49 @@ void exec_one(Cursor &c) {
             // One rule for the allocation-free entry point, whatever happens to fit its fixed array: the many-row
             // fp16 GEMM (whose operands live in a workspace sized by the shape) is never taken there.
             p.small_workspace_only = g.no_alloc;
+            if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
+            break;
+        }
+        case DJ_OP_Q8_LINEAR_ROPE: {
+            // [op, x, weight, qOut, M, K, d, flags, gamma, bias, beta, kCache, vCache, state, cos, sin, H, hd, maxSeq, layer]
+            const int64_t m = w[4], k = w[5], d = w[6], H = w[16], hd = w[17], max_seq = w[18], layer = w[19];
+            const int flags = w[7];
+            if (m <= 1 || k <= 0 || d <= 0 || H <= 0 || hd <= 0 || (hd & 3) || H * hd != d || max_seq <= 0 || layer < 0)
+                fail("OP_Q8_LINEAR_ROPE: bad shape");
+            if (flags & ~(DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM | DJ_LIN_BIAS)) fail("OP_Q8_LINEAR_ROPE: only a norm prologue and a bias go with it");
+            const bool ln = flags & DJ_LIN_LAYERNORM;
+            if (ln && (flags & DJ_LIN_RMSNORM)) fail("OP_Q8_LINEAR_ROPE: RMSNORM and LAYERNORM are exclusive");
+            if (g.no_alloc || !q8_gemm_f16_rope_ok((int)m, (int)d, (int)k))
+                fail("OP_Q8_LINEAR_ROPE: this shape does not run on the fp16 GEMM (deepj_hip_q8_linear_rope_ok); use Q8_LINEAR + ROPE_KV_STORE");
+            const int64_t rows = 3 * d, per_layer = H * max_seq * hd;
+            Q8Linear p;
+            p.x = buf(w[1], m * k, op, "x");
+            const float *wq = buf(w[2], (q8_bytes((int)k, (int)rows) + 3) / 4, op, "weight");
+            p.wq = reinterpret_cast<const int8_t *>(wq);
+            p.scales = reinterpret_cast<const float *>(p.wq + q8_scale_offset_bytes((int)k, (int)rows));
+            p.out = nullptr;
+            p.m = (int)m; p.k = (int)k; p.n = (int)rows; p.flags = flags;
+            p.gamma = (flags & (DJ_LIN_RMSNORM | DJ_LIN_LAYERNORM)) ? buf(w[8], k, op, "gamma") : nullptr;
+            p.bias = (flags & DJ_LIN_BIAS) ? buf(w[9], rows, op, "bias") : nullptr;
+            p.beta = ln ? buf(w[10], k, op, "beta") : nullptr;
+            p.bias2 = nullptr; p.residual = nullptr;
+            p.rope.q = buf(w[3], m * d, op, "qOut");
+            p.rope.k_cache = buf(w[11], (layer + 1) * per_layer, op, "kCache") + layer * per_layer;
+            p.rope.v_cache = buf(w[12], (layer + 1) * per_layer, op, "vCache") + layer * per_layer;
+            p.rope.state = reinterpret_cast<const int32_t *>(buf(w[13], 4, op, "state"));
+            p.rope.cos_t = buf(w[14], max_seq * (hd / 2), op, "cos");
+            p.rope.sin_t = buf(w[15], max_seq * (hd / 2), op, "sin");
+            p.rope.hd = (int)hd; p.rope.d = (int)d; p.rope.max_seq = (int)max_seq;
+            auto pit = g.prepared.find(w[2]);
+            if (pit != g.prepared.end() && pit->second.k == k && pit->second.rows == rows)
+                p.prepared = buf(pit->second.id, q8_prepared_floats((int)k, (int)rows), op, "prepared weights");
+            if (p.prepared && run && g.capture_into) {
+                const std::pair<int32_t, int32_t> pr(w[2], pit->second.id);
+                auto &own = g.capture_into->self_prepared;
+                if (std::find(own.begin(), own.end(), pr) == own.end()) g.capture_into->prepared.push_back(pr);
+            }
+            const int64_t ws = q8_linear_preferred_workspace_floats((int)m, (int)k, (int)rows, flags, p.prepared != nullptr);
+            if (c.dry) c.ws_need = std::max(c.ws_need, ws);
             if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
             break;
         }
@@ -779,6 +823,7 @@ const char *op_name(int op) {
         case DJ_OP_SILU_MUL: return "OP_SILU_MUL";
         case DJ_OP_EMBED_GATHER: return "OP_EMBED_GATHER";
         case DJ_OP_ROPE_KV_STORE: return "OP_ROPE_KV_STORE";
+        case DJ_OP_Q8_LINEAR_ROPE: return "OP_Q8_LINEAR_ROPE";
         case DJ_OP_ATTENTION: return "OP_ATTENTION";
         case DJ_OP_ARGMAX_ROWS: return "OP_ARGMAX_ROWS";
         case DJ_OP_DECODE_ADVANCE: return "OP_DECODE_ADVANCE";
@@ -1019,6 +1064,11 @@ void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_ro
     if (tile_rows) *tile_rows = tr;
     if (tile_cols) *tile_cols = tc;
     if (k_shares) *k_shares = ks;
+}
+
+int32_t deepj_hip_q8_linear_rope_ok(int32_t m, int32_t k, int32_t d) {
+    if (m <= 1 || k <= 0 || d <= 0) return 0;
+    return q8_gemm_f16_rope_ok(m, d, k) ? 1 : 0;
 }
 
 int32_t deepj_hip_q8_gemm_f16_extents(int32_t m, int32_t k, int32_t rows, int32_t tile_rows, int32_t tile_cols, int64_t *reach3, int64_t *size3) {

@@ -143,6 +143,15 @@ class Stream:
     def stream_read(self, src, sink, n): return self.emit(op.OP_STREAM_READ, src, sink, n)
     def nop(self, grid=1): return self.emit(op.OP_NOP, grid)
     def q8_prepare(self, w, prepared, k, rows): return self.emit(op.OP_Q8_PREPARE, w, prepared, k, rows)
+
+    def q8_linear_rope(self, x, w, q_out, m, k, d, k_cache, v_cache, state, cos, sin, H, hd, max_seq, layer, *, gamma=-1,
+                       bias=-1, beta=-1):
+        """The q | k | v projection (weight rows 3 d) with ROPE_KV_STORE as its epilogue (HipNative.q8LinearRopeOk says
+        for which shapes)."""
+        layernorm = beta >= 0
+        flags = ((op.LIN_LAYERNORM if layernorm else (op.LIN_RMSNORM if gamma >= 0 else 0)) | (op.LIN_BIAS if bias >= 0 else 0))
+        return self.emit(op.OP_Q8_LINEAR_ROPE, x, w, q_out, m, k, d, flags, gamma, bias, beta, k_cache, v_cache, state, cos, sin,
+                         H, hd, max_seq, layer)
     def matmul(self, a, b, out, m, n, k): return self.emit(op.OP_MATMUL, a, b, out, m, n, k)
 
     # execution -----------------------------------------------------------------

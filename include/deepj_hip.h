@@ -202,13 +202,21 @@ enum {
      *     to, or the destination of Q8_QUANTIZE / COPY / FILL - the ways Q8 data gets into a buffer; an op that writes
      *     floats over a Q8 weight (which no longer is one then) does not end it.  A graph captured before that keeps the
      *     copy it was captured with.  Results are the same with and without it.
+     * Q8_LINEAR_ROPE [op, x, weight, qOut, M, K, d, flags, gamma, bias, beta, kCache, vCache, state, cos, sin, H, hd, maxSeq, layer]
+     *     The fused q | k | v projection of a prompt (weight rows 3 d = 3 H hd, flags RMSNORM / LAYERNORM / BIAS as in
+     *     Q8_LINEAR) with ROPE_KV_STORE as its epilogue: row r is the token at position state[0] + r; its queries go
+     *     rotated to qOut [M x d], its keys rotated and its values as they are into the caches of `layer` - one launch
+     *     and one pass over the [M x 3 d] product less than Q8_LINEAR followed by ROPE_KV_STORE, same results to the
+     *     last bit or two of the rotation.  Only for shapes the fp16 GEMM takes with an unshared K
+     *     (deepj_hip_q8_linear_rope_ok(M, K, d) != 0) and not through deepj_hip_flush_ops_noalloc; refused otherwise.
      */
     DJ_OP_Q8_QUANTIZE = 64, DJ_OP_Q8_DEQUANTIZE = 65, DJ_OP_Q8_LINEAR = 66, DJ_OP_RMSNORM = 67,
     DJ_OP_SILU_MUL = 68, DJ_OP_EMBED_GATHER = 69, DJ_OP_ROPE_KV_STORE = 70, DJ_OP_ATTENTION = 71,
     DJ_OP_ARGMAX_ROWS = 72, DJ_OP_DECODE_ADVANCE = 73, DJ_OP_COPY = 74, DJ_OP_FILL = 75,
     DJ_OP_ROPE_ROWS = 76, DJ_OP_ATTENTION_KV = 77, DJ_OP_DECODE_NEXT = 78, DJ_OP_ATTN_DECODE = 79,
     DJ_OP_APPEND_ROWS = 80, DJ_OP_Q8_LINEAR_DYN = 81, /* 82 unused */ DJ_OP_LAYERNORM = 83,
-    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85, DJ_OP_STREAM_READ = 86, DJ_OP_NOP = 87, DJ_OP_Q8_PREPARE = 88
+    DJ_OP_ADD_POSITIONS = 84, DJ_OP_ATTN_DECODE_RECORDS = 85, DJ_OP_STREAM_READ = 86, DJ_OP_NOP = 87, DJ_OP_Q8_PREPARE = 88,
+    DJ_OP_Q8_LINEAR_ROPE = 89
 };
 
 enum { DJ_LIN_RMSNORM = 1, DJ_LIN_BIAS = 2, DJ_LIN_RESIDUAL = 4, DJ_LIN_SWIGLU = 8, DJ_LIN_LAYERNORM = 16,
@@ -229,6 +237,9 @@ int64_t deepj_hip_q8_floats(int32_t k, int32_t rows);
  * No counterpart in the reference, whose weights are fp32 (J/layers/Linear.java:9-24). */
 int64_t deepj_hip_q8_prepared_floats(int32_t k, int32_t rows);
 int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);
+/* 1 when Q8_LINEAR_ROPE takes a projection of M rows over K inputs to 3 d outputs, 0 when the caller has to record
+ * Q8_LINEAR and ROPE_KV_STORE instead */
+int32_t deepj_hip_q8_linear_rope_ok(int32_t m, int32_t k, int32_t d);
 /* the same with the tile's columns (256 or 192) and the number of workgroups that share a tile's K (1: none) */
 void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares);
 /* Host arithmetic only (no GPU call): the last byte + 1 that the fp16 GEMM's direct global -> LDS loads reach in its three

@@ -355,3 +355,62 @@ def test_graph_with_prepared_weights_is_refused_once_the_weights_change(dev):
         HipNative.graphDestroy(uses_copy)
         HipNative.graphDestroy(own_copy)
     dev.release(src, wq, xb, ob, prep)
+
+
+@pytest.mark.parametrize("m,k,H,hd,norm", [(512, 2048, 32, 64, "rms"), (300, 512, 24, 128, "layer"), (260, 384, 96, 32, None)])
+def test_qkv_projection_with_rope_and_cache_append_as_its_epilogue(dev, m, k, H, hd, norm):
+    """OP_Q8_LINEAR_ROPE against OP_Q8_LINEAR followed by OP_ROPE_KV_STORE on the same buffers: rotated queries, the
+    rows appended to both caches of the layer (and nothing else in them touched), from a position inside the cache."""
+    d, max_seq, layers, layer, pos0 = H * hd, 640, 2, 1, 37
+    assert HipNative.q8LinearRopeOk(m, k, d)
+    x = JavaRandom(71).tensor(m, k, 1.0)
+    w = JavaRandom(72).tensor(k, 3 * d, 0.05)
+    b = JavaRandom(73).tensor(1, 3 * d, 0.2)
+    gamma = (1.0 + JavaRandom(74).tensor(1, k, 0.1)).astype(np.float32)
+    beta = JavaRandom(75).tensor(1, k, 0.1)
+    cos, sin = ref.rope_tables(hd, max_seq)
+    wq, _ = quantised(dev, w)
+    xb, bb, gb, beb = dev.upload(x), dev.upload(b), dev.upload(gamma), dev.upload(beta)
+    cos_b, sin_b = dev.upload(cos), dev.upload(sin)
+    state = dev.upload(np.array([pos0, 0, 0, 0], np.int32))
+    kw = {"bias": bb}
+    if norm == "rms":
+        kw["gamma"] = gb
+    elif norm == "layer":
+        kw["gamma"], kw["beta"] = gb, beb
+    cache_floats = layers * H * max_seq * hd
+    results = []
+    for fused in (False, True):
+        kc, vc, qo = dev.alloc(cache_floats), dev.alloc(cache_floats), dev.alloc(m * d)
+        Stream().fill(kc, 0x40400000, cache_floats).fill(vc, 0x40800000, cache_floats).fill(qo, 0, m * d).run()
+        if fused:
+            Stream().q8_linear_rope(xb, wq, qo, m, k, d, kc, vc, state, cos_b, sin_b, H, hd, max_seq, layer, **kw).run()
+        else:
+            qkv = dev.alloc(m * 3 * d)
+            Stream().q8_linear(xb, wq, qkv, m, k, 3 * d, **kw).rope_kv_store(qkv, qo, kc, vc, state, cos_b, sin_b, m, H, hd, max_seq, layer).run()
+            dev.release(qkv)
+        results.append((dev.download(qo, (m, d)), dev.download(kc, (layers, H, max_seq, hd)), dev.download(vc, (layers, H, max_seq, hd))))
+        dev.release(kc, vc, qo)
+    (q0, k0, v0), (q1, k1, v1) = results
+    assert np.array_equal(v0, v1)                                         # values are stored as they are
+    assert_close(q0, q1, atol=1e-6, rtol=1e-6, what="rotated queries")
+    assert_close(k0, k1, atol=1e-6, rtol=1e-6, what="key cache")
+    assert np.all(k1[0] == 3.0) and np.all(v1[0] == 4.0)                  # the other layer is untouched
+    assert np.all(k1[1][:, :pos0] == 3.0) and np.all(k1[1][:, pos0 + m:] == 3.0)
+    assert np.all(v1[1][:, :pos0] == 4.0) and np.all(v1[1][:, pos0 + m:] == 4.0)
+    dev.release(xb, bb, gb, beb, cos_b, sin_b, state, wq)
+
+
+def test_rope_epilogue_is_refused_where_the_fp16_gemm_is_not_taken(dev):
+    m, k, H, hd = 64, 256, 4, 64                                           # too few rows for the fp16 GEMM
+    d, max_seq = H * hd, 128
+    assert not HipNative.q8LinearRopeOk(m, k, d)
+    wq, _ = quantised(dev, JavaRandom(76).tensor(k, 3 * d, 0.05))
+    cos, sin = ref.rope_tables(hd, max_seq)
+    xb, qo = dev.upload(JavaRandom(77).tensor(m, k, 1.0)), dev.alloc(m * d)
+    kc, vc = dev.alloc(H * max_seq * hd), dev.alloc(H * max_seq * hd)
+    state, cos_b, sin_b = dev.upload(np.zeros(4, np.int32)), dev.upload(cos), dev.upload(sin)
+    with pytest.raises(RuntimeError, match="does not run on the fp16 GEMM"):
+        Stream().q8_linear_rope(xb, wq, qo, m, k, d, kc, vc, state, cos_b, sin_b, H, hd, max_seq, 0).run()
+    with pytest.raises(RuntimeError, match="bad shape"):
+        Stream().q8_linear_rope(xb, wq, qo, 512, k, d, kc, vc, state, cos_b, sin_b, H + 1, hd, max_seq, 0).run()
