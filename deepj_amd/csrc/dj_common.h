@@ -108,6 +108,15 @@ void launch_argmax_rows(hipStream_t s, const float *a, int32_t *out, int rows, i
 void launch_matmul_f32(hipStream_t s, const float *a, const float *b, float *out, int m, int n, int k);
 
 // kernels_q8.hip
+// Two consecutive fp16 GEMMs of a stream, the second normalising (RMSNorm) and multiplying the first one's output: when
+// the first shares its tiles' K among workgroups, the kernel that adds their partial products also writes the second
+// one's activations in its layout, and the second skips its own split.
+struct GemmChain {
+    const float *next_gamma = nullptr;   // to the first launch: the gain the next GEMM normalises this output with
+    bool left_planes = false;            // from the first launch: it left the next GEMM's activations in the workspace
+    bool planes_ready = false;           // to the second launch: they are there
+};
+
 struct Q8Linear {
     const float *x; const int8_t *wq; const float *scales; float *out;
     int m, k, n, flags;
@@ -117,6 +126,7 @@ struct Q8Linear {
     const int32_t *m_dev = nullptr;   // GEMM path only: live row count = min(m, m_dev[0] + m_extra)
     int m_extra = 0;
     const float *prepared = nullptr;  // the weights in the fp16 GEMM's layout (launch_q8_prepare), or null: converted per call
+    GemmChain *chain = nullptr;       // fp16 GEMM only
     RopeStore rope;                   // fp16 GEMM only: out = nullptr, the q | k | v row goes through RoPE to q and the caches
     bool small_workspace_only = false; // the caller's workspace cannot grow: stay on the kernels that need M * K floats at most
 };
@@ -147,7 +157,7 @@ void launch_q8_prepare(hipStream_t s, const int8_t *wq, const float *scales, flo
 void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
                         const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
                         const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats,
-                        const RopeStore *rope = nullptr);
+                        const RopeStore *rope = nullptr, GemmChain *chain = nullptr);
 bool q8_gemm_f16_rope_ok(int m, int d, int k);
 
 // kernels_attn.hip

@@ -529,10 +529,16 @@ __global__ void __launch_bounds__(256) k_sum_partials(const float *__restrict__ 
 // (the weights' padding is zero as well, but 0 x garbage could be a NaN).  The grid covers the rows the GEMM's tiles
 // read, which may go past m: those rows only feed output rows that are never stored, and are written as zeros so that
 // the GEMM never multiplies what an earlier user of the workspace left there.
-template <int NORM>
+// SUM: the row is not read from x but put together first - the sum over `splits` slabs of partial products of a
+// K-sharing GEMM, plus bias and residual in the order that GEMM's own epilogue uses - and written to sum_out as that
+// GEMM's result; what follows is the next GEMM's prologue on it.  One kernel where the two GEMMs would otherwise launch
+// one each (the sum of the slabs, the split of the rows).  Rows that fit the register path only.
+struct SplitSum { const float *partial; int splits; int64_t slab; const float *bias, *residual; float *sum_out; };
+
+template <int NORM, bool SUM = false>
 __global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
                                                    uint16_t *__restrict__ planes, float *__restrict__ unscale, int m, int k, int kp, int pitch,
-                                                   int64_t plane_elems) {
+                                                   int64_t plane_elems, const SplitSum sum) {
 #pragma clang fp contract(off)
     __shared__ float red[4];
     const int row = blockIdx.x, t = threadIdx.x;
@@ -571,7 +577,7 @@ __global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, 
     };
     uint16_t *hi = planes + (int64_t)row * pitch, *lo = hi + plane_elems;
     constexpr int NV = 8;                                            // 128-bit words a thread keeps of one row
-    if ((k & 3) == 0 && k == kp && k <= 256 * 4 * NV) {
+    if (SUM || ((k & 3) == 0 && k == kp && k <= 256 * 4 * NV)) {
         // the row stays in registers: one pass over memory
         const int n4 = k >> 2;
         const float4 *row4 = reinterpret_cast<const float4 *>(xr);
@@ -580,6 +586,30 @@ __global__ void __launch_bounds__(256) k_split_f16(const float *__restrict__ x, 
 #pragma unroll
         for (int j = 0; j < NV; j++) {
             const int i = t + j * 256;
+            if constexpr (SUM) {
+                v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (i < n4) {
+                    const float4 *p4 = reinterpret_cast<const float4 *>(sum.partial + (int64_t)row * k) + i;
+                    float4 a = *p4;
+                    for (int z = 1; z < sum.splits; z++) {
+                        const float4 q = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p4) + (int64_t)z * sum.slab);
+                        a.x += q.x; a.y += q.y; a.z += q.z; a.w += q.w;
+                    }
+                    if (sum.bias) {
+                        const float4 b = reinterpret_cast<const float4 *>(sum.bias)[i];
+                        a.x = a.x + b.x; a.y = a.y + b.y; a.z = a.z + b.z; a.w = a.w + b.w;
+                    }
+                    if (sum.residual) {
+                        const float4 r = reinterpret_cast<const float4 *>(sum.residual + (int64_t)row * k)[i];
+                        a.x = r.x + a.x; a.y = r.y + a.y; a.z = r.z + a.z; a.w = r.w + a.w;
+                    }
+                    reinterpret_cast<float4 *>(sum.sum_out + (int64_t)row * k)[i] = a;
+                    v[j] = a;
+                }
+                if (NORM == 1) s1 += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+                if (NORM == 2) s1 += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+                continue;
+            }
             v[j] = i < n4 ? row4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
             if (NORM == 1) s1 += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
             if (NORM == 2) s1 += (v[j].x + v[j].y) + (v[j].z + v[j].w);
@@ -807,7 +837,7 @@ void q8_gemm_f16_configure() {
 void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const float *beta, const int8_t *wq, const float *scales,
                         const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
                         const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats,
-                        const RopeStore *rope) {
+                        const RopeStore *rope, GemmChain *chain) {
     if (!q8_gemm_f16_shape_ok(m, n_rows, k)) fail("q8_gemm_f16: shape outside this kernel's range");
     if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
@@ -824,7 +854,9 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
     // gamma alone: RMSNorm of the rows first; gamma and beta: LayerNorm
     auto split = !gamma ? k_split_f16<0> : beta ? k_split_f16<2> : k_split_f16<1>;
     // (the helpers are ordinary launches: per-kernel timing of this op, launch_kernel's business, is the GEMM's)
-    launch_kernel(split, dim3(m_read), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch);
+    // (a K-sharing GEMM right before this one may have left these rows here already: GemmChain)
+    if (!(chain && chain->planes_ready))
+        launch_kernel(split, dim3(m_read), dim3(256), 0, s, x, gamma, beta, planes, unscale, m, k, kp, pitch, (int64_t)m_pad * pitch, SplitSum{});
     if (!prepared) {
         launch_q8_prepare(s, wq, scales, w, k, n_rows);
         prepared = w;
@@ -847,7 +879,20 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
             if (roped) launch_kernel((k_gemm_q8_f16_m64<4, true>), grid, dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
             else launch_kernel((k_gemm_q8_f16_m64<4>), grid, dim3(256), (size_t)kStages * stage64_bytes(4), s, a);
         }
-        if (plan.splits > 1) {
+        // The next GEMM of the stream normalises this one's output (RMSNorm) and runs on these kernels too: the sum of
+        // the K shares and that GEMM's activation split are one row-wise kernel, which leaves the planes where the next
+        // launch looks for them - at the start of the workspace, below this launch's slabs.
+        const int kp_next = q8_padded_k(n_rows);
+        const int64_t next_floats = round_up((int64_t)m_pad * (kp_next + 64), 64) + round_up(m_pad, 64);
+        if (plan.splits > 1 && chain && chain->next_gamma && !gelu && !swiglu && !interleaved_bias && (n_rows & 3) == 0 &&
+            n_rows == kp_next && n_rows <= 8192 && w - workspace >= next_floats) {
+            uint16_t *planes_next = reinterpret_cast<uint16_t *>(workspace);
+            float *unscale_next = workspace + round_up((int64_t)m_pad * (kp_next + 64), 64);
+            launch_kernel((k_split_f16<1, true>), dim3(m_pad), dim3(256), 0, s, (const float *)nullptr, chain->next_gamma, (const float *)nullptr,
+                          planes_next, unscale_next, m, n_rows, kp_next, kp_next + 64, (int64_t)m_pad * (kp_next + 64),
+                          SplitSum{w, plan.splits, (int64_t)m * n_rows, bias, residual, out});
+            chain->left_planes = true;
+        } else if (plan.splits > 1) {
             const int64_t mn4 = (int64_t)m * n_rows / 4;
             launch_kernel(k_sum_partials, dim3((unsigned)std::min<int64_t>((mn4 + 255) / 256, 4096)), dim3(256), 0, s, (const float *)w, out, plan.splits,
                                mn4, n_rows / 4, a.ep);

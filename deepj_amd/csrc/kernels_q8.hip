@@ -731,7 +731,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     if (!p.m_dev && !p.small_workspace_only && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
         launch_q8_gemm_f16(s, p.x, gamma, beta, p.wq, p.scales, p.prepared, p.out, p.m, p.k, n_rows, bias, swiglu ? bias2 : nullptr,
                            swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, workspace, workspace_floats,
-                           rope ? &p.rope : nullptr);
+                           rope ? &p.rope : nullptr, p.chain);
         return;
     }
     if (rope) fail("q8_linear: the RoPE epilogue exists on the fp16 GEMM only (deepj_hip_q8_linear_rope_ok says for which shapes)");

@@ -64,6 +64,9 @@ struct Runtime {
     int32_t next_graph = 1;
     unsigned *attn_counters = nullptr;             // kAttnCounterHeads zeroed words: decode attention's split arrivals
     unsigned char *static_scratch = nullptr;       // device address of `scratch` below on g.device
+    // Set by a K-sharing fp16 GEMM that also wrote the activations of the op right behind it in that op's layout
+    // (GemmChain): which op of which stream, reading which buffer through which gain.  Good for that one op only.
+    struct ChainSlot { const int32_t *cmd = nullptr; int32_t pos = -1, x_id = -1, gamma_id = -1; int64_t m = 0, k = 0; bool valid = false; } chain;
     bool no_alloc = false;                         // inside deepj_hip_flush_ops_noalloc: nothing may allocate
     std::vector<std::pair<int32_t, void *>> *track = nullptr;   // graph capture: buffers the dry pass resolves
     Graph *capture_into = nullptr;                               // graph capture: the graph the run pass records for
@@ -268,6 +271,13 @@ void exec_one(Cursor &c) {
     const int op = w[0];
     hipStream_t s = g.stream;
     const bool run = !c.dry;
+    const Runtime::ChainSlot was = g.chain;
+    if (run) g.chain.valid = false;
+    // this op is the one a GemmChain's first launch prepared the activations of (x, gain, shape as it saw them)
+    auto chained = [&](int32_t x_id, int32_t gamma_id, int flags, int64_t m, int64_t k) {
+        return run && was.valid && was.cmd == c.cmd && was.pos == c.pos && was.x_id == x_id && was.gamma_id == gamma_id && was.m == m &&
+               was.k == k && (flags & DJ_LIN_RMSNORM) && !(flags & DJ_LIN_LAYERNORM);
+    };
     switch (op) {
         case DJ_OP_ADD: case DJ_OP_SUBTRACT: case DJ_OP_MULTIPLY: case DJ_OP_DIVIDE: case DJ_OP_RELU_BACKWARD:
         case DJ_OP_GELU_BACKWARD: {
@@ -473,7 +483,32 @@ void exec_one(Cursor &c) {
             // One rule for the allocation-free entry point, whatever happens to fit its fixed array: the many-row
             // fp16 GEMM (whose operands live in a workspace sized by the shape) is never taken there.
             p.small_workspace_only = g.no_alloc;
+            GemmChain chain;
+            int32_t next_gamma_id = -1;
+            const int32_t next_pos = c.pos + stride_of(op);
+            if (run && m > 1 && !g.no_alloc && !merge) {
+                chain.planes_ready = chained(w[1], w[8], flags, m, k);
+                // the op right behind this one normalises this output (RMSNorm) and multiplies it on the fp16 GEMM: the
+                // launch may leave that op's activations ready (it does when this one shares its tiles' K)
+                if (next_pos < c.len && !sw) {
+                    const int32_t *nw = c.cmd + next_pos;
+                    const bool n_rope = nw[0] == DJ_OP_Q8_LINEAR_ROPE;
+                    if ((nw[0] == DJ_OP_Q8_LINEAR || n_rope) && nw[1] == w[3] && nw[4] == m && nw[5] == n && (nw[7] & DJ_LIN_RMSNORM) &&
+                        !(nw[7] & (DJ_LIN_LAYERNORM | DJ_LIN_ATTN_MERGE))) {
+                        const int64_t n_rows = n_rope ? 3 * (int64_t)nw[6] : ((nw[7] & DJ_LIN_SWIGLU) ? 2 * (int64_t)nw[6] : (int64_t)nw[6]);
+                        if (n_rows > 0 && n_rows < (1 << 30) && (n_rope ? q8_gemm_f16_rope_ok((int)m, nw[6], (int)n) : q8_gemm_f16_shape_ok((int)m, (int)n_rows, (int)n))) {
+                            next_gamma_id = nw[8];
+                            chain.next_gamma = buf(next_gamma_id, n, op, "the next op's gamma");
+                        }
+                    }
+                }
+                p.chain = &chain;
+            }
             if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
+            if (chain.left_planes) {
+                g.chain.cmd = c.cmd; g.chain.pos = next_pos; g.chain.x_id = w[3]; g.chain.gamma_id = next_gamma_id;
+                g.chain.m = m; g.chain.k = n; g.chain.valid = true;
+            }
             break;
         }
         case DJ_OP_Q8_LINEAR_ROPE: {
@@ -516,6 +551,9 @@ void exec_one(Cursor &c) {
             }
             const int64_t ws = q8_linear_preferred_workspace_floats((int)m, (int)k, (int)rows, flags, p.prepared != nullptr);
             if (c.dry) c.ws_need = std::max(c.ws_need, ws);
+            GemmChain chain;
+            chain.planes_ready = chained(w[1], w[8], flags, m, k);
+            p.chain = &chain;
             if (run) launch_q8_linear(s, p, g.workspace, g.workspace_floats);
             break;
         }
