@@ -414,3 +414,51 @@ def test_rope_epilogue_is_refused_where_the_fp16_gemm_is_not_taken(dev):
         Stream().q8_linear_rope(xb, wq, qo, m, k, d, kc, vc, state, cos_b, sin_b, H, hd, max_seq, 0).run()
     with pytest.raises(RuntimeError, match="bad shape"):
         Stream().q8_linear_rope(xb, wq, qo, 512, k, d, kc, vc, state, cos_b, sin_b, H + 1, hd, max_seq, 0).run()
+
+
+def test_a_shared_k_gemm_prepares_the_next_normalised_gemm_without_changing_a_bit(dev):
+    """Two consecutive ops, the second an RMSNorm'd projection of the first one's output: in one stream the first op's
+    sum kernel also writes the second's activation planes (one dispatch instead of two); run as two separate streams
+    each op does its own part.  Same bits either way, for a plain and a q | k | v + RoPE second op."""
+    m, d, dff, H, hd, max_seq = 512, 2048, 1024, 32, 64, 600
+    assert HipNative.q8GemmTile(m, d, d)[2] > 1
+    x = JavaRandom(81).tensor(m, d, 1.0)
+    res = JavaRandom(82).tensor(m, d, 1.0)
+    gamma = (1.0 + JavaRandom(83).tensor(1, d, 0.1)).astype(np.float32)
+    bias = JavaRandom(84).tensor(1, d, 0.2)
+    w1, _ = quantised(dev, JavaRandom(85).tensor(d, d, 0.03))
+    w2, _ = quantised(dev, JavaRandom(86).tensor(d, 2 * dff, 0.03))
+    w3, _ = quantised(dev, JavaRandom(87).tensor(d, 3 * d, 0.03))
+    cos, sin = ref.rope_tables(hd, max_seq)
+    xb, rb, gb, bb = dev.upload(x), dev.upload(res), dev.upload(gamma), dev.upload(bias)
+    cos_b, sin_b, state = dev.upload(cos), dev.upload(sin), dev.upload(np.array([5, 0, 0, 0], np.int32))
+    mid, out, qo = dev.alloc(m * d), dev.alloc(m * dff), dev.alloc(m * d)
+    kc, vc = dev.alloc(H * max_seq * hd), dev.alloc(H * max_seq * hd)
+
+    first = Stream().q8_linear(xb, w1, mid, m, d, d, bias=bb, residual=rb)
+    second = Stream().q8_linear(mid, w2, out, m, d, dff, gamma=gb, swiglu=True)
+    second_rope = Stream().q8_linear_rope(mid, w3, qo, m, d, d, kc, vc, state, cos_b, sin_b, H, hd, max_seq, 0, gamma=gb)
+
+    first.run(); second.run(); second_rope.run()
+    want = (dev.download(mid, (m, d)), dev.download(out, (m, dff)), dev.download(qo, (m, d)), dev.download(kc, (H, max_seq, hd)))
+    for buf_id, n in ((mid, m * d), (out, m * dff), (qo, m * d)):
+        Stream().fill(buf_id, 0, n).run()
+    both = Stream()
+    both.words = first.words + second.words
+    both.run()
+    assert np.array_equal(dev.download(mid, (m, d)), want[0]) and np.array_equal(dev.download(out, (m, dff)), want[1])
+    _, _, count = HipNative.profileOps(both.array(), 2, detail=True)
+    # split, weight conversion, GEMM, sum + next split | weight conversion, GEMM, sum (it shares K too) - alone: 4
+    assert list(count) == [4, 3] and list(HipNative.profileOps(second.array(), 2, detail=True)[2]) == [4]
+    Stream().fill(mid, 0, m * d).run()
+    both.words = first.words + second_rope.words
+    both.run()
+    assert np.array_equal(dev.download(mid, (m, d)), want[0]) and np.array_equal(dev.download(qo, (m, d)), want[2])
+    assert np.array_equal(dev.download(kc, (H, max_seq, hd)), want[3])
+    # an op in between, or another gain, and the second op splits its rows itself
+    other = dev.upload((gamma * 1.5).astype(np.float32))
+    both.words = first.words + Stream().q8_linear(mid, w2, out, m, d, dff, gamma=other, swiglu=True).words
+    both.run()
+    with_other = dev.download(out, (m, dff))
+    Stream().q8_linear(mid, w2, out, m, d, dff, gamma=other, swiglu=True).run()
+    assert np.array_equal(dev.download(out, (m, dff)), with_other) and not np.array_equal(with_other, want[1])
