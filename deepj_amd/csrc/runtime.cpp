@@ -816,6 +816,7 @@ void exec_one(Cursor &c) {
 
 void walk(const int32_t *cmd, int32_t len, bool dry, int64_t *ws_need) {
     Cursor c{cmd, len, 0, dry, 0};
+    g.chain.valid = false;          // nothing carries over from an earlier stream (or from one that ended in an error)
     while (c.pos < len) {
         int op = cmd[c.pos];
         int stride = stride_of(op);
@@ -1203,6 +1204,7 @@ int deepj_hip_profile_ops(const int32_t *cmd, int32_t len, int32_t iters, float 
         try {
             for (auto &e : ev) DJ_HIP(hipEventCreate(&e));
             for (int it = 0; it < iters; it++) {
+                g.chain.valid = false;
                 for (int i = 0; i < n; i++) {
                     Cursor c{cmd, len, starts[(size_t)i], false, 0};
                     g_launch_timing.pairs = ev.data() + (size_t)per_op * i;
