@@ -85,6 +85,15 @@ __device__ __forceinline__ void load_to_lds4(const void *base, uint32_t off, uin
 }
 #pragma clang diagnostic pop
 
+// Timeline of one launch, for tuning builds only (-DDJ_TRACE; never in the shipped library): every wavefront leaves
+// 100 MHz time stamps at its start, at its first product, after its K loop and after its epilogue.
+#ifdef DJ_TRACE
+__device__ unsigned long long g_gemm_trace[4 * 16384];
+#define DJ_GSTAMP(i) do { const int wg_ = (blockIdx.z * gridDim.x + blockIdx.x) * 4 + wave; if (lane == 0 && wg_ < 16384) g_gemm_trace[wg_ * 4 + (i)] = wall_clock64(); } while (0)
+#else
+#define DJ_GSTAMP(i) do {} while (0)
+#endif
+
 // Workgroup -> tile.  Workgroups go to the eight XCDs (each with its own L2) round-robin by their linear index, so index L
 // runs on XCD L % 8.  All row tiles of one column tile get indices that agree mod 8: the column tile's weights - the
 // bulk of the traffic - are then fetched into one L2 instead of up to eight.  Groups of eight column tiles; the grid is
@@ -98,10 +107,21 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int 
 
 // One tile row of a wavefront's block: acc[tn][e] is C[row0 + 8 (e / 4) + 4 half + e % 4][col0 + 32 tn + l32], TNW tiles
 // wide.  The 32 x 32 TNW floats go through LDS that belongs to this wavefront alone (16 KB) and come back as rows of
-// float4 (8 TNW lanes per row, two rows per round), which get the row's power of two, bias / GELU / residual or the
-// SwiGLU pairing.
+// float4 (8 TNW lanes per row, two rows per round), which get bias / GELU / residual or the SwiGLU pairing; the row's
+// power of two is applied before the trip through LDS.
+// The powers of two of the 16 rows a lane holds of the tile row at row0 (four runs of four rows): requested together
+// and applied on the way into LDS, so that the row loop holds no load a store would wait for.
+struct RowFactors { float4 run[4]; };
+__device__ __forceinline__ RowFactors load_row_factors(const GemmF16Args &a, int row0, int lane) {
+    RowFactors f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) f.run[j] = *reinterpret_cast<const float4 *>(a.unscale + row0 + 8 * j + 4 * (lane >> 5));
+    return f;
+}
+
 template <int TNW, bool ROPE = false>
 __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stage_f, const float (&acc)[TNW][16], int row0, int col0, int lane) {
+    const RowFactors factors = load_row_factors(a, row0, lane);
     constexpr int W = 32 * TNW, LPR = 8 * TNW;                         // floats per row; lanes per row
     const GemmEpilogue &ep = a.ep;
     const int out_n = ep.swiglu ? a.n >> 1 : a.n;
@@ -109,7 +129,11 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
 #pragma unroll
     for (int tn = 0; tn < TNW; tn++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * W + 32 * tn + l32] = acc[tn][e];
+        for (int e = 0; e < 16; e++) {
+            const float4 u = factors.run[e >> 2];
+            const float us = (e & 3) == 0 ? u.x : (e & 3) == 1 ? u.y : (e & 3) == 2 ? u.z : u.w;
+            stage_f[(8 * (e >> 2) + 4 * half + (e & 3)) * W + 32 * tn + l32] = acc[tn][e] * us;
+        }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     const int rsel = lane / LPR, c4 = lane % LPR;                      // this lane's row of the pair, and its float4 in the row
     const bool active = rsel < 2;
@@ -140,8 +164,6 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
         const int rl = i * 2 + rsel, row = row0 + rl;
         if (!active || row >= a.m || col >= a.n) continue;
         float4 v = *reinterpret_cast<const float4 *>(stage_f + rl * W + c4 * 4);
-        const float us = a.unscale[row];
-        v.x = v.x * us; v.y = v.y * us; v.z = v.z * us; v.w = v.w * us;
         if (ep.bias) { v.x = v.x + b4.x; v.y = v.y + b4.y; v.z = v.z + b4.z; v.w = v.w + b4.w; }
         if constexpr (ROPE) { rope_store(ep.rope, rc, v, row, pos0, tab[i]); continue; }
         if (ep.swiglu) {
@@ -178,6 +200,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
     int m_tile, n_tile;
     if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
+    DJ_GSTAMP(0);
     const int m0 = m_tile * TM, n0 = n_tile * kTn;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
@@ -307,11 +330,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         for (int tn = 0; tn < TNW - 1; tn++) { read_w(0, tn, a0); read_w(1, tn, a0); }
         for (int tn = 0; tn < TNW - 1; tn++) sc[tn] = *reinterpret_cast<const float *>(a0.s + tn * 128);
     }
+    DJ_GSTAMP(1);
     int stage = 0;
     for (int step = 0; step < steps; step++) {
         k_step(step, stage);
         stage = stage == 2 ? 0 : stage + 1;
     }
+    DJ_GSTAMP(2);
     // the last tile's scaling; its scale (the last column of the last step) is still in place
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[1][TNW - 1][e] = fmaf(g[1][e], sc[TNW - 1], acc[1][TNW - 1][e]);
@@ -323,6 +348,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     float *stage_f = reinterpret_cast<float *>(lds + wave * (32 * 128 * 4));
 #pragma unroll
     for (int tm = 0; tm < 2; tm++) store_tile_row<TNW, ROPE>(a, stage_f, acc[tm], m0 + wm * 64 + 32 * tm, n0 + wn * (32 * TNW), lane);
+    DJ_GSTAMP(3);
 }
 
 // The same product on a 64-row workgroup tile, 256 (TNW = 4) or 192 (TNW = 3) columns wide, for problems whose 128-row
@@ -349,6 +375,7 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
     int m_tile, n_tile;
     if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
+    DJ_GSTAMP(0);
     const int m0 = m_tile * TM64, n0 = n_tile * kTn;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
@@ -454,6 +481,7 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     }
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
+    DJ_GSTAMP(1);
     int stage = 0, step = 0;
     for (; step + 1 < steps; step += 2) {
         const int st1 = stage == 2 ? 0 : stage + 1;
@@ -462,6 +490,7 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
         stage = st1 == 2 ? 0 : st1 + 1;
     }
     if (step < steps) k_step(S0{}, step, stage);
+    DJ_GSTAMP(2);
     // the last tile's scaling: the last column of the last step, whose set (and partial-sum register) follow that step's parity
     {
         const bool odd = (steps - 1) & 1;
@@ -479,9 +508,11 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
         b.out = a.partial + (int64_t)blockIdx.z * a.m * a.n;
         b.ep = GemmEpilogue{nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0};
         store_tile_row<TNW>(b, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
+        DJ_GSTAMP(3);
         return;
     }
     store_tile_row<TNW, ROPE>(a, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
+    DJ_GSTAMP(3);
 }
 
 // out = epilogue(sum over the splits of partial[z]) on float4s: bias, GELU, residual or the SwiGLU pairing as in
@@ -905,5 +936,11 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
         else launch_kernel((k_gemm_q8_f16<4>), dim3(grid_x), dim3(256), (size_t)kStages * stage128_bytes(4), s, a);
     }
 }
+
+#ifdef DJ_TRACE
+extern "C" int deepj_hip_debug_gemm_trace(unsigned long long *out, int n) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_gemm_trace), (size_t)n * sizeof(unsigned long long));
+}
+#endif
 
 }  // namespace dj
