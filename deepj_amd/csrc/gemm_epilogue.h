@@ -30,6 +30,17 @@ struct GemmEpilogue {
     RopeStore rope;         // fp16 Q8 GEMM only
 };
 
+// A finished tile of a plain or SwiGLU epilogue leaves with streaming (non-temporal) stores: no workgroup of the launch
+// reads it again, and lines a kernel leaves dirty in an XCD's L2 are written back when the kernel ends, with every
+// compute unit waiting (the prompt's gate/up GEMM at 512 rows: 66.8 -> 65.8 us).  The consumer then reads from HBM
+// rather than from the memory-side cache, which costs it about as much where it is a bandwidth-bound helper kernel (the
+// sum of K shares) and more where it is the attention kernel - so the RoPE epilogue keeps ordinary stores (attention
+// 21.7 -> 23.2 us with streaming ones).  Write-through (agent-scope) stores were slower throughout.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_streaming(float *p, float4 v) { __builtin_nontemporal_store((floatx4){v.x, v.y, v.z, v.w}, reinterpret_cast<floatx4 *>(p)); }
+__device__ __forceinline__ void store_streaming(float *p, float2 v) { __builtin_nontemporal_store((floatx2){v.x, v.y}, reinterpret_cast<floatx2 *>(p)); }
+
 // Where the four columns col .. col + 3 of a q | k | v row go: fixed for a lane over the rows of its tile.
 struct RopeColumn { int region, cc, head, within; };
 __device__ __forceinline__ RopeColumn rope_column(const RopeStore &r, int col) {

@@ -171,7 +171,7 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
             float2 o;
             o.x = v.x * (1.0f / (1.0f + expf(-v.x))) * v.y;
             o.y = v.z * (1.0f / (1.0f + expf(-v.z))) * v.w;
-            *reinterpret_cast<float2 *>(a.out + (int64_t)row * out_n + (col >> 1)) = o;
+            store_streaming(a.out + (int64_t)row * out_n + (col >> 1), o);
             continue;
         }
         if (ep.gelu) { v.x = gemm_gelu(v.x); v.y = gemm_gelu(v.y); v.z = gemm_gelu(v.z); v.w = gemm_gelu(v.w); }
@@ -179,7 +179,7 @@ __device__ __forceinline__ void store_tile_row(const GemmF16Args &a, float *stag
             const float4 r = *reinterpret_cast<const float4 *>(ep.residual + (int64_t)row * a.n + col);
             v.x = r.x + v.x; v.y = r.y + v.y; v.z = r.z + v.z; v.w = r.w + v.w;
         }
-        *reinterpret_cast<float4 *>(a.out + (int64_t)row * a.n + col) = v;
+        store_streaming(a.out + (int64_t)row * a.n + col, v);
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                  // the rows are in registers before anything overwrites them
 }
