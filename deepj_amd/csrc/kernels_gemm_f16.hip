@@ -67,7 +67,7 @@ struct GemmF16Args {
     int m, n, m_pad, n_pad, kp, pitch;
     int m_tiles, n_tiles;       // tiles of the launched kernel's size along M and N
     GemmEpilogue ep;
-    int split_steps;            // 64-row kernel only: K steps per workgroup along blockIdx.z (0: all of K, no partial sums)
+    int split_steps;            // 64-row kernel only: K steps per share of a tile (0: all of K, no partial sums); gridDim.z shares
     float *partial;             // [gridDim.z][m][n] partial products when split_steps > 0
 };
 
@@ -102,6 +102,24 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int 
     const int per_group = 8 * m_tiles, g = blockIdx.x / per_group, r = blockIdx.x % per_group;
     n_tile = g * 8 + (r & 7);
     m_tile = r >> 3;
+    return n_tile < n_tiles;
+}
+
+// The same for a launch whose tiles share K among gridDim.z workgroups (share z takes K steps [z, z + 1) * split_steps).
+// With the mapping above every XCD would run all shares and all row tiles of its column tiles and so fetch ALL activation
+// planes - eight times the planes in all.  When the share count divides eight, an XCD instead takes ONE share and every
+// (8 / shares)-th column tile: it fetches that share's quarter (half, eighth) of the planes and an eighth of the weights,
+// as before.
+__device__ __forceinline__ bool tile_of_share(int m_tiles, int n_tiles, int &m_tile, int &n_tile, int &z) {
+    const int shares = gridDim.z;
+    if (shares == 1 || (8 % shares) != 0) {
+        z = blockIdx.z;
+        return tile_of_workgroup(m_tiles, n_tiles, m_tile, n_tile);
+    }
+    const int idx = blockIdx.z * gridDim.x + blockIdx.x, c = idx & 7, r = idx >> 3;     // gridDim.x is a multiple of 8: XCD c
+    z = c % shares;
+    n_tile = c / shares + (8 / shares) * (r / m_tiles);
+    m_tile = r % m_tiles;
     return n_tile < n_tiles;
 }
 
@@ -373,8 +391,8 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     extern __shared__ __align__(16) unsigned char lds[];
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
-    int m_tile, n_tile;
-    if (!tile_of_workgroup(a.m_tiles, a.n_tiles, m_tile, n_tile)) return;
+    int m_tile, n_tile, share;
+    if (!tile_of_share(a.m_tiles, a.n_tiles, m_tile, n_tile, share)) return;
     DJ_GSTAMP(0);
     const int m0 = m_tile * TM64, n0 = n_tile * kTn;
     const int64_t plane_elems = (int64_t)a.m_pad * a.pitch;
@@ -403,8 +421,8 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     }
     const unsigned char *s_base = reinterpret_cast<const unsigned char *>(a.scales_t) + (int64_t)(n0 + wave * 64) * 4;
     const uint32_t s_dst = kXs64 + kW + wave * 256;
-    // this workgroup's share of K: all of it, or split_steps steps from blockIdx.z * split_steps (a partial product)
-    const int all_steps = a.kp / 32, first = a.split_steps ? (int)blockIdx.z * a.split_steps : 0;
+    // this workgroup's share of K: all of it, or split_steps steps from share * split_steps (a partial product)
+    const int all_steps = a.kp / 32, first = a.split_steps ? share * a.split_steps : 0;
     const int steps = a.split_steps ? min(a.split_steps, all_steps - first) : all_steps, last = first + steps - 1;
     auto load_one = [&](int i, int step, int stage) {
         const uint32_t sb = lds0 + stage * kStage64;
@@ -505,7 +523,7 @@ __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
     if (a.split_steps) {
         // a partial product: the bare sums (times the row's power of two) into this split's slab; k_sum_partials finishes them
         GemmF16Args b = a;
-        b.out = a.partial + (int64_t)blockIdx.z * a.m * a.n;
+        b.out = a.partial + (int64_t)share * a.m * a.n;
         b.ep = GemmEpilogue{nullptr, nullptr, nullptr, 0, nullptr, 0, 0, 0};
         store_tile_row<TNW>(b, stage_f, acc, m0 + wm * 32, n0 + wn * 32 * TNW, lane);
         DJ_GSTAMP(3);
