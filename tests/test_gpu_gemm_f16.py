@@ -77,6 +77,25 @@ def test_plain_product_ragged_shapes(dev, m, k, n, tile):
     assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear M={m} K={k} N={n}")
 
 
+@pytest.mark.parametrize("m,k,n,shares", [(256, 4096, 2048, 8), (512, 2048, 2048, 4), (384, 4096, 2048, 5), (320, 2048, 4096, 3),
+                                           (300, 4096, 2044, 6)])
+def test_every_way_the_shares_of_k_are_dealt_to_the_xcds(dev, m, k, n, shares):
+    """A tile's K shares go to workgroups by one of two rules: share counts that divide eight put one share on each XCD
+    (eight and four here), the others keep every share of a column tile together (six, five and three).  Each must cover every
+    (row tile, column tile, share) exactly once: a tile missed or taken twice shows as a wrong block of the product."""
+    assert HipNative.q8GemmTile(m, k, n) == (64, 256, shares)
+    w = JavaRandom(41).tensor(k, n, 0.02)
+    x = JavaRandom(42).tensor(m, k, 1.0)
+    b = JavaRandom(43).tensor(1, n, 0.3)
+    wq, deq = quantised(dev, w)
+    exp = ref.add_row_vector(ref.matmul(x, deq), b)
+    xb, bb, ob = dev.upload(x), dev.upload(b), dev.alloc(m * n)
+    Stream().q8_linear(xb, wq, ob, m, k, n, bias=bb).run()
+    got = dev.download(ob, (m, n))
+    dev.release(xb, bb, ob, wq)
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear M={m} K={k} N={n}, K shared by {shares}")
+
+
 def test_random_shapes_both_tiles_and_shared_k(dev):
     """Seeded random (M, K, N) over the kernel's whole domain - M not a multiple of 64, K not a multiple of 32, N only a
     multiple of 4 - until each of the three ways the library takes a problem (128-row tiles, 64-row tiles, 64-row tiles
