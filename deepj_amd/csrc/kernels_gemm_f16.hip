@@ -18,7 +18,7 @@
 // (64 x 256 or 64 x 192, further down) for those whose large tiles would leave compute units idle, optionally with a
 // tile's K shared by several workgroups and k_sum_partials adding their partial products in a fixed order;
 // q8_gemm_f16_plan chooses.  A workgroup's tile follows from its index so that the workgroups of one column tile
-// run on one XCD (tile_of_workgroup).
+// run on one XCD (tile_of_workgroup), and those of one K share too where K is shared (tile_of_share).
 //
 // Shape.  Workgroup tile 128 x 256, 256 threads = 4 wavefronts (2 x 2), one wavefront per SIMD; a wavefront owns
 // 64 x 128 of C = 8 MFMA tiles of 32 x 32 = 128 fp32 accumulators per lane, kept in ordinary vector registers because
