@@ -319,8 +319,10 @@ def c2_sweep(iters: int = 10, cpu: bool = True):
                                        ", fp16 x 2) + k_split_f16 + k_q8_to_f16") if tile else "k_gemm_q8 (bf16 x 3)",
                             "flops": flops, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
                             "frac_of_mfma_peak": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4)})
-                if tile:
+                ptile, ptile_cols, pshares = HipNative.q8GemmTilePrepared(m, k, n)
+                if ptile:
                     # with the weight kept in the GEMM's own layout (OP_Q8_PREPARE), as the decode driver keeps them
+                    # (fewer than 256 rows reach the fp16 GEMM only this way)
                     prep = [dev.alloc(HipNative.q8PreparedFloats(k, n)) for _ in use[:2]]
                     ps = Stream()
                     for q, pb in zip(use, prep):
@@ -331,7 +333,8 @@ def c2_sweep(iters: int = 10, cpu: bool = True):
                         prepared.q8_linear(x, q, out, m, k, n)
                     pus = period_us(prepared, len(use[:2]))
                     row.update({"prepared_us": round(pus, 2), "prepared_TFLOPs": round(flops / pus / 1e6, 1),
-                                "prepared_frac_of_mfma_peak": round(flops / pus / 1e6 / MFMA_PEAK_TFLOPS, 4)})
+                                "prepared_frac_of_mfma_peak": round(flops / pus / 1e6 / MFMA_PEAK_TFLOPS, 4),
+                                "prepared_kernel": f"k_gemm_q8_f16 ({ptile} x {ptile_cols} tiles" + (f", K shared by {pshares}" if pshares > 1 else "") + ", fp16 x 2) + k_split_f16"})
                     dev.release(*prep)       # releasing a prepared copy ends its association with the weight
             if ref is not None:
                 reps = 1 if m * k * n > 2e9 else 3      # (the oracle multiplies the fp32 weights, as CpuBackend.matmul does)

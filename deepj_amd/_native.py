@@ -48,6 +48,8 @@ def _bind(lib: C.CDLL) -> None:
     lib.deepj_hip_q8_gemm_path.restype = C.c_int32
     lib.deepj_hip_q8_gemm_tile.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
     lib.deepj_hip_q8_gemm_tile.restype = None
+    lib.deepj_hip_q8_gemm_tile_prepared.argtypes = [C.c_int32, C.c_int32, C.c_int32, _i32p, _i32p, _i32p]
+    lib.deepj_hip_q8_gemm_tile_prepared.restype = None
     lib.deepj_hip_q8_linear_rope_ok.argtypes = [C.c_int32, C.c_int32, C.c_int32]
     lib.deepj_hip_q8_linear_rope_ok.restype = C.c_int32
     lib.deepj_hip_clock_probe.argtypes = [_i32p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
@@ -181,6 +183,13 @@ class HipNative:
         """(tile rows, tile columns, workgroups sharing a tile's K) of the fp16 GEMM for this problem; rows 0: not taken."""
         r, c, s = C.c_int32(), C.c_int32(), C.c_int32()
         library().deepj_hip_q8_gemm_tile(m, k, rows, C.byref(r), C.byref(c), C.byref(s))
+        return r.value, c.value, s.value
+
+    @staticmethod
+    def q8GemmTilePrepared(m: int, k: int, rows: int):
+        """The same for a weight already in the fp16 GEMM's layout (OP_Q8_PREPARE): taken from 16 rows on."""
+        r, c, s = C.c_int32(), C.c_int32(), C.c_int32()
+        library().deepj_hip_q8_gemm_tile_prepared(m, k, rows, C.byref(r), C.byref(c), C.byref(s))
         return r.value, c.value, s.value
 
     @staticmethod

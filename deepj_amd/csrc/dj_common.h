@@ -141,9 +141,9 @@ int64_t q8_linear_workspace_floats(int m, int k, int n, int flags);
 int64_t q8_linear_preferred_workspace_floats(int m, int k, int n, int flags, bool prepared);
 
 // kernels_gemm_f16.hip: the many-row Q8 GEMM on fp16 matrix cores (two-piece activations, direct loads to LDS)
-bool q8_gemm_f16_shape_ok(int m, int n_rows, int k);
-int q8_gemm_f16_tile_rows(int m, int n_rows, int k);   // 128 or 64 rows per workgroup tile, 0: not for these kernels
-void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares);
+bool q8_gemm_f16_shape_ok(int m, int n_rows, int k, bool prepared = false);   // prepared: the weights are in these kernels' layout already (fewer than 256 rows take them only then)
+int q8_gemm_f16_tile_rows(int m, int n_rows, int k, bool prepared = false);   // 128 or 64 rows per workgroup tile, 0: not for these kernels
+void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares, bool prepared = false);
 // bytes the direct loads of a launch with this tile reach in {planes, fp16 weights, transposed scales} and bytes those
 // hold; false when any load would pass its buffer
 bool q8_gemm_f16_extents(int m, int n_rows, int k, int tile_rows, int tile_cols, int64_t reach[3], int64_t size[3]);

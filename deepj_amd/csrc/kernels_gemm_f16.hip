@@ -772,13 +772,32 @@ struct GemmF16Plan { int tile_rows, tile_cols, splits; };
 
 constexpr int kNPad = 768;      // weight rows of a prepared buffer are padded to a multiple of both tile widths
 
-GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
+constexpr int kMinRowsPrepared = 16;     // fewer rows than this stay on the bf16 kernels even with prepared weights
+constexpr int kMinSplitStepsFewRows = 8; // K steps per share below 256 rows (weight streaming counts there, not the tile's fixed cost)
+
+GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k, bool prepared) {
     // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels; =128, =128192, =64 or =192 force the 128 x 256,
     // 128 x 192, 64 x 256 or 64 x 192 tile (for comparisons)
     static const int forced = [] { const char *e = getenv("DEEPJ_HIP_GEMM_F16"); return e ? atoi(e) : -1; }();
     if (forced == 0) return {0, 0, 1};
     // four columns per lane in the epilogue need n_rows % 4 == 0
-    if (m < 256 || (n_rows & 3) != 0 || k < 64) return {0, 0, 1};
+    if ((n_rows & 3) != 0 || k < 64) return {0, 0, 1};
+    // Fewer than 256 rows: only when the weights are already in these kernels' layout (a conversion per call costs more
+    // than the launch gains), on 64-row tiles, and only for wide outputs - where the tiles alone, or with a few shares of
+    // K, make enough workgroups to stream the weights (64 rows x 11008 outputs over K 4096: 28.4 us against 46.6 on the
+    // bf16 kernels; 128 x 11264 over K 2048: 27.5 against 47.6; 192 x 6144: 25.8 against 47.8).  Narrow outputs would need
+    // eight shares, whose partial products cost more than they gain (64 x 2048 over K 2048: 16.4 against 11.6), unless K
+    // is long (255 x 2048 over K 5632: 30.1 against 44.5).
+    if (m < 256) {
+        if (!prepared || m < kMinRowsPrepared || forced > 0) return {0, 0, 1};
+        const int64_t r64 = (m + TM64 - 1) / TM64, tw = r64 * ((n_rows + 255) / 256), tn = r64 * ((n_rows + 191) / 192);
+        const int steps = q8_padded_k(k) / 32;
+        if (!(tn >= 48 || (tn >= 40 && steps >= 128))) return {0, 0, 1};
+        auto shares_of = [&](int64_t tiles) { return tiles >= 256 ? 1 : (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(8, 256 / tiles), steps / kMinSplitStepsFewRows)); };
+        const int sw = shares_of(tw), sn = shares_of(tn);
+        const int64_t wgw = std::min<int64_t>(tw * sw, 256), wgn = std::min<int64_t>(tn * sn, 256);
+        return wgn > wgw ? GemmF16Plan{64, 192, sn} : GemmF16Plan{64, 256, sw};
+    }
     const int64_t rows128 = (m + TM - 1) / TM, rows64 = (m + TM64 - 1) / TM64, cols256 = (n_rows + 255) / 256, cols192 = (n_rows + 191) / 192;
     const int64_t t128 = rows128 * cols256, t128n = rows128 * cols192, t64 = rows64 * cols256, t64n = rows64 * cols192;
     if (forced == 128 || forced == 128192 || forced == 64 || forced == 192) {
@@ -808,15 +827,15 @@ GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k) {
     return {0, 0, 1};
 }
 
-int q8_gemm_f16_tile_rows(int m, int n_rows, int k) { return q8_gemm_f16_plan(m, n_rows, k).tile_rows; }
+int q8_gemm_f16_tile_rows(int m, int n_rows, int k, bool prepared) { return q8_gemm_f16_plan(m, n_rows, k, prepared).tile_rows; }
 // the fused q | k | v projection with RoPE and the cache append as its epilogue: on these kernels, K not shared
 bool q8_gemm_f16_rope_ok(int m, int d, int k) {
-    const GemmF16Plan p = q8_gemm_f16_plan(m, 3 * d, k);
+    const GemmF16Plan p = q8_gemm_f16_plan(m, 3 * d, k, false);      // (256 rows and more: whatever the weights' state)
     return p.tile_rows != 0 && p.splits == 1;
 }
-bool q8_gemm_f16_shape_ok(int m, int n_rows, int k) { return q8_gemm_f16_tile_rows(m, n_rows, k) != 0; }
-void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares) {
-    const GemmF16Plan p = q8_gemm_f16_plan(m, n_rows, k);
+bool q8_gemm_f16_shape_ok(int m, int n_rows, int k, bool prepared) { return q8_gemm_f16_tile_rows(m, n_rows, k, prepared) != 0; }
+void q8_gemm_f16_tile(int m, int n_rows, int k, int *tile_rows, int *tile_cols, int *k_shares, bool prepared) {
+    const GemmF16Plan p = q8_gemm_f16_plan(m, n_rows, k, prepared);
     if (tile_rows) *tile_rows = p.tile_rows;
     if (tile_cols) *tile_cols = p.tile_cols;
     if (k_shares) *k_shares = p.splits;
@@ -834,7 +853,7 @@ int64_t q8_prepared_floats(int k, int n_rows) {
 // floats of workspace: planes, row factors and, unless the caller holds prepared weights, those
 int64_t q8_gemm_f16_workspace_floats(int m, int n_rows, int k, bool prepared) {
     const int64_t kp = q8_padded_k(k), pitch = kp + 64, m_pad = round_up(m, TM);
-    const int splits = q8_gemm_f16_plan(m, n_rows, k).splits;
+    const int splits = q8_gemm_f16_plan(m, n_rows, k, prepared).splits;
     return round_up(m_pad * pitch, 64) + round_up(m_pad, 64) + (prepared ? 0 : q8_prepared_floats(k, n_rows)) +
            (splits > 1 ? round_up((int64_t)splits * m * n_rows, 64) : 0);
 }
@@ -887,11 +906,11 @@ void launch_q8_gemm_f16(hipStream_t s, const float *x, const float *gamma, const
                         const float *prepared, float *out, int m, int k, int n_rows, const float *bias, const float *bias2,
                         const float *residual, int interleaved_bias, int gelu, int swiglu, float *workspace, int64_t workspace_floats,
                         const RopeStore *rope, GemmChain *chain) {
-    if (!q8_gemm_f16_shape_ok(m, n_rows, k)) fail("q8_gemm_f16: shape outside this kernel's range");
+    if (!q8_gemm_f16_shape_ok(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: shape outside this kernel's range");
     if (workspace_floats < q8_gemm_f16_workspace_floats(m, n_rows, k, prepared != nullptr)) fail("q8_gemm_f16: workspace too small");
     if (swiglu && ((n_rows & 1) || residual || gelu)) fail("q8_gemm_f16: the SwiGLU epilogue needs an even row count and takes no residual or GELU");
     const int kp = q8_padded_k(k), pitch = kp + 64, m_pad = (int)round_up(m, TM), n_pad = (int)round_up(n_rows, kNPad);
-    const GemmF16Plan plan = q8_gemm_f16_plan(m, n_rows, k);
+    const GemmF16Plan plan = q8_gemm_f16_plan(m, n_rows, k, prepared != nullptr);
     if (rope && (plan.splits > 1 || swiglu || gelu || residual || n_rows != 3 * rope->d || (rope->hd & 3) || rope->d % rope->hd))
         fail("q8_gemm_f16: the RoPE epilogue needs an unshared K, N = 3 d and no other epilogue than a bias");
     int64_t reach[3], size[3];

@@ -682,7 +682,7 @@ int64_t q8_linear_preferred_workspace_floats(int m, int k, int n, int flags, boo
     const int64_t ws = q8_linear_workspace_floats(m, k, n, flags);
     const int n_rows = (flags & DJ_LIN_SWIGLU) ? 2 * n : n;
     const bool mv = (m == 1) && matvec_supported(k);
-    if (!mv && q8_gemm_f16_shape_ok(m, n_rows, k)) return std::max(ws, q8_gemm_f16_workspace_floats(m, n_rows, k, prepared));
+    if (!mv && q8_gemm_f16_shape_ok(m, n_rows, k, prepared)) return std::max(ws, q8_gemm_f16_workspace_floats(m, n_rows, k, prepared));
     if (!mv) return ws + q8_gemm_workspace_floats(m, n_rows, k);      // the partial products of a K-sharing launch
     return ws;
 }
@@ -728,7 +728,7 @@ void launch_q8_linear(hipStream_t s, const Q8Linear &p, float *workspace, int64_
     // normalisation happens on the rows' way into that layout
     const int n_rows = swiglu ? 2 * p.n : p.n;
     const bool rope = p.rope.q != nullptr;
-    if (!p.m_dev && !p.small_workspace_only && q8_gemm_f16_shape_ok(p.m, n_rows, p.k) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
+    if (!p.m_dev && !p.small_workspace_only && q8_gemm_f16_shape_ok(p.m, n_rows, p.k, p.prepared != nullptr) && workspace_floats >= q8_gemm_f16_workspace_floats(p.m, n_rows, p.k, p.prepared != nullptr)) {
         launch_q8_gemm_f16(s, p.x, gamma, beta, p.wq, p.scales, p.prepared, p.out, p.m, p.k, n_rows, bias, swiglu ? bias2 : nullptr,
                            swiglu ? nullptr : residual, swiglu ? 1 : 0, swiglu ? 0 : gelu, swiglu ? 1 : 0, workspace, workspace_floats,
                            rope ? &p.rope : nullptr, p.chain);

@@ -467,13 +467,13 @@ Stream decode_stream(Runner &r, bool sample_on_device) {
     return s;
 }
 
-// A long prompt runs its projections on the GEMM that loads fp16 weights straight into LDS.  The first such prompt
-// writes the weights once in that layout (about 2 bytes per weight more, kept until the runner goes) instead of every
+// A prompt of some length runs its projections on the GEMM that loads fp16 weights straight into LDS.  The first such
+// prompt writes the weights once in that layout (about 2 bytes per weight more, kept until the runner goes) instead of every
 // call converting them into the workspace - layer by layer while the byte budget lasts; the layers past it convert on
 // every call (same results, 40 us or so per layer and prompt slower).  (finalize()'s warm-up pass runs long prompts
 // when maxSeqLen allows them, so with the warm-up on the copies exist from the start.)
 void ensure_prepared(Runner &r, int n) {
-    if (r.prepared_done || n < 256) return;
+    if (r.prepared_done || n < 64) return;      // (with the copies in place the GEMM takes prompts from 16 rows on where its plan says so)
     r.prepared_done = true;
     const Config &c = r.cfg;
     const int d = c.d;

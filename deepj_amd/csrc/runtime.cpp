@@ -1105,6 +1105,14 @@ void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_ro
     if (k_shares) *k_shares = ks;
 }
 
+void deepj_hip_q8_gemm_tile_prepared(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares) {
+    int tr = 0, tc = 0, ks = 1;
+    if (m > 1 && k > 0 && rows > 0) q8_gemm_f16_tile(m, rows, k, &tr, &tc, &ks, true);
+    if (tile_rows) *tile_rows = tr;
+    if (tile_cols) *tile_cols = tc;
+    if (k_shares) *k_shares = ks;
+}
+
 int32_t deepj_hip_q8_linear_rope_ok(int32_t m, int32_t k, int32_t d) {
     if (m <= 1 || k <= 0 || d <= 0) return 0;
     return q8_gemm_f16_rope_ok(m, d, k) ? 1 : 0;

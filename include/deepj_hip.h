@@ -242,6 +242,9 @@ int32_t deepj_hip_q8_gemm_path(int32_t m, int32_t k, int32_t rows);
 int32_t deepj_hip_q8_linear_rope_ok(int32_t m, int32_t k, int32_t d);
 /* the same with the tile's columns (256 or 192) and the number of workgroups that share a tile's K (1: none) */
 void deepj_hip_q8_gemm_tile(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares);
+/* the same for a weight that Q8_PREPARE has written in the fp16 GEMM's layout: from 16 rows on instead of 256 (64-row tiles,
+ * K shared so that as many workgroups as possible stream weights) */
+void deepj_hip_q8_gemm_tile_prepared(int32_t m, int32_t k, int32_t rows, int32_t *tile_rows, int32_t *tile_cols, int32_t *k_shares);
 /* Host arithmetic only (no GPU call): the last byte + 1 that the fp16 GEMM's direct global -> LDS loads reach in its three
  * operand buffers {activation planes, fp16 weights, transposed scales} for a tile of tile_rows x tile_cols (128 or 64 rows
  * by 256 or 192 columns; tile_rows 0: the tile the library would choose), and the bytes those buffers hold.  Returns 1

@@ -49,7 +49,7 @@ def test_reach_matches_a_lane_by_lane_enumeration(tile):
 
 
 def test_every_load_stays_inside_over_the_shape_space():
-    ms = [256, 257, 300, 319, 320, 384, 448, 511, 512, 513, 1000, 1024, 2048, 4096]
+    ms = [16, 17, 63, 64, 65, 100, 128, 129, 192, 255, 256, 257, 300, 319, 320, 384, 448, 511, 512, 513, 1000, 1024, 2048, 4096]
     ks = [64, 65, 96, 100, 2048, 2080, 4096, 5632, 11008]
     ns = [4, 64, 188, 192, 196, 252, 256, 260, 764, 768, 772, 1536, 2048, 2052, 3072, 4096, 5632, 6144, 11008, 11264, 32000]
     checked = 0

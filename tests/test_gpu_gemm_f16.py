@@ -96,6 +96,65 @@ def test_every_way_the_shares_of_k_are_dealt_to_the_xcds(dev, m, k, n, shares):
     assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"Q8 linear M={m} K={k} N={n}, K shared by {shares}")
 
 
+@pytest.mark.parametrize("m,k,n,tile,epilogue", [
+    (64, 4096, 11008, (64, 192, 4), "bias"),              # a short prompt against a wide projection: four shares of K
+    (16, 2048, 5632, (64, 192, 4), "swiglu"),             # the fewest rows taken; three quarters of a tile's rows are padding
+    (100, 2048, 6144, (64, 192, 4), "rms_bias"),          # ragged rows, the RMSNorm prologue
+    (200, 1000, 11268, (64, 192, 1), "residual"),         # ragged everything, K not shared
+    (255, 5632, 2048, (64, 256, 8), "bias_residual"),     # a narrow output that qualifies through its long K: eight shares
+])
+def test_fewer_than_256_rows_on_prepared_weights(dev, m, k, n, tile, epilogue):
+    """With the weights already in the fp16 GEMM's layout the library takes prompts from 16 rows on, where its plan
+    expects enough workgroups (deepj_hip_q8_gemm_tile_prepared); without them the same shapes stay on the bf16 kernels.
+    Both against the oracle."""
+    swiglu = epilogue == "swiglu"
+    n_rows = 2 * n if swiglu else n
+    assert HipNative.q8GemmTile(m, k, n_rows) == (0, 0, 1)
+    assert HipNative.q8GemmTilePrepared(m, k, n_rows) == tile
+    x = JavaRandom(51).tensor(m, k, 1.0)
+    b = JavaRandom(53).tensor(1, n, 0.3)
+    r = JavaRandom(54).tensor(m, n, 1.0)
+    g = (1.0 + 0.1 * JavaRandom(55).tensor(1, k, 1.0)).astype(np.float32)
+    xb, ob = dev.upload(x), dev.alloc(m * n)
+    kw = {}
+    if swiglu:
+        wg, wu = JavaRandom(52).tensor(k, n, 0.03), JavaRandom(56).tensor(k, n, 0.03)
+        inter = np.empty((k, 2 * n), np.float32)
+        inter[:, 0::2], inter[:, 1::2] = wg, wu
+        wq, deq = quantised(dev, inter)
+        exp = ref.multiply(ref.silu(ref.matmul(x, np.ascontiguousarray(deq[:, 0::2]))), ref.matmul(x, np.ascontiguousarray(deq[:, 1::2])))
+        kw["swiglu"] = True
+    else:
+        wq, deq = quantised(dev, JavaRandom(52).tensor(k, n, 0.03))
+        xin = x
+        if epilogue.startswith("rms"):
+            xin = ref.rmsnorm(x, g)
+            kw["gamma"] = dev.upload(g)
+        exp = ref.matmul(xin, deq)
+        if "bias" in epilogue:
+            exp = ref.add_row_vector(exp, b)
+            kw["bias"] = dev.upload(b)
+        if "residual" in epilogue:
+            exp = ref.add(r, exp)
+            kw["residual"] = dev.upload(r)
+    op = Stream().q8_linear(xb, wq, ob, m, k, n, **kw)
+    op.run()
+    unprepared = dev.download(ob, (m, n))
+    assert_close(exp, unprepared, atol=gate(exp), rtol=1e-4, what=f"bf16 kernels M={m} K={k} N={n} {epilogue}")
+    prep = dev.alloc(HipNative.q8PreparedFloats(k, n_rows))
+    Stream().q8_prepare(wq, prep, k, n_rows).run()
+    counts = HipNative.profileOps(op.array(), 1, detail=True)[2]
+    assert counts[0] == (1 if tile[2] == 1 else 2) + 1        # activation split, GEMM, and the sum of the shares
+    op.run()
+    got = dev.download(ob, (m, n))
+    assert_close(exp, got, atol=gate(exp), rtol=1e-4, what=f"fp16 GEMM on prepared weights M={m} K={k} N={n} {epilogue}")
+    dev.release(xb, ob, wq, prep, *kw_buffers(kw))
+
+
+def kw_buffers(kw):
+    return [v for v in kw.values() if not isinstance(v, bool)]
+
+
 def test_random_shapes_both_tiles_and_shared_k(dev):
     """Seeded random (M, K, N) over the kernel's whole domain - M not a multiple of 64, K not a multiple of 32, N only a
     multiple of 4 - until each of the three ways the library takes a problem (128-row tiles, 64-row tiles, 64-row tiles
