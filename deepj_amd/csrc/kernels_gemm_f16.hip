@@ -380,7 +380,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 constexpr int TM64 = 64;
 constexpr int kXs64 = 2 * TM64 * 64;
 constexpr int stage64_bytes(int tnw) { return kXs64 + 64 * tnw * 64 + 1024; }
-constexpr int kMinSplitSteps = 16;          // K steps a workgroup must at least have when several share a tile's K
+constexpr int kMinSplitSteps = 8;           // K steps a workgroup must at least have when several share a tile's K
 
 template <int TNW, bool ROPE = false>
 __global__ void __launch_bounds__(256) k_gemm_q8_f16_m64(const GemmF16Args a) {
@@ -773,7 +773,6 @@ struct GemmF16Plan { int tile_rows, tile_cols, splits; };
 constexpr int kNPad = 768;      // weight rows of a prepared buffer are padded to a multiple of both tile widths
 
 constexpr int kMinRowsPrepared = 16;     // fewer rows than this stay on the bf16 kernels even with prepared weights
-constexpr int kMinSplitStepsFewRows = 8; // K steps per share below 256 rows (weight streaming counts there, not the tile's fixed cost)
 
 GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k, bool prepared) {
     // DEEPJ_HIP_GEMM_F16=0 keeps every GEMM on the bf16 kernels; =128, =128192, =64 or =192 force the 128 x 256,
@@ -782,22 +781,9 @@ GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k, bool prepared) {
     if (forced == 0) return {0, 0, 1};
     // four columns per lane in the epilogue need n_rows % 4 == 0
     if ((n_rows & 3) != 0 || k < 64) return {0, 0, 1};
-    // Fewer than 256 rows: only when the weights are already in these kernels' layout (a conversion per call costs more
-    // than the launch gains), on 64-row tiles, and only for wide outputs - where the tiles alone, or with a few shares of
-    // K, make enough workgroups to stream the weights (64 rows x 11008 outputs over K 4096: 28.4 us against 46.6 on the
-    // bf16 kernels; 128 x 11264 over K 2048: 27.5 against 47.6; 192 x 6144: 25.8 against 47.8).  Narrow outputs would need
-    // eight shares, whose partial products cost more than they gain (64 x 2048 over K 2048: 16.4 against 11.6), unless K
-    // is long (255 x 2048 over K 5632: 30.1 against 44.5).
-    if (m < 256) {
-        if (!prepared || m < kMinRowsPrepared || forced > 0) return {0, 0, 1};
-        const int64_t r64 = (m + TM64 - 1) / TM64, tw = r64 * ((n_rows + 255) / 256), tn = r64 * ((n_rows + 191) / 192);
-        const int steps = q8_padded_k(k) / 32;
-        if (!(tn >= 48 || (tn >= 40 && steps >= 128))) return {0, 0, 1};
-        auto shares_of = [&](int64_t tiles) { return tiles >= 256 ? 1 : (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(8, 256 / tiles), steps / kMinSplitStepsFewRows)); };
-        const int sw = shares_of(tw), sn = shares_of(tn);
-        const int64_t wgw = std::min<int64_t>(tw * sw, 256), wgn = std::min<int64_t>(tn * sn, 256);
-        return wgn > wgw ? GemmF16Plan{64, 192, sn} : GemmF16Plan{64, 256, sw};
-    }
+    // Fewer than 256 rows: only when the weights are already in these kernels' layout - a conversion per call costs more
+    // than the launch gains.
+    if (m < 256 && (!prepared || m < kMinRowsPrepared || forced > 0)) return {0, 0, 1};
     const int64_t rows128 = (m + TM - 1) / TM, rows64 = (m + TM64 - 1) / TM64, cols256 = (n_rows + 255) / 256, cols192 = (n_rows + 191) / 192;
     const int64_t t128 = rows128 * cols256, t128n = rows128 * cols192, t64 = rows64 * cols256, t64n = rows64 * cols192;
     if (forced == 128 || forced == 128192 || forced == 64 || forced == 192) {
@@ -817,14 +803,19 @@ GemmF16Plan q8_gemm_f16_plan(int m, int n_rows, int k, bool prepared) {
         if (t128 >= 160 && c128 <= c64 && c128 <= c64n) return {128, 256, 1};
         return c64n < c64 ? GemmF16Plan{64, 192, 1} : GemmF16Plan{64, 256, 1};
     }
-    // few tiles but a long K (512 x 2048 output over K 5632: 64 tiles, 71 us on the bf16 kernel, 47 us as 4 x 64
-    // workgroups): several workgroups per tile, each with a share of K of at least kMinSplitSteps steps, their partial
-    // products summed by a second kernel.  (512 x 2048 over K 2048, 64 tiles: four shares of 16 steps, GEMM 18.4 us,
-    // 27.4 with the activation split and the sum, against 30.3 on the bf16 kernel; three shares 29.4, two a tie.)
+    // Few tiles: several workgroups per tile, each with a share of K of at least kMinSplitSteps steps, their partial
+    // products summed by a second kernel - as many workgroups as that allows, on the tile width that gives more of them
+    // (the wider one unless the narrower gives 5 % more).  Worth it when there is enough work to stream: K of 1536 or more
+    // (512 x 2048 over K 1024: 25 us against 17.5 on the bf16 kernels) and 48 narrow tiles or more, or 40 with a long K.  Measured against the bf16 kernels (us, prepared weights): 512 x 2048 over K 5632
+    // 44 / 68; 512 x 2048 over K 2048 29 / 28; 256 x 6144 over K 2048 (two shares) 29 / 49; 320 x 2048 over K 2048 (six
+    // shares) 23 / 26; 64 x 11008 over K 4096 28 / 47; 128 x 11264 over K 2048 27 / 48; 255 x 2048 over K 5632 30 / 45.
+    // Below those bounds the partial products cost more than the launch gains (256 x 2048 over K 2048: 23 / 19; 64 x 2048
+    // over K 2048, eight shares: 16 / 12).
     const int steps = q8_padded_k(k) / 32;
-    const int splits = (int)std::min<int64_t>(std::min<int64_t>(8, 256 / t64), steps / kMinSplitSteps);
-    if (t64 >= 32 && splits >= 3) return {64, 256, splits};
-    return {0, 0, 1};
+    if (steps < 48 || !(t64n >= 48 || (t64n >= 40 && steps >= 128))) return {0, 0, 1};
+    auto shares_of = [&](int64_t tiles) { return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(8, 256 / tiles), steps / kMinSplitSteps)); };
+    const int sw = shares_of(t64), sn = shares_of(t64n);
+    return (double)(t64n * sn) > 1.05 * (double)(t64 * sw) ? GemmF16Plan{64, 192, sn} : GemmF16Plan{64, 256, sw};
 }
 
 int q8_gemm_f16_tile_rows(int m, int n_rows, int k, bool prepared) { return q8_gemm_f16_plan(m, n_rows, k, prepared).tile_rows; }

@@ -49,7 +49,14 @@ def test_path_query_matches_the_documented_rule():
     assert HipNative.q8GemmPath(2048, 4096, 4096) == 128      # 16 x 16
     assert HipNative.q8GemmPath(512, 2048, 6144) == 64        # 96 such tiles would idle most of the chip: 192 of 64 x 256
     assert HipNative.q8GemmPath(512, 2048, 2048) == 64        # 64 even of those: four workgroups share each tile's K
-    assert HipNative.q8GemmPath(512, 1024, 2048) == 0         # ... when K is long enough for shares of 16 steps: else the bf16 kernels
+    assert HipNative.q8GemmPath(512, 1024, 2048) == 0         # ... when K is 1536 or more: else the bf16 kernels
+    assert HipNative.q8GemmTile(256, 2048, 6144) == (64, 192, 2)     # 128 narrow tiles, two shares each: every compute unit
+    assert HipNative.q8GemmTile(320, 2048, 2048) == (64, 256, 6)     # shares of at least eight K steps
+    assert HipNative.q8GemmTile(256, 2048, 2048) == (0, 0, 1)        # too little to stream for eight shares' partial products
+    assert HipNative.q8GemmTile(128, 2048, 11264) == (0, 0, 1)       # fewer than 256 rows: not without prepared weights
+    assert HipNative.q8GemmTilePrepared(128, 2048, 11264) == (64, 192, 2)
+    assert HipNative.q8GemmTilePrepared(15, 2048, 11264) == (0, 0, 1)
+    assert HipNative.q8GemmTilePrepared(64, 2048, 2048) == (0, 0, 1)
     assert HipNative.q8GemmPath(512, 5632, 2048) == 64        # the same 64 tiles over a long K: four workgroups share each
     assert HipNative.q8GemmTile(512, 5632, 2048) == (64, 256, 4)
     assert HipNative.q8GemmTile(512, 2048, 6144) == (64, 192, 1)     # 256 tiles: one per compute unit
@@ -287,10 +294,9 @@ def test_swiglu_and_norm_prologues(dev, norm, dff, tile):
 
 def test_swiglu_on_partial_products_of_a_shared_k(dev):
     """A few-tile gate/up projection over a long K runs as several workgroups per tile; the kernel that adds their
-    partial products applies the interleaved biases and the SwiGLU pairing (a DeepSeek block at 256 rows has this
-    shape)."""
-    m, d, dff = 256, 2048, 1024
-    assert HipNative.q8GemmTile(m, d, 2 * dff) == (64, 256, 4)
+    partial products applies the interleaved biases and the SwiGLU pairing."""
+    m, d, dff = 320, 2048, 1024
+    assert HipNative.q8GemmTile(m, d, 2 * dff) == (64, 256, 6)
     x = JavaRandom(51).tensor(m, d, 1.0)
     gamma = (1.0 + JavaRandom(52).tensor(1, d, 0.1)).astype(np.float32)
     wg, wu = JavaRandom(53).tensor(d, dff, 0.03), JavaRandom(54).tensor(d, dff, 0.03)
