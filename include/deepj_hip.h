@@ -56,8 +56,8 @@ int deepj_hip_flush_ops(const int32_t *cmd, int32_t len);
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same streams and
  * the same kernels and bits as deepj_hip_flush_ops, with ONE exception: a Q8_LINEAR of more than one row always
  * runs as a single launch of the bf16 GEMM here, where flush_ops - with a workspace sized by the shape - takes
- * the fp16 GEMM (256 rows and more, enough tiles) or lets several workgroups share a tile's K (few tiles, long K),
- * prepared weights or not; both meet the per-op tolerance against the CPU backend, their bits differ.  The
+ * the fp16 GEMM (256 rows and more - 16 and more with prepared weights - and enough tiles) or lets several workgroups
+ * share a tile's K (few tiles, long K); both meet the per-op tolerance against the CPU backend, their bits differ.  The
  * device scratch the kernels need - the workspace that Q8_LINEAR with a norm
  * prologue and M > 1 writes its normalised rows to, and the arrival counters of the split decode attention
  * (ATTENTION / ATTENTION_KV with S = 1, ATTN_DECODE) - is a fixed array inside the library's code object instead
@@ -286,9 +286,10 @@ int deepj_runner_init_seeded(void *runner, int64_t seed, int32_t threads);  /* n
 /* new GPTModel(cfg, seed) with GPTConfig.initScale = init_scale (J/models/gpt/GPTModel.java:27-46,76-81) */
 int deepj_runner_init_seeded_gpt(void *runner, int64_t seed, float init_scale, int32_t threads);
 /* Bytes a runner may spend on fp16 copies of its weights for the many-row (prompt) GEMM, which reads them in that
- * form: -1 (default) no limit - a copy of every layer, written at the first prompt of 256 rows or more (+ 2 bytes
+ * form: -1 (default) no limit - a copy of every layer, written at the first prompt of 64 rows or more (+ 2 bytes
  * per weight); 0 none - every call converts into the workspace; otherwise layers in order while the budget lasts.
- * Results are bit-identical whatever the budget.  deepj_runner_prepared_bytes: what the copies take now. */
+ * Prompts of 256 rows and more give the same bits whatever the budget; shorter ones take the fp16 GEMM only where a
+ * copy exists (the bf16 kernels otherwise: same tolerance, other last bits).  deepj_runner_prepared_bytes: what the copies take now. */
 int deepj_runner_set_prepared_budget(void *runner, int64_t bytes);
 int64_t deepj_runner_prepared_bytes(void *runner);
 int deepj_runner_finalize(void *runner);

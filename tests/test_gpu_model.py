@@ -370,3 +370,41 @@ def test_generate_slides_the_window_past_max_seq_len():
             assert np.array_equal(got, exp), cls.__name__
         finally:
             gpu.close(); cpu.close()
+
+
+def test_short_and_chunked_prompts_on_prepared_weights_against_the_oracle():
+    """With prepared (fp16) copies of the weights the prompt GEMM takes prompts from 16 rows on where the projection is
+    wide enough - here q | k | v and gate/up of a d = 2048 model - and the bf16 kernels take the rest.  A 200-token
+    prompt in one piece, the same prompt as chunks of 128 + 40 + 17 + 15 rows, and the one-piece prompt with no copies
+    at all (every GEMM below 256 rows on the bf16 kernels) against the oracle's forward: same logits within the gate,
+    same next tokens."""
+    cfg = LlamaConfig(vocabSize=512, maxSeqLen=256, dModel=2048, nHeads=16, nLayers=2, dFF=5632)
+    assert HipNative.q8GemmTilePrepared(128, 2048, 3 * 2048)[0] == 64 and HipNative.q8GemmTile(128, 2048, 3 * 2048)[0] == 0
+    assert HipNative.q8GemmTilePrepared(40, 2048, 2 * 5632)[0] == 64 and HipNative.q8GemmTilePrepared(15, 2048, 2 * 5632)[0] == 0
+    ref.set_threads(ref.default_threads())
+    gpu, cpu = LlamaModel(cfg, 42), oracle_model(cfg, 42)
+    try:
+        prompt = ref.JavaRandom(9).ints(200, 512)
+        exp = cpu.forward(prompt)
+        assert gpu.preparedBytes() > 0                          # the warm-up pass left the copies
+        whole = gpu.forward(prompt)
+        gpu.reset()
+        pos = 0
+        for n in (128, 40, 17, 15):
+            gpu.prefill(prompt[pos:pos + n], choose_next=False)
+            pos += n
+        chunked_last = gpu.lastLogits()
+        gpu.setPreparedBudget(0)                                # no copies: the bf16 kernels for every short GEMM
+        assert gpu.preparedBytes() == 0
+        plain = gpu.forward(prompt)
+        assert gpu.preparedBytes() == 0
+        for name, got in (("prepared", whole), ("no copies", plain)):
+            err = float(np.max(np.abs(got - exp)))
+            print(f"\n[d2048 L2, 200-token prompt, {name}] logits max-abs error {err:.2e}")
+            assert err <= 1e-3, (name, err)
+            assert np.array_equal(np.argmax(got, axis=1), np.argmax(exp, axis=1)), name
+        assert float(np.max(np.abs(chunked_last - exp[-1]))) <= 1e-3
+        assert int(np.argmax(chunked_last)) == int(np.argmax(exp[-1]))
+    finally:
+        gpu.close()
+        ref.set_threads(1)
