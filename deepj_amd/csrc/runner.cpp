@@ -480,7 +480,9 @@ void ensure_prepared(Runner &r, int n) {
     Stream s;
     bool room = true;
     auto prepare = [&](int32_t w, int k, int rows) {
-        if (!room || w < 0 || !deepj_hip_q8_gemm_path(c.max_seq, k, rows)) return;
+        int32_t tile_rows = 0;      // would the longest prompt reach the fp16 GEMM with a copy in place?
+        deepj_hip_q8_gemm_tile_prepared(c.max_seq, k, rows, &tile_rows, nullptr, nullptr);
+        if (!room || w < 0 || !tile_rows) return;
         const int64_t floats = deepj_hip_q8_prepared_floats(k, rows);
         if (r.prepared_budget >= 0 && r.prepared_bytes + 4 * floats > r.prepared_budget) { room = false; return; }
         int32_t p = r.alloc(floats);
